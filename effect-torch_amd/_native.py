@@ -1,0 +1,96 @@
+"""ctypes binding of ``lib/libet_hip.so`` (the C ABI declared in ``include/et_hip.h``).
+
+The library is loaded from inside the package directory only. There is no CPU
+fallback: if the shared object is missing this module raises on import of
+``lib()``, and every operator fails loudly without it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libet_hip.so")
+
+# et_status
+OK, ERR_UNSUPPORTED, ERR_EXECUTION, ERR_CANCELLED, ERR_UNAVAILABLE, ERR_INVALID = range(6)
+# et_dtype
+DTYPE_F32, DTYPE_F64, DTYPE_F16, DTYPE_BF16, DTYPE_U8, DTYPE_U32, DTYPE_I64 = range(7)
+# et_activation_mode
+ACT_F32, ACT_INT8 = 0, 1
+STATUS_BYTES = 16
+
+
+class EtTensor(ctypes.Structure):
+    """``et_tensor`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("dtype", ctypes.c_int32),
+        ("rank", ctypes.c_int32),
+        ("shape", ctypes.POINTER(ctypes.c_uint64)),
+        ("strides", ctypes.POINTER(ctypes.c_uint64)),
+        ("offset", ctypes.c_uint64),
+    ]
+
+
+# Every symbol include/et_hip.h declares: name -> (restype, argtypes).
+_vp, _u64, _i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32
+_T = ctypes.POINTER(EtTensor)
+_PP = ctypes.POINTER(ctypes.c_void_p)
+SIGNATURES = {
+    "et_hip_is_available": (ctypes.c_int, []),
+    "et_hip_codec_name": (ctypes.c_char_p, [_i32]),
+    "et_hip_block_values": (_u64, [_i32]),
+    "et_hip_block_bytes": (_u64, [_i32]),
+    "et_hip_encoded_row_bytes": (_u64, [_i32, _u64]),
+    "et_hip_linear_requirements": (ctypes.c_int, [_T, _T, _T, _i32, _u64, _u64, _i32, _PP]),
+    "et_hip_linear_plan_destroy": (None, [_vp]),
+    "et_hip_linear_plan_output_rank": (_i32, [_vp]),
+    "et_hip_linear_plan_output_shape": (None, [_vp, ctypes.POINTER(_u64)]),
+    "et_hip_linear_plan_vectors": (_u64, [_vp]),
+    "et_hip_linear_plan_output_bytes": (_u64, [_vp]),
+    "et_hip_linear_plan_workspace_bytes": (_u64, [_vp]),
+    "et_hip_linear_plan_kernel": (ctypes.c_char_p, [_vp]),
+    "et_hip_linear_plan_algorithmic_bytes": (_u64, [_vp]),
+    "et_hip_linear_into": (ctypes.c_int, [_vp, _T, _T, _T, _T, _vp, _u64, _vp, _vp]),
+    "et_hip_linear_plan_create": (ctypes.c_int, [_i32, _u64, _u64, _u64, _i32, _i32, _PP]),
+    "et_hip_linear_enqueue": (ctypes.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
+    "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
+    "et_hip_embedding_plan_destroy": (None, [_vp]),
+    "et_hip_embedding_plan_output_rank": (_i32, [_vp]),
+    "et_hip_embedding_plan_output_shape": (None, [_vp, ctypes.POINTER(_u64)]),
+    "et_hip_embedding_plan_output_bytes": (_u64, [_vp]),
+    "et_hip_embedding_into": (ctypes.c_int, [_vp, _T, _T, _T, _vp, _vp, _vp]),
+    "et_hip_embedding_status_check": (ctypes.c_int, [_vp, _vp]),
+    "et_hip_dequantize_rows": (ctypes.c_int, [_i32, _u64, _u64, _vp, _vp, _vp]),
+    "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
+    "et_hip_last_error": (ctypes.c_char_p, []),
+}
+
+_lib = None
+
+
+class NativeLibraryMissing(ImportError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """Loads the built HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise NativeLibraryMissing(
+                f"{LIB_PATH} is missing: build it with `python effect-torch_amd/build.py` "
+                "(there is no fallback implementation)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().et_hip_last_error().decode()

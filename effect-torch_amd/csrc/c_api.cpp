@@ -1,0 +1,303 @@
+// extern "C" surface of libet_hip.so (declared in include/et_hip.h). Thin
+// wrappers: convert descriptors, catch every C++ exception, keep the last
+// error message per thread.
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <exception>
+#include <new>
+#include <string>
+
+#include "et_codecs.h"
+#include "et_hip.h"
+#include "kernels.h"
+#include "quantized.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int set_error(int status, const std::string& message) {
+    g_last_error = message;
+    return status;
+}
+
+template <class F>
+int guarded(F&& body) {
+    try {
+        std::string error;
+        const int status = body(&error);
+        if (status != ET_OK) g_last_error = error;
+        return status;
+    } catch (const std::bad_alloc&) {
+        return set_error(ET_ERR_EXECUTION, "out of host memory");
+    } catch (const std::exception& e) {
+        return set_error(ET_ERR_EXECUTION, e.what());
+    } catch (...) {
+        return set_error(ET_ERR_EXECUTION, "unknown C++ exception");
+    }
+}
+
+using et::quantized::TensorView;
+
+}  // namespace
+
+extern "C" {
+
+int et_hip_is_available(void) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    hipDeviceProp_t props;
+    if (hipGetDeviceProperties(&props, device) != hipSuccess) return 0;
+    return std::strncmp(props.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+}
+
+const char* et_hip_codec_name(int32_t codec) { return et::codec_name(codec); }
+uint64_t et_hip_block_values(int32_t codec) { return et::block_values(codec); }
+uint64_t et_hip_block_bytes(int32_t codec) { return et::block_bytes(codec); }
+
+uint64_t et_hip_encoded_row_bytes(int32_t codec, uint64_t columns) {
+    const uint64_t values = et::block_values(codec);
+    if (values == 0 || columns % values != 0) return 0;
+    const uint64_t blocks = columns / values;
+    const uint64_t bytes = et::block_bytes(codec);
+    if (blocks != 0 && bytes > UINT64_MAX / blocks) return 0;
+    return blocks * bytes;
+}
+
+int et_hip_linear_requirements(const et_tensor* input, const et_tensor* weight, const et_tensor* bias,
+                               int32_t codec, uint64_t rows, uint64_t columns,
+                               int32_t activation_mode, et_linear_plan** out) {
+    return guarded([&](std::string* error) -> int {
+        if (out == nullptr) {
+            *error = "quantized_linear: output plan pointer is NULL";
+            return ET_ERR_INVALID;
+        }
+        *out = nullptr;
+        TensorView in, w, b;
+        if (!TensorView::from_c(input, &in, error) || !TensorView::from_c(weight, &w, error) ||
+            (bias != nullptr && !TensorView::from_c(bias, &b, error))) {
+            *error = "quantized_linear: " + *error;
+            return ET_ERR_INVALID;
+        }
+        auto* plan = new et_linear_plan();
+        const int status = et::quantized::linear_requirements(in, w, bias ? &b : nullptr, codec, rows,
+                                                              columns, activation_mode, plan, error);
+        if (status != ET_OK) {
+            delete plan;
+            return status;
+        }
+        *out = plan;
+        return ET_OK;
+    });
+}
+
+int et_hip_linear_plan_create(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
+                              int32_t has_bias, int32_t activation_mode, et_linear_plan** out) {
+    return guarded([&](std::string* error) -> int {
+        if (out == nullptr) {
+            *error = "quantized_linear: output plan pointer is NULL";
+            return ET_ERR_INVALID;
+        }
+        *out = nullptr;
+        auto* plan = new et_linear_plan();
+        const int status = et::quantized::linear_plan_from_sizes(codec, rows, columns, vectors,
+                                                                 has_bias != 0, activation_mode, plan,
+                                                                 error);
+        if (status != ET_OK) {
+            delete plan;
+            return status;
+        }
+        *out = plan;
+        return ET_OK;
+    });
+}
+
+void et_hip_linear_plan_destroy(et_linear_plan* plan) { delete plan; }
+
+int32_t et_hip_linear_plan_output_rank(const et_linear_plan* plan) {
+    return plan ? static_cast<int32_t>(plan->output_shape.size()) : 0;
+}
+void et_hip_linear_plan_output_shape(const et_linear_plan* plan, uint64_t* shape) {
+    if (plan == nullptr || shape == nullptr) return;
+    for (size_t d = 0; d < plan->output_shape.size(); d++) shape[d] = plan->output_shape[d];
+}
+uint64_t et_hip_linear_plan_vectors(const et_linear_plan* plan) { return plan ? plan->vectors : 0; }
+uint64_t et_hip_linear_plan_output_bytes(const et_linear_plan* plan) {
+    return plan ? plan->output_bytes : 0;
+}
+uint64_t et_hip_linear_plan_workspace_bytes(const et_linear_plan* plan) {
+    return plan ? plan->workspace_bytes : 0;
+}
+const char* et_hip_linear_plan_kernel(const et_linear_plan* plan) {
+    return plan ? et::quantized::kernel_name(*plan) : "";
+}
+uint64_t et_hip_linear_plan_algorithmic_bytes(const et_linear_plan* plan) {
+    if (plan == nullptr) return 0;
+    return plan->rows * plan->encoded_row_bytes + 4 * plan->vectors * plan->columns +
+           4 * plan->vectors * plan->rows + (plan->has_bias ? 4 * plan->rows : 0);
+}
+
+int et_hip_linear_into(const et_linear_plan* plan, const et_tensor* input, const et_tensor* weight,
+                       const et_tensor* bias, const et_tensor* destination, void* workspace,
+                       uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        TensorView in, w, b, dst;
+        if (!TensorView::from_c(input, &in, error) || !TensorView::from_c(weight, &w, error) ||
+            (bias != nullptr && !TensorView::from_c(bias, &b, error)) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "quantized_linear: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_into(*plan, in, w, bias ? &b : nullptr, dst, workspace,
+                                          workspace_bytes, stream, cancel, error);
+    });
+}
+
+int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
+                          const uint8_t* weight, const float* bias, float* y, void* workspace,
+                          uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_enqueue(*plan, x, x_row_stride, weight, bias, y, workspace,
+                                             workspace_bytes, stream, cancel, error);
+    });
+}
+
+int et_hip_embedding_requirements(const et_tensor* indexes, const et_tensor* weight, int32_t codec,
+                                  uint64_t rows, uint64_t columns, et_embedding_plan** out) {
+    return guarded([&](std::string* error) -> int {
+        if (out == nullptr) {
+            *error = "quantized_embedding: output plan pointer is NULL";
+            return ET_ERR_INVALID;
+        }
+        *out = nullptr;
+        TensorView idx, w;
+        if (!TensorView::from_c(indexes, &idx, error) || !TensorView::from_c(weight, &w, error)) {
+            *error = "quantized_embedding: " + *error;
+            return ET_ERR_INVALID;
+        }
+        auto* plan = new et_embedding_plan();
+        const int status =
+            et::quantized::embedding_requirements(idx, w, codec, rows, columns, plan, error);
+        if (status != ET_OK) {
+            delete plan;
+            return status;
+        }
+        *out = plan;
+        return ET_OK;
+    });
+}
+
+void et_hip_embedding_plan_destroy(et_embedding_plan* plan) { delete plan; }
+int32_t et_hip_embedding_plan_output_rank(const et_embedding_plan* plan) {
+    return plan ? static_cast<int32_t>(plan->output_shape.size()) : 0;
+}
+void et_hip_embedding_plan_output_shape(const et_embedding_plan* plan, uint64_t* shape) {
+    if (plan == nullptr || shape == nullptr) return;
+    for (size_t d = 0; d < plan->output_shape.size(); d++) shape[d] = plan->output_shape[d];
+}
+uint64_t et_hip_embedding_plan_output_bytes(const et_embedding_plan* plan) {
+    return plan ? plan->output_bytes : 0;
+}
+
+int et_hip_embedding_into(const et_embedding_plan* plan, const et_tensor* indexes,
+                          const et_tensor* weight, const et_tensor* destination, void* status,
+                          void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_embedding: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        TensorView idx, w, dst;
+        if (!TensorView::from_c(indexes, &idx, error) || !TensorView::from_c(weight, &w, error) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "quantized_embedding: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::embedding_into(*plan, idx, w, dst, status, stream, cancel, error);
+    });
+}
+
+int et_hip_embedding_status_check(const et_embedding_plan* plan, const void* status_host) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr || status_host == nullptr) {
+            *error = "quantized_embedding: plan or status is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::embedding_status_check(*plan, status_host, error);
+    });
+}
+
+int et_hip_dequantize_rows(int32_t codec, uint64_t rows, uint64_t columns, const uint8_t* weight,
+                           float* out, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        const char* name = et::codec_name(codec);
+        if (name == nullptr) {
+            *error = "dequantize_rows: unknown codec " + std::to_string(codec);
+            return ET_ERR_INVALID;
+        }
+        if (et_hip_encoded_row_bytes(codec, columns) == 0 && columns != 0) {
+            *error = "dequantize_rows: logical row width " + std::to_string(columns) +
+                     " is invalid for " + name;
+            return ET_ERR_UNSUPPORTED;
+        }
+        if (rows == 0 || columns == 0) return ET_OK;
+        if (weight == nullptr || out == nullptr || reinterpret_cast<uintptr_t>(out) % 16 != 0) {
+            *error = "dequantize_rows: operands must be non-NULL and the output 16-byte aligned";
+            return ET_ERR_INVALID;
+        }
+        et::IndexLayout layout;
+        std::memset(&layout, 0, sizeof layout);
+        layout.contiguous = 1;
+        const hipError_t status = et::dequantize_rows(codec, weight, nullptr, 0, layout, rows, rows,
+                                                      columns, out, nullptr,
+                                                      static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("dequantize_rows: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
+int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (columns % 32 != 0) {
+            *error = "quantize_activations: columns must be a multiple of 32";
+            return ET_ERR_UNSUPPORTED;
+        }
+        if (vectors == 0 || columns == 0) return ET_OK;
+        if (x == nullptr || q == nullptr || scale == nullptr ||
+            reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_row_stride % 4 != 0 ||
+            reinterpret_cast<uintptr_t>(q) % 4 != 0) {
+            *error = "quantize_activations: operands must be non-NULL and 16-byte aligned";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status = et::quantize_activations(x, x_row_stride, vectors, columns, q, scale,
+                                                           sum, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("quantize_activations: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
+const char* et_hip_last_error(void) { return g_last_error.c_str(); }
+
+}  // extern "C"

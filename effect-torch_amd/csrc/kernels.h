@@ -1,0 +1,62 @@
+// Launchers of the gfx950 kernels. Host-callable; every function enqueues on
+// `stream` and returns the launch status without synchronising.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+
+namespace et {
+
+constexpr int kMaxRank = 8;
+
+// Strided view of an index (or input) tensor, passed to kernels by value.
+struct IndexLayout {
+    int32_t rank;
+    int32_t contiguous;
+    uint64_t offset;
+    uint64_t shape[kMaxRank];
+    uint64_t strides[kMaxRank];
+};
+
+// ---- dequant.hip -----------------------------------------------------------
+// out[p, :] = decode(W[index[p], :]); indexes == nullptr decodes rows 0..out_rows.
+hipError_t dequantize_rows(int32_t codec, const uint8_t* weight, const void* indexes,
+                           int index_is_i64, const IndexLayout& layout, uint64_t out_rows,
+                           uint64_t table_rows, uint64_t columns, float* out, void* status,
+                           hipStream_t stream);
+
+// ---- gemv_generic.hip (gather) ------------------------------------------------
+// dst[i] = src[source_index(layout, i)] for i < count (f32): densifies a
+// strided activation view into the workspace.
+hipError_t gather_f32(const float* src, const IndexLayout& layout, uint64_t count, float* dst,
+                      hipStream_t stream);
+
+// ---- gemv_fast.hip: activation-stationary dequant-GEMV (Q4_K, Q4_0, Q8_0) ----
+// y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r]) for v < vectors.
+// x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
+uint32_t gemv_fast_max_vectors(int32_t codec);
+bool gemv_fast_supported(int32_t codec, uint64_t columns, uint32_t vectors);
+hipError_t gemv_fast(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                     const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
+                     hipStream_t stream);
+
+// ---- gemv_generic.hip: every codec, any whole number of blocks, vectors <= 4 ----
+constexpr uint32_t kGemvGenericMaxVectors = 4;
+hipError_t gemv_generic(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                        const float* bias, float* y, uint64_t rows, uint64_t columns,
+                        uint32_t vectors, hipStream_t stream);
+
+// ---- quantize_act.hip --------------------------------------------------------
+// q [vectors, columns] int8; scale and sum TRANSPOSED: [columns/32, round_up(vectors, 32)].
+hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                hipStream_t stream);
+
+// ---- gemm_i8.hip: int8-activation MFMA contraction ---------------------------
+bool gemm_i8_supported(int32_t codec, uint64_t columns);
+hipError_t gemm_i8(int32_t codec, const uint8_t* weight, const int8_t* q, const float* scale,
+                   const int32_t* sum, const float* bias, float* y, uint64_t rows,
+                   uint64_t columns, uint64_t vectors, hipStream_t stream);
+
+}  // namespace et

@@ -1,0 +1,97 @@
+// int8 activation quantiser: stage 1 of the int8-activation path.
+//
+// For each vector v and each 32-column block b:
+//     amax  = max |x|                      scale[b, v] = amax / 127
+//     inv   = amax > 0 ? 127 / amax : 0    q = clamp(rint(x * inv), -127, 127)
+//     sum[b, v] = sum of q (int32)
+// Both divisions are IEEE-correct and rint rounds to nearest even, so the
+// integers and scales are bit-identical to a CPU evaluation of the same
+// formulas. The reference has no int8 activation path; these semantics are
+// this library's own.
+//
+// Layout: q is [vectors, columns] int8 (row-major, what the MFMA operand loads
+// want); scale and sum are stored TRANSPOSED, [columns/32, stride] with
+// stride = vectors rounded up to a multiple of 32, so that the GEMM epilogue
+// reads the scales of four consecutive vectors with one 16-byte load and a
+// 32-vector tile never reads past the array. Entries at m >= vectors are
+// never written and never influence a stored output.
+//
+// Eight lanes share a block: each loads one float4, the absmax and the sum are
+// folded across the eight with DPP, each lane packs its four int8 into a dword.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "kernels.h"
+
+namespace et {
+namespace {
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x,
+                                                       uint64_t x_row_stride, uint32_t vectors,
+                                                       uint32_t columns, int8_t* __restrict__ q,
+                                                       float* __restrict__ scale,
+                                                       int32_t* __restrict__ sum) {
+    const uint32_t quads_per_row = columns >> 2;
+    const uint64_t total = static_cast<uint64_t>(vectors) * quads_per_row;  // multiple of 8
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+    for (uint64_t item = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
+         item += stride) {
+        const uint32_t v = static_cast<uint32_t>(item / quads_per_row);
+        const uint32_t quad = static_cast<uint32_t>(item - static_cast<uint64_t>(v) * quads_per_row);
+        const float4 in = *reinterpret_cast<const float4*>(x + v * x_row_stride + 4u * quad);
+        float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
+        amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
+        amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
+        amax = fmaxf(amax, dpp_f32<0x141>(amax));  // row_half_mirror: the other quad of the 8
+        const float inv = amax > 0.f ? 127.f / amax : 0.f;
+        int qi[4];
+        const float values[4] = {in.x, in.y, in.z, in.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float r = rintf(values[i] * inv);
+            r = fminf(fmaxf(r, -127.f), 127.f);
+            qi[i] = static_cast<int>(r);
+        }
+        int total_q = (qi[0] + qi[1]) + (qi[2] + qi[3]);
+        total_q += dpp_i32<0xB1>(total_q);
+        total_q += dpp_i32<0x4E>(total_q);
+        total_q += dpp_i32<0x141>(total_q);
+        const uint32_t packed = (static_cast<uint32_t>(qi[0]) & 0xffu) |
+                                ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
+                                ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
+                                ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
+        reinterpret_cast<uint32_t*>(q)[static_cast<uint64_t>(v) * quads_per_row + quad] = packed;
+        if ((quad & 7u) == 0) {
+            const uint64_t slot = static_cast<uint64_t>(quad >> 3) * ((vectors + 31u) & ~31u) + v;
+            scale[slot] = amax / 127.f;
+            if (sum != nullptr) sum[slot] = total_q;
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                hipStream_t stream) {
+    const uint64_t total = vectors * (columns >> 2);
+    if (total == 0) return hipSuccess;
+    uint64_t blocks = (total + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(quantize_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream, x,
+                       x_row_stride, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
+                       scale, sum);
+    return hipGetLastError();
+}
+
+}  // namespace et

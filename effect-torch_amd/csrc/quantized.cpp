@@ -1,0 +1,550 @@
+// Host side of the quantized operators (plan + execute). See quantized.h.
+#include "quantized.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <limits>
+#include <sstream>
+
+#include "et_codecs.h"
+#include "kernels.h"
+
+namespace et {
+namespace quantized {
+namespace {
+
+constexpr uint64_t kMax = std::numeric_limits<uint64_t>::max();
+
+bool checked_mul(uint64_t a, uint64_t b, uint64_t* out) {
+    if (a != 0 && b > kMax / a) return false;
+    *out = a * b;
+    return true;
+}
+
+// checked_product, crates/runtime-cpu/src/quantized.rs:44-49
+bool checked_product(const std::vector<uint64_t>& values, uint64_t* out) {
+    uint64_t total = 1;
+    for (uint64_t value : values)
+        if (!checked_mul(total, value, &total)) return false;
+    *out = total;
+    return true;
+}
+
+const char* dtype_name(int32_t dtype) {  // DType::name, crates/runtime/src/dtype.rs:38-48
+    switch (dtype) {
+        case ET_DTYPE_F32: return "f32";
+        case ET_DTYPE_F64: return "f64";
+        case ET_DTYPE_F16: return "f16";
+        case ET_DTYPE_BF16: return "bf16";
+        case ET_DTYPE_U8: return "u8";
+        case ET_DTYPE_U32: return "u32";
+        case ET_DTYPE_I64: return "i64";
+        default: return "?";
+    }
+}
+
+// Rust's `{:?}` of a slice of integers: "[2, 512]".
+std::string debug_shape(const std::vector<uint64_t>& shape) {
+    std::ostringstream out;
+    out << "[";
+    for (size_t i = 0; i < shape.size(); i++) out << (i ? ", " : "") << shape[i];
+    out << "]";
+    return out.str();
+}
+
+int fail(std::string* error, int status, const std::string& message) {
+    if (error != nullptr) *error = message;
+    return status;
+}
+
+uint64_t align_up(uint64_t value, uint64_t alignment) {
+    return (value + alignment - 1) / alignment * alignment;
+}
+
+// GgmlKQuant::encoded_row_bytes (crates/runtime/src/gguf.rs:245-250): false = None.
+bool encoded_row_bytes(int32_t codec, uint64_t columns, uint64_t* out) {
+    const uint64_t values = block_values(codec);
+    if (values == 0 || columns % values != 0) return false;
+    return checked_mul(columns / values, block_bytes(codec), out);
+}
+
+// validate_weight, crates/runtime-cpu/src/quantized.rs:266-292
+int validate_weight(const char* operation, const TensorView& weight, int32_t codec, uint64_t rows,
+                    uint64_t columns, uint64_t* row_bytes, std::string* error) {
+    const char* name = codec_name(codec);
+    if (name == nullptr)
+        return fail(error, ET_ERR_INVALID,
+                    std::string(operation) + ": unknown codec " + std::to_string(codec));
+    if (!encoded_row_bytes(codec, columns, row_bytes))
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    std::string(operation) + ": logical row width " + std::to_string(columns) +
+                        " is invalid for " + name);
+    uint64_t total;
+    if (!checked_mul(rows, *row_bytes, &total))
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    std::string(operation) + ": packed weight byte size overflow");
+    if (weight.dtype != ET_DTYPE_U8 || weight.shape.size() != 2 || weight.shape[0] != rows ||
+        weight.shape[1] != *row_bytes || !weight.is_contiguous() || weight.offset != 0)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    std::string(operation) + ": expected exact contiguous packed " + name +
+                        " weight [" + std::to_string(rows) + ", " + std::to_string(*row_bytes) +
+                        "] u8");
+    return ET_OK;
+}
+
+// Chooses the kernel for (codec, columns, vectors, mode) and lays out the workspace.
+// cf. linear_kernel_kind, crates/runtime-metal/src/quantized.rs:1204-1220.
+int select_kernel(et_linear_plan* plan, std::string* error) {
+    plan->gather_offset = plan->gather_bytes = 0;
+    plan->q_offset = plan->scale_offset = plan->sum_offset = plan->bias_offset = 0;
+    plan->workspace_bytes = 0;
+    plan->vectors_per_launch = 0;
+    if (plan->vectors == 0 || plan->rows == 0) {
+        plan->kernel = LinearKernel::kNone;
+        return ET_OK;
+    }
+    if (plan->rows > 0xffffffffull || plan->columns > 0xffffffffull || plan->vectors > 0xffffffffull)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "quantized_linear: rows, columns and vectors must each fit 32 bits");
+    uint64_t cursor = 0;
+    // Space to densify a strided or misaligned f32 input.
+    plan->gather_offset = 0;
+    plan->gather_bytes = plan->vectors * plan->columns * 4u;
+    cursor = align_up(plan->gather_bytes, 256);
+    plan->bias_offset = cursor;  // dense copy of a strided bias
+    cursor = align_up(cursor + plan->rows * 4u, 256);
+    if (plan->activation_mode == ET_ACT_INT8) {
+        if (!gemm_i8_supported(plan->codec, plan->columns))
+            return fail(error, ET_ERR_UNSUPPORTED,
+                        std::string("quantized_linear: int8 activation mode is not available for ") +
+                            codec_name(plan->codec));
+        plan->kernel = LinearKernel::kGemmI8;
+        plan->q_offset = cursor;
+        cursor = align_up(cursor + plan->vectors * plan->columns, 256);
+        plan->scale_offset = cursor;
+        const uint64_t padded_vectors = align_up(plan->vectors, 32);  // [columns/32, padded] tables
+        cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
+        plan->sum_offset = cursor;
+        cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
+    } else if (plan->activation_mode == ET_ACT_F32) {
+        const uint32_t fast_max = gemv_fast_max_vectors(plan->codec);
+        const uint32_t per_launch =
+            static_cast<uint32_t>(plan->vectors < fast_max ? plan->vectors : fast_max);
+        if (fast_max != 0 && gemv_fast_supported(plan->codec, plan->columns, per_launch)) {
+            plan->kernel = LinearKernel::kGemvFast;
+            plan->vectors_per_launch = per_launch;
+        } else {
+            plan->kernel = LinearKernel::kGemvGeneric;
+            plan->vectors_per_launch = kGemvGenericMaxVectors;
+        }
+    } else {
+        return fail(error, ET_ERR_INVALID, "quantized_linear: unknown activation mode " +
+                                               std::to_string(plan->activation_mode));
+    }
+    plan->workspace_bytes = cursor;
+    return ET_OK;
+}
+
+hipStream_t as_stream(void* stream) { return static_cast<hipStream_t>(stream); }
+
+int hip_failure(std::string* error, const char* operation, hipError_t status) {
+    return fail(error, ET_ERR_EXECUTION,
+                std::string(operation) + ": HIP error: " + hipGetErrorString(status));
+}
+
+bool cancelled(const volatile int32_t* cancel) { return cancel != nullptr && *cancel != 0; }
+
+// A view is "row-dense" when it can be read as [vectors, columns] with unit
+// trailing stride and one common stride between consecutive vectors.
+bool row_dense(const TensorView& input, uint64_t* row_stride) {
+    const size_t rank = input.shape.size();
+    const uint64_t columns = input.shape[rank - 1];
+    if (columns > 1 && input.strides[rank - 1] != 1) return false;
+    bool have = false;
+    uint64_t stride = columns, expected = 0;
+    for (size_t d = rank - 1; d-- > 0;) {
+        if (input.shape[d] == 1) continue;
+        if (!have) {
+            have = true;
+            stride = input.strides[d];
+            if (!checked_mul(stride, input.shape[d], &expected)) return false;
+        } else {
+            if (input.strides[d] != expected) return false;
+            if (!checked_mul(expected, input.shape[d], &expected)) return false;
+        }
+    }
+    *row_stride = stride;
+    return true;
+}
+
+IndexLayout make_layout(const TensorView& view) {
+    IndexLayout layout;
+    std::memset(&layout, 0, sizeof layout);
+    layout.rank = static_cast<int32_t>(view.shape.size());
+    layout.contiguous = view.is_contiguous() ? 1 : 0;
+    layout.offset = view.offset;
+    for (size_t d = 0; d < view.shape.size(); d++) {
+        layout.shape[d] = view.shape[d];
+        layout.strides[d] = view.strides[d];
+    }
+    return layout;
+}
+
+}  // namespace
+
+bool TensorView::from_c(const et_tensor* tensor, TensorView* out, std::string* error) {
+    if (tensor == nullptr) {
+        if (error) *error = "tensor descriptor is NULL";
+        return false;
+    }
+    if (tensor->rank < 0 || tensor->rank > kMaxRank || (tensor->rank > 0 && tensor->shape == nullptr)) {
+        if (error) *error = "tensor rank must be 0.." + std::to_string(kMaxRank) + " with a shape array";
+        return false;
+    }
+    out->data = tensor->data;
+    out->dtype = tensor->dtype;
+    out->offset = tensor->offset;
+    out->shape.assign(tensor->shape, tensor->shape + tensor->rank);
+    if (tensor->strides != nullptr) {
+        out->strides.assign(tensor->strides, tensor->strides + tensor->rank);
+    } else {
+        // Layout::contiguous, crates/runtime/src/layout.rs:53-67
+        out->strides.assign(tensor->rank, 0);
+        uint64_t acc = 1;
+        for (int d = tensor->rank - 1; d >= 0; d--) {
+            out->strides[d] = acc;
+            if (d != 0 && !checked_mul(acc, out->shape[d], &acc)) {
+                if (error) *error = "layout stride overflow";
+                return false;
+            }
+        }
+    }
+    return true;
+}
+
+bool TensorView::is_contiguous() const {
+    uint64_t acc = 1;
+    for (size_t d = shape.size(); d-- > 0;) {
+        if (shape[d] != 1 && strides[d] != acc) return false;
+        if (d != 0 && !checked_mul(acc, shape[d], &acc)) return false;
+    }
+    return true;
+}
+
+const char* kernel_name(const et_linear_plan& plan) {
+    switch (plan.kernel) {
+        case LinearKernel::kNone: return "none";
+        case LinearKernel::kGemvFast: return "gemv_fast";
+        case LinearKernel::kGemvGeneric: return "gemv_generic";
+        case LinearKernel::kGemmI8: return "quantize_act+gemm_i8";
+    }
+    return "?";
+}
+
+int linear_requirements(const TensorView& input, const TensorView& weight, const TensorView* bias,
+                        int32_t codec, uint64_t rows, uint64_t columns, int32_t activation_mode,
+                        et_linear_plan* plan, std::string* error) {
+    if (input.dtype != ET_DTYPE_F32 || input.shape.size() < 2)
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: input must be rank >= 2 f32");
+    if (input.shape.back() != columns)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "quantized_linear: expected input trailing width " + std::to_string(columns) +
+                        ", got " + debug_shape(input.shape));
+    uint64_t elements;
+    if (!checked_product(input.shape, &elements))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: element count overflow");
+    uint64_t row_bytes = 0;
+    if (int status = validate_weight("quantized_linear", weight, codec, rows, columns, &row_bytes, error))
+        return status;
+    if (bias != nullptr) {
+        if (bias->dtype != ET_DTYPE_F32 || bias->shape.size() != 1 || bias->shape[0] != rows)
+            return fail(error, ET_ERR_UNSUPPORTED,
+                        "quantized_linear: bias must be [" + std::to_string(rows) + "] f32, got " +
+                            debug_shape(bias->shape) + " " + dtype_name(bias->dtype));
+    }
+    plan->codec = codec;
+    plan->rows = rows;
+    plan->columns = columns;
+    plan->encoded_row_bytes = row_bytes;
+    plan->has_bias = bias != nullptr;
+    plan->activation_mode = activation_mode;
+    plan->input_shape = input.shape;
+    plan->output_shape = input.shape;
+    plan->output_shape.back() = rows;
+    uint64_t out_elements;
+    if (!checked_product(plan->output_shape, &out_elements))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: element count overflow");
+    if (!checked_mul(out_elements, 4, &plan->output_bytes))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: output byte size overflow");
+    std::vector<uint64_t> leading(input.shape.begin(), input.shape.end() - 1);
+    if (!checked_product(leading, &plan->vectors))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: element count overflow");
+    return select_kernel(plan, error);
+}
+
+int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
+                           bool has_bias, int32_t activation_mode, et_linear_plan* plan,
+                           std::string* error) {
+    TensorView input;
+    input.dtype = ET_DTYPE_F32;
+    input.shape = {vectors, columns};
+    input.strides = {columns, 1};
+    uint64_t row_bytes = 0;
+    TensorView weight;
+    weight.dtype = ET_DTYPE_U8;
+    if (!encoded_row_bytes(codec, columns, &row_bytes)) row_bytes = 0;  // reported by validate_weight
+    weight.shape = {rows, row_bytes};
+    weight.strides = {row_bytes, 1};
+    TensorView bias;
+    bias.dtype = ET_DTYPE_F32;
+    bias.shape = {rows};
+    bias.strides = {1};
+    return linear_requirements(input, weight, has_bias ? &bias : nullptr, codec, rows, columns,
+                               activation_mode, plan, error);
+}
+
+int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
+                   const uint8_t* weight, const float* bias, float* y, void* workspace,
+                   uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                   std::string* error) {
+    if ((bias != nullptr) != plan.has_bias)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias does not match the immutable plan");
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (plan.kernel == LinearKernel::kNone) return ET_OK;  // empty output: no dispatch
+    if (x == nullptr || weight == nullptr || y == nullptr)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: NULL operand");
+    hipStream_t s = as_stream(stream);
+    auto* scratch = static_cast<uint8_t*>(workspace);
+
+    // The kernels read activations with 16-byte loads.
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (x_row_stride % 4 == 0) &&
+                         x_row_stride >= plan.columns;
+    if (!aligned) {
+        if (scratch == nullptr || workspace_bytes < plan.gather_offset + plan.gather_bytes)
+            return fail(error, ET_ERR_EXECUTION,
+                        "quantized_linear: input rows are not 16-byte aligned and the workspace (" +
+                            std::to_string(workspace_bytes) + " bytes) cannot hold a dense copy");
+        IndexLayout layout;
+        std::memset(&layout, 0, sizeof layout);
+        layout.rank = 2;
+        layout.shape[0] = plan.vectors;
+        layout.shape[1] = plan.columns;
+        layout.strides[0] = x_row_stride;
+        layout.strides[1] = 1;
+        float* dense = reinterpret_cast<float*>(scratch + plan.gather_offset);
+        if (hipError_t status = gather_f32(x, layout, plan.vectors * plan.columns, dense, s))
+            return hip_failure(error, "quantized_linear", status);
+        x = dense;
+        x_row_stride = plan.columns;
+    }
+
+    if (plan.kernel == LinearKernel::kGemmI8) {
+        if (scratch == nullptr || workspace_bytes < plan.workspace_bytes)
+            return fail(error, ET_ERR_EXECUTION,
+                        "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                            " bytes is smaller than the planned " +
+                            std::to_string(plan.workspace_bytes));
+        auto* q = reinterpret_cast<int8_t*>(scratch + plan.q_offset);
+        auto* scale = reinterpret_cast<float*>(scratch + plan.scale_offset);
+        auto* sum = reinterpret_cast<int32_t*>(scratch + plan.sum_offset);
+        if (hipError_t status =
+                quantize_activations(x, x_row_stride, plan.vectors, plan.columns, q, scale, sum, s))
+            return hip_failure(error, "quantized_linear", status);
+        if (hipError_t status = gemm_i8(plan.codec, weight, q, scale, sum, bias, y, plan.rows,
+                                        plan.columns, plan.vectors, s))
+            return hip_failure(error, "quantized_linear", status);
+        return ET_OK;
+    }
+
+    for (uint64_t v0 = 0; v0 < plan.vectors; v0 += plan.vectors_per_launch) {
+        const uint32_t count = static_cast<uint32_t>(
+            plan.vectors - v0 < plan.vectors_per_launch ? plan.vectors - v0 : plan.vectors_per_launch);
+        const float* xv = x + v0 * x_row_stride;
+        float* yv = y + v0 * plan.rows;
+        hipError_t status;
+        if (plan.kernel == LinearKernel::kGemvFast && gemv_fast_supported(plan.codec, plan.columns, count))
+            status = gemv_fast(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
+                               count, s);
+        else
+            status = gemv_generic(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows,
+                                  plan.columns, count, s);
+        if (status != hipSuccess) return hip_failure(error, "quantized_linear", status);
+    }
+    return ET_OK;
+}
+
+// validate_linear_execution + linear_into, crates/runtime-cpu/src/quantized.rs:367-499
+int linear_into(const et_linear_plan& plan, const TensorView& input, const TensorView& weight,
+                const TensorView* bias, const TensorView& destination, void* workspace,
+                uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                std::string* error) {
+    if (input.dtype != ET_DTYPE_F32 || input.shape.size() < 2 || input.shape.back() != plan.columns)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: input does not match the immutable plan");
+    std::vector<uint64_t> leading(input.shape.begin(), input.shape.end() - 1);
+    uint64_t vectors;
+    if (!checked_product(leading, &vectors))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: element count overflow");
+    uint64_t output_elements, output_bytes;
+    if (!checked_mul(vectors, plan.rows, &output_elements))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: output element count overflow");
+    if (!checked_mul(output_elements, 4, &output_bytes))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: output byte size overflow");
+    uint64_t row_bytes;
+    if (int status = validate_weight("quantized_linear", weight, plan.codec, plan.rows, plan.columns,
+                                     &row_bytes, error))
+        return status;
+    if ((bias != nullptr) != plan.has_bias ||
+        (bias != nullptr && (bias->dtype != ET_DTYPE_F32 || bias->shape.size() != 1 ||
+                             bias->shape[0] != plan.rows)))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias does not match the immutable plan");
+    bool shape_ok = destination.dtype == ET_DTYPE_F32 &&
+                    destination.shape.size() == input.shape.size() &&
+                    destination.shape.back() == plan.rows;
+    for (size_t d = 0; shape_ok && d + 1 < input.shape.size(); d++)
+        shape_ok = destination.shape[d] == input.shape[d];
+    if (!shape_ok)
+        return fail(error, ET_ERR_EXECUTION,
+                    "quantized_linear: destination does not match the logical node shape");
+    // The plan froze the vector count through its shapes; a different count needs a new plan.
+    if (vectors != plan.vectors)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: input does not match the immutable plan");
+    // CpuDestination is an exclusive dense output (crates/runtime-cpu/src/tensor.rs:743-760).
+    if (!destination.is_contiguous() || destination.offset != 0)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: destination must be contiguous with zero offset");
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (plan.kernel == LinearKernel::kNone) return ET_OK;
+
+    hipStream_t s = as_stream(stream);
+    const float* x = static_cast<const float*>(input.data);
+    uint64_t x_row_stride = plan.columns;
+    const float* bias_data = nullptr;
+    if (bias != nullptr) {
+        // bias[source_index(layout, row)]: a strided [rows] view is densified too.
+        if (bias->is_contiguous()) {
+            bias_data = static_cast<const float*>(bias->data) + bias->offset;
+        } else {
+            auto* scratch = static_cast<uint8_t*>(workspace);
+            if (scratch == nullptr || workspace_bytes < plan.workspace_bytes)
+                return fail(error, ET_ERR_EXECUTION,
+                            "quantized_linear: strided bias needs the planned workspace of " +
+                                std::to_string(plan.workspace_bytes) + " bytes");
+            float* dense = reinterpret_cast<float*>(scratch + plan.bias_offset);
+            if (hipError_t status = gather_f32(static_cast<const float*>(bias->data),
+                                               make_layout(*bias), plan.rows, dense, s))
+                return hip_failure(error, "quantized_linear", status);
+            bias_data = dense;
+        }
+    }
+    uint64_t stride;
+    if (row_dense(input, &stride)) {
+        x = static_cast<const float*>(input.data) + input.offset;
+        x_row_stride = stride;
+    } else {
+        auto* scratch = static_cast<uint8_t*>(workspace);
+        if (scratch == nullptr || workspace_bytes < plan.gather_offset + plan.gather_bytes)
+            return fail(error, ET_ERR_EXECUTION,
+                        "quantized_linear: strided input needs a workspace of at least " +
+                            std::to_string(plan.gather_offset + plan.gather_bytes) + " bytes");
+        float* dense = reinterpret_cast<float*>(scratch + plan.gather_offset);
+        const IndexLayout layout = make_layout(input);
+        if (hipError_t status = gather_f32(static_cast<const float*>(input.data), layout,
+                                           plan.vectors * plan.columns, dense, s))
+            return hip_failure(error, "quantized_linear", status);
+        x = dense;
+        x_row_stride = plan.columns;
+    }
+    return linear_enqueue(plan, x, x_row_stride, static_cast<const uint8_t*>(weight.data), bias_data,
+                          static_cast<float*>(const_cast<void*>(destination.data)), workspace,
+                          workspace_bytes, stream, cancel, error);
+}
+
+int embedding_requirements(const TensorView& indexes, const TensorView& weight, int32_t codec,
+                           uint64_t rows, uint64_t columns, et_embedding_plan* plan,
+                           std::string* error) {
+    if (indexes.dtype != ET_DTYPE_U32 && indexes.dtype != ET_DTYPE_I64)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    std::string("quantized_embedding: indexes must be u32 or i64, got ") +
+                        dtype_name(indexes.dtype));
+    uint64_t count;
+    if (!checked_product(indexes.shape, &count))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_embedding: element count overflow");
+    uint64_t row_bytes = 0;
+    if (int status = validate_weight("quantized_embedding", weight, codec, rows, columns, &row_bytes, error))
+        return status;
+    plan->codec = codec;
+    plan->rows = rows;
+    plan->columns = columns;
+    plan->encoded_row_bytes = row_bytes;
+    plan->index_shape = indexes.shape;
+    plan->index_dtype = indexes.dtype;
+    plan->output_shape = indexes.shape;
+    plan->output_shape.push_back(columns);
+    plan->count = count;
+    uint64_t out_elements;
+    if (!checked_product(plan->output_shape, &out_elements))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_embedding: element count overflow");
+    if (!checked_mul(out_elements, 4, &plan->output_bytes))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_embedding: output byte size overflow");
+    return ET_OK;
+}
+
+// validate_embedding_execution + embedding_into, crates/runtime-cpu/src/quantized.rs:501-616
+int embedding_into(const et_embedding_plan& plan, const TensorView& indexes,
+                   const TensorView& weight, const TensorView& destination, void* status,
+                   void* stream, const volatile int32_t* cancel, std::string* error) {
+    if (indexes.dtype != ET_DTYPE_U32 && indexes.dtype != ET_DTYPE_I64)
+        return fail(error, ET_ERR_EXECUTION, "quantized_embedding: indexes do not match the immutable plan");
+    uint64_t count;
+    if (!checked_product(indexes.shape, &count))
+        return fail(error, ET_ERR_EXECUTION, "quantized_embedding: element count overflow");
+    uint64_t output_elements, output_bytes;
+    if (!checked_mul(count, plan.columns, &output_elements))
+        return fail(error, ET_ERR_EXECUTION, "quantized_embedding: output element count overflow");
+    if (!checked_mul(output_elements, 4, &output_bytes))
+        return fail(error, ET_ERR_EXECUTION, "quantized_embedding: output byte size overflow");
+    uint64_t row_bytes;
+    if (int rc = validate_weight("quantized_embedding", weight, plan.codec, plan.rows, plan.columns,
+                                 &row_bytes, error))
+        return rc;
+    bool shape_ok = destination.dtype == ET_DTYPE_F32 &&
+                    destination.shape.size() == indexes.shape.size() + 1 &&
+                    destination.shape.back() == plan.columns;
+    for (size_t d = 0; shape_ok && d < indexes.shape.size(); d++)
+        shape_ok = destination.shape[d] == indexes.shape[d];
+    if (!shape_ok)
+        return fail(error, ET_ERR_EXECUTION,
+                    "quantized_embedding: destination does not match the logical node shape");
+    if (!destination.is_contiguous() || destination.offset != 0)
+        return fail(error, ET_ERR_EXECUTION,
+                    "quantized_embedding: destination must be contiguous with zero offset");
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (count == 0 || plan.columns == 0) return ET_OK;
+    if (status == nullptr)
+        return fail(error, ET_ERR_INVALID, "quantized_embedding: a device status block is required");
+    if (reinterpret_cast<uintptr_t>(destination.data) % 16 != 0)
+        return fail(error, ET_ERR_EXECUTION, "quantized_embedding: destination must be 16-byte aligned");
+    const IndexLayout layout = make_layout(indexes);
+    if (hipError_t rc = dequantize_rows(plan.codec, static_cast<const uint8_t*>(weight.data),
+                                        indexes.data, indexes.dtype == ET_DTYPE_I64 ? 1 : 0, layout,
+                                        count, plan.rows, plan.columns,
+                                        static_cast<float*>(const_cast<void*>(destination.data)), status,
+                                        as_stream(stream)))
+        return hip_failure(error, "quantized_embedding", rc);
+    return ET_OK;
+}
+
+int embedding_status_check(const et_embedding_plan& plan, const void* status_host,
+                           std::string* error) {
+    uint64_t words[2];
+    std::memcpy(words, status_host, sizeof words);
+    if (words[0] == kMax) return ET_OK;
+    // crates/runtime-cpu/src/quantized.rs:570-583: i64 values print signed, u32 unsigned.
+    const long long value = static_cast<long long>(words[1]);
+    return fail(error, ET_ERR_EXECUTION,
+                "quantized_embedding: index " + std::to_string(value) + " is outside 0.." +
+                    std::to_string(plan.rows));
+}
+
+}  // namespace quantized
+}  // namespace et

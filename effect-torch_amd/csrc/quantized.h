@@ -1,0 +1,100 @@
+// Host side of the quantized operators: the plan / execute pair a backend
+// crate of the reference exposes to its executable, restated over device
+// buffers. Names, argument meaning and error text follow
+// crates/runtime-cpu/src/quantized.rs (linear_requirements :297-336,
+// validate_linear_execution :367-415, linear_into :419-499,
+// embedding_requirements :340-365, embedding_into :546-616).
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "et_hip.h"
+
+namespace et {
+namespace quantized {
+
+// Reference Tensor = storage + Layout (crates/runtime/src/layout.rs).
+struct TensorView {
+    const void* data = nullptr;
+    int32_t dtype = ET_DTYPE_F32;
+    std::vector<uint64_t> shape;
+    std::vector<uint64_t> strides;  // always materialised
+    uint64_t offset = 0;
+
+    static bool from_c(const et_tensor* tensor, TensorView* out, std::string* error);
+    bool is_contiguous() const;  // Layout::is_contiguous, layout.rs:110-124
+};
+
+enum class LinearKernel {
+    kNone,         // empty output: nothing is enqueued
+    kGemvFast,     // activation-stationary dequant-GEMV (gemv_fast.hip)
+    kGemvGeneric,  // portable dequant-GEMV (gemv_generic.hip)
+    kGemmI8,       // quantize_act.hip + gemm_i8.hip
+};
+
+}  // namespace quantized
+}  // namespace et
+
+// The opaque plan types of the C ABI.
+struct et_linear_plan {
+    int32_t codec;
+    uint64_t rows, columns, encoded_row_bytes;
+    bool has_bias;
+    int32_t activation_mode;
+    std::vector<uint64_t> input_shape;   // empty for plans made from raw sizes
+    std::vector<uint64_t> output_shape;
+    uint64_t vectors;
+    uint64_t output_bytes;
+    et::quantized::LinearKernel kernel;
+    uint32_t vectors_per_launch;
+    // workspace sections (byte offsets), all 256-byte aligned
+    uint64_t gather_offset, gather_bytes;  // densified f32 input
+    uint64_t bias_offset;                  // densified f32 bias
+    uint64_t q_offset, scale_offset, sum_offset;
+    uint64_t workspace_bytes;
+};
+
+struct et_embedding_plan {
+    int32_t codec;
+    uint64_t rows, columns, encoded_row_bytes;
+    std::vector<uint64_t> index_shape;
+    int32_t index_dtype;
+    std::vector<uint64_t> output_shape;
+    uint64_t count;
+    uint64_t output_bytes;
+};
+
+namespace et {
+namespace quantized {
+
+// Every function returns an et_status and, on failure, leaves the message in *error.
+int linear_requirements(const TensorView& input, const TensorView& weight, const TensorView* bias,
+                        int32_t codec, uint64_t rows, uint64_t columns, int32_t activation_mode,
+                        et_linear_plan* plan, std::string* error);
+int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
+                           bool has_bias, int32_t activation_mode, et_linear_plan* plan,
+                           std::string* error);
+int linear_into(const et_linear_plan& plan, const TensorView& input, const TensorView& weight,
+                const TensorView* bias, const TensorView& destination, void* workspace,
+                uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                std::string* error);
+int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
+                   const uint8_t* weight, const float* bias, float* y, void* workspace,
+                   uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                   std::string* error);
+
+int embedding_requirements(const TensorView& indexes, const TensorView& weight, int32_t codec,
+                           uint64_t rows, uint64_t columns, et_embedding_plan* plan,
+                           std::string* error);
+int embedding_into(const et_embedding_plan& plan, const TensorView& indexes,
+                   const TensorView& weight, const TensorView& destination, void* status,
+                   void* stream, const volatile int32_t* cancel, std::string* error);
+int embedding_status_check(const et_embedding_plan& plan, const void* status_host,
+                           std::string* error);
+
+const char* kernel_name(const et_linear_plan& plan);
+
+}  // namespace quantized
+}  // namespace et

@@ -1,0 +1,327 @@
+"""Host-side mirror of the reference's quantized operator pair, over torch device tensors.
+
+Same names, argument meaning and error text as the backend crates of the
+reference (crates/runtime-cpu/src/quantized.rs): ``linear_requirements``
+(:297-336) plans and validates, ``linear_into`` (:419-499) executes into a
+caller-provided destination; ``embedding_requirements`` (:340-365) and
+``embedding_into`` (:546-616) likewise. Errors the reference returns as
+``Err(String)`` are raised as :class:`QuantizedError` carrying the same text.
+
+torch is used for device memory and streams only; all arithmetic happens in
+``libet_hip.so`` behind the C ABI of ``include/et_hip.h``.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+from typing import Optional, Sequence
+
+import torch
+
+from . import _native as N
+
+
+class GgmlQuant(enum.IntEnum):
+    """GGML tensor type codes; Q2_K..Q6_K are the reference's ``GgmlKQuant``
+    (crates/runtime/src/gguf.rs:199-205)."""
+
+    Q4_0 = 2
+    Q8_0 = 8
+    Q2_K = 10
+    Q3_K = 11
+    Q4_K = 12
+    Q5_K = 13
+    Q6_K = 14
+
+    @property
+    def ggml_name(self) -> str:  # GgmlKQuant::name, gguf.rs:208-217
+        return N.lib().et_hip_codec_name(int(self)).decode()
+
+    @classmethod
+    def from_name(cls, name: str) -> Optional["GgmlQuant"]:  # gguf.rs:220-230
+        for member in cls:
+            if member.ggml_name == name:
+                return member
+        return None
+
+    @property
+    def block_values(self) -> int:
+        return N.lib().et_hip_block_values(int(self))
+
+    @property
+    def block_bytes(self) -> int:  # quantized.rs:60-68
+        return N.lib().et_hip_block_bytes(int(self))
+
+    def encoded_row_bytes(self, columns: int) -> Optional[int]:  # gguf.rs:245-250
+        value = N.lib().et_hip_encoded_row_bytes(int(self), columns)
+        return None if value == 0 and columns != 0 else value
+
+
+class ActivationMode(enum.IntEnum):
+    F32 = N.ACT_F32
+    INT8 = N.ACT_INT8
+
+
+class QuantizedError(RuntimeError):
+    """An ``Err(String)`` of the reference operator; ``status`` is the et_status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(message)
+        self.status = status
+
+
+class Cancelled(QuantizedError):
+    """``"operation aborted"`` (crates/runtime-cpu/src/quantized.rs:451-453)."""
+
+
+_DTYPES = {
+    torch.float32: N.DTYPE_F32,
+    torch.float64: N.DTYPE_F64,
+    torch.float16: N.DTYPE_F16,
+    torch.bfloat16: N.DTYPE_BF16,
+    torch.uint8: N.DTYPE_U8,
+    torch.uint32: N.DTYPE_U32,
+    torch.int64: N.DTYPE_I64,
+}
+
+
+def _check(status: int) -> None:
+    if status == N.OK:
+        return
+    message = N.last_error()
+    if status == N.ERR_CANCELLED:
+        raise Cancelled(status, message)
+    raise QuantizedError(status, message)
+
+
+class _Desc:
+    """Keeps the ctypes arrays of an ``et_tensor`` alive."""
+
+    def __init__(self, tensor: torch.Tensor):
+        if tensor.dtype not in _DTYPES:
+            raise QuantizedError(N.ERR_UNSUPPORTED, f"unsupported dtype {tensor.dtype}")
+        rank = tensor.dim()
+        self.shape = (ctypes.c_uint64 * max(rank, 1))(*tensor.shape)
+        self.strides = (ctypes.c_uint64 * max(rank, 1))(*tensor.stride())
+        storage_ptr = tensor.untyped_storage().data_ptr() if tensor.numel() or tensor.device.type != "meta" else 0
+        self.struct = N.EtTensor(storage_ptr, _DTYPES[tensor.dtype], rank, self.shape, self.strides,
+                                 tensor.storage_offset())
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.struct)
+
+
+def _desc(tensor: Optional[torch.Tensor]):
+    return None if tensor is None else _Desc(tensor)
+
+
+def _ref(desc: Optional[_Desc]):
+    return None if desc is None else desc.ref
+
+
+def _stream_handle(stream) -> int:
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return stream.cuda_stream if hasattr(stream, "cuda_stream") else int(stream)
+
+
+class CancellationFlag:
+    """Host flag polled before work is enqueued (crates/runtime/src/cancellation.rs:18-35)."""
+
+    def __init__(self):
+        self._value = ctypes.c_int32(0)
+
+    def cancel(self) -> None:
+        self._value.value = 1
+
+    def is_cancelled(self) -> bool:
+        return self._value.value != 0
+
+    @property
+    def ptr(self):
+        return ctypes.cast(ctypes.byref(self._value), ctypes.c_void_p)
+
+
+class QuantizedRequirements:
+    """Frozen plan of one quantized linear (crates/runtime-cpu/src/quantized.rs:35-42)."""
+
+    def __init__(self, handle: int, codec: GgmlQuant, rows: int, columns: int):
+        self._handle = ctypes.c_void_p(handle)
+        self.codec, self.rows, self.columns = codec, rows, columns
+        lib = N.lib()
+        rank = lib.et_hip_linear_plan_output_rank(self._handle)
+        shape = (ctypes.c_uint64 * max(rank, 1))()
+        lib.et_hip_linear_plan_output_shape(self._handle, shape)
+        self.output_shape = tuple(shape[i] for i in range(rank))
+        self.vectors = lib.et_hip_linear_plan_vectors(self._handle)
+        self.output_bytes = lib.et_hip_linear_plan_output_bytes(self._handle)
+        self.workspace_bytes = lib.et_hip_linear_plan_workspace_bytes(self._handle)
+        self.kernel = lib.et_hip_linear_plan_kernel(self._handle).decode()
+        self.algorithmic_bytes = lib.et_hip_linear_plan_algorithmic_bytes(self._handle)
+
+    def __del__(self):
+        handle, self._handle = getattr(self, "_handle", None), None
+        if handle:
+            try:
+                N.lib().et_hip_linear_plan_destroy(handle)
+            except Exception:
+                pass
+
+
+class EmbeddingRequirements:
+    def __init__(self, handle: int, codec: GgmlQuant, rows: int, columns: int):
+        self._handle = ctypes.c_void_p(handle)
+        self.codec, self.rows, self.columns = codec, rows, columns
+        lib = N.lib()
+        rank = lib.et_hip_embedding_plan_output_rank(self._handle)
+        shape = (ctypes.c_uint64 * max(rank, 1))()
+        lib.et_hip_embedding_plan_output_shape(self._handle, shape)
+        self.output_shape = tuple(shape[i] for i in range(rank))
+        self.output_bytes = lib.et_hip_embedding_plan_output_bytes(self._handle)
+
+    def __del__(self):
+        handle, self._handle = getattr(self, "_handle", None), None
+        if handle:
+            try:
+                N.lib().et_hip_embedding_plan_destroy(handle)
+            except Exception:
+                pass
+
+
+def is_available() -> bool:
+    """A gfx950 device is visible (cf. isAvailable, native-addon.ts:266)."""
+    return bool(N.lib().et_hip_is_available())
+
+
+def linear_requirements(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                        codec: GgmlQuant, weight_shape: Sequence[int],
+                        activation_mode: ActivationMode = ActivationMode.F32) -> QuantizedRequirements:
+    """Plan step (crates/runtime-cpu/src/quantized.rs:297-336). Reads metadata only."""
+    rows, columns = weight_shape
+    descs = (_desc(input), _desc(weight), _desc(bias))
+    out = ctypes.c_void_p()
+    _check(N.lib().et_hip_linear_requirements(_ref(descs[0]), _ref(descs[1]), _ref(descs[2]),
+                                              int(codec), rows, columns, int(activation_mode),
+                                              ctypes.byref(out)))
+    return QuantizedRequirements(out.value, GgmlQuant(codec), rows, columns)
+
+
+def linear_into(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                codec: GgmlQuant, destination: torch.Tensor, requirements: QuantizedRequirements,
+                cancelled: Optional[CancellationFlag] = None, *,
+                workspace: Optional[torch.Tensor] = None, stream=None) -> None:
+    """Execute step (crates/runtime-cpu/src/quantized.rs:419-499): enqueues on ``stream``."""
+    if int(codec) != int(requirements.codec):
+        raise QuantizedError(N.ERR_EXECUTION, "quantized_linear: codec does not match the immutable plan")
+    descs = (_desc(input), _desc(weight), _desc(bias), _desc(destination))
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _check(N.lib().et_hip_linear_into(requirements._handle, _ref(descs[0]), _ref(descs[1]),
+                                      _ref(descs[2]), _ref(descs[3]), ws_ptr, ws_bytes,
+                                      _stream_handle(stream),
+                                      cancelled.ptr if cancelled is not None else None))
+
+
+def quantized_linear(input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                     codec: GgmlQuant, weight_shape: Sequence[int],
+                     activation_mode: ActivationMode = ActivationMode.F32) -> torch.Tensor:
+    """Plan + allocate + execute, for callers that do not manage buffers themselves."""
+    requirements = linear_requirements(input, weight, bias, codec, weight_shape, activation_mode)
+    destination = torch.empty(requirements.output_shape, dtype=torch.float32, device=input.device)
+    workspace = None
+    if requirements.workspace_bytes:
+        workspace = torch.empty(requirements.workspace_bytes, dtype=torch.uint8, device=input.device)
+    linear_into(input, weight, bias, codec, destination, requirements, workspace=workspace)
+    return destination
+
+
+def embedding_requirements(indexes: torch.Tensor, weight: torch.Tensor, codec: GgmlQuant,
+                           weight_shape: Sequence[int]) -> EmbeddingRequirements:
+    """Plan step (crates/runtime-cpu/src/quantized.rs:340-365)."""
+    rows, columns = weight_shape
+    descs = (_desc(indexes), _desc(weight))
+    out = ctypes.c_void_p()
+    _check(N.lib().et_hip_embedding_requirements(_ref(descs[0]), _ref(descs[1]), int(codec), rows,
+                                                 columns, ctypes.byref(out)))
+    return EmbeddingRequirements(out.value, GgmlQuant(codec), rows, columns)
+
+
+def embedding_into(indexes: torch.Tensor, weight: torch.Tensor, codec: GgmlQuant,
+                   destination: torch.Tensor, requirements: EmbeddingRequirements,
+                   cancelled: Optional[CancellationFlag] = None, *, stream=None,
+                   synchronize: bool = True) -> Optional[torch.Tensor]:
+    """Execute step (crates/runtime-cpu/src/quantized.rs:546-616).
+
+    The kernel skips out-of-range indexes and records the first one in a device
+    status block. With ``synchronize`` (default) the stream is drained and the
+    reference's error is raised here; otherwise the status tensor is returned
+    for :func:`embedding_status_check` after the caller's own fence.
+    """
+    if int(codec) != int(requirements.codec):
+        raise QuantizedError(N.ERR_EXECUTION, "quantized_embedding: codec does not match the immutable plan")
+    status = torch.empty(N.STATUS_BYTES, dtype=torch.uint8, device=destination.device)
+    descs = (_desc(indexes), _desc(weight), _desc(destination))
+    _check(N.lib().et_hip_embedding_into(requirements._handle, _ref(descs[0]), _ref(descs[1]),
+                                         _ref(descs[2]), status.data_ptr(), _stream_handle(stream),
+                                         cancelled.ptr if cancelled is not None else None))
+    if not synchronize:
+        return status
+    embedding_status_check(requirements, status)
+    return None
+
+
+def embedding_status_check(requirements: EmbeddingRequirements, status: torch.Tensor) -> None:
+    host = status.cpu().numpy().tobytes()  # synchronises with the producing stream
+    buf = ctypes.create_string_buffer(host, N.STATUS_BYTES)
+    _check(N.lib().et_hip_embedding_status_check(requirements._handle, buf))
+
+
+def dequantize_rows(weight: torch.Tensor, codec: GgmlQuant, weight_shape: Sequence[int],
+                    stream=None) -> torch.Tensor:
+    """Bit-exact decode of every row: ``[rows, columns]`` f32."""
+    rows, columns = weight_shape
+    out = torch.empty((rows, columns), dtype=torch.float32, device=weight.device)
+    _check(N.lib().et_hip_dequantize_rows(int(codec), rows, columns, weight.data_ptr(),
+                                          out.data_ptr(), _stream_handle(stream)))
+    return out
+
+
+def quantize_activations(x: torch.Tensor, stream=None):
+    """int8 activation quantiser: returns (q int8 [M, K], scale f32 [K/32, M], sum i32 [K/32, M]).
+
+    The library writes the two tables with a row stride of M rounded up to 32;
+    the returned tensors are views of the first M columns."""
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1
+    vectors, columns = x.shape
+    padded = (vectors + 31) // 32 * 32
+    q = torch.empty((vectors, columns), dtype=torch.int8, device=x.device)
+    scale = torch.zeros((columns // 32, padded), dtype=torch.float32, device=x.device)
+    total = torch.zeros((columns // 32, padded), dtype=torch.int32, device=x.device)
+    _check(N.lib().et_hip_quantize_activations(x.data_ptr(), x.stride(0), vectors, columns,
+                                               q.data_ptr(), scale.data_ptr(), total.data_ptr(),
+                                               _stream_handle(stream)))
+    return q, scale[:, :vectors], total[:, :vectors]
+
+
+class RawLinear:
+    """Raw-pointer plan/enqueue pair (``et_hip_linear_plan_create`` / ``et_hip_linear_enqueue``)
+    for dense ``[vectors, columns]`` inputs; what a timing loop or a graph capture uses."""
+
+    def __init__(self, codec: GgmlQuant, rows: int, columns: int, vectors: int, has_bias: bool = False,
+                 activation_mode: ActivationMode = ActivationMode.F32):
+        out = ctypes.c_void_p()
+        _check(N.lib().et_hip_linear_plan_create(int(codec), rows, columns, vectors, int(has_bias),
+                                                 int(activation_mode), ctypes.byref(out)))
+        self.requirements = QuantizedRequirements(out.value, GgmlQuant(codec), rows, columns)
+
+    def enqueue(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                y: torch.Tensor, workspace: Optional[torch.Tensor] = None, stream=None,
+                cancelled: Optional[CancellationFlag] = None) -> None:
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+        _check(N.lib().et_hip_linear_enqueue(self.requirements._handle, x.data_ptr(), x.stride(0),
+                                             weight.data_ptr(),
+                                             bias.data_ptr() if bias is not None else None,
+                                             y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream),
+                                             cancelled.ptr if cancelled is not None else None))

@@ -1,0 +1,219 @@
+/*
+ * et_hip.h - C ABI of the MI355X (gfx950) quantized-GGUF matmul backend.
+ *
+ * This is the boundary a `runtime-hip` backend crate binds over FFI. It mirrors
+ * the per-operator free-function pair every backend crate of the reference
+ * exposes to its executable: a *plan* step that validates geometry and freezes
+ * an immutable requirements object, and an allocation-free *execute* step that
+ * re-validates against the plan and runs (CPU) or enqueues (GPU):
+ *
+ *   reference (crates/runtime-cpu/src/quantized.rs)        this header
+ *   ------------------------------------------------       ---------------------------------
+ *   linear_requirements            :297-336                et_hip_linear_requirements
+ *   linear_into                    :419-499                et_hip_linear_into
+ *   embedding_requirements         :340-365                et_hip_embedding_requirements
+ *   embedding_into                 :546-616                et_hip_embedding_into (+ _status_check)
+ *   GgmlKQuant::encoded_row_bytes  crates/runtime/src/gguf.rs:245-250   et_hip_encoded_row_bytes
+ *   warm_linear_exact              crates/runtime-metal/src/quantized.rs:1226   (done inside the plan step)
+ *   isAvailable                    packages/backend-cpu/src/internal/native-addon.ts:266   et_hip_is_available
+ *
+ * Conventions
+ *   - All `data` pointers are DEVICE pointers to caller-owned, pre-allocated
+ *     memory. No entry point allocates or frees device memory; execute entry
+ *     points allocate nothing at all. Scratch comes in as `workspace`.
+ *   - Execute entry points ENQUEUE on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream) and return without synchronising.
+ *   - Return value 0 = ok; otherwise an et_status whose categories follow the
+ *     reference's BackendError taxonomy (crates/runtime/src/error.rs:25-68).
+ *     The message, worded like the reference's `Err(String)`, is available
+ *     from et_hip_last_error() on the calling thread.
+ *   - `cancel` is an optional host flag (the reference's CancellationFlag,
+ *     crates/runtime/src/cancellation.rs:18-35). It is polled before anything
+ *     is enqueued; a set flag yields ET_ERR_CANCELLED / "operation aborted".
+ *     Kernels already enqueued are not pre-empted.
+ *   - No C++ exception crosses this boundary.
+ */
+#ifndef ET_HIP_H
+#define ET_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GGML tensor type codes. 10..14 = the reference's GgmlKQuant
+ * (crates/runtime/src/gguf.rs:199-205, codes :278-291). 2 and 8 are the legacy
+ * ggml block formats, which the reference does not implement. */
+typedef enum {
+    ET_CODEC_Q4_0 = 2,
+    ET_CODEC_Q8_0 = 8,
+    ET_CODEC_Q2_K = 10,
+    ET_CODEC_Q3_K = 11,
+    ET_CODEC_Q4_K = 12,
+    ET_CODEC_Q5_K = 13,
+    ET_CODEC_Q6_K = 14
+} et_codec;
+
+/* Element types, in the order of the reference's DType (crates/runtime/src/dtype.rs:13-21). */
+typedef enum {
+    ET_DTYPE_F32 = 0,
+    ET_DTYPE_F64 = 1,
+    ET_DTYPE_F16 = 2,
+    ET_DTYPE_BF16 = 3,
+    ET_DTYPE_U8 = 4,
+    ET_DTYPE_U32 = 5,
+    ET_DTYPE_I64 = 6
+} et_dtype;
+
+typedef enum {
+    ET_OK = 0,
+    ET_ERR_UNSUPPORTED = 1, /* geometry / dtype / layout the operator does not accept */
+    ET_ERR_EXECUTION = 2,   /* a HIP call failed, or operands do not match the frozen plan */
+    ET_ERR_CANCELLED = 3,   /* "operation aborted" */
+    ET_ERR_UNAVAILABLE = 4, /* no usable gfx950 device */
+    ET_ERR_INVALID = 5      /* NULL where a pointer is required, unknown enum value */
+} et_status;
+
+/* How activations enter the contraction. */
+typedef enum {
+    ET_ACT_F32 = 0, /* f32 activations, f32 accumulate; tolerance 1e-3 against the CPU path */
+    ET_ACT_INT8 = 1 /* activations quantised on the fly to int8 per 32 columns with an f32
+                       absmax scale, int8 MFMA, f32 block-scale epilogue; tolerance 2e-2.
+                       The reference has no such mode. */
+} et_activation_mode;
+
+/* A strided view of caller-owned storage, in ELEMENTS - the reference's Tensor
+ * = buffer + Layout{shape, strides, offset} (crates/runtime/src/layout.rs).
+ * `strides == NULL` means row-major contiguous. */
+typedef struct {
+    const void* data;       /* device pointer to the start of the STORAGE (not of the view) */
+    int32_t dtype;          /* et_dtype */
+    int32_t rank;
+    const uint64_t* shape;  /* host array, `rank` entries */
+    const uint64_t* strides; /* host array, `rank` entries, or NULL */
+    uint64_t offset;        /* view offset into the storage */
+} et_tensor;
+
+typedef struct et_linear_plan et_linear_plan;       /* opaque, immutable, host memory */
+typedef struct et_embedding_plan et_embedding_plan; /* opaque, immutable, host memory */
+
+/* ---- availability and codec tables -------------------------------------- */
+
+/* 1 when a gfx950 device is visible and the library's kernels can run on it.
+ * cf. isAvailable (packages/backend-cpu/src/internal/native-addon.ts:266). */
+int et_hip_is_available(void);
+
+/* "Q4_K", ... or NULL. cf. GgmlKQuant::name (crates/runtime/src/gguf.rs:208-217). */
+const char* et_hip_codec_name(int32_t codec);
+/* Values per block (256 for K-quants, 32 for Q8_0 / Q4_0); 0 = unknown codec. */
+uint64_t et_hip_block_values(int32_t codec);
+/* Bytes per block. cf. block_bytes (crates/runtime-cpu/src/quantized.rs:60-68). */
+uint64_t et_hip_block_bytes(int32_t codec);
+/* Packed bytes of one logical row; 0 when `columns` is not a whole number of
+ * blocks or the product overflows. cf. GgmlKQuant::encoded_row_bytes
+ * (crates/runtime/src/gguf.rs:245-250). */
+uint64_t et_hip_encoded_row_bytes(int32_t codec, uint64_t columns);
+
+/* ---- quantized_linear ---------------------------------------------------- */
+
+/* Plan step = linear_requirements (crates/runtime-cpu/src/quantized.rs:297-336)
+ * + kernel selection by (codec, vectors, mode) (cf. linear_kernel_kind,
+ * crates/runtime-metal/src/quantized.rs:1204-1220).
+ *   input  f32, rank >= 2, trailing width = columns, any strides
+ *   weight u8, exactly [rows, encoded_row_bytes], contiguous, offset 0
+ *   bias   NULL or f32 [rows]
+ * Only metadata is read; `data` pointers may be NULL here. */
+int et_hip_linear_requirements(const et_tensor* input, const et_tensor* weight,
+                               const et_tensor* bias, int32_t codec, uint64_t rows,
+                               uint64_t columns, int32_t activation_mode, et_linear_plan** out);
+
+void et_hip_linear_plan_destroy(et_linear_plan* plan);
+
+/* Plan queries (QuantizedRequirements, crates/runtime-cpu/src/quantized.rs:35-42;
+ * LinearRequirements, crates/runtime-metal/src/quantized.rs:45-68). */
+int32_t et_hip_linear_plan_output_rank(const et_linear_plan* plan);
+/* Writes output_rank entries. */
+void et_hip_linear_plan_output_shape(const et_linear_plan* plan, uint64_t* shape);
+uint64_t et_hip_linear_plan_vectors(const et_linear_plan* plan);
+uint64_t et_hip_linear_plan_output_bytes(const et_linear_plan* plan);
+/* Device scratch the execute step needs (int8 activations, gathered strided
+ * input); the caller allocates at least this many bytes, 256-byte aligned. May be 0. */
+uint64_t et_hip_linear_plan_workspace_bytes(const et_linear_plan* plan);
+/* Name of the selected kernel variant, for profiles and diagnostics. */
+const char* et_hip_linear_plan_kernel(const et_linear_plan* plan);
+/* Algorithmic bytes of one execution: packed weight + f32 input + f32 output (+ bias). */
+uint64_t et_hip_linear_plan_algorithmic_bytes(const et_linear_plan* plan);
+
+/* Execute step = linear_into (crates/runtime-cpu/src/quantized.rs:419-499):
+ * re-validates the operands against the plan (validate_linear_execution,
+ * :367-415), then enqueues. destination: f32, contiguous, offset 0, shape =
+ * input shape with the trailing dim replaced by rows. */
+int et_hip_linear_into(const et_linear_plan* plan, const et_tensor* input, const et_tensor* weight,
+                       const et_tensor* bias, const et_tensor* destination, void* workspace,
+                       uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel);
+
+/* Raw-pointer form of the same pair for callers that hold dense buffers:
+ * x is [vectors, columns] f32 with `x_row_stride` elements between vectors,
+ * y is dense [vectors, rows] f32. Same validation of (codec, rows, columns). */
+int et_hip_linear_plan_create(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
+                              int32_t has_bias, int32_t activation_mode, et_linear_plan** out);
+int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
+                          const uint8_t* weight, const float* bias, float* y, void* workspace,
+                          uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel);
+
+/* ---- quantized_embedding (= bit-exact dequantisation of selected rows) ---- */
+
+/* Plan step = embedding_requirements (crates/runtime-cpu/src/quantized.rs:340-365).
+ * indexes: u32 or i64, any shape and strides. */
+int et_hip_embedding_requirements(const et_tensor* indexes, const et_tensor* weight, int32_t codec,
+                                  uint64_t rows, uint64_t columns, et_embedding_plan** out);
+void et_hip_embedding_plan_destroy(et_embedding_plan* plan);
+int32_t et_hip_embedding_plan_output_rank(const et_embedding_plan* plan);
+void et_hip_embedding_plan_output_shape(const et_embedding_plan* plan, uint64_t* shape);
+uint64_t et_hip_embedding_plan_output_bytes(const et_embedding_plan* plan);
+
+/* Execute step = embedding_into (crates/runtime-cpu/src/quantized.rs:546-616).
+ * destination: f32 [indexes.., columns], contiguous, offset 0. Every value is
+ * bit-identical to the CPU decode. An index outside 0..rows cannot fail the
+ * call (the kernel is already enqueued): the row is skipped and the device
+ * `status` block (ET_HIP_STATUS_BYTES bytes, zeroed by this call on `stream`)
+ * records it, as the reference's Metal backend does
+ * (crates/runtime-metal/src/quantized.rs:1103-1129). `status` may be NULL when
+ * `indexes` is NULL (= decode every row in order). */
+#define ET_HIP_STATUS_BYTES 16
+int et_hip_embedding_into(const et_embedding_plan* plan, const et_tensor* indexes,
+                          const et_tensor* weight, const et_tensor* destination, void* status,
+                          void* stream, const volatile int32_t* cancel);
+/* After the stream has completed and `status` has been copied to the host:
+ * 0, or ET_ERR_EXECUTION with "quantized_embedding: index {i} is outside 0..{rows}"
+ * (crates/runtime-cpu/src/quantized.rs:570-583). */
+int et_hip_embedding_status_check(const et_embedding_plan* plan, const void* status_host);
+
+/* Raw-pointer dequantisation of whole rows: out[r, :] = decode(W[r, :]) for
+ * r in [0, rows). Bit-exact. cf. decode_block (crates/runtime-cpu/src/quantized.rs:90-111). */
+int et_hip_dequantize_rows(int32_t codec, uint64_t rows, uint64_t columns, const uint8_t* weight,
+                           float* out, void* stream);
+
+/* ---- int8 activation quantiser (stage 1 of ET_ACT_INT8) ------------------- */
+
+/* The activation quantiser on its own, exposed so that tests can check the
+ * stage separately: q is int8 [vectors, columns]; scale (f32) and sum (i32, may
+ * be NULL) are TRANSPOSED tables [columns/32, stride] with stride = vectors
+ * rounded up to a multiple of 32 (entries at m >= vectors are not written).
+ *   amax = max|x| over the 32-block; scale = amax / 127;
+ *   q = clamp(rint(x * (amax > 0 ? 127 / amax : 0)), -127, 127); sum = sum of q.
+ * No counterpart in the reference. */
+int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                void* stream);
+
+/* ---- errors -------------------------------------------------------------- */
+
+/* Message of the last failed call on this thread ("" if none). */
+const char* et_hip_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ET_HIP_H */

@@ -1,0 +1,314 @@
+"""GPU parity: the HIP path behind the C ABI against the CPU oracle on the same seeded inputs.
+
+Bars: decoded weights bit-exact; f32-activation outputs within
+``|a-b| <= 1e-3 * max(|b|, 1)`` (the reference's own form,
+crates/runtime-metal/src/executable.rs:8372-8381, at the tolerance the workload
+states); the int8-activation path equals its own CPU restatement within the
+same 1e-3 bar (integer dots are exact, only the f32 summation order differs)
+and stays within ``2e-2 * max(|b|, rms(b))`` of the f32 reference.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import packers
+import ref_fixtures as rf
+from effect_torch_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+ALL = oracle.ALL_CODECS
+K_QUANTS = oracle.K_QUANTS
+
+
+def close(got, want, tol=1e-3):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    bound = tol * np.maximum(np.abs(want), 1.0)
+    bad = np.abs(got - want) > bound
+    assert not bad.any(), (f"{bad.sum()} of {bad.size} outside {tol}: max |err| "
+                           f"{np.abs(got - want).max():.4g} at {np.unravel_index(np.argmax(np.abs(got - want)), got.shape)}")
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def to_dev(array, device):
+    return torch.from_numpy(np.ascontiguousarray(array)).to(device)
+
+
+def finite_random_weight(codec, rows, columns, rng):
+    """Uniform random bytes everywhere; fp16 fields forced finite (any sign, subnormals included)."""
+    w = rng.integers(0, 256, (rows * columns // synth.BLOCK_VALUES[codec], synth.BLOCK_BYTES[codec]),
+                     dtype=np.uint8)
+    for off in synth._FP16_FIELDS[codec]:
+        hi = w[:, off + 1]
+        hi[(hi & 0x7C) == 0x7C] &= 0xBF  # exponent 31 (inf/nan) -> exponent 15 or 23
+    return w.reshape(rows, -1)
+
+
+# --------------------------------------------------------------------------- dequant
+
+@pytest.mark.parametrize("codec", K_QUANTS)
+def test_dequant_reference_fixtures(et, device, codec):
+    block = rf.FIXTURES[codec]["bytes"]
+    w = np.tile(block, 6).reshape(3, -1)
+    out = et.dequantize_rows(to_dev(w, device), et.GgmlQuant(codec), (3, 512)).cpu().numpy()
+    want = np.tile(rf.expected_values(codec), 6).reshape(3, 512)
+    assert np.array_equal(bits(out), bits(want))
+
+
+@pytest.mark.parametrize("codec", ALL)
+def test_dequant_bit_exact_on_packed_random_fields(et, device, codec):
+    rng = np.random.default_rng(500 + codec)
+    values = oracle.block_values(codec)
+    per_row = 512 // values
+    blocks = [packers.random_block(codec, rng) for _ in range(64 * per_row)]
+    w = np.concatenate([b for b, _ in blocks]).reshape(64, -1)
+    want = np.concatenate([v for _, v in blocks]).reshape(64, 512)
+    out = et.dequantize_rows(to_dev(w, device), et.GgmlQuant(codec), (64, 512)).cpu().numpy()
+    assert np.array_equal(bits(out), bits(want))
+    assert np.array_equal(bits(out), bits(oracle.decode_rows(codec, w, 512)))
+
+
+@pytest.mark.parametrize("codec", ALL)
+def test_dequant_bit_exact_on_random_bytes(et, device, codec):
+    rng = np.random.default_rng(600 + codec)
+    rows, columns = 257, 2048
+    w = finite_random_weight(codec, rows, columns, rng)
+    out = et.dequantize_rows(to_dev(w, device), et.GgmlQuant(codec), (rows, columns)).cpu().numpy()
+    assert np.array_equal(bits(out), bits(oracle.decode_rows(codec, w, columns)))
+
+
+def test_dequant_full_size_q4k_matches_oracle_checksum(et, device):
+    rng = np.random.default_rng(0xE77C0DE2)
+    rows, columns = 14336, 4096
+    w = synth.random_weight(synth.Q4_K, rows, columns, rng)
+    out = et.dequantize_rows(to_dev(w, device), et.GgmlQuant.Q4_K, (rows, columns))
+    got = out.cpu().numpy()
+    want = oracle.decode_rows(oracle.Q4_K, w, columns)
+    assert np.array_equal(bits(got), bits(want))
+
+
+# --------------------------------------------------------------------------- embedding
+
+@pytest.mark.parametrize("index_dtype", [torch.uint32, torch.int64])
+def test_embedding_kat(et, device, index_dtype):
+    # quantized.rs:867-897
+    table = np.zeros((3, 176), np.uint8)
+    table[1] = rf.FIXTURES[rf.Q5_K]["bytes"]
+    indexes = torch.tensor([1, 1], dtype=index_dtype).to(device)
+    w = to_dev(table, device)
+    plan = et.embedding_requirements(indexes, w, et.GgmlQuant.Q5_K, (3, 256))
+    out = torch.full(plan.output_shape, float("nan"), dtype=torch.float32, device=device)
+    et.embedding_into(indexes, w, et.GgmlQuant.Q5_K, out, plan)
+    want = rf.expected_values(rf.Q5_K)
+    got = out.cpu().numpy()
+    assert np.array_equal(got[0], want) and np.array_equal(got[1], want)
+
+
+@pytest.mark.parametrize("codec", ALL)
+def test_embedding_strided_indexes_all_codecs(et, device, codec):
+    rng = np.random.default_rng(700 + codec)
+    rows, columns = 50, 1024
+    table = finite_random_weight(codec, rows, columns, rng)
+    storage = rng.integers(0, rows, 64).astype(np.int64)
+    view = torch.from_numpy(storage).to(device)[4:].reshape(10, 6)[::2, 1:5]  # [5, 4], strided
+    w = to_dev(table, device)
+    plan = et.embedding_requirements(view, w, et.GgmlQuant(codec), (rows, columns))
+    assert plan.output_shape == (5, 4, columns)
+    out = torch.empty(plan.output_shape, dtype=torch.float32, device=device)
+    et.embedding_into(view, w, et.GgmlQuant(codec), out, plan)
+    want = oracle.embedding_into(codec, rows, columns, np.ascontiguousarray(view.cpu().numpy()), table)
+    assert np.array_equal(bits(out.cpu().numpy()), bits(want))
+
+
+@pytest.mark.parametrize("bad", [-1, 1, 2**40])
+def test_embedding_reports_out_of_range_indexes(et, device, bad):
+    # quantized.rs:899-921
+    table = to_dev(rf.FIXTURES[rf.Q2_K]["bytes"].reshape(1, 84), device)
+    indexes = torch.tensor([0, bad, 0, 7], dtype=torch.int64, device=device)
+    plan = et.embedding_requirements(indexes, table, et.GgmlQuant.Q2_K, (1, 256))
+    out = torch.zeros(plan.output_shape, dtype=torch.float32, device=device)
+    with pytest.raises(et.QuantizedError) as info:
+        et.embedding_into(indexes, table, et.GgmlQuant.Q2_K, out, plan)
+    assert str(info.value) == f"quantized_embedding: index {bad} is outside 0..1"
+    # valid rows were still decoded, the bad ones skipped
+    got = out.cpu().numpy()
+    assert np.array_equal(got[0], rf.expected_values(rf.Q2_K)) and not got[1].any()
+    u32 = torch.tensor([0, 5], dtype=torch.uint32).to(device)
+    plan = et.embedding_requirements(u32, table, et.GgmlQuant.Q2_K, (1, 256))
+    with pytest.raises(et.QuantizedError, match="index 5 is outside 0..1"):
+        et.embedding_into(u32, table, et.GgmlQuant.Q2_K, torch.zeros((2, 256), device=device), plan)
+
+
+# --------------------------------------------------------------------------- f32-activation linear
+
+def run_linear(et, device, codec, rows, columns, x, weight, bias=None, mode=None):
+    mode = et.ActivationMode.F32 if mode is None else mode
+    xt = x if isinstance(x, torch.Tensor) else to_dev(x, device)
+    bt = None if bias is None else to_dev(bias, device)
+    y = et.quantized_linear(xt, to_dev(weight, device), bt, et.GgmlQuant(codec), (rows, columns), mode)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def test_linear_kats(et, device):
+    # quantized.rs:827-865 and executable.rs:4881-4918
+    x = np.zeros(1024, np.float32)
+    x[:576] = 1.0
+    weight = np.tile(rf.FIXTURES[rf.Q4_K]["bytes"], 4).reshape(2, 288)
+    y = run_linear(et, device, oracle.Q4_K, 2, 512, x.reshape(2, 512), weight, np.array([0.5, -0.5], np.float32))
+    assert y.tolist() == [[4096.5, 4095.5], [512.5, 511.5]]
+    weight = np.tile(rf.FIXTURES[rf.Q4_K]["bytes"], 3).reshape(3, 144)
+    y = run_linear(et, device, oracle.Q4_K, 3, 256, np.ones((1, 256), np.float32), weight)
+    assert y.tolist() == [[2048.0, 2048.0, 2048.0]]
+
+
+@pytest.mark.parametrize("codec", K_QUANTS)
+@pytest.mark.parametrize("vectors", [1, 3, 4, 5, 16, 17])
+def test_linear_cross_backend_protocol(et, device, codec, vectors):
+    # crates/runtime-metal/src/executable.rs:8458-8505, at the reference's own 1e-4
+    columns = 512
+    i = np.arange(vectors * columns)
+    x = (((i * 7 + i // columns * 3) % 17).astype(np.float32) * np.float32(0.125) - np.float32(1.0))
+    x = x.reshape(vectors, columns)
+    weight = np.tile(rf.FIXTURES[codec]["bytes"], 4).reshape(2, -1)
+    bias = np.array([0.25, -0.5], np.float32) if vectors == 1 else None
+    got = run_linear(et, device, codec, 2, columns, x, weight, bias)
+    want = oracle.linear_into(codec, 2, columns, x, weight, bias)
+    close(got, want, 1e-4)
+
+
+@pytest.mark.parametrize("codec", ALL)
+@pytest.mark.parametrize("rows,columns", [(1, 256), (37, 512), (130, 4096), (64, 14336), (9, 1280)])
+@pytest.mark.parametrize("vectors", [1, 2, 3, 4, 7])
+def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
+    rng = np.random.default_rng(rows * 131 + columns + vectors + codec)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    bias = rng.standard_normal(rows).astype(np.float32) if (rows + vectors) % 2 else None
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias)
+    want = oracle.linear_into(codec, rows, columns, x, weight, bias)
+    assert got.shape == (vectors, rows)
+    close(got, want)
+
+
+@pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0, oracle.Q6_K])
+def test_linear_unit_vectors_select_decoded_weights(et, device, codec):
+    rng = np.random.default_rng(800 + codec)
+    rows, columns = 33, 4096
+    weight = synth.random_weight(codec, rows, columns, rng)
+    dense = oracle.decode_rows(codec, weight, columns)
+    picks = rng.choice(columns, 4, replace=False)
+    x = np.zeros((4, columns), np.float32)
+    x[np.arange(4), picks] = 1.0
+    got = run_linear(et, device, codec, rows, columns, x, weight)
+    # factored forms may differ from the decoded value by a rounding or two, never more
+    assert np.allclose(got, dense[:, picks].T, rtol=4e-6, atol=1e-6)
+
+
+def test_linear_strided_and_high_rank_inputs(et, device):
+    rng = np.random.default_rng(900)
+    rows, columns = 40, 1024
+    weight = synth.random_weight(synth.Q4_K, rows, columns, rng)
+    w = to_dev(weight, device)
+    Q4 = et.GgmlQuant.Q4_K
+    # every second row of a [10, K] buffer, at a storage offset that breaks 16-byte alignment
+    storage = torch.from_numpy(rng.standard_normal(3 + 10 * columns).astype(np.float32)).to(device)
+    view = storage[3:].reshape(10, columns)[::2]
+    got = et.quantized_linear(view, w, None, Q4, (rows, columns)).cpu().numpy()
+    close(got, oracle.linear_into(oracle.Q4_K, rows, columns, view.cpu().numpy(), weight))
+    # transposed (non unit trailing stride) view
+    base = torch.from_numpy(rng.standard_normal((columns, 3)).astype(np.float32)).to(device)
+    got = et.quantized_linear(base.T, w, None, Q4, (rows, columns)).cpu().numpy()
+    close(got, oracle.linear_into(oracle.Q4_K, rows, columns, np.ascontiguousarray(base.T.cpu().numpy()), weight))
+    # rank 3, with a strided bias
+    x3 = torch.from_numpy(rng.standard_normal((2, 3, columns)).astype(np.float32)).to(device)
+    bias2 = torch.from_numpy(rng.standard_normal(2 * rows).astype(np.float32)).to(device)
+    got = et.quantized_linear(x3, w, bias2[::2], Q4, (rows, columns)).cpu().numpy()
+    assert got.shape == (2, 3, rows)
+    want = oracle.linear_into(oracle.Q4_K, rows, columns, x3.cpu().numpy(), weight, bias2[::2].cpu().numpy().copy())
+    close(got, want)
+    # empty batch: nothing is dispatched
+    empty = et.quantized_linear(torch.zeros((0, columns), device=device), w, None, Q4, (rows, columns))
+    assert empty.shape == (0, rows)
+
+
+FULL = [("q8_0_gemv_4096x4096", 1), ("q4_0_gemv_11008x4096", 1), ("q4_0_gemv_11008x4096", 4),
+        ("q4_0_gemv_11008x4096", 8), ("q4_k_gemv_14336x4096", 1)]
+
+
+@pytest.mark.parametrize("name,vectors", FULL)
+def test_linear_full_size_configs(et, device, name, vectors):
+    cfg = synth.CONFIGS[name]
+    rng = np.random.default_rng(cfg["seed"])
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(vectors, cfg["columns"], rng, cfg["x_scale"])
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight)
+    want = oracle.linear_into(cfg["codec"], cfg["rows"], cfg["columns"], x, weight)
+    close(got, want)
+
+
+@pytest.mark.parametrize("vectors", [16, 64])
+def test_linear_full_size_q4k_batched_row_ranges(et, device, vectors):
+    cfg = synth.CONFIGS["q4_k_gemv_14336x4096"]
+    rng = np.random.default_rng(cfg["seed"] + vectors)
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(vectors, cfg["columns"], rng)
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight)
+    for begin in (0, 7000, cfg["rows"] - 96):
+        want = oracle.linear_rows(cfg["codec"], cfg["rows"], cfg["columns"], x, weight, None, begin, begin + 96)
+        close(got[:, begin:begin + 96], want[:, begin:begin + 96])
+    # linearity in the activations, over all rows: y(a) + y(b) ~ y(a + b)
+    x2 = synth.random_activations(vectors, cfg["columns"], rng)
+    y2 = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x2, weight)
+    y12 = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x + x2, weight)
+    close(y12, got.astype(np.float64) + y2, 2e-3)
+
+
+# --------------------------------------------------------------------------- int8-activation path
+
+@pytest.mark.parametrize("vectors,columns", [(1, 32), (5, 4096), (33, 14336), (512, 256)])
+def test_activation_quantiser_is_bit_exact(et, device, vectors, columns):
+    rng = np.random.default_rng(vectors + columns)
+    x = synth.random_activations(vectors, columns, rng, 0.5)
+    x[0, :32] = 0.0
+    q, scale, total = et.quantize_activations(to_dev(x, device))
+    wq, wscale, wtotal = oracle.quantize_q8(x)
+    assert np.array_equal(q.cpu().numpy(), wq)
+    assert np.array_equal(bits(scale.cpu().numpy().T), bits(wscale))
+    assert np.array_equal(total.cpu().numpy().T, wtotal)
+
+
+@pytest.mark.parametrize("codec", [oracle.Q8_0, oracle.Q4_0, oracle.Q4_K])
+@pytest.mark.parametrize("vectors,rows,columns", [(16, 128, 512), (64, 200, 4096), (33, 37, 1024),
+                                                  (512, 96, 2048), (1, 5, 256)])
+def test_int8_path_matches_its_oracle(et, device, codec, vectors, rows, columns):
+    rng = np.random.default_rng(codec * 7 + vectors + rows)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng, 0.5)
+    bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias, et.ActivationMode.INT8)
+    q, scale, total = oracle.quantize_q8(x)
+    want = oracle.linear_q8_rows(codec, rows, columns, q, scale, total, weight, bias)
+    close(got, want)
+    ref = oracle.linear_into(codec, rows, columns, x, weight, bias)
+    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2, axis=1, keepdims=True))
+    assert np.all(np.abs(got - ref) <= 2e-2 * np.maximum(np.abs(ref), rms))
+
+
+def test_int8_full_size_prefill_row_ranges(et, device):
+    cfg = synth.CONFIGS["q8_0_gemm_i8_512x14336x4096"]
+    rng = np.random.default_rng(cfg["seed"])
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(512, cfg["columns"], rng, cfg["x_scale"])
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight, None,
+                     et.ActivationMode.INT8)
+    q, scale, total = oracle.quantize_q8(x)
+    for begin in (0, 2048, cfg["rows"] - 16):
+        want = oracle.linear_q8_rows(cfg["codec"], cfg["rows"], cfg["columns"], q, scale, total, weight,
+                                     None, begin, begin + 16)
+        close(got[:, begin:begin + 16], want[:, begin:begin + 16])

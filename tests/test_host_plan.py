@@ -1,0 +1,153 @@
+"""Host logic of the C ABI, without a GPU: the library loads, exports every
+symbol the header declares, and the plan step validates like the reference's
+linear_requirements / embedding_requirements (crates/runtime-cpu/src/quantized.rs:297-365;
+test cases of :923-978 and crates/graph/src/lib.rs:3523-3579).
+
+Plans read metadata only, so tensors here live on the CPU or are zero-sized;
+nothing is ever launched.
+"""
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(et):
+    from effect_torch_amd import _native
+    header = open(os.path.join(ROOT, "include", "et_hip.h")).read()
+    declared = set(re.findall(r"\b(et_hip_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _native.lib()
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} is declared in et_hip.h but not exported"
+    assert declared == set(_native.SIGNATURES), declared ^ set(_native.SIGNATURES)
+
+
+def test_codec_tables(et):
+    Q = et.GgmlQuant
+    assert [(q.ggml_name, q.block_bytes) for q in (Q.Q2_K, Q.Q3_K, Q.Q4_K, Q.Q5_K, Q.Q6_K)] == [
+        ("Q2_K", 84), ("Q3_K", 110), ("Q4_K", 144), ("Q5_K", 176), ("Q6_K", 210)]
+    assert (Q.Q8_0.block_bytes, Q.Q4_0.block_bytes) == (34, 18)
+    assert Q.Q4_K.encoded_row_bytes(512) == 288      # gguf.rs:1117-1181
+    assert Q.Q4_K.encoded_row_bytes(255) is None
+    assert Q.Q4_K.encoded_row_bytes(14336) == 8064
+    assert Q.from_name("Q5_K") is Q.Q5_K and Q.from_name("Q9_K") is None
+
+
+def _w(rows, row_bytes):
+    return torch.zeros((rows, row_bytes), dtype=torch.uint8)
+
+
+def test_linear_plan_shapes(et):
+    # crates/graph/src/lib.rs:3523-3579: x [2,256], W [3,144] u8, Q4_K -> [2,3] f32
+    plan = et.linear_requirements(torch.zeros(2, 256), _w(3, 144), None, et.GgmlQuant.Q4_K, (3, 256))
+    assert plan.output_shape == (2, 3) and plan.vectors == 2
+    assert plan.output_bytes == 24  # crates/runtime-metal/src/quantized.rs:1393-1449
+    plan = et.linear_requirements(torch.zeros(2, 5, 512), _w(7, 288), torch.zeros(7), et.GgmlQuant.Q4_K, (7, 512))
+    assert plan.output_shape == (2, 5, 7) and plan.vectors == 10
+    assert plan.kernel == "gemv_fast"
+    assert plan.algorithmic_bytes == 7 * 288 + 4 * 10 * 512 + 4 * 10 * 7 + 4 * 7
+    plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 210), None, et.GgmlQuant.Q6_K, (2, 256))
+    assert plan.kernel == "gemv_generic"
+    plan = et.linear_requirements(torch.zeros(64, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256),
+                                  et.ActivationMode.INT8)
+    assert plan.kernel == "quantize_act+gemm_i8" and plan.workspace_bytes > 64 * 256
+    # empty output: nothing to dispatch
+    plan = et.linear_requirements(torch.zeros(0, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256))
+    assert plan.output_shape == (0, 2) and plan.kernel == "none"
+
+
+def test_linear_plan_rejects_malformed_geometry(et):
+    Q4 = et.GgmlQuant.Q4_K
+    x = torch.zeros(1, 256)
+    with pytest.raises(et.QuantizedError, match="input must be rank >= 2 f32"):
+        et.linear_requirements(torch.zeros(256), _w(1, 144), None, Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match="input must be rank >= 2 f32"):
+        et.linear_requirements(torch.zeros(1, 256, dtype=torch.float16), _w(1, 144), None, Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match=r"expected input trailing width 256, got \[1, 512\]"):
+        et.linear_requirements(torch.zeros(1, 512), _w(1, 144), None, Q4, (1, 256))
+    # wrong rank / width-1 / offset view -> "exact contiguous" (quantized.rs:923-960)
+    with pytest.raises(et.QuantizedError, match="exact contiguous"):
+        et.linear_requirements(x, torch.zeros(144, dtype=torch.uint8), None, Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match="exact contiguous"):
+        et.linear_requirements(x, _w(1, 143), None, Q4, (1, 256))
+    offset_view = torch.zeros(145, dtype=torch.uint8)[1:].reshape(1, 144)
+    with pytest.raises(et.QuantizedError, match=r"expected exact contiguous packed Q4_K weight \[1, 144\] u8"):
+        et.linear_requirements(x, offset_view, None, Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match="exact contiguous"):
+        et.linear_requirements(x, torch.zeros((1, 288), dtype=torch.uint8)[:, ::2], None, Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match="exact contiguous"):
+        et.linear_requirements(x, torch.zeros((1, 144), dtype=torch.float16), None, Q4, (1, 256))
+    # wrong codec for the bytes: graph/lib.rs:3570-3579
+    with pytest.raises(et.QuantizedError, match=r"expected exact contiguous packed Q5_K weight \[3, 176\] u8"):
+        et.linear_requirements(torch.zeros(2, 256), _w(3, 144), None, et.GgmlQuant.Q5_K, (3, 256))
+    with pytest.raises(et.QuantizedError, match="logical row width 255 is invalid for Q4_K"):
+        et.linear_requirements(torch.zeros(1, 255), _w(1, 0), None, Q4, (1, 255))
+    with pytest.raises(et.QuantizedError, match="byte size overflow"):
+        et.linear_requirements(x, torch.zeros(144, dtype=torch.uint8), None, Q4, (2**64 - 1, 256))
+    with pytest.raises(et.QuantizedError, match=r"bias must be \[1\] f32, got \[2\] f32"):
+        et.linear_requirements(x, _w(1, 144), torch.zeros(2), Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match=r"bias must be \[1\] f32, got \[1\] f64"):
+        et.linear_requirements(x, _w(1, 144), torch.zeros(1, dtype=torch.float64), Q4, (1, 256))
+    with pytest.raises(et.QuantizedError, match="int8 activation mode is not available for Q6_K"):
+        et.linear_requirements(x, _w(1, 210), None, et.GgmlQuant.Q6_K, (1, 256), et.ActivationMode.INT8)
+
+
+def test_embedding_plan(et):
+    Q5 = et.GgmlQuant.Q5_K
+    plan = et.embedding_requirements(torch.zeros((2, 3), dtype=torch.int64), _w(3, 176), Q5, (3, 256))
+    assert plan.output_shape == (2, 3, 256) and plan.output_bytes == 2 * 3 * 256 * 4
+    plan = et.embedding_requirements(torch.zeros(2, dtype=torch.uint32), _w(3, 176), Q5, (3, 256))
+    assert plan.output_shape == (2, 256)
+    with pytest.raises(et.QuantizedError, match="indexes must be u32 or i64, got f32"):
+        et.embedding_requirements(torch.zeros(2), _w(3, 176), Q5, (3, 256))
+    with pytest.raises(et.QuantizedError, match="quantized_embedding: expected exact contiguous"):
+        et.embedding_requirements(torch.zeros(2, dtype=torch.int64), _w(3, 175), Q5, (3, 256))
+    with pytest.raises(et.QuantizedError, match="quantized_embedding: logical row width 100"):
+        et.embedding_requirements(torch.zeros(2, dtype=torch.int64), _w(3, 0), Q5, (3, 100))
+
+
+def test_execute_revalidates_against_the_plan_and_observes_cancellation(et):
+    # validate_linear_execution (quantized.rs:367-415) runs before anything is
+    # enqueued, so these never reach a device.
+    Q4 = et.GgmlQuant.Q4_K
+    plan = et.linear_requirements(torch.zeros(2, 256), _w(3, 144), None, Q4, (3, 256))
+    dst = torch.zeros(2, 3)
+    with pytest.raises(et.QuantizedError, match="input does not match the immutable plan"):
+        et.linear_into(torch.zeros(2, 512), _w(3, 144), None, Q4, dst, plan, stream=0)
+    with pytest.raises(et.QuantizedError, match="exact contiguous"):
+        et.linear_into(torch.zeros(2, 256), _w(3, 143), None, Q4, dst, plan, stream=0)
+    with pytest.raises(et.QuantizedError, match="bias does not match the immutable plan"):
+        et.linear_into(torch.zeros(2, 256), _w(3, 144), torch.zeros(3), Q4, dst, plan, stream=0)
+    with pytest.raises(et.QuantizedError, match="destination does not match the logical node shape"):
+        et.linear_into(torch.zeros(2, 256), _w(3, 144), None, Q4, torch.zeros(2, 4), plan, stream=0)
+    flag = et.CancellationFlag()
+    flag.cancel()
+    with pytest.raises(et.Cancelled) as info:
+        et.linear_into(torch.zeros(2, 256), _w(3, 144), None, Q4, dst, plan, flag, stream=0)
+    assert str(info.value) == "operation aborted"  # quantized.rs:980-1000
+    eplan = et.embedding_requirements(torch.zeros(1, dtype=torch.uint32), _w(1, 210), et.GgmlQuant.Q6_K, (1, 256))
+    from effect_torch_amd import _native as N
+    import ctypes
+    from effect_torch_amd.quantized import _Desc
+    descs = (_Desc(torch.zeros(1, dtype=torch.uint32)), _Desc(_w(1, 210)), _Desc(torch.zeros(1, 256)))
+    status = N.lib().et_hip_embedding_into(eplan._handle, descs[0].ref, descs[1].ref, descs[2].ref,
+                                           None, None, flag.ptr)
+    assert status == N.ERR_CANCELLED and N.last_error() == "operation aborted"
+
+
+def test_embedding_status_wording(et):
+    # quantized.rs:899-921: "... index {i} is outside 0..{rows}"
+    import ctypes
+    import struct
+    from effect_torch_amd import _native as N
+    plan = et.embedding_requirements(torch.zeros(1, dtype=torch.int64), _w(1, 84), et.GgmlQuant.Q2_K, (1, 256))
+    ok = ctypes.create_string_buffer(struct.pack("<Qq", 2**64 - 1, 0), 16)
+    assert N.lib().et_hip_embedding_status_check(plan._handle, ok) == N.OK
+    for value in (-1, 1):
+        bad = ctypes.create_string_buffer(struct.pack("<Qq", 0, value), 16)
+        assert N.lib().et_hip_embedding_status_check(plan._handle, bad) == N.ERR_EXECUTION
+        assert N.last_error() == f"quantized_embedding: index {value} is outside 0..1"
