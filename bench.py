@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-GGUF matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--vectors M]
+
+A "step" is one pass of the hot path over one batch of synthetic input: one
+``quantized_linear`` of the chosen workload, enqueued through the C ABI. The
+default workload is the headline one: Q4_K dequant-GEMV, W 14336 x 4096, one
+activation vector (M = 1). Inputs are resident in HBM before the timed region.
+
+Cold HBM, not cache: the packed weight of every workload here fits the 256 MB
+Infinity Cache, so consecutive steps rotate over enough distinct weight copies
+(> 512 MiB in total) that no step can find its weight in a cache. ``--hot``
+times the same buffer over and over instead (labelled, never the headline).
+
+The K timed steps are captured once into a HIP graph (the launches go through
+the C ABI on the capturing stream) and replayed, so the device sees K kernels
+back to back without host launch gaps; HIP events on that stream bracket the
+replay. One JSON line is printed at the end.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published (5.0 POP/s)
+ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=2000)
+    p.add_argument("--warmup", type=int, default=200)
+    p.add_argument("--workload", default="q4_k_gemv_14336x4096",
+                   help="one of effect_torch_amd.synth.CONFIGS")
+    p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
+    p.add_argument("--mode", choices=["f32", "int8"], default=None)
+    p.add_argument("--hot", action="store_true", help="reuse one weight buffer (cache-resident; not the headline)")
+    p.add_argument("--no-graph", action="store_true", help="enqueue the steps one by one instead of replaying a HIP graph")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--cpu-seconds", type=float, default=10.0)
+    return p.parse_args()
+
+
+def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
+    """Times the CPU oracle (a C restatement of the reference's scalar loop,
+    crates/runtime-cpu/src/quantized.rs:447-498) on one host core over a bounded
+    sample of the same workload."""
+    import numpy as np
+    import oracle
+
+    rows, columns, codec = cfg["rows"], cfg["columns"], cfg["codec"]
+    # Size the sample from a small probe: whole calls if one fits the budget, else a row range.
+    probe_rows = min(rows, 64)
+    t0 = time.perf_counter()
+    oracle.linear_rows(codec, rows, columns, x[:1], weight, None, 0, probe_rows)
+    per_row_vector = max((time.perf_counter() - t0) / probe_rows, 1e-9)
+    full_call = per_row_vector * rows * vectors
+    if full_call <= seconds:
+        sample_rows, calls = rows, max(1, int(seconds / full_call))
+    else:
+        sample_rows, calls = max(16, int(seconds / (per_row_vector * vectors))), 1
+        sample_rows = min(sample_rows, rows)
+    y = np.zeros((vectors, rows), dtype=np.float32)
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        oracle.linear_rows(codec, rows, columns, x, weight, None, 0, sample_rows, out=y)
+    elapsed = time.perf_counter() - t0
+    seconds_per_call = elapsed / calls * (rows / sample_rows)
+    what = (f"{calls} full call(s) of the same workload" if sample_rows == rows else
+            f"rows 0..{sample_rows} of {rows} of one call, scaled by {rows / sample_rows:.1f}")
+    return {
+        "value": round(algorithmic_bytes / seconds_per_call / 1e9, 4),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"{what}; {elapsed:.1f} s of CPU work; f32 activations, scalar C restatement of the "
+                  f"reference's single-threaded loop ({seconds_per_call * 1e3:.1f} ms per call)",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import __graft_entry__ as entry
+
+    et = entry.load_package()
+    from effect_torch_amd import synth
+
+    if args.workload not in synth.CONFIGS:
+        sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)}")
+    cfg = synth.CONFIGS[args.workload]
+    vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
+    mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")
+    mode = et.ActivationMode.INT8 if mode_name == "int8" else et.ActivationMode.F32
+    codec = et.GgmlQuant(cfg["codec"])
+    rows, columns = cfg["rows"], cfg["columns"]
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    assert et.is_available(), "the visible GPU is not gfx950"
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    rng = np.random.default_rng(cfg["seed"])
+    weight_host = synth.random_weight(cfg["codec"], rows, columns, rng)
+    x_host = synth.random_activations(vectors, columns, rng, cfg["x_scale"])
+    weight_bytes = weight_host.size
+
+    copies = 1 if args.hot else max(2, -(-ROTATE_BYTES // weight_bytes))
+    base = torch.from_numpy(weight_host).to(device)
+    weights = [base]
+    for i in range(1, copies):
+        # Distinct buffers with distinct contents (rows rolled by i), same distribution.
+        weights.append(torch.roll(base, shifts=i, dims=0).contiguous())
+    x = torch.from_numpy(x_host).to(device)
+    ys = [torch.empty((vectors, rows), dtype=torch.float32, device=device) for _ in range(min(copies, 4))]
+
+    linear = et.RawLinear(codec, rows, columns, vectors, False, mode)
+    req = linear.requirements
+    workspace = (torch.empty(req.workspace_bytes, dtype=torch.uint8, device=device)
+                 if mode_name == "int8" else None)
+    algorithmic_bytes = req.algorithmic_bytes
+
+    def step(i):
+        linear.enqueue(x, weights[i % copies], None, ys[i % len(ys)], workspace)
+
+    # Parity gate before any timing: the first buffer against the CPU oracle on a row range.
+    import oracle
+    step(0)
+    torch.cuda.synchronize()
+    check_rows = min(rows, 256)
+    got = ys[0].cpu().numpy()[:, :check_rows]
+    if mode_name == "int8":
+        q, s, t = oracle.quantize_q8(x_host)
+        want = oracle.linear_q8_rows(cfg["codec"], rows, columns, q, s, t, weight_host, None, 0, check_rows)
+    else:
+        want = oracle.linear_rows(cfg["codec"], rows, columns, x_host, weight_host, None, 0, check_rows)
+    want = want[:, :check_rows]
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= 1e-3 * np.maximum(np.abs(want), 1.0) + 4e-5 * rms), \
+        f"parity gate failed: max |err| {err.max():.4g}"
+
+    stream = torch.cuda.current_stream()
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(args.steps):
+                    step(i)
+            graph.replay()  # one untimed replay
+            torch.cuda.synchronize()
+        except Exception as exc:  # noqa: BLE001 - report and fall back to plain enqueues
+            print(f"HIP graph capture failed ({exc}); timing plain enqueues", file=sys.stderr)
+            graph = None
+            torch.cuda.synchronize()
+
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    start.record(stream)
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(args.steps):
+            step(i)
+    stop.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    gpu_ms = start.elapsed_time(stop)
+    ms_per_step = gpu_ms / args.steps
+    seconds_per_step = ms_per_step * 1e-3
+
+    gbs = algorithmic_bytes / seconds_per_step / 1e9
+    ops = 2.0 * vectors * rows * columns
+    if mode_name == "int8" and vectors >= 256:
+        roofline = {"bound": "mfma", "achieved": round(ops / seconds_per_step / 1e12, 3),
+                    "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
+                    "frac": round(ops / seconds_per_step / 1e12 / INT8_PEAK_TOPS, 4), "traffic": None}
+    else:
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+    roofline["kernel"] = req.kernel
+    roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes
+    roofline["avg_launch_us"] = round(ms_per_step * 1e3, 3)
+
+    result = {
+        "metric": "Q4_K dequant-GEMV HBM GB/s (% peak) at 14336x4096; batched decode tok/s"
+                  if args.workload == "q4_k_gemv_14336x4096" else f"{args.workload} GB/s",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8" if mode_name == "int8" else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload} M={vectors} ({codec.ggml_name} W {rows}x{columns}, {mode_name} activations)",
+            "weights": "hot: one buffer, cache resident" if args.hot else
+                       f"cold: rotating over {copies} distinct weight buffers ({copies * weight_bytes >> 20} MiB)",
+            "launch": "hipgraph replay of the K steps" if graph is not None else "K plain enqueues",
+            "percent_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+            "host_wall_ms": round(wall * 1e3, 3),
+        },
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg, vectors, mode_name, weight_host, x_host,
+                                              args.cpu_seconds, algorithmic_bytes)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -16,7 +16,9 @@ BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q2_K: 84, Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6
 # byte offsets of the fp16 fields of a block
 _FP16_FIELDS = {Q4_0: (0,), Q8_0: (0,), Q2_K: (80, 82), Q3_K: (108,), Q4_K: (0, 2), Q5_K: (0, 2),
                 Q6_K: (208,)}
-DEFAULT_SCALE = {Q4_0: 0.02, Q8_0: 0.01, Q2_K: 0.01, Q3_K: 0.01, Q4_K: 0.01, Q5_K: 0.01, Q6_K: 0.01}
+# Q4_0 / Q8_0 / Q4_K: the scales the workload definitions name. The others are chosen so
+# that decoded weights have a comparable magnitude (a few units).
+DEFAULT_SCALE = {Q4_0: 0.02, Q8_0: 0.01, Q2_K: 0.1, Q3_K: 0.05, Q4_K: 0.01, Q5_K: 0.005, Q6_K: 0.002}
 
 
 def row_bytes(codec: int, columns: int) -> int:

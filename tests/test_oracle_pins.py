@@ -293,9 +293,11 @@ def test_linear_q8_against_integer_brute_force_and_f32_reference(codec):
     xq = (q.reshape(vectors, -1, 32).astype(np.float64) * scale[:, :, None].astype(np.float64))
     model = xq.reshape(vectors, columns) @ dense.T
     assert np.allclose(got, model, rtol=0, atol=2e-4 * np.abs(dense).max() * np.sqrt(columns))
-    # and it stays within 2e-2 of the f32-activation reference, relative to the
-    # larger of |ref| and the RMS of that vector's outputs (int8 rounding noise
-    # scales with |w|.|x|, not with the possibly tiny individual output)
-    ref = oracle.linear_into(codec, rows, columns, x, weight)
-    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2, axis=1, keepdims=True))
-    assert np.all(np.abs(got - ref) <= 2e-2 * np.maximum(np.abs(ref), rms))
+    # and it stays within 2e-2 of the f32-activation reference: per vector, in
+    # relative L2 and elementwise against the vector's peak output (int8 rounding
+    # noise scales with |w|.|x|, not with the possibly tiny individual output)
+    ref = oracle.linear_into(codec, rows, columns, x, weight).astype(np.float64)
+    l2 = np.linalg.norm(got - ref, axis=1) / np.linalg.norm(ref, axis=1)
+    assert np.all(l2 <= 2e-2)
+    peak = np.abs(ref).max(axis=1, keepdims=True)
+    assert np.all(np.abs(got - ref) <= 2e-2 * np.maximum(np.abs(ref), peak))
