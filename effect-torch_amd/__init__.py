@@ -13,6 +13,8 @@ from .quantized import (  # noqa: F401
     QuantizedError,
     QuantizedRequirements,
     RawLinear,
+    calibration_copy,
+    calibration_read,
     dequantize_rows,
     embedding_into,
     embedding_requirements,

@@ -28,9 +28,11 @@ COMMON = [
 SOURCES = {
     "dequant.hip": ["-ffp-contract=off"],
     "gemv_fast.hip": [],
+    "gemv_limb.hip": [],
     "gemv_generic.hip": [],
     "quantize_act.hip": ["-ffp-contract=off"],
     "gemm_i8.hip": [],
+    "calibrate.hip": [],
     "quantized.cpp": [],
     "c_api.cpp": [],
 }

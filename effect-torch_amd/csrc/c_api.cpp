@@ -298,6 +298,41 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
     });
 }
 
+int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
+                            void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (src == nullptr || sink == nullptr || workgroups == 0 ||
+            reinterpret_cast<uintptr_t>(src) % 16 != 0) {
+            *error = "calibration_read: source must be 16-byte aligned, sink non-NULL, workgroups > 0";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status =
+            et::calibration_read(src, bytes, sink, workgroups, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("calibration_read: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
+int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (src == nullptr || dst == nullptr || reinterpret_cast<uintptr_t>(src) % 16 != 0 ||
+            reinterpret_cast<uintptr_t>(dst) % 16 != 0) {
+            *error = "calibration_copy: buffers must be non-NULL and 16-byte aligned";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status =
+            et::calibration_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("calibration_copy: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
 const char* et_hip_last_error(void) { return g_last_error.c_str(); }
 
 }  // extern "C"

@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 
 #include "et_codecs.h"
 #include "gemv_common.h"
@@ -412,10 +414,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_kernel(
 
 template <class T, int M, int R, int WAVES, int NK>
 hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
-                  float* y, uint32_t rows, uint32_t columns, hipStream_t stream) {
+                  float* y, uint32_t rows, uint32_t columns, hipStream_t stream, uint32_t rpw = 0) {
     constexpr int RG = WAVES / NK;
     // One contiguous range of rows per CU, rounded to whole iterations.
-    uint32_t rows_per_wg = (rows + 255u) / 256u;
+    uint32_t rows_per_wg = rpw ? rpw : (rows + 255u) / 256u;
     rows_per_wg = ((rows_per_wg + RG * R - 1) / (RG * R)) * (RG * R);
     const uint32_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL((gemv_kernel<T, M, R, WAVES, NK>), dim3(grid), dim3(64 * WAVES), 0, stream,
@@ -458,6 +460,21 @@ hipError_t gemv_fast(int32_t codec, const uint8_t* weight, const float* x, uint6
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
                      hipStream_t stream) {
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
+    if (codec == kQ4_K && vectors == 1 && k <= 4096 && getenv("ET_EXP")) {  // EXPERIMENT HOOK
+        int w = 4, r = 2, rpw = 0;
+        sscanf(getenv("ET_EXP"), "%d,%d,%d", &w, &r, &rpw);
+        using T = Q4KTraits<false>;
+        if (w == 4 && r == 2) return launch<T, 1, 2, 4, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 4 && r == 1) return launch<T, 1, 1, 4, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 4 && r == 4) return launch<T, 1, 4, 4, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 8 && r == 2) return launch<T, 1, 2, 8, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 8 && r == 1) return launch<T, 1, 1, 8, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 8 && r == 4) return launch<T, 1, 4, 8, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 16 && r == 1) return launch<T, 1, 1, 16, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 12 && r == 1) return launch<T, 1, 1, 12, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        if (w == 12 && r == 2) return launch<T, 1, 2, 12, 1>(weight, x, x_row_stride, bias, y, n, k, stream, rpw);
+        return hipErrorInvalidValue;
+    }
     if (codec == kQ4_K) {
         switch (vectors) {
             case 1: return launch_slices<Q4KTraits<false>, 1, 2>(weight, x, x_row_stride, bias, y, n, k, stream);

@@ -1,0 +1,636 @@
+// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q4_0, Q8_0; 1-4 vectors):
+//     y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r])
+//
+// Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499)
+// with decode_q4_k (:180-199) in factored form; Q4_0 / Q8_0 follow the public
+// ggml block layouts. f32-accurate: the result agrees with the scalar f32 loop
+// within 1e-3 (in fact to a few 1e-6 relative).
+//
+// Why integers. The kernel is HBM-bound (0.56 - 1.06 bytes per weight), and on
+// CDNA4 the obvious f32 formulation (byte -> float convert + FMA per weight) is
+// VALU-bound before it is HBM-bound: ~2.4 vector ops per weight. Here each f32
+// activation is converted ONCE per workgroup to a 24-bit fixed-point integer
+// with a shared scale per 64 columns, X = rint(x * 127 * 2^16 / max|x|), and X
+// is cut into three signed 8-bit limbs,
+//     x ~= s * (65536*x1 + 256*x2 + x3),   |residual| <= 6.0e-8 * max|x|,
+// i.e. to f32 precision. The weights' quants - already small integers - meet
+// the limbs in v_dot4_i32_i8: 4 multiply-adds per op, three ops per four
+// weights, exact int32 accumulation. Block scales are applied to the integer
+// sums in f32 afterwards. ~1.3 vector ops per weight.
+//
+// Work split (activation-stationary): a lane owns 64 consecutive columns (one
+// 32-byte pair of a Q4_K super-block, or two Q4_0 / Q8_0 blocks), keeps their
+// limbs in registers for its whole life, and streams weight rows past them with
+// 16-byte loads. A wave covers 4096 columns, NK waves a row; their partial sums
+// meet in LDS. A workgroup walks a contiguous range of rows.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+#include "et_codecs.h"
+#include "gemv_common.h"
+#include "kernels.h"
+
+#ifdef ET_TRACE
+// Debug build only: per-wave timestamps (100 MHz wall clock), kept in registers
+// and written once at the end of the wave.
+__device__ unsigned long long* g_et_trace = nullptr;
+#define ET_STAMP_DECL unsigned long long et_stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define ET_STAMP(k) et_stamps[k] = wall_clock64()
+#define ET_STAMP_FLUSH()                                                                         \
+    do {                                                                                         \
+        if (g_et_trace != nullptr && (threadIdx.x & 63u) == 0)                                   \
+            for (int k_ = 0; k_ < 8; k_++)                                                       \
+                g_et_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + k_] = \
+                    et_stamps[k_];                                                               \
+    } while (0)
+extern "C" int et_dbg_set_trace(unsigned long long* buffer) {
+    return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(g_et_trace), &buffer, sizeof buffer));
+}
+#else
+#define ET_STAMP_DECL
+#define ET_STAMP(k) do {} while (0)
+#define ET_STAMP_FLUSH() do {} while (0)
+#endif
+
+namespace et {
+namespace {
+
+constexpr int kChunk = 64;                       // columns a lane owns
+constexpr uint32_t kSliceColumns = 64 * kChunk;  // columns a wave covers
+constexpr uint32_t kSliceQuads = kSliceColumns / 4;
+
+// Per-vector lane state: the limbs of the lane's 64 activations and their sums.
+struct XLimbs {
+    int limb[3][16];  // limb[k][j]: bytes = limb k of elements 4j..4j+3 of the chunk;
+                      // limb 0 is the least significant (weight 1), limb 2 the most (65536)
+    float s;          // value of one unit of limb 0
+    float sum[2];     // exact f32 sums of elements 0..31 and 32..63
+};
+
+constexpr float kLimbRange = 8323072.0f;  // 127 * 2^16: |X| <= this
+
+// LDS slot (in 16-byte units) of limb unit u = 4*chunk + j: the XOR spreads the
+// eight lanes that read in one pass over all banks; writes of consecutive dwords
+// stay conflict-free because it only permutes within aligned groups of four units.
+__device__ __forceinline__ uint32_t limb_slot(uint32_t u) { return u ^ ((u >> 3) & 3u); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+struct alignas(16) StageMemory {
+    uint32_t limbs[3][kSliceQuads];  // [limb][swizzled dword]
+    float unit[64];
+    float sum[2][64];
+};
+
+// Splits one float4 of a slice into limbs and stores them in LDS. Float4 number f
+// of the slice belongs to thread f % THREADS; sixteen consecutive lanes (one DPP
+// row) hold one 64-column chunk, so the chunk's maximum and its two 32-column
+// sums are folded across lanes with DPP. Must be called by whole waves.
+//
+// X = rint(x * inv) is an exact integer of at most 24 bits. Adding 0x8080 and
+// flipping the top bit of the two low bytes turns its bytes into balanced
+// digits: X = 65536*x1 + 256*x2 + x3 with every x_k a signed byte.
+__device__ __forceinline__ void stage_quad(StageMemory& stage, float4 v, uint32_t f) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, dpp<0xB1>(amax));   // quad_perm [1,0,3,2]
+    amax = fmaxf(amax, dpp<0x4E>(amax));   // quad_perm [2,3,0,1]
+    amax = fmaxf(amax, dpp<0x141>(amax));  // row_half_mirror
+    amax = fmaxf(amax, dpp<0x140>(amax));  // row_mirror: all 16 lanes hold the chunk's max
+    float total = (v.x + v.y) + (v.z + v.w);
+    total += dpp<0xB1>(total);
+    total += dpp<0x4E>(total);
+    total += dpp<0x141>(total);  // sum over the lane's 8-lane half = 32 columns
+    // 1 ulp of the reciprocal moves |X| by at most 1, far inside the headroom of the limbs.
+    const bool nonzero = amax >= 1e-30f;
+    const float inv = nonzero ? kLimbRange * __builtin_amdgcn_rcpf(amax) : 0.f;
+    const float unit = nonzero ? amax * (1.0f / kLimbRange) : 0.f;
+    const int x0 = static_cast<int>(rintf(v.x * inv)) + 0x8080;
+    const int x1 = static_cast<int>(rintf(v.y * inv)) + 0x8080;
+    const int x2 = static_cast<int>(rintf(v.z * inv)) + 0x8080;
+    const int x3 = static_cast<int>(rintf(v.w * inv)) + 0x8080;
+    // 4x3 byte transpose: limb k of the four elements into one dword.
+    const uint32_t a = __builtin_amdgcn_perm(x1, x0, 0x05010400u);  // x0.b0 x1.b0 x0.b1 x1.b1
+    const uint32_t b = __builtin_amdgcn_perm(x3, x2, 0x05010400u);
+    const uint32_t c = __builtin_amdgcn_perm(x1, x0, 0x0c0c0602u);  // x0.b2 x1.b2 0 0
+    const uint32_t d = __builtin_amdgcn_perm(x3, x2, 0x0c0c0602u);
+    const uint32_t limb0 = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
+    const uint32_t limb1 = __builtin_amdgcn_perm(b, a, 0x07060302u) ^ 0x80808080u;
+    const uint32_t limb2 = __builtin_amdgcn_perm(d, c, 0x05040100u);
+    const uint32_t slot = limb_slot(f >> 2) * 4u + (f & 3u);
+    stage.limbs[0][slot] = limb0;
+    stage.limbs[1][slot] = limb1;
+    stage.limbs[2][slot] = limb2;
+    const uint32_t chunk = f >> 4;
+    if ((f & 15u) == 0u) stage.unit[chunk] = unit;
+    if ((f & 7u) == 0u) stage.sum[(f >> 3) & 1u][chunk] = total;
+}
+
+__device__ __forceinline__ void load_limbs(const StageMemory& stage, uint32_t lane, bool active,
+                                           XLimbs& out) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint4 v = *reinterpret_cast<const uint4*>(&stage.limbs[k][limb_slot(4u * lane + j) * 4u]);
+            out.limb[k][4 * j + 0] = active ? static_cast<int>(v.x) : 0;
+            out.limb[k][4 * j + 1] = active ? static_cast<int>(v.y) : 0;
+            out.limb[k][4 * j + 2] = active ? static_cast<int>(v.z) : 0;
+            out.limb[k][4 * j + 3] = active ? static_cast<int>(v.w) : 0;
+        }
+    }
+    out.s = active ? stage.unit[lane] : 0.f;
+    out.sum[0] = active ? stage.sum[0][lane] : 0.f;
+    out.sum[1] = active ? stage.sum[1][lane] : 0.f;
+}
+
+// s * (D0 + 256*D1 + 65536*D2) for the integer dots D_k of the three limbs.
+__device__ __forceinline__ float limb_value(const XLimbs& x, int d0, int d1, int d2) {
+    float v = static_cast<float>(d0);
+    v = fmaf(256.0f, static_cast<float>(d1), v);
+    v = fmaf(65536.0f, static_cast<float>(d2), v);
+    return x.s * v;
+}
+
+// ---------------------------------------------------------------------------
+// Codec traits: what a lane loads per row and how it folds it with the limbs.
+// ---------------------------------------------------------------------------
+
+struct Q4KLimb {
+    struct Lane {
+        uint32_t offset;  // byte offset of the lane's block within a row
+        uint32_t p;       // pair within the block
+    };
+    struct Data {
+        uint4 header;  // d, dmin, scales[12]
+        uint4 q[2];    // the pair's 32 bytes of quants
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 8) * 144u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) {
+        return Lane{(chunk >> 2) * 144u, chunk & 3u};
+    }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        const uint8_t* base = row + lane.offset;
+        data.header = *reinterpret_cast<const uint4*>(base);
+        data.q[0] = *reinterpret_cast<const uint4*>(base + 16 + 32 * lane.p);
+        data.q[1] = *reinterpret_cast<const uint4*>(base + 32 + 32 * lane.p);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
+                                                const XLimbs (&x)[M], float (&value)[M]) {
+        const uint32_t w[8] = {data.q[0].x, data.q[0].y, data.q[0].z, data.q[0].w,
+                               data.q[1].x, data.q[1].y, data.q[1].z, data.q[1].w};
+        int lo[M][3], hi[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int k = 0; k < 3; k++) lo[m][k] = hi[m][k] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            // low nibbles: elements 4j..4j+3 of sub-block 2p; high nibbles: of sub-block 2p+1
+            const int ql = static_cast<int>(w[j] & 0x0f0f0f0fu);
+            const int qh = static_cast<int>((w[j] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    lo[m][k] = __builtin_amdgcn_sdot4(ql, x[m].limb[k][j], lo[m][k], false);
+                    hi[m][k] = __builtin_amdgcn_sdot4(qh, x[m].limb[k][8 + j], hi[m][k], false);
+                }
+        }
+        // (scale, min) of sub-blocks 2p, 2p+1: crates/runtime-cpu/src/quantized.rs:77-86
+        const uint32_t shift = (lane.p & 1u) * 16u;
+        const uint32_t a = data.header.y >> shift, b = data.header.z >> shift, c = data.header.w >> shift;
+        uint32_t sc, mn;
+        if (lane.p < 2) {
+            sc = a & 0x3f3fu;
+            mn = b & 0x3f3fu;
+        } else {
+            sc = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+            mn = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+        }
+        const float sc_lo = static_cast<float>(sc & 0xffu), sc_hi = static_cast<float>((sc >> 8) & 0xffu);
+        const float m_lo = static_cast<float>(mn & 0xffu), m_hi = static_cast<float>((mn >> 8) & 0xffu);
+        const float d = half_bits_to_float(data.header.x & 0xffffu);
+        const float dmin = half_bits_to_float(data.header.x >> 16);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            // sub-block scales first, limb weights second, one f32 scale last
+            // (as floats: the dots are below 2^17 and convert exactly; a 32-bit
+            // integer multiply would run at quarter rate)
+            const float i1 = fmaf(sc_hi, static_cast<float>(hi[m][0]), sc_lo * static_cast<float>(lo[m][0]));
+            const float i2 = fmaf(sc_hi, static_cast<float>(hi[m][1]), sc_lo * static_cast<float>(lo[m][1]));
+            const float i3 = fmaf(sc_hi, static_cast<float>(hi[m][2]), sc_lo * static_cast<float>(lo[m][2]));
+            const float pos = x[m].s * fmaf(65536.0f, i3, fmaf(256.0f, i2, i1));
+            const float neg = fmaf(m_lo, x[m].sum[0], m_hi * x[m].sum[1]);
+            value[m] = d * pos - dmin * neg;
+        }
+    }
+};
+
+struct __attribute__((packed, aligned(4))) Dwords9 {
+    uint32_t v[9];
+};
+struct __attribute__((packed, aligned(4))) Dwords17 {
+    uint32_t v[17];
+};
+
+// Q4_0: two 18-byte blocks = 36 bytes = 9 dwords (dword aligned when columns % 64 == 0).
+struct Q40Limb {
+    struct Lane {
+        uint32_t offset;
+    };
+    struct Data {
+        Dwords9 raw;
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 5) * 18u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) { return Lane{chunk * 36u}; }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        data.raw = *reinterpret_cast<const Dwords9*>(row + lane.offset);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane&, const XLimbs (&x)[M],
+                                                float (&value)[M]) {
+        const uint32_t* w = data.raw.v;
+        int da_[M][3], db_[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int k = 0; k < 3; k++) da_[m][k] = db_[m][k] = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            // block A: bytes 2..17 of the pair (2 bytes off dword alignment); block B: bytes 20..35.
+            // Byte j's low nibble is element j, its high nibble element j + 16.
+            const uint32_t qa = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
+            const uint32_t qb = w[5 + i];
+            const int al = static_cast<int>(qa & 0x0f0f0f0fu), ah = static_cast<int>((qa >> 4) & 0x0f0f0f0fu);
+            const int bl = static_cast<int>(qb & 0x0f0f0f0fu), bh = static_cast<int>((qb >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    da_[m][k] = __builtin_amdgcn_sdot4(al, x[m].limb[k][i], da_[m][k], false);
+                    da_[m][k] = __builtin_amdgcn_sdot4(ah, x[m].limb[k][4 + i], da_[m][k], false);
+                    db_[m][k] = __builtin_amdgcn_sdot4(bl, x[m].limb[k][8 + i], db_[m][k], false);
+                    db_[m][k] = __builtin_amdgcn_sdot4(bh, x[m].limb[k][12 + i], db_[m][k], false);
+                }
+        }
+        const float da = half_bits_to_float(w[0] & 0xffffu);
+        const float db = half_bits_to_float(w[4] >> 16);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            // value = d * (nibble - 8): the -8 meets the chunk's activation sums once
+            const float va = limb_value(x[m], da_[m][0], da_[m][1], da_[m][2]) - 8.f * x[m].sum[0];
+            const float vb = limb_value(x[m], db_[m][0], db_[m][1], db_[m][2]) - 8.f * x[m].sum[1];
+            value[m] = da * va + db * vb;
+        }
+    }
+};
+
+// Q8_0: two 34-byte blocks = 68 bytes = 17 dwords (dword aligned when columns % 64 == 0).
+struct Q80Limb {
+    struct Lane {
+        uint32_t offset;
+    };
+    struct Data {
+        Dwords17 raw;
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 5) * 34u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) { return Lane{chunk * 68u}; }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        data.raw = *reinterpret_cast<const Dwords17*>(row + lane.offset);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane&, const XLimbs (&x)[M],
+                                                float (&value)[M]) {
+        const uint32_t* w = data.raw.v;
+        int da_[M][3], db_[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int k = 0; k < 3; k++) da_[m][k] = db_[m][k] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int qa = static_cast<int>(__builtin_amdgcn_alignbit(w[i + 1], w[i], 16));  // bytes 2..33
+            const int qb = static_cast<int>(w[9 + i]);                                        // bytes 36..67
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    da_[m][k] = __builtin_amdgcn_sdot4(qa, x[m].limb[k][i], da_[m][k], false);
+                    db_[m][k] = __builtin_amdgcn_sdot4(qb, x[m].limb[k][8 + i], db_[m][k], false);
+                }
+        }
+        const float da = half_bits_to_float(w[0] & 0xffffu);
+        const float db = half_bits_to_float(w[8] >> 16);
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            value[m] = da * limb_value(x[m], da_[m][0], da_[m][1], da_[m][2]) +
+                       db * limb_value(x[m], db_[m][0], db_[m][1], db_[m][2]);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// The kernel. M vectors, R rows per wave iteration, WAVES waves per workgroup,
+// NK waves per row (so WAVES / NK row groups per workgroup).
+//
+// A 33 MB GEMV lasts only a few microseconds, comparable to a handful of HBM
+// round trips, so what counts is how early the whole weight matrix is in
+// flight. LOOP = false is the single-shot form: every wave requests ALL its rows
+// (R <= 8) as its very first instructions after the activation loads, then
+// prepares the activations while the weights travel, then folds the rows as
+// they arrive. LOOP = true keeps two R-row buffers in ping-pong for shapes
+// whose rows per wave do not fit registers.
+// ---------------------------------------------------------------------------
+template <class T, int M, int R, int WAVES, int NK, bool LOOP>
+__global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
+    const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
+    const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
+    uint32_t rows_per_wg) {
+    constexpr int RG = WAVES / NK;
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int NI = (kSliceQuads + THREADS - 1) / THREADS;  // float4s per thread and slice
+    __shared__ StageMemory stage[M];
+    __shared__ float partial[2][RG][NK][R][M];
+    const uint32_t lane_id = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t slice = wave % NK;
+    const uint32_t group = wave / NK;
+    const uint32_t all_quads = columns >> 2;
+
+    // Activation loads first: they are served by L2 and must not queue behind
+    // the weight loads (a wave's loads complete in order).
+    auto load_x = [&](uint32_t s, float4 (&xv)[M][NI]) {
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                const uint32_t f = threadIdx.x + i * THREADS;
+                const uint32_t quad = s * kSliceQuads + f;
+                xv[m][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (f < kSliceQuads && quad < all_quads)
+                    xv[m][i] = reinterpret_cast<const float4*>(x + m * x_row_stride)[quad];
+            }
+    };
+    ET_STAMP_DECL;
+    ET_STAMP(0);
+    float4 xv[M][NI];
+    load_x(0, xv);
+
+    const uint32_t chunk = slice * 64u + lane_id;  // which 64-column stretch of the row
+    const bool active = chunk < columns / kChunk;
+    const typename T::Lane lane = T::lane_setup(active ? chunk : 0u);
+    const uint64_t row_bytes = T::row_bytes(columns);
+
+    const uint32_t wg_row0 = blockIdx.x * rows_per_wg;
+    const uint32_t wg_row_end = min(wg_row0 + rows_per_wg, rows);
+    const uint32_t iterations = LOOP ? (wg_row_end - wg_row0 + RG * R - 1) / (RG * R) : 1u;
+
+    auto load_row = [&](uint32_t it, int r, typename T::Data& data) {
+        uint32_t row = wg_row0 + (it * RG + group) * R + r;
+        row = min(row, rows - 1);  // rows past the end re-read a valid row and are discarded
+        T::load(weight + row * row_bytes, lane, data);
+    };
+    auto load_rows = [&](uint32_t it, typename T::Data (&data)[R]) {
+#pragma unroll
+        for (int r = 0; r < R; r++) load_row(it, r, data[r]);
+    };
+
+    // Order of the prologue. A wave that issues a load while the CU's memory
+    // queue is full stalls, and so does everything behind the load in program
+    // order; once the weights of a whole CU are requested the queue stays full
+    // for microseconds. The activations, which the whole workgroup needs before
+    // the first multiply, therefore go first: (1) activation loads, (2) ONE row
+    // of weights, so that HBM has work during the activation round trip,
+    // (3) split the activations as soon as they are back, (4) barrier, (5) only
+    // then the rest of the rows, which may stall freely.
+    typename T::Data current[R];
+    load_row(0, 0, current[0]);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Activations: limbs in LDS -> registers, one 4096-column slice at a time.
+    XLimbs xr[M];
+    for (uint32_t s = 0; s < NK; s++) {
+        if (s != 0) {
+            __syncthreads();
+            load_x(s, xv);
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                const uint32_t f = threadIdx.x + i * THREADS;
+                if (f < kSliceQuads) stage_quad(stage[m], xv[m][i], f);  // wave-uniform condition
+            }
+        ET_STAMP(1);
+        __syncthreads();
+        ET_STAMP(2);
+        if (s == slice) {
+#pragma unroll
+            for (int m = 0; m < M; m++) load_limbs(stage[m], lane_id, active, xr[m]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#ifdef ET_TRACE
+    asm volatile("" ::"v"(xr[0].limb[2][15]), "v"(xr[0].sum[1]));
+    ET_STAMP(3);
+#endif
+
+    // Writes the outputs of iteration `it` from the per-row totals.
+    auto write_rows = [&](uint32_t it, const float (&total)[R][M]) {
+        const uint32_t row0 = wg_row0 + (it * RG + group) * R;
+        if (NK == 1) {
+            if (lane_id == 0) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const uint32_t row = row0 + r;
+                    if (row < wg_row_end) {
+                        const float b = bias != nullptr ? bias[row] : 0.f;
+#pragma unroll
+                        for (int m = 0; m < M; m++)
+                            y[static_cast<uint64_t>(m) * rows + row] =
+                                bias != nullptr ? total[r][m] + b : total[r][m];
+                    }
+                }
+            }
+        } else {
+            const uint32_t parity = it & 1u;
+            if (lane_id == 0) {
+#pragma unroll
+                for (int r = 0; r < R; r++)
+#pragma unroll
+                    for (int m = 0; m < M; m++) partial[parity][group][slice][r][m] = total[r][m];
+            }
+            __syncthreads();
+            if (slice == 0 && lane_id < R * M) {
+                const uint32_t r = lane_id / M, m = lane_id - r * M;
+                const uint32_t row = row0 + r;
+                if (row < wg_row_end) {
+                    float value = 0.f;
+                    for (int s = 0; s < NK; s++) value += partial[parity][group][s][r][m];
+                    if (bias != nullptr) value += bias[row];
+                    y[static_cast<uint64_t>(m) * rows + row] = value;
+                }
+            }
+        }
+    };
+    auto fold_row = [&](const typename T::Data& data, float (&total)[M]) {
+        float value[M];
+        T::template fold<M>(data, lane, xr, value);
+#pragma unroll
+        for (int m = 0; m < M; m++) total[m] = wave_sum(active ? value[m] : 0.f);
+    };
+
+    if (!LOOP) {
+        // Request row r+1, then fold row r: a request that stalls on a full
+        // queue stalls behind useful work, and rows are folded as they arrive.
+        float total[R][M];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (r + 1 < R) load_row(0, r + 1, current[r + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            fold_row(current[r], total[r]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        ET_STAMP(5);
+        write_rows(0, total);
+        ET_STAMP(6);
+        ET_STAMP_FLUSH();
+    } else {
+        // Two R-row buffers in ping-pong. Row 0 of the first is already on its way.
+        typename T::Data other[R];
+#pragma unroll
+        for (int r = 1; r < R; r++) load_row(0, r, current[r]);
+        float total[R][M];
+        for (uint32_t it = 0; it < iterations; it += 2) {
+            if (it + 1 < iterations) load_rows(it + 1, other);
+#pragma unroll
+            for (int r = 0; r < R; r++) fold_row(current[r], total[r]);
+            write_rows(it, total);
+            if (it + 1 < iterations) {
+                if (it + 2 < iterations) load_rows(it + 2, current);
+#pragma unroll
+                for (int r = 0; r < R; r++) fold_row(other[r], total[r]);
+                write_rows(it + 1, total);
+            }
+        }
+        ET_STAMP(6);
+        ET_STAMP_FLUSH();
+    }
+}
+
+template <class T, int M, int R, int WAVES, int NK, bool LOOP>
+hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
+                  float* y, uint32_t rows, uint32_t columns, uint32_t rows_per_wg, hipStream_t stream) {
+    const uint32_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    hipLaunchKernelGGL((gemv_limb_kernel<T, M, R, WAVES, NK, LOOP>), dim3(grid), dim3(64 * WAVES), 0,
+                       stream, weight, x, x_row_stride, bias, y, rows, columns, rows_per_wg);
+    return hipGetLastError();
+}
+
+// Picks rows per workgroup and the single-shot depth for WAVES / NK row groups.
+template <class T, int M, int WAVES, int NK>
+hipError_t launch_rows(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
+                       float* y, uint32_t rows, uint32_t columns, hipStream_t stream,
+                       uint32_t force_depth = 0) {
+    constexpr uint32_t RG = WAVES / NK;
+    // One contiguous range of rows per CU; a wave takes ceil(range / RG) of them.
+    const uint32_t share = (rows + 255u) / 256u;
+    uint32_t depth = (share + RG - 1) / RG;
+    if (force_depth) depth = force_depth;
+    // Registers bound the single-shot depth: 4 rows with more than 8 waves (128 VGPRs), else 8.
+    constexpr uint32_t kMaxDepth = (WAVES > 8 || M > 1) ? 4 : 8;
+#define ET_SHOT(D)                                                                               \
+    case D:                                                                                      \
+        return launch<T, M, D, WAVES, NK, false>(weight, x, x_row_stride, bias, y, rows, columns, \
+                                                 RG * D, stream)
+    if (depth <= kMaxDepth) {
+        switch (depth) {
+            ET_SHOT(1);
+            ET_SHOT(2);
+            ET_SHOT(3);
+            ET_SHOT(4);
+            default: break;
+        }
+        if (kMaxDepth == 8) {
+            switch (depth) {
+                case 5: return launch<T, M, (kMaxDepth == 8 ? 5 : 1), WAVES, NK, false>(weight, x, x_row_stride, bias, y, rows, columns, RG * 5, stream);
+                case 6: return launch<T, M, (kMaxDepth == 8 ? 6 : 1), WAVES, NK, false>(weight, x, x_row_stride, bias, y, rows, columns, RG * 6, stream);
+                case 7: return launch<T, M, (kMaxDepth == 8 ? 7 : 1), WAVES, NK, false>(weight, x, x_row_stride, bias, y, rows, columns, RG * 7, stream);
+                case 8: return launch<T, M, (kMaxDepth == 8 ? 8 : 1), WAVES, NK, false>(weight, x, x_row_stride, bias, y, rows, columns, RG * 8, stream);
+                default: break;
+            }
+        }
+    }
+#undef ET_SHOT
+    // Too many rows per wave for registers: loop with two 2-row buffers.
+    const uint32_t rows_per_wg = ((share + RG * 2 - 1) / (RG * 2)) * (RG * 2);
+    return launch<T, M, 2, WAVES, NK, true>(weight, x, x_row_stride, bias, y, rows, columns,
+                                            rows_per_wg, stream);
+}
+
+template <class T, int M>
+hipError_t launch_slices(const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                         const float* bias, float* y, uint32_t rows, uint32_t columns,
+                         hipStream_t stream) {
+    const uint32_t slices = (columns + kSliceColumns - 1) / kSliceColumns;
+    if (slices <= 1) {
+        if (M == 1 && getenv("ET_EXP")) {  // EXPERIMENT HOOK "waves,depth"
+            int w = 8, d = 0;
+            sscanf(getenv("ET_EXP"), "%d,%d", &w, &d);
+            if (w == 14) return launch_rows<T, 1, 14, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream, d);
+            if (w == 16) return launch_rows<T, 1, 16, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream, d);
+        }
+        return launch_rows<T, M, 8, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    }
+    if (slices <= 2) return launch_rows<T, M, 8, 2>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    if (slices <= 4) return launch_rows<T, M, 8, 4>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    if (slices <= 8) return launch_rows<T, M, 8, 8>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    return launch_rows<T, M, 16, 16>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+}
+
+template <class T>
+hipError_t launch_vectors(const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                          const float* bias, float* y, uint32_t rows, uint32_t columns,
+                          uint32_t vectors, hipStream_t stream) {
+    switch (vectors) {
+        case 1: return launch_slices<T, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+        case 2: return launch_slices<T, 2>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+        case 3: return launch_slices<T, 3>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors) {
+    if (vectors == 0 || vectors > kGemvLimbMaxVectors || columns == 0 || columns > 65536u) return false;
+    if (codec == kQ4_K) return columns % 256 == 0;
+    if (codec == kQ4_0 || codec == kQ8_0) return columns % 64 == 0;
+    return false;
+}
+
+hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                     const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
+                     hipStream_t stream) {
+    const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
+    switch (codec) {
+        case kQ4_K: return launch_vectors<Q4KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ4_0: return launch_vectors<Q40Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ8_0: return launch_vectors<Q80Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace et

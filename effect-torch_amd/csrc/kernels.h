@@ -41,6 +41,14 @@ hipError_t gemv_fast(int32_t codec, const uint8_t* weight, const float* x, uint6
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
                      hipStream_t stream);
 
+// ---- gemv_limb.hip: dequant-GEMV on v_dot4_i32_i8 over 3-limb activations -----
+// Same contract as gemv_fast; f32-accurate. Preferred wherever it applies.
+constexpr uint32_t kGemvLimbMaxVectors = 3;
+bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors);
+hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                     const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
+                     hipStream_t stream);
+
 // ---- gemv_generic.hip: every codec, any whole number of blocks, vectors <= 4 ----
 constexpr uint32_t kGemvGenericMaxVectors = 4;
 hipError_t gemv_generic(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
@@ -58,5 +66,11 @@ bool gemm_i8_supported(int32_t codec, uint64_t columns);
 hipError_t gemm_i8(int32_t codec, const uint8_t* weight, const int8_t* q, const float* scale,
                    const int32_t* sum, const float* bias, float* y, uint64_t rows,
                    uint64_t columns, uint64_t vectors, hipStream_t stream);
+
+// ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
+// sink must hold `workgroups` words.
+hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
+                            hipStream_t stream);
+hipError_t calibration_copy(const void* src, void* dst, uint64_t bytes, hipStream_t stream);
 
 }  // namespace et

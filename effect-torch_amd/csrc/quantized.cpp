@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <sstream>
@@ -128,10 +129,15 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         plan->sum_offset = cursor;
         cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
     } else if (plan->activation_mode == ET_ACT_F32) {
+        const uint32_t limb_launch = static_cast<uint32_t>(
+            plan->vectors < kGemvLimbMaxVectors ? plan->vectors : kGemvLimbMaxVectors);
         const uint32_t fast_max = gemv_fast_max_vectors(plan->codec);
         const uint32_t per_launch =
             static_cast<uint32_t>(plan->vectors < fast_max ? plan->vectors : fast_max);
-        if (fast_max != 0 && gemv_fast_supported(plan->codec, plan->columns, per_launch)) {
+        if (getenv("ET_NO_LIMB") == nullptr && gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
+            plan->kernel = LinearKernel::kGemvLimb;
+            plan->vectors_per_launch = limb_launch;
+        } else if (fast_max != 0 && gemv_fast_supported(plan->codec, plan->columns, per_launch)) {
             plan->kernel = LinearKernel::kGemvFast;
             plan->vectors_per_launch = per_launch;
         } else {
@@ -235,6 +241,7 @@ bool TensorView::is_contiguous() const {
 const char* kernel_name(const et_linear_plan& plan) {
     switch (plan.kernel) {
         case LinearKernel::kNone: return "none";
+        case LinearKernel::kGemvLimb: return "gemv_limb";
         case LinearKernel::kGemvFast: return "gemv_fast";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
         case LinearKernel::kGemmI8: return "quantize_act+gemm_i8";
@@ -363,7 +370,10 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         const float* xv = x + v0 * x_row_stride;
         float* yv = y + v0 * plan.rows;
         hipError_t status;
-        if (plan.kernel == LinearKernel::kGemvFast && gemv_fast_supported(plan.codec, plan.columns, count))
+        if (plan.kernel == LinearKernel::kGemvLimb && gemv_limb_supported(plan.codec, plan.columns, count))
+            status = gemv_limb(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
+                               count, s);
+        else if (plan.kernel == LinearKernel::kGemvFast && gemv_fast_supported(plan.codec, plan.columns, count))
             status = gemv_fast(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
                                count, s);
         else

@@ -325,3 +325,16 @@ class RawLinear:
                                              bias.data_ptr() if bias is not None else None,
                                              y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream),
                                              cancelled.ptr if cancelled is not None else None))
+
+
+def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
+    """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""
+    assert sink.numel() >= workgroups and sink.element_size() == 4
+    _check(N.lib().et_hip_calibration_read(src.data_ptr(), src.numel() * src.element_size(),
+                                           sink.data_ptr(), workgroups, _stream_handle(stream)))
+
+
+def calibration_copy(src: torch.Tensor, dst: torch.Tensor, stream=None) -> None:
+    """Plain copy ``dst <- src`` (measurement aid, ``et_hip_calibration_copy``)."""
+    _check(N.lib().et_hip_calibration_copy(src.data_ptr(), dst.data_ptr(),
+                                           src.numel() * src.element_size(), _stream_handle(stream)))

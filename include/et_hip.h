@@ -208,6 +208,18 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
                                 uint64_t columns, int8_t* q, float* scale, int32_t* sum,
                                 void* stream);
 
+/* ---- measurement aids ----------------------------------------------------- */
+
+/* A plain streaming read (`workgroups` workgroups of 256 lanes, each a
+ * contiguous range, 16-byte loads; `sink` receives one word per workgroup) and a
+ * plain 16-byte copy, both of `bytes` rounded down to 16. They measure the
+ * bandwidth this device delivers to a kernel of a given footprint and calibrate
+ * hardware counters against a known number of bytes. They have no counterpart
+ * in the reference and are not part of the operator path. */
+int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
+                            void* stream);
+int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* stream);
+
 /* ---- errors -------------------------------------------------------------- */
 
 /* Message of the last failed call on this thread ("" if none). */
