@@ -33,6 +33,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published (5.0 POP/s)
 ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
+# counters' reading for a plain copy of known size. These cannot be collected from inside this
+# script; the runs and their figures are in profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md.
+MEASURED_TRAFFIC = {("q4_k_gemv_14336x4096", 1, "f32"): 33338900}
+
 
 def parse_args():
     p = argparse.ArgumentParser()
@@ -87,6 +92,77 @@ def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
     }
 
 
+def time_steps(step, steps, warmup, use_graph):
+    """Warm up, then time exactly `steps` calls of step(i) on torch's current stream
+    (a HIP graph replay unless disabled); returns (ms per step, graph used, wall seconds)."""
+    import torch
+
+    stream = torch.cuda.current_stream()
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    graph = None
+    if use_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(steps):
+                    step(i)
+            graph.replay()  # one untimed replay
+            torch.cuda.synchronize()
+        except Exception as exc:  # noqa: BLE001 - report and fall back to plain enqueues
+            print(f"HIP graph capture failed ({exc}); timing plain enqueues", file=sys.stderr)
+            graph = None
+            torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    start.record(stream)
+    if graph is not None:
+        graph.replay()
+    else:
+        for i in range(steps):
+            step(i)
+    stop.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    return start.elapsed_time(stop) / steps, graph is not None, wall
+
+
+def calibrate(args, et):
+    """Plain streaming read / copy of the headline weight's size: the bandwidth the device
+    delivers to a kernel of that footprint, and the reference for counter calibration."""
+    import torch
+
+    device = torch.device("cuda:0")
+    nbytes = 14336 * 2304  # the packed Q4_K 14336 x 4096 weight
+    copies = 1 if args.hot else -(-ROTATE_BYTES // nbytes)
+    buffers = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=device) for _ in range(copies)]
+    workgroups = 512
+    sink = torch.zeros(4 * workgroups, dtype=torch.int32, device=device)
+    dst = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    if args.workload == "calibrate_read":
+        step = lambda i: et.calibration_read(buffers[i % copies], sink, workgroups)  # noqa: E731
+        moved = nbytes
+    else:
+        step = lambda i: et.calibration_copy(buffers[i % copies], dst)  # noqa: E731
+        moved = 2 * nbytes
+    ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    gbs = moved / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": f"{args.workload} GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload} of {nbytes} bytes ({'hot' if args.hot else 'cold, %d buffers' % copies})",
+                   "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": moved, "avg_launch_us": round(ms * 1e3, 3)},
+    }))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -101,8 +177,11 @@ def main():
     et = entry.load_package()
     from effect_torch_amd import synth
 
+    if args.workload in ("calibrate_read", "calibrate_copy"):
+        return calibrate(args, et)
     if args.workload not in synth.CONFIGS:
-        sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)}")
+        sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
+                 "or calibrate_read / calibrate_copy")
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")
@@ -155,40 +234,7 @@ def main():
     assert np.all(err <= 1e-3 * np.maximum(np.abs(want), 1.0) + 4e-5 * rms), \
         f"parity gate failed: max |err| {err.max():.4g}"
 
-    stream = torch.cuda.current_stream()
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-
-    graph = None
-    if not args.no_graph:
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                for i in range(args.steps):
-                    step(i)
-            graph.replay()  # one untimed replay
-            torch.cuda.synchronize()
-        except Exception as exc:  # noqa: BLE001 - report and fall back to plain enqueues
-            print(f"HIP graph capture failed ({exc}); timing plain enqueues", file=sys.stderr)
-            graph = None
-            torch.cuda.synchronize()
-
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    wall0 = time.perf_counter()
-    start.record(stream)
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(args.steps):
-            step(i)
-    stop.record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    gpu_ms = start.elapsed_time(stop)
-    ms_per_step = gpu_ms / args.steps
+    ms_per_step, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
     seconds_per_step = ms_per_step * 1e-3
 
     gbs = algorithmic_bytes / seconds_per_step / 1e9
@@ -200,6 +246,7 @@ def main():
     else:
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+    roofline["traffic"] = MEASURED_TRAFFIC.get((args.workload, vectors, mode_name))
     roofline["kernel"] = req.kernel
     roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes
     roofline["avg_launch_us"] = round(ms_per_step * 1e3, 3)
@@ -222,7 +269,7 @@ def main():
             "workload": f"{args.workload} M={vectors} ({codec.ggml_name} W {rows}x{columns}, {mode_name} activations)",
             "weights": "hot: one buffer, cache resident" if args.hot else
                        f"cold: rotating over {copies} distinct weight buffers ({copies * weight_bytes >> 20} MiB)",
-            "launch": "hipgraph replay of the K steps" if graph is not None else "K plain enqueues",
+            "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues",
             "percent_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
             "host_wall_ms": round(wall * 1e3, 3),
         },

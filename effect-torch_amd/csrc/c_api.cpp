@@ -301,7 +301,7 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             void* stream) {
     return guarded([&](std::string* error) -> int {
-        if (src == nullptr || sink == nullptr || workgroups == 0 ||
+        if (src == nullptr || sink == nullptr || workgroups == 0 || (bytes >> 36) != 0 ||
             reinterpret_cast<uintptr_t>(src) % 16 != 0) {
             *error = "calibration_read: source must be 16-byte aligned, sink non-NULL, workgroups > 0";
             return ET_ERR_INVALID;

@@ -8,41 +8,36 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstdio>
-#include <cstdlib>
 
 #include "kernels.h"
 
 namespace et {
 namespace {
 
-// Each workgroup streams a contiguous range with 16-byte loads, UNROLL in flight per lane.
-template <int UNROLL, int THREADS = 256>
-__global__ __launch_bounds__(THREADS) void read_kernel(const uint4* __restrict__ src, uint64_t quads,
+// Each workgroup streams a contiguous range with 16-byte loads, four in flight
+// per lane. The XOR of everything read leaves through one word per wave, so the
+// loads cannot be removed; there is no barrier and no atomic on the way out.
+__global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ src, uint32_t quads,
                                                    uint32_t* __restrict__ sink) {
-    const uint64_t per_wg = (quads + gridDim.x - 1) / gridDim.x;
-    const uint64_t begin = blockIdx.x * per_wg;
-    const uint64_t end = begin + per_wg < quads ? begin + per_wg : quads;
+    const uint32_t per_wg = (quads + gridDim.x - 1) / gridDim.x;
+    const uint32_t begin = blockIdx.x * per_wg;
+    const uint32_t end = min(begin + per_wg, quads);
     uint32_t acc = 0;
-    uint64_t i = begin + threadIdx.x;
-    for (; i + (UNROLL - 1) * static_cast<uint64_t>(THREADS) < end; i += UNROLL * static_cast<uint64_t>(THREADS)) {
-        uint4 v[UNROLL];
+    uint32_t i = begin + threadIdx.x;
+    for (; i + 3 * 256u < end; i += 4 * 256u) {
+        uint4 v[4];
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) v[u] = src[i + u * static_cast<uint64_t>(THREADS)];
+        for (int u = 0; u < 4; u++) v[u] = src[i + u * 256u];
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+        for (int u = 0; u < 4; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
     }
-    for (; i < end; i += static_cast<uint64_t>(THREADS)) {
+    for (; i < end; i += 256u) {
         const uint4 v = src[i];
         acc ^= v.x ^ v.y ^ v.z ^ v.w;
     }
-    // The sum is data dependent, so the loads cannot be removed; one word per workgroup leaves.
-    __shared__ uint32_t folded;
-    if (threadIdx.x == 0) folded = 0;
-    __syncthreads();
-    atomicXor(&folded, acc);
-    __syncthreads();
-    if (threadIdx.x == 0) sink[blockIdx.x] = folded;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) acc ^= __shfl_xor(acc, offset);
+    if ((threadIdx.x & 63u) == 0) sink[blockIdx.x * 4u + (threadIdx.x >> 6)] = acc;
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src,
@@ -56,21 +51,8 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             hipStream_t stream) {
     if (bytes < 16) return hipSuccess;
-    if (const char* exp = getenv("ET_CAL")) {  // EXPERIMENT HOOK: "unroll,threads"
-        int u = 4, t = 256;
-        sscanf(exp, "%d,%d", &u, &t);
-#define ET_CASE(U, T)                                                                          \
-    if (u == U && t == T) {                                                                    \
-        hipLaunchKernelGGL((read_kernel<U, T>), dim3(workgroups), dim3(T), 0, stream,          \
-                           static_cast<const uint4*>(src), bytes / 16, sink);                  \
-        return hipGetLastError();                                                              \
-    }
-        ET_CASE(8, 256) ET_CASE(16, 256) ET_CASE(4, 512) ET_CASE(8, 512) ET_CASE(4, 1024) ET_CASE(8, 1024)
-        ET_CASE(2, 1024) ET_CASE(16, 512) ET_CASE(2, 512) ET_CASE(1, 1024) ET_CASE(16, 64) ET_CASE(32, 64) ET_CASE(8, 64) ET_CASE(8, 128) ET_CASE(16, 128)
-#undef ET_CASE
-    }
-    hipLaunchKernelGGL((read_kernel<4, 256>), dim3(workgroups), dim3(256), 0, stream,
-                       static_cast<const uint4*>(src), bytes / 16, sink);
+    hipLaunchKernelGGL(read_kernel, dim3(workgroups), dim3(256), 0, stream,
+                       static_cast<const uint4*>(src), static_cast<uint32_t>(bytes / 16), sink);
     return hipGetLastError();
 }
 

@@ -68,7 +68,7 @@ hipError_t gemm_i8(int32_t codec, const uint8_t* weight, const int8_t* q, const 
                    uint64_t columns, uint64_t vectors, hipStream_t stream);
 
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
-// sink must hold `workgroups` words.
+// sink must hold 4 * `workgroups` words; bytes < 2^36.
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             hipStream_t stream);
 hipError_t calibration_copy(const void* src, void* dst, uint64_t bytes, hipStream_t stream);

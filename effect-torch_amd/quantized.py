@@ -329,7 +329,7 @@ class RawLinear:
 
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""
-    assert sink.numel() >= workgroups and sink.element_size() == 4
+    assert sink.numel() >= 4 * workgroups and sink.element_size() == 4
     _check(N.lib().et_hip_calibration_read(src.data_ptr(), src.numel() * src.element_size(),
                                            sink.data_ptr(), workgroups, _stream_handle(stream)))
 

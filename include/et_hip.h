@@ -211,7 +211,8 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 /* ---- measurement aids ----------------------------------------------------- */
 
 /* A plain streaming read (`workgroups` workgroups of 256 lanes, each a
- * contiguous range, 16-byte loads; `sink` receives one word per workgroup) and a
+ * contiguous range, 16-byte loads; `sink` receives four words per workgroup; at
+ * most 2^36 bytes) and a
  * plain 16-byte copy, both of `bytes` rounded down to 16. They measure the
  * bandwidth this device delivers to a kernel of a given footprint and calibrate
  * hardware counters against a known number of bytes. They have no counterpart
