@@ -27,7 +27,6 @@ COMMON = [
 # dequant.hip must round every multiply and subtract separately (bit-exact decode).
 SOURCES = {
     "dequant.hip": ["-ffp-contract=off"],
-    "gemv_fast.hip": [],
     "gemv_limb.hip": [],
     "gemv_generic.hip": [],
     "quantize_act.hip": ["-ffp-contract=off"],

@@ -32,17 +32,9 @@ hipError_t dequantize_rows(int32_t codec, const uint8_t* weight, const void* ind
 hipError_t gather_f32(const float* src, const IndexLayout& layout, uint64_t count, float* dst,
                       hipStream_t stream);
 
-// ---- gemv_fast.hip: activation-stationary dequant-GEMV (Q4_K, Q4_0, Q8_0) ----
-// y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r]) for v < vectors.
-// x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
-uint32_t gemv_fast_max_vectors(int32_t codec);
-bool gemv_fast_supported(int32_t codec, uint64_t columns, uint32_t vectors);
-hipError_t gemv_fast(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
-                     const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
-                     hipStream_t stream);
-
 // ---- gemv_limb.hip: dequant-GEMV on v_dot4_i32_i8 over 3-limb activations -----
-// Same contract as gemv_fast; f32-accurate. Preferred wherever it applies.
+// y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r]) for v < vectors; f32-accurate.
+// x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
 constexpr uint32_t kGemvLimbMaxVectors = 3;
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors);
 hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,

@@ -3,7 +3,6 @@
 
 #include <hip/hip_runtime_api.h>
 
-#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <sstream>
@@ -131,15 +130,9 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     } else if (plan->activation_mode == ET_ACT_F32) {
         const uint32_t limb_launch = static_cast<uint32_t>(
             plan->vectors < kGemvLimbMaxVectors ? plan->vectors : kGemvLimbMaxVectors);
-        const uint32_t fast_max = gemv_fast_max_vectors(plan->codec);
-        const uint32_t per_launch =
-            static_cast<uint32_t>(plan->vectors < fast_max ? plan->vectors : fast_max);
-        if (getenv("ET_NO_LIMB") == nullptr && gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
+        if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
             plan->kernel = LinearKernel::kGemvLimb;
             plan->vectors_per_launch = limb_launch;
-        } else if (fast_max != 0 && gemv_fast_supported(plan->codec, plan->columns, per_launch)) {
-            plan->kernel = LinearKernel::kGemvFast;
-            plan->vectors_per_launch = per_launch;
         } else {
             plan->kernel = LinearKernel::kGemvGeneric;
             plan->vectors_per_launch = kGemvGenericMaxVectors;
@@ -242,7 +235,6 @@ const char* kernel_name(const et_linear_plan& plan) {
     switch (plan.kernel) {
         case LinearKernel::kNone: return "none";
         case LinearKernel::kGemvLimb: return "gemv_limb";
-        case LinearKernel::kGemvFast: return "gemv_fast";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
         case LinearKernel::kGemmI8: return "quantize_act+gemm_i8";
     }
@@ -372,9 +364,6 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         hipError_t status;
         if (plan.kernel == LinearKernel::kGemvLimb && gemv_limb_supported(plan.codec, plan.columns, count))
             status = gemv_limb(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
-                               count, s);
-        else if (plan.kernel == LinearKernel::kGemvFast && gemv_fast_supported(plan.codec, plan.columns, count))
-            status = gemv_fast(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
                                count, s);
         else
             status = gemv_generic(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows,

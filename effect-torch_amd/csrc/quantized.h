@@ -30,7 +30,6 @@ struct TensorView {
 enum class LinearKernel {
     kNone,         // empty output: nothing is enqueued
     kGemvLimb,     // dequant-GEMV on integer dot products (gemv_limb.hip)
-    kGemvFast,     // activation-stationary f32 dequant-GEMV (gemv_fast.hip)
     kGemvGeneric,  // portable dequant-GEMV (gemv_generic.hip)
     kGemmI8,       // quantize_act.hip + gemm_i8.hip
 };
