@@ -48,15 +48,23 @@ hipError_t gemv_generic(int32_t codec, const uint8_t* weight, const float* x, ui
                         uint32_t vectors, hipStream_t stream);
 
 // ---- quantize_act.hip --------------------------------------------------------
-// q [vectors, columns] int8; scale and sum TRANSPOSED: [columns/32, round_up(vectors, 32)].
+// limbs = 1: q [vectors, columns] int8, scale = max|x| / 127 per vector and 32 columns.
+// limbs = 3: three byte planes q + limb * limb_stride of 24-bit fixed-point activations,
+//            scale = max|x| / (127 * 65536).
+// scale, sum (int32 block sums, may be null) and xsum (f32: scale * sum, may be null) are
+// TRANSPOSED: [columns/32, round_up(vectors, 32)].
 hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
-                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
-                                hipStream_t stream);
+                                uint64_t columns, int limbs, int8_t* q, uint64_t limb_stride,
+                                float* scale, int32_t* sum, float* xsum, hipStream_t stream);
 
-// ---- gemm_i8.hip: int8-activation MFMA contraction ---------------------------
+// ---- gemm_i8.hip: matrix-core contraction over quantised activations ------------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
-hipError_t gemm_i8(int32_t codec, const uint8_t* weight, const int8_t* q, const float* scale,
-                   const int32_t* sum, const float* bias, float* y, uint64_t rows,
+// From this many vectors on, f32-mode requests use the matrix cores (3-limb activations).
+constexpr uint32_t kGemmMinVectors = 4;
+// table_stride = round_up(vectors, 32): row pitch of the scale and xsum tables.
+hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const int8_t* q,
+                   uint64_t limb_stride, const float* scale, const float* xsum,
+                   uint32_t table_stride, const float* bias, float* y, uint64_t rows,
                    uint64_t columns, uint64_t vectors, hipStream_t stream);
 
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------

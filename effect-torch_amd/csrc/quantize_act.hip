@@ -1,4 +1,4 @@
-// int8 activation quantiser: stage 1 of the int8-activation path.
+// Activation quantiser: stage 1 of the matrix-core paths.
 //
 // For each vector v and each 32-column block b:
 //     amax  = max |x|                      scale[b, v] = amax / 127
@@ -7,7 +7,9 @@
 // Both divisions are IEEE-correct and rint rounds to nearest even, so the
 // integers and scales are bit-identical to a CPU evaluation of the same
 // formulas. The reference has no int8 activation path; these semantics are
-// this library's own.
+// this library's own. A second variant writes 24-bit fixed-point activations as
+// three byte planes (range 127 * 2^16 instead of 127), which the same matrix-core
+// kernel contracts limb by limb with f32-level accuracy.
 //
 // Layout: q is [vectors, columns] int8 (row-major, what the MFMA operand loads
 // want); scale and sum are stored TRANSPOSED, [columns/32, stride] with
@@ -36,11 +38,19 @@ __device__ __forceinline__ int dpp_i32(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
 }
 
+// LIMBS = 1: q = clamp(rint(x * 127/amax)), scale = amax / 127.
+// LIMBS = 3: X = clamp(rint(x * 8323072/amax)) as three balanced signed bytes
+//            (X = 65536*x2 + 256*x1 + x0, planes q + limb * limb_stride), scale = amax / 8323072.
+// sum (int32, may be null) receives the block's integer sum, xsum (f32, may be null)
+// scale * sum: the activation block sum as the quantised operand represents it.
+template <int LIMBS>
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x,
                                                        uint64_t x_row_stride, uint32_t vectors,
                                                        uint32_t columns, int8_t* __restrict__ q,
-                                                       float* __restrict__ scale,
-                                                       int32_t* __restrict__ sum) {
+                                                       uint64_t limb_stride, float* __restrict__ scale,
+                                                       int32_t* __restrict__ sum,
+                                                       float* __restrict__ xsum) {
+    constexpr float kRange = LIMBS == 1 ? 127.f : 8323072.f;  // 127 * 2^16
     const uint32_t quads_per_row = columns >> 2;
     const uint64_t total = static_cast<uint64_t>(vectors) * quads_per_row;  // multiple of 8
     const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
@@ -53,28 +63,46 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
         amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
         amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
         amax = fmaxf(amax, dpp_f32<0x141>(amax));  // row_half_mirror: the other quad of the 8
-        const float inv = amax > 0.f ? 127.f / amax : 0.f;
+        const float inv = amax > 0.f ? kRange / amax : 0.f;
         int qi[4];
         const float values[4] = {in.x, in.y, in.z, in.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             float r = rintf(values[i] * inv);
-            r = fminf(fmaxf(r, -127.f), 127.f);
+            r = fminf(fmaxf(r, -kRange), kRange);
             qi[i] = static_cast<int>(r);
         }
         int total_q = (qi[0] + qi[1]) + (qi[2] + qi[3]);
         total_q += dpp_i32<0xB1>(total_q);
         total_q += dpp_i32<0x4E>(total_q);
         total_q += dpp_i32<0x141>(total_q);
-        const uint32_t packed = (static_cast<uint32_t>(qi[0]) & 0xffu) |
-                                ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
-                                ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
-                                ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
-        reinterpret_cast<uint32_t*>(q)[static_cast<uint64_t>(v) * quads_per_row + quad] = packed;
+        const uint64_t word = static_cast<uint64_t>(v) * quads_per_row + quad;
+        if constexpr (LIMBS == 1) {
+            const uint32_t packed = (static_cast<uint32_t>(qi[0]) & 0xffu) |
+                                    ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
+                                    ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
+                                    ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
+            reinterpret_cast<uint32_t*>(q)[word] = packed;
+        } else {
+            // X + 0x808080 = (x2+128)<<16 | (x1+128)<<8 | (x0+128), every x in [-128, 127]
+            uint32_t u[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) u[i] = static_cast<uint32_t>(qi[i] + 0x808080);
+#pragma unroll
+            for (int limb = 0; limb < 3; limb++) {
+                const uint32_t packed = ((u[0] >> (8 * limb)) & 0xffu) |
+                                        (((u[1] >> (8 * limb)) & 0xffu) << 8) |
+                                        (((u[2] >> (8 * limb)) & 0xffu) << 16) |
+                                        (((u[3] >> (8 * limb)) & 0xffu) << 24);
+                reinterpret_cast<uint32_t*>(q + limb * limb_stride)[word] = packed ^ 0x80808080u;
+            }
+        }
         if ((quad & 7u) == 0) {
             const uint64_t slot = static_cast<uint64_t>(quad >> 3) * ((vectors + 31u) & ~31u) + v;
-            scale[slot] = amax / 127.f;
+            const float unit = amax / kRange;
+            scale[slot] = unit;
             if (sum != nullptr) sum[slot] = total_q;
+            if (xsum != nullptr) xsum[slot] = unit * static_cast<float>(total_q);
         }
     }
 }
@@ -82,15 +110,22 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 }  // namespace
 
 hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
-                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
-                                hipStream_t stream) {
+                                uint64_t columns, int limbs, int8_t* q, uint64_t limb_stride,
+                                float* scale, int32_t* sum, float* xsum, hipStream_t stream) {
     const uint64_t total = vectors * (columns >> 2);
     if (total == 0) return hipSuccess;
+    if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
     uint64_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
-    hipLaunchKernelGGL(quantize_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream, x,
-                       x_row_stride, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
-                       scale, sum);
+    const dim3 grid(static_cast<uint32_t>(blocks));
+    if (limbs == 1)
+        hipLaunchKernelGGL(quantize_kernel<1>, grid, dim3(256), 0, stream, x, x_row_stride,
+                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
+                           limb_stride, scale, sum, xsum);
+    else
+        hipLaunchKernelGGL(quantize_kernel<3>, grid, dim3(256), 0, stream, x, x_row_stride,
+                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
+                           limb_stride, scale, sum, xsum);
     return hipGetLastError();
 }
 

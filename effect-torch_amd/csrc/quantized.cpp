@@ -114,23 +114,28 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     cursor = align_up(plan->gather_bytes, 256);
     plan->bias_offset = cursor;  // dense copy of a strided bias
     cursor = align_up(cursor + plan->rows * 4u, 256);
-    if (plan->activation_mode == ET_ACT_INT8) {
-        if (!gemm_i8_supported(plan->codec, plan->columns))
-            return fail(error, ET_ERR_UNSUPPORTED,
-                        std::string("quantized_linear: int8 activation mode is not available for ") +
-                            codec_name(plan->codec));
-        plan->kernel = LinearKernel::kGemmI8;
+    const auto plan_matrix_core = [&](LinearKernel kernel, uint64_t limbs) {
+        plan->kernel = kernel;
         plan->q_offset = cursor;
-        cursor = align_up(cursor + plan->vectors * plan->columns, 256);
+        cursor = align_up(cursor + limbs * plan->vectors * plan->columns, 256);
         plan->scale_offset = cursor;
         const uint64_t padded_vectors = align_up(plan->vectors, 32);  // [columns/32, padded] tables
         cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
         plan->sum_offset = cursor;
         cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
+    };
+    if (plan->activation_mode == ET_ACT_INT8) {
+        if (!gemm_i8_supported(plan->codec, plan->columns))
+            return fail(error, ET_ERR_UNSUPPORTED,
+                        std::string("quantized_linear: int8 activation mode is not available for ") +
+                            codec_name(plan->codec));
+        plan_matrix_core(LinearKernel::kGemmI8, 1);
     } else if (plan->activation_mode == ET_ACT_F32) {
         const uint32_t limb_launch = static_cast<uint32_t>(
             plan->vectors < kGemvLimbMaxVectors ? plan->vectors : kGemvLimbMaxVectors);
-        if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
+        if (plan->vectors >= kGemmMinVectors && gemm_i8_supported(plan->codec, plan->columns)) {
+            plan_matrix_core(LinearKernel::kGemmLimb, 3);
+        } else if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
             plan->kernel = LinearKernel::kGemvLimb;
             plan->vectors_per_launch = limb_launch;
         } else {
@@ -237,6 +242,7 @@ const char* kernel_name(const et_linear_plan& plan) {
         case LinearKernel::kGemvLimb: return "gemv_limb";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
         case LinearKernel::kGemmI8: return "quantize_act+gemm_i8";
+        case LinearKernel::kGemmLimb: return "quantize_limbs+gemm_i8";
     }
     return "?";
 }
@@ -338,20 +344,23 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         x_row_stride = plan.columns;
     }
 
-    if (plan.kernel == LinearKernel::kGemmI8) {
+    if (plan.kernel == LinearKernel::kGemmI8 || plan.kernel == LinearKernel::kGemmLimb) {
         if (scratch == nullptr || workspace_bytes < plan.workspace_bytes)
             return fail(error, ET_ERR_EXECUTION,
                         "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
                             " bytes is smaller than the planned " +
                             std::to_string(plan.workspace_bytes));
+        const int limbs = plan.kernel == LinearKernel::kGemmI8 ? 1 : 3;
+        const uint64_t limb_stride = plan.vectors * plan.columns;
+        const uint32_t table_stride = static_cast<uint32_t>(align_up(plan.vectors, 32));
         auto* q = reinterpret_cast<int8_t*>(scratch + plan.q_offset);
         auto* scale = reinterpret_cast<float*>(scratch + plan.scale_offset);
-        auto* sum = reinterpret_cast<int32_t*>(scratch + plan.sum_offset);
-        if (hipError_t status =
-                quantize_activations(x, x_row_stride, plan.vectors, plan.columns, q, scale, sum, s))
+        auto* xsum = reinterpret_cast<float*>(scratch + plan.sum_offset);
+        if (hipError_t status = quantize_activations(x, x_row_stride, plan.vectors, plan.columns, limbs,
+                                                     q, limb_stride, scale, nullptr, xsum, s))
             return hip_failure(error, "quantized_linear", status);
-        if (hipError_t status = gemm_i8(plan.codec, weight, q, scale, sum, bias, y, plan.rows,
-                                        plan.columns, plan.vectors, s))
+        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, q, limb_stride, scale, xsum,
+                                        table_stride, bias, y, plan.rows, plan.columns, plan.vectors, s))
             return hip_failure(error, "quantized_linear", status);
         return ET_OK;
     }

@@ -31,7 +31,8 @@ enum class LinearKernel {
     kNone,         // empty output: nothing is enqueued
     kGemvLimb,     // dequant-GEMV on integer dot products (gemv_limb.hip)
     kGemvGeneric,  // portable dequant-GEMV (gemv_generic.hip)
-    kGemmI8,       // quantize_act.hip + gemm_i8.hip
+    kGemmI8,       // int8 activations: quantize_act.hip + gemm_i8.hip
+    kGemmLimb,     // f32-accurate 3-limb activations on the same matrix-core kernel
 };
 
 }  // namespace quantized

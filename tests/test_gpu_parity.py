@@ -208,6 +208,30 @@ def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
     close(got, exact, oracle_noise=0)
 
 
+@pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0])
+@pytest.mark.parametrize("vectors,rows,columns", [(4, 129, 256), (8, 64, 2304), (33, 1, 512), (65, 300, 1024),
+                                                  (100, 130, 4096), (130, 257, 768), (200, 63, 256)])
+def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, rows, columns):
+    # four or more vectors: 3-limb activations on the matrix cores; ragged tiles on every side,
+    # one and several stages of eight blocks, a partial last stage for the 32-wide codecs
+    if codec != oracle.Q4_K:
+        columns += 32
+    rng = np.random.default_rng(codec * 11 + vectors + rows + columns)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    x[vectors // 2, :64] = 0.0  # all-zero blocks: unit 0
+    bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
+    plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
+                                  None, et.GgmlQuant(codec), (rows, columns))
+    assert plan.kernel == "quantize_limbs+gemm_i8"
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias)
+    close(got, oracle.linear_into(codec, rows, columns, x, weight, bias))
+    exact = x.astype(np.float64) @ oracle.decode_rows(codec, weight, columns).astype(np.float64).T
+    if bias is not None:
+        exact = exact + bias.astype(np.float64)
+    close(got, exact, oracle_noise=0)
+
+
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0, oracle.Q6_K])
 def test_linear_unit_vectors_select_decoded_weights(et, device, codec):
     rng = np.random.default_rng(800 + codec)
@@ -314,7 +338,8 @@ def test_activation_quantiser_is_bit_exact(et, device, vectors, columns):
 
 @pytest.mark.parametrize("codec", [oracle.Q8_0, oracle.Q4_0, oracle.Q4_K])
 @pytest.mark.parametrize("vectors,rows,columns", [(16, 128, 512), (64, 200, 4096), (33, 37, 1024),
-                                                  (512, 96, 2048), (1, 5, 256)])
+                                                  (512, 96, 2048), (1, 5, 256), (97, 129, 768),
+                                                  (130, 300, 2304)])
 def test_int8_path_matches_its_oracle(et, device, codec, vectors, rows, columns):
     rng = np.random.default_rng(codec * 7 + vectors + rows)
     weight = synth.random_weight(codec, rows, columns, rng)
