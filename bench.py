@@ -211,7 +211,7 @@ def main():
     linear = et.RawLinear(codec, rows, columns, vectors, False, mode)
     req = linear.requirements
     workspace = (torch.empty(req.workspace_bytes, dtype=torch.uint8, device=device)
-                 if mode_name == "int8" else None)
+                 if req.workspace_bytes else None)
     algorithmic_bytes = req.algorithmic_bytes
 
     def step(i):

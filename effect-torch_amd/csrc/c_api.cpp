@@ -288,8 +288,8 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
             *error = "quantize_activations: operands must be non-NULL and 16-byte aligned";
             return ET_ERR_INVALID;
         }
-        const hipError_t status = et::quantize_activations(
-            x, x_row_stride, vectors, columns, 1, q, 0, scale, sum, nullptr, static_cast<hipStream_t>(stream));
+        const hipError_t status = et::quantize_activations(x, x_row_stride, vectors, columns, q, scale,
+                                                           sum, static_cast<hipStream_t>(stream));
         if (status != hipSuccess) {
             *error = std::string("quantize_activations: HIP error: ") + hipGetErrorString(status);
             return ET_ERR_EXECUTION;

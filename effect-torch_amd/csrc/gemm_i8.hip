@@ -5,10 +5,11 @@
 //   Q4_K:  y[m, n] = sum_g (d*sc_g)[n] * s[m,g] * (sum_i nib * qx)  -  sum_g (dmin*m_g)[n] * xf[m,g]
 // b / g index 32-column blocks; xf[m, g] is the block's activation sum in f32.
 // The inner sums are exact int32 from v_mfma_i32_32x32x32_i8, whose K = 32 is
-// exactly one quantisation block; the block scales are applied by an f32
-// epilogue on the VALU after every MFMA. The Q4_K "min" term is a small f32
-// GEMM of its own (inner dimension K/32) and runs on v_mfma_f32_32x32x2f32
-// straight into a second accumulator, with no epilogue.
+// exactly one quantisation block. The block scales are applied in f32 after every
+// MFMA: the 32x32 tile of scale products s[m] * d[n] is itself a rank-1 matrix
+// product and comes from v_mfma_f32_32x32x2f32 in the result layout, so the VALU
+// epilogue is one convert and one FMA per element. The Q4_K "min" term is a small
+// f32 GEMM of its own (inner dimension K/32) and accumulates on the same f32 MFMA.
 //
 // Two activation formats feed the same kernel (quantize_act.hip makes both):
 //   LIMBS = 1  int8 activations, one scale per vector and 32 columns (the
@@ -22,19 +23,30 @@
 // uses f32 simdgroup MMA, crates/runtime-metal/src/quantized.rs:1016-1097); the
 // contraction computed is linear_into's (crates/runtime-cpu/src/quantized.rs:419-499).
 //
-// Tiling. A workgroup of four waves owns BN weight rows x BM = 32*MT vectors and
-// walks K in stages of eight blocks (256 columns, one Q4_K super-block).
-//   KSPLIT = 1: BN = 128, each wave 32 rows, all eight blocks of a stage.
-//   KSPLIT = 2: BN = 64, two waves share 32 rows and take four blocks each; their
-//               accumulators meet in LDS at the end. Used when there are too few
-//               128-row tiles to fill 256 CUs.
-// Activations of a stage go global -> registers -> LDS (XOR-swizzled rows, so the
-// 16-byte MFMA operand reads are conflict free) one stage ahead of their use.
-// Weights never touch LDS: each packed byte is needed by exactly one lane, which
-// loads it one stage ahead into registers; MFMA operand roles are A = activations,
-// B = weights, so a lane of the 32x32 result holds one weight row (its block
-// scale is one value) and sixteen vectors, and every result register row is
-// stored as 128 contiguous bytes of y.
+// Tiling. A workgroup owns 64 weight rows x 32*MT vectors and walks K in stages of
+// eight blocks (256 columns, one Q4_K super-block). Eight consumer waves run the
+// MFMAs: KSPLIT = 4 of them share 32 weight rows and split the eight blocks of every
+// stage between them; their accumulators meet in LDS at the end. Two more waves
+// only move activations (below).
+//
+// Streaming. With few vectors the kernel is bound by weight bytes from HBM, and what
+// matters is how many bytes each CU keeps in flight. Both operand streams run AHEAD
+// stages in front of the MFMAs:
+//   activations  arrive as ready-made stage blobs (see kernels.h) and are copied
+//                global -> LDS by global_load_lds, 16 bytes per lane, into a ring of
+//                AHEAD + 1 slots, by the two loader waves, which do nothing else;
+//   weights      never touch LDS: each packed byte is needed by exactly one lane of a
+//                consumer wave, which loads it into a ring of AHEAD + 1 register sets.
+// The split into loader and consumer waves is what keeps both streams deep. Loads
+// return in order and are counted per wave; a wave that mixes global_load_lds with
+// loads into registers gets a full wait (vmcnt 0) from the compiler before every use
+// of a loaded register, which drains the pipeline once per stage. Kept in separate
+// waves, the loaders wait with an explicit count and the consumers' waits are the
+// compiler's exact ones. One s_barrier per stage joins the two.
+//
+// MFMA operand roles: A = activations, B = weights. A lane of the 32x32 result holds
+// one weight row n = lane % 32 and sixteen vectors m = 8*(r/4) + 4*(lane/32) + r%4,
+// and every result register row is stored as 128 contiguous bytes of y.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -54,12 +66,7 @@ struct __attribute__((packed, aligned(2))) Bytes16 {
     uint32_t v[4];
 };
 
-constexpr int kStageBlocks = 8;                   // 32-column blocks per stage
-constexpr int kStageBytes = 32 * kStageBlocks;    // int8 activations per vector and stage
-constexpr int kChunksPerRow = kStageBytes / 16;   // 16-byte chunks per vector and stage
-
-// Position of 16-byte chunk c of vector-row m inside its 256-byte LDS row.
-__device__ __forceinline__ uint32_t x_chunk_slot(uint32_t m, uint32_t c) { return c ^ (m & 15u); }
+constexpr int kStageBlocks = 8;  // 32-column blocks per stage
 
 // Packed weights one lane holds for NB consecutive blocks of its row (its 16-column half).
 template <int CODEC, int NB>
@@ -72,6 +79,12 @@ struct StageWeights<kQ4_K, NB> {
     uint4 header;     // d, dmin, scales[12]
     uint4 q[NB / 2];  // pair p: bytes 16*half .. +16 of its 32
 };
+
+// VMEM instructions load_stage_weights issues (for the counted wait).
+template <int CODEC, int NB>
+constexpr int weight_loads() {
+    return CODEC == kQ4_K ? 1 + NB / 2 : 2 * NB;
+}
 
 // first_block: index of the first 32-column block to load; blocks: how many of the NB exist.
 template <int CODEC, int NB>
@@ -131,8 +144,8 @@ __device__ __forceinline__ v4i weight_operand(const StageWeights<CODEC, NB>& w, 
 }
 
 // (scale, min) of Q4_K sub-block g (crates/runtime-cpu/src/quantized.rs:77-86).
-__device__ __forceinline__ void q4k_scale_min(const uint4& header, int g, float& scale, float& min) {
-    const uint32_t shift = 8u * (g & 3);
+__device__ __forceinline__ void q4k_scale_min(const uint4& header, uint32_t g, float& scale, float& min) {
+    const uint32_t shift = 8u * (g & 3u);
     const uint32_t s0 = (header.y >> shift) & 0xffu;  // scales[g & 3]
     const uint32_t s1 = (header.z >> shift) & 0xffu;  // scales[4 + (g & 3)]
     const uint32_t s2 = (header.w >> shift) & 0xffu;  // scales[8 + (g & 3)]
@@ -142,101 +155,120 @@ __device__ __forceinline__ void q4k_scale_min(const uint4& header, int g, float&
     min = static_cast<float>(mn);
 }
 
-template <int MT, int LIMBS>
-struct alignas(16) StageLds {
-    uint8_t x[LIMBS][32 * MT][kStageBytes];  // [limb][vector][swizzled chunks]
-    float scale[kStageBlocks][32 * MT];
-    float xsum[kStageBlocks][32 * MT];
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) {
+    return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
+}
+
+constexpr int kConsumers = 8;  // waves that run the MFMAs: two per SIMD
+constexpr int kLoaders = 2;    // waves that only copy activation blobs into LDS
+constexpr int kThreads = 64 * (kConsumers + kLoaders);
+
+template <int CODEC, int MT, int LIMBS, int KSPLIT, int AHEAD>
+struct Shape {
+    static constexpr int kDepth = AHEAD + 1;
+    static constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);
+    static constexpr uint32_t kSlotBytes = MT * kBlob;
+    // One global_load_lds moves 1 KiB per wave.
+    static constexpr int kPieces = kSlotBytes / 1024;
+    static constexpr int kRounds = kPieces / kLoaders;
+    static_assert(kPieces % kLoaders == 0, "equal shares for the loader waves");
+    static constexpr int kBlocksPerWave = kStageBlocks / KSPLIT;
+    static constexpr int kRowGroups = kConsumers / KSPLIT;  // 32-row groups per workgroup
+    static constexpr uint32_t kRows = 32 * kRowGroups;
+    // vmcnt is a 6-bit counter: a smaller bound only waits for more than necessary.
+    static constexpr int kLoaderWait = (AHEAD - 1) * kRounds < 63 ? (AHEAD - 1) * kRounds : 63;
+    static constexpr uint32_t kExchangeBytes = (KSPLIT - 1) * kRowGroups * MT * 16 * 64 * 4;
+    static constexpr uint32_t kLdsBytes =
+        kDepth * kSlotBytes > kExchangeBytes ? kDepth * kSlotBytes : kExchangeBytes;
 };
 
-template <int CODEC, int MT, int LIMBS, int KSPLIT>
-__global__ __launch_bounds__(256) void gemm_i8_kernel(
-    const uint8_t* __restrict__ weight, const int8_t* __restrict__ q, uint64_t limb_stride,
-    const float* __restrict__ scale, const float* __restrict__ xsum, uint32_t table_stride,
+template <int CODEC, int MT, int LIMBS, int KSPLIT, int AHEAD>
+__global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
+    const uint8_t* weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
-    uint32_t vectors) {
-    constexpr int BM = 32 * MT;
-    constexpr int BN = 128 / KSPLIT;
-    constexpr int kXChunks = LIMBS * BM * kChunksPerRow;  // 16-byte chunks of a stage
-    constexpr int kXPerThread = (kXChunks + 255) / 256;
-    constexpr int kTableQuads = kStageBlocks * BM / 4;    // float4s of one table per stage
-    constexpr int kTablePerThread = (kTableQuads + 255) / 256;
-    constexpr int kBlocksPerWave = kStageBlocks / KSPLIT;
-    __shared__ StageLds<MT, LIMBS> lds;
+    uint32_t vectors, uint32_t row_tiles, uint32_t vector_groups) {
+    using S = Shape<CODEC, MT, LIMBS, KSPLIT, AHEAD>;
+    constexpr int NB = S::kBlocksPerWave;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    // Workgroups are handed to the eight XCDs round-robin. All vector groups of one row tile
+    // go to the same XCD, next to each other in time, so the second one finds the weights in L2.
+    const uint32_t xcd = blockIdx.x & 7u, turn = blockIdx.x >> 3;
+    const uint32_t row_tile = (turn / vector_groups) * 8u + xcd;
+    const uint32_t vector_group = turn % vector_groups;
+    if (row_tile >= row_tiles) return;
 
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t half = lane >> 5;
-    const uint32_t wave_n = KSPLIT == 1 ? wave : (wave & 1u);
-    const uint32_t wave_k = KSPLIT == 1 ? 0u : (wave >> 1);
-    const uint32_t n0 = blockIdx.x * BN + wave_n * 32u;
-    const uint32_t m0 = blockIdx.y * BM;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: uniform branches
+    const uint32_t tile0 = vector_group * MT;
     const uint32_t xblocks = columns >> 5;
     const uint32_t stages = (xblocks + kStageBlocks - 1) / kStageBlocks;
+    // Both loops run a whole number of ring turns; the stages past the end are empty.
+    const uint32_t padded_stages = (stages + S::kDepth - 1) / S::kDepth * S::kDepth;
+
+    if (wave >= static_cast<uint32_t>(kConsumers)) {
+        // ---- loader waves ---------------------------------------------------------
+        // Copy the activation blobs of stage s + AHEAD into ring slot (s + AHEAD) % kDepth while
+        // the consumers contract stage s. One barrier per stage, matched by the consumers':
+        // passing it says "stage s is in LDS" to them and "slot of stage s - 1 is free" to us.
+        const uint32_t loader = wave - kConsumers;
+        const auto request = [&](uint32_t stage) {
+            const uint32_t s = min(stage, stages - 1u);  // past the end: a copy nobody reads
+            const uint32_t slot = stage % S::kDepth;
+#pragma unroll
+            for (int i = 0; i < S::kRounds; i++) {
+                const uint32_t piece = i * kLoaders + loader;  // 1 KiB pieces of the slot
+                const uint32_t t = piece / (S::kBlob / 1024u), within = piece % (S::kBlob / 1024u);
+                const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
+                const uint8_t* src = tiles + (static_cast<uint64_t>(s) * vector_tiles + tile) * S::kBlob +
+                                     within * 1024u + lane * 16u;
+                uint8_t* dst = lds + slot * S::kSlotBytes + piece * 1024u;  // + 16 * lane by the hardware
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
+                                                 reinterpret_cast<uint4*>(dst), 16, 0, 0);
+            }
+        };
+        for (uint32_t a = 0; a < static_cast<uint32_t>(AHEAD); a++) request(a);
+        for (uint32_t stage = 0; stage < padded_stages; stage++) {
+            // Loads return in order: all but the newest AHEAD - 1 requests have landed.
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kLoaderWait));
+            __builtin_amdgcn_s_barrier();
+            request(stage + AHEAD);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));  // nothing may still write the ring
+        if constexpr (KSPLIT > 1) {
+            __builtin_amdgcn_s_barrier();  // the consumers' two exchange barriers
+            __builtin_amdgcn_s_barrier();
+        }
+        return;
+    }
+
+    // ---- consumer waves -----------------------------------------------------------
+    const uint32_t half = lane >> 5;
+    const uint32_t wave_n = wave % S::kRowGroups;
+    const uint32_t wave_k = wave / S::kRowGroups;
+    const uint32_t n0 = row_tile * S::kRows + wave_n * 32u;
+    const uint32_t m0 = tile0 * 32u;
 
     // This lane's weight row. Rows past the end are clamped for loads, masked at stores.
     const uint32_t n = min(n0 + (lane & 31u), rows - 1u);
     const uint64_t row_bytes = static_cast<uint64_t>(columns / block_values(CODEC)) * block_bytes(CODEC);
     const uint8_t* w_row = weight + n * row_bytes;
 
-    // ---- staging helpers --------------------------------------------------
-    uint4 x_regs[kXPerThread];
-    float4 s_regs[kTablePerThread], f_regs[kTablePerThread];
-    auto load_x_regs = [&](uint32_t stage) {
-        const uint32_t k0 = stage * kStageBytes;
-#pragma unroll
-        for (int i = 0; i < kXPerThread; i++) {
-            const uint32_t c = threadIdx.x + i * 256u;
-            x_regs[i] = make_uint4(0u, 0u, 0u, 0u);
-            if (c < static_cast<uint32_t>(kXChunks)) {
-                const uint32_t limb = c / (BM * kChunksPerRow);
-                const uint32_t rest = c - limb * (BM * kChunksPerRow);
-                const uint32_t m = rest / kChunksPerRow, chunk = rest % kChunksPerRow;
-                const uint32_t column = k0 + 16u * chunk;
-                if (m0 + m < vectors && column < columns)
-                    x_regs[i] = *reinterpret_cast<const uint4*>(
-                        q + limb * limb_stride + static_cast<uint64_t>(m0 + m) * columns + column);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < kTablePerThread; i++) {
-            const uint32_t t = threadIdx.x + i * 256u;
-            s_regs[i] = f_regs[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (t < static_cast<uint32_t>(kTableQuads)) {
-                const uint32_t b = t / (BM / 4), quad = t % (BM / 4);
-                const uint32_t block = stage * kStageBlocks + b;
-                if (block < xblocks && m0 + 4u * quad < table_stride) {
-                    // The tables are padded to a multiple of 32 vectors: whole quads are inside.
-                    const uint64_t at = static_cast<uint64_t>(block) * table_stride + m0 + 4u * quad;
-                    s_regs[i] = *reinterpret_cast<const float4*>(scale + at);
-                    f_regs[i] = *reinterpret_cast<const float4*>(xsum + at);
-                }
-            }
-        }
+    // Blocks of stage `stage` this wave contracts: first .. first + count (count may be 0).
+    const auto wave_first = [&](uint32_t stage) { return stage * kStageBlocks + wave_k * NB; };
+    const auto wave_count = [&](uint32_t stage) {
+        const uint32_t first = wave_first(stage);
+        return first < xblocks ? min(xblocks - first, static_cast<uint32_t>(NB)) : 0u;
     };
-    auto store_x_regs = [&]() {
-#pragma unroll
-        for (int i = 0; i < kXPerThread; i++) {
-            const uint32_t c = threadIdx.x + i * 256u;
-            if (c < static_cast<uint32_t>(kXChunks)) {
-                const uint32_t limb = c / (BM * kChunksPerRow);
-                const uint32_t rest = c - limb * (BM * kChunksPerRow);
-                const uint32_t m = rest / kChunksPerRow, chunk = rest % kChunksPerRow;
-                *reinterpret_cast<uint4*>(&lds.x[limb][m][16u * x_chunk_slot(m, chunk)]) = x_regs[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < kTablePerThread; i++) {
-            const uint32_t t = threadIdx.x + i * 256u;
-            if (t < static_cast<uint32_t>(kTableQuads)) {
-                const uint32_t b = t / (BM / 4), quad = t % (BM / 4);
-                *reinterpret_cast<float4*>(&lds.scale[b][4u * quad]) = s_regs[i];
-                *reinterpret_cast<float4*>(&lds.xsum[b][4u * quad]) = f_regs[i];
-            }
-        }
+    // Requests this lane's weights of a stage (past the end: the last stage again, unused).
+    const auto request = [&](uint32_t stage, StageWeights<CODEC, NB>& w) {
+        const uint32_t s = min(stage, stages - 1u);
+        uint32_t first = wave_first(s), count = wave_count(s);
+        if (count == 0) first = 0;  // a wave with no blocks in a partial last stage: any valid address
+        load_stage_weights<CODEC, NB>(w_row, first, count, half, w);
     };
 
-    // ---- accumulators -------------------------------------------------------
     float acc[MT][16];
     v16f acc_min[MT];
 #pragma unroll
@@ -246,82 +278,63 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(
             acc[t][r] = 0.f;
             acc_min[t][r] = 0.f;
         }
-    v16i zero;
+    v16i zero_i;
+    v16f zero_f;
 #pragma unroll
-    for (int r = 0; r < 16; r++) zero[r] = 0;
+    for (int r = 0; r < 16; r++) {
+        zero_i[r] = 0;
+        zero_f[r] = 0.f;
+    }
 
-    // Blocks of stage `stage` this wave contracts: wave_first(stage) .. +wave_count(stage).
-    const auto wave_first = [&](uint32_t stage) { return stage * kStageBlocks + wave_k * kBlocksPerWave; };
-    const auto wave_count = [&](uint32_t stage) {
-        const uint32_t first = wave_first(stage);
-        return first < xblocks ? min(xblocks - first, static_cast<uint32_t>(kBlocksPerWave)) : 0u;
-    };
-    StageWeights<CODEC, kBlocksPerWave> w_next;
-    load_x_regs(0);
-    load_stage_weights<CODEC, kBlocksPerWave>(w_row, wave_first(0), wave_count(0), half, w_next);
-
-    for (uint32_t stage = 0; stage < stages; stage++) {
-        __syncthreads();  // the previous stage has been read
-        store_x_regs();
-        const StageWeights<CODEC, kBlocksPerWave> w = w_next;
-        __syncthreads();
-        if (stage + 1 < stages) {
-            load_x_regs(stage + 1);
-            load_stage_weights<CODEC, kBlocksPerWave>(w_row, wave_first(stage + 1), wave_count(stage + 1),
-                                                      half, w_next);
-        }
+    // Contracts stage `stage` from its LDS slot and the weight registers `w`.
+    const auto contract = [&](uint32_t stage, const StageWeights<CODEC, NB>& w) {
         const uint32_t stage_blocks = wave_count(stage);
-        const uint32_t b_base = wave_k * kBlocksPerWave;  // first block of this wave inside the stage
-
+        const uint32_t b_base = wave_k * NB;  // first block of this wave inside the stage
+        const uint8_t* base = lds + (stage % S::kDepth) * S::kSlotBytes;
         float d_block = 0.f, dmin_block = 0.f;
         if constexpr (CODEC == kQ4_K) {
             d_block = half_bits_to_float(w.header.x & 0xffffu);
             dmin_block = half_bits_to_float(w.header.x >> 16);
         }
 #pragma unroll
-        for (int bb = 0; bb < kBlocksPerWave; bb++) {
+        for (int bb = 0; bb < NB; bb++) {
             if (static_cast<uint32_t>(bb) < stage_blocks) {  // wave-uniform
-                const uint32_t b = b_base + bb;  // block inside the stage: LDS row and chunk index
-                const v4i bw = weight_operand<CODEC, kBlocksPerWave>(w, bb, half);
+                const uint32_t b = b_base + bb;              // block inside the stage
+                const v4i bw = weight_operand<CODEC, NB>(w, bb, half);
                 float w_scale;
                 if constexpr (CODEC == kQ4_K) {
                     float sc, mn;
-                    q4k_scale_min(w.header, static_cast<int>(b), sc, mn);
+                    q4k_scale_min(w.header, b, sc, mn);
                     w_scale = d_block * sc;
                 } else {
                     w_scale = half_bits_to_float(w.d[bb]);
                 }
+                // rank-1 operands: only the k = 0 half carries values
+                const float w_operand = half == 0 ? w_scale : 0.f;
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
-                    const uint32_t m = 32u * t + (lane & 31u);
-                    // block scales of the sixteen vectors this lane accumulates
-                    float sd[16];
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const float4 s4 =
-                            *reinterpret_cast<const float4*>(&lds.scale[b][32 * t + 8 * g + 4 * half]);
-                        sd[4 * g + 0] = s4.x * w_scale;
-                        sd[4 * g + 1] = s4.y * w_scale;
-                        sd[4 * g + 2] = s4.z * w_scale;
-                        sd[4 * g + 3] = s4.w * w_scale;
-                    }
-                    const uint32_t slot = 16u * x_chunk_slot(m, 2u * b + half);
+                    const uint8_t* blob = base + t * S::kBlob;
+                    const float x_scale =
+                        *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
+                    const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale : 0.f, w_operand,
+                                                                         zero_f, 0, 0, 0);
+                    const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
                     if constexpr (LIMBS == 1) {
-                        const v4i ax = *reinterpret_cast<const v4i*>(&lds.x[0][m][slot]);
-                        const v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(ax, bw, zero, 0, 0, 0);
+                        const v4i ax = *reinterpret_cast<const v4i*>(chunk);
+                        const v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(ax, bw, zero_i, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++)
                             acc[t][r] = fmaf(static_cast<float>(c[r]), sd[r], acc[t][r]);
                     } else {
-                        const v4i a0 = *reinterpret_cast<const v4i*>(&lds.x[0][m][slot]);
-                        const v4i a1 = *reinterpret_cast<const v4i*>(&lds.x[LIMBS > 1 ? 1 : 0][m][slot]);
-                        const v4i a2 = *reinterpret_cast<const v4i*>(&lds.x[LIMBS > 2 ? 2 : 0][m][slot]);
-                        const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bw, zero, 0, 0, 0);
-                        const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bw, zero, 0, 0, 0);
-                        const v16i c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a2, bw, zero, 0, 0, 0);
+                        const v4i a0 = *reinterpret_cast<const v4i*>(chunk);
+                        const v4i a1 = *reinterpret_cast<const v4i*>(chunk + 8192u);
+                        const v4i a2 = *reinterpret_cast<const v4i*>(chunk + 16384u);
+                        const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bw, zero_i, 0, 0, 0);
+                        const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bw, zero_i, 0, 0, 0);
+                        const v16i c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a2, bw, zero_i, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
-                            // |c0 + 256 c1| < 2^26 stays exact in int32; the top limb joins in f32
+                            // |c0 + 256 c1| < 2^28 is exact in int32; the top limb joins in f32
                             const float low = static_cast<float>(c0[r] + (c1[r] << 8));
                             const float all = fmaf(65536.0f, static_cast<float>(c2[r]), low);
                             acc[t][r] = fmaf(all, sd[r], acc[t][r]);
@@ -331,44 +344,82 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(
             }
         }
         if constexpr (CODEC == kQ4_K) {
-            // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g], K = 2 per MFMA,
-            // lane half h supplies sub-block 2j + h.
+          if (stage_blocks > 0) {
+            // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
+            // lane half h supplies sub-block 2j + h. (Q4_K stages are whole: all blocks or none.)
 #pragma unroll
-            for (int jj = 0; jj < 4 / KSPLIT; jj++) {
-                const int j = jj + static_cast<int>(wave_k) * (4 / KSPLIT);  // sub-block pair of the stage
-                float sc0, mn0, sc1, mn1;
-                q4k_scale_min(w.header, 2 * j, sc0, mn0);
-                q4k_scale_min(w.header, 2 * j + 1, sc1, mn1);
-                const float b_operand = dmin_block * (half ? mn1 : mn0);
+            for (int jj = 0; jj < NB / 2; jj++) {
+                const uint32_t g = b_base + 2u * jj + half;
+                float sc, mn;
+                q4k_scale_min(w.header, g, sc, mn);
+                const float b_operand = dmin_block * mn;
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
-                    const float a_operand = lds.xsum[2 * j + half][32 * t + (lane & 31u)];
+                    const float a_operand = *reinterpret_cast<const float*>(
+                        base + t * S::kBlob + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
                     acc_min[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc_min[t], 0, 0, 0);
                 }
             }
+          }
+        }
+    };
+
+    StageWeights<CODEC, NB> ring[S::kDepth];
+#pragma unroll
+    for (int a = 0; a < AHEAD; a++) {
+        request(a, ring[a]);
+        // Oldest stage first: the waits count back from the newest load. (`weight` is not
+        // declared __restrict__ so that this compiler barrier orders its loads.)
+        asm volatile("" ::: "memory");
+    }
+
+    // The ring position of a stage is a compile-time constant only if the loop is unrolled by
+    // the ring size. The bodies carry no early exit (stages past the end contract nothing):
+    // any extra edge in the loop's control flow makes the compiler assume that fewer loads
+    // were issued behind a weight register and wait for more than it has to.
+    for (uint32_t s0 = 0; s0 < padded_stages; s0 += S::kDepth) {
+#pragma unroll
+        for (int d = 0; d < S::kDepth; d++) {
+            const uint32_t stage = s0 + d;
+            // Stage `stage` is in LDS; every consumer is done with stage - 1.
+            // (A plain s_barrier: __syncthreads() adds a fence that waits for every load in flight.)
+            __builtin_amdgcn_s_barrier();
+            request(stage + AHEAD, ring[(d + AHEAD) % S::kDepth]);
+            __builtin_amdgcn_sched_barrier(0);
+            contract(stage, ring[d]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
-    // ---- combine the K halves, add bias, store --------------------------------
-    if constexpr (KSPLIT == 2) {
-        __syncthreads();
-        float* exchange = reinterpret_cast<float*>(&lds);  // [2 (wave_n)][MT*16][64 lanes]
-        static_assert(sizeof(StageLds<MT, LIMBS>) >= 2u * MT * 16u * 64u * 4u, "exchange buffer");
-        if (wave_k == 1) {
+    // ---- combine the K shares, add bias, store ----------------------------------
+    if constexpr (KSPLIT > 1) {
+        __syncthreads();  // the loaders arrive here with nothing in flight: the ring is free
+        float* exchange = reinterpret_cast<float*>(lds);  // [wave_k - 1][wave_n][MT * 16][64 lanes]
+        if (wave_k > 0) {
 #pragma unroll
             for (int t = 0; t < MT; t++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const float value = CODEC == kQ4_K ? acc[t][r] - acc_min[t][r] : acc[t][r];
-                    exchange[((wave_n * MT + t) * 16 + r) * 64 + lane] = value;
+                    exchange[((((wave_k - 1u) * S::kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane] = value;
                 }
         }
         __syncthreads();
-        if (wave_k == 1) return;
+        if (wave_k > 0) return;
 #pragma unroll
         for (int t = 0; t < MT; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[t][r] += exchange[((wave_n * MT + t) * 16 + r) * 64 + lane];
+            for (int r = 0; r < 16; r++) {
+                if constexpr (CODEC == kQ4_K) acc[t][r] -= acc_min[t][r];
+#pragma unroll
+                for (int k = 1; k < KSPLIT; k++)
+                    acc[t][r] += exchange[((((k - 1) * S::kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane];
+            }
+    } else if constexpr (CODEC == kQ4_K) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][r] -= acc_min[t][r];
     }
     const uint32_t n_out = n0 + (lane & 31u);
     if (n_out < rows) {
@@ -379,7 +430,7 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(
             for (int r = 0; r < 16; r++) {
                 const uint32_t m = m0 + 32u * t + 8u * (r >> 2) + 4u * half + (r & 3u);
                 if (m < vectors) {
-                    float value = CODEC == kQ4_K ? acc[t][r] - acc_min[t][r] : acc[t][r];
+                    float value = acc[t][r];
                     if (bias != nullptr) value += bias_value;
                     y[static_cast<uint64_t>(m) * rows + n_out] = value;
                 }
@@ -387,42 +438,43 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(
     }
 }
 
-template <int CODEC, int MT, int LIMBS, int KSPLIT>
-hipError_t launch(const uint8_t* weight, const int8_t* q, uint64_t limb_stride, const float* scale,
-                  const float* xsum, uint32_t table_stride, const float* bias, float* y, uint32_t rows,
-                  uint32_t columns, uint32_t vectors, hipStream_t stream) {
-    constexpr uint32_t BN = 128 / KSPLIT, BM = 32 * MT;
-    const dim3 grid((rows + BN - 1) / BN, (vectors + BM - 1) / BM);
-    hipLaunchKernelGGL((gemm_i8_kernel<CODEC, MT, LIMBS, KSPLIT>), grid, dim3(256), 0, stream, weight, q,
-                       limb_stride, scale, xsum, table_stride, bias, y, rows, columns, vectors);
+template <int CODEC, int MT, int LIMBS, int KSPLIT, int AHEAD>
+hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
+                  uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+    using S = Shape<CODEC, MT, LIMBS, KSPLIT, AHEAD>;
+    static_assert(S::kLdsBytes <= 160 * 1024, "LDS of a gfx950 CU");
+    const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, KSPLIT, AHEAD>;
+    // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
+    static bool allowed[64] = {};
+    int device = 0;
+    if (hipError_t status = hipGetDevice(&device)) return status;
+    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+    if (!allowed[device]) {
+        if (hipError_t status =
+                hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes))
+            return status;
+        allowed[device] = true;
+    }
+    const uint32_t vector_tiles = (vectors + 31u) / 32u;
+    const uint32_t vector_groups = (vector_tiles + MT - 1) / MT;
+    const uint32_t row_tiles = (rows + S::kRows - 1) / S::kRows;
+    const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_groups;
+    if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream,
+                       weight, tiles, vector_tiles, bias, y, rows, columns, vectors, row_tiles,
+                       vector_groups);
     return hipGetLastError();
 }
 
-template <int CODEC, int LIMBS>
-hipError_t launch_shape(const uint8_t* weight, const int8_t* q, uint64_t limb_stride,
-                        const float* scale, const float* xsum, uint32_t table_stride,
-                        const float* bias, float* y, uint32_t rows, uint32_t columns,
-                        uint32_t vectors, hipStream_t stream) {
-    // Few vectors: one tile of vectors, 64-row workgroups so that N/64 of them fill the CUs.
-    // Many vectors: 128 rows x 64 or 128 vectors per workgroup.
-    constexpr int kMaxTiles = LIMBS == 1 ? 4 : 2;  // LDS: 32*MT vectors x 256 B x LIMBS
-#define ET_GO(MT, KS) \
-    return launch<CODEC, MT, LIMBS, KS>(weight, q, limb_stride, scale, xsum, table_stride, bias, y, rows, columns, vectors, stream)
-    const bool few_row_tiles = (rows + 127u) / 128u * ((vectors + 32u * kMaxTiles - 1) / (32u * kMaxTiles)) < 192u;
-    if (vectors <= 32) {
-        if (few_row_tiles) ET_GO(1, 2);
-        ET_GO(1, 1);
-    }
-    if (vectors <= 64 || kMaxTiles == 2) {
-        if (few_row_tiles) ET_GO(2, 2);
-        ET_GO(2, 1);
-    }
-    if constexpr (kMaxTiles == 4) {
-        if (vectors <= 96) ET_GO(3, 1);
-        ET_GO(4, 1);
-    }
-#undef ET_GO
-    return hipErrorInvalidValue;
+template <int CODEC>
+hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const float* bias,
+                        float* y, uint32_t rows, uint32_t columns, uint32_t vectors,
+                        hipStream_t stream) {
+    // Three limbs: one 32-vector tile per workgroup (28 KiB of activations per stage), 3 stages ahead.
+    if (limbs == 3) return launch<CODEC, 1, 3, 4, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    if (vectors <= 32) return launch<CODEC, 1, 1, 4, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    return launch<CODEC, 2, 1, 4, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
 }
 
 }  // namespace
@@ -433,25 +485,18 @@ bool gemm_i8_supported(int32_t codec, uint64_t columns) {
     return false;
 }
 
-hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const int8_t* q,
-                   uint64_t limb_stride, const float* scale, const float* xsum,
-                   uint32_t table_stride, const float* bias, float* y, uint64_t rows,
-                   uint64_t columns, uint64_t vectors, hipStream_t stream) {
+hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
+                   const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
+                   hipStream_t stream) {
+    if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns),
                    m = static_cast<uint32_t>(vectors);
-#define ET_CODEC(C)                                                                                  \
-    case C:                                                                                          \
-        return limbs == 1 ? launch_shape<C, 1>(weight, q, limb_stride, scale, xsum, table_stride, bias, \
-                                               y, n, k, m, stream)                                   \
-                          : launch_shape<C, 3>(weight, q, limb_stride, scale, xsum, table_stride, bias, \
-                                               y, n, k, m, stream)
     switch (codec) {
-        ET_CODEC(kQ8_0);
-        ET_CODEC(kQ4_0);
-        ET_CODEC(kQ4_K);
+        case kQ8_0: return launch_codec<kQ8_0>(limbs, weight, tiles, bias, y, n, k, m, stream);
+        case kQ4_0: return launch_codec<kQ4_0>(limbs, weight, tiles, bias, y, n, k, m, stream);
+        case kQ4_K: return launch_codec<kQ4_K>(limbs, weight, tiles, bias, y, n, k, m, stream);
         default: return hipErrorInvalidValue;
     }
-#undef ET_CODEC
 }
 
 }  // namespace et

@@ -48,24 +48,34 @@ hipError_t gemv_generic(int32_t codec, const uint8_t* weight, const float* x, ui
                         uint32_t vectors, hipStream_t stream);
 
 // ---- quantize_act.hip --------------------------------------------------------
-// limbs = 1: q [vectors, columns] int8, scale = max|x| / 127 per vector and 32 columns.
-// limbs = 3: three byte planes q + limb * limb_stride of 24-bit fixed-point activations,
-//            scale = max|x| / (127 * 65536).
-// scale, sum (int32 block sums, may be null) and xsum (f32: scale * sum, may be null) are
-// TRANSPOSED: [columns/32, round_up(vectors, 32)].
+// Public layout: q [vectors, columns] int8, scale = max|x| / 127 per vector and 32 columns,
+// scale and sum (int32 block sums, may be null) TRANSPOSED: [columns/32, round_up(vectors, 32)].
 hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
-                                uint64_t columns, int limbs, int8_t* q, uint64_t limb_stride,
-                                float* scale, int32_t* sum, float* xsum, hipStream_t stream);
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                hipStream_t stream);
 
-// ---- gemm_i8.hip: matrix-core contraction over quantised activations ------------
+// Tiled layout for gemm_i8: blob (stage s, tile t) at ((s * tiles) + t) * tile_blob_bytes(limbs),
+// stages = ceil(columns / 256), tiles = ceil(vectors / 32). Inside a blob:
+//   limb l, 16-column chunk c (0..15), vector m (0..31): 16 int8 at  l*8192 + c*512 + m*16
+//   scale[block b (0..7)][m] f32 at  limbs*8192 + b*128 + m*4
+//   xsum [b][m] f32 (scale * integer block sum) at  limbs*8192 + 1024 + b*128 + m*4
+// and padding up to a multiple of 4096 bytes.
+// limbs = 1: int8 activations, scale = max|x| / 127.
+// limbs = 3: 24-bit fixed point in three balanced signed bytes, scale = max|x| / (127 * 65536).
+constexpr uint32_t tile_blob_bytes(int limbs) { return limbs == 1 ? 12288u : 28672u; }
+constexpr uint64_t tile_workspace_bytes(int limbs, uint64_t vectors, uint64_t columns) {
+    return ((columns + 255) / 256) * ((vectors + 31) / 32) * tile_blob_bytes(limbs);
+}
+hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vectors, uint64_t columns,
+                          int limbs, uint8_t* tiles, hipStream_t stream);
+
+// ---- gemm_i8.hip: matrix-core contraction over quantised activation tiles ---------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
 // From this many vectors on, f32-mode requests use the matrix cores (3-limb activations).
 constexpr uint32_t kGemmMinVectors = 4;
-// table_stride = round_up(vectors, 32): row pitch of the scale and xsum tables.
-hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const int8_t* q,
-                   uint64_t limb_stride, const float* scale, const float* xsum,
-                   uint32_t table_stride, const float* bias, float* y, uint64_t rows,
-                   uint64_t columns, uint64_t vectors, hipStream_t stream);
+hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
+                   const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
+                   hipStream_t stream);
 
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
 // sink must hold 4 * `workgroups` words; bytes < 2^36.

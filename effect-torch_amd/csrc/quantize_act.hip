@@ -11,12 +11,13 @@
 // three byte planes (range 127 * 2^16 instead of 127), which the same matrix-core
 // kernel contracts limb by limb with f32-level accuracy.
 //
-// Layout: q is [vectors, columns] int8 (row-major, what the MFMA operand loads
-// want); scale and sum are stored TRANSPOSED, [columns/32, stride] with
-// stride = vectors rounded up to a multiple of 32, so that the GEMM epilogue
-// reads the scales of four consecutive vectors with one 16-byte load and a
-// 32-vector tile never reads past the array. Entries at m >= vectors are
-// never written and never influence a stored output.
+// Two output layouts. The public one: q [vectors, columns] int8 row-major, scale and
+// sum TRANSPOSED, [columns/32, stride] with stride = vectors rounded up to a multiple
+// of 32 (entries at m >= vectors are never written). The one the matrix-core kernel
+// streams: a blob per (256-column stage, 32-vector tile) that holds the stage's
+// operands in exactly the order the kernel wants them in LDS, so that staging is a
+// linear copy (see tile_blob_bytes in kernels.h). Vectors at m >= vectors inside a
+// tile are never written and never influence a stored output.
 //
 // Eight lanes share a block: each loads one float4, the absmax and the sum are
 // folded across the eight with DPP, each lane packs its four int8 into a dword.
@@ -40,25 +41,28 @@ __device__ __forceinline__ int dpp_i32(int v) {
 
 // LIMBS = 1: q = clamp(rint(x * 127/amax)), scale = amax / 127.
 // LIMBS = 3: X = clamp(rint(x * 8323072/amax)) as three balanced signed bytes
-//            (X = 65536*x2 + 256*x1 + x0, planes q + limb * limb_stride), scale = amax / 8323072.
-// sum (int32, may be null) receives the block's integer sum, xsum (f32, may be null)
-// scale * sum: the activation block sum as the quantised operand represents it.
-template <int LIMBS>
+//            (X = 65536*x2 + 256*x1 + x0), scale = amax / 8323072.
+// TILED = false: q [vectors, columns], scale and sum transposed tables (the public layout).
+// TILED = true:  one blob per (256-column stage, 32-vector tile), see tile_blob_bytes();
+//                columns are padded with zeros to whole stages.
+template <int LIMBS, bool TILED>
 __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ x,
                                                        uint64_t x_row_stride, uint32_t vectors,
                                                        uint32_t columns, int8_t* __restrict__ q,
-                                                       uint64_t limb_stride, float* __restrict__ scale,
-                                                       int32_t* __restrict__ sum,
-                                                       float* __restrict__ xsum) {
+                                                       float* __restrict__ scale,
+                                                       int32_t* __restrict__ sum) {
     constexpr float kRange = LIMBS == 1 ? 127.f : 8323072.f;  // 127 * 2^16
-    const uint32_t quads_per_row = columns >> 2;
+    const uint32_t padded_columns = TILED ? (columns + 255u) & ~255u : columns;
+    const uint32_t quads_per_row = padded_columns >> 2;
+    const uint32_t vector_tiles = (vectors + 31u) >> 5;
     const uint64_t total = static_cast<uint64_t>(vectors) * quads_per_row;  // multiple of 8
     const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
     for (uint64_t item = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
          item += stride) {
         const uint32_t v = static_cast<uint32_t>(item / quads_per_row);
         const uint32_t quad = static_cast<uint32_t>(item - static_cast<uint64_t>(v) * quads_per_row);
-        const float4 in = *reinterpret_cast<const float4*>(x + v * x_row_stride + 4u * quad);
+        float4 in = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (4u * quad < columns) in = *reinterpret_cast<const float4*>(x + v * x_row_stride + 4u * quad);
         float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
         amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
         amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
@@ -76,56 +80,82 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
         total_q += dpp_i32<0xB1>(total_q);
         total_q += dpp_i32<0x4E>(total_q);
         total_q += dpp_i32<0x141>(total_q);
-        const uint64_t word = static_cast<uint64_t>(v) * quads_per_row + quad;
+        // limb planes: X + 0x808080 = (x2+128)<<16 | (x1+128)<<8 | (x0+128), every x in [-128, 127]
+        uint32_t packed[LIMBS];
         if constexpr (LIMBS == 1) {
-            const uint32_t packed = (static_cast<uint32_t>(qi[0]) & 0xffu) |
-                                    ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
-                                    ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
-                                    ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
-            reinterpret_cast<uint32_t*>(q)[word] = packed;
+            packed[0] = (static_cast<uint32_t>(qi[0]) & 0xffu) | ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
+                        ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
+                        ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
         } else {
-            // X + 0x808080 = (x2+128)<<16 | (x1+128)<<8 | (x0+128), every x in [-128, 127]
             uint32_t u[4];
 #pragma unroll
             for (int i = 0; i < 4; i++) u[i] = static_cast<uint32_t>(qi[i] + 0x808080);
 #pragma unroll
-            for (int limb = 0; limb < 3; limb++) {
-                const uint32_t packed = ((u[0] >> (8 * limb)) & 0xffu) |
-                                        (((u[1] >> (8 * limb)) & 0xffu) << 8) |
-                                        (((u[2] >> (8 * limb)) & 0xffu) << 16) |
-                                        (((u[3] >> (8 * limb)) & 0xffu) << 24);
-                reinterpret_cast<uint32_t*>(q + limb * limb_stride)[word] = packed ^ 0x80808080u;
+            for (int limb = 0; limb < LIMBS; limb++)
+                packed[limb] = (((u[0] >> (8 * limb)) & 0xffu) | (((u[1] >> (8 * limb)) & 0xffu) << 8) |
+                                (((u[2] >> (8 * limb)) & 0xffu) << 16) |
+                                (((u[3] >> (8 * limb)) & 0xffu) << 24)) ^ 0x80808080u;
+        }
+        const float unit = amax / kRange;
+        if constexpr (TILED) {
+            constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);
+            const uint32_t stage = quad >> 6, chunk = (quad & 63u) >> 2, dword = quad & 3u;
+            uint8_t* blob = reinterpret_cast<uint8_t*>(q) +
+                            (static_cast<uint64_t>(stage) * vector_tiles + (v >> 5)) * kBlob;
+#pragma unroll
+            for (int limb = 0; limb < LIMBS; limb++)
+                *reinterpret_cast<uint32_t*>(blob + limb * 8192u + chunk * 512u + (v & 31u) * 16u + dword * 4u) =
+                    packed[limb];
+            if ((quad & 7u) == 0) {
+                float* tables = reinterpret_cast<float*>(blob + LIMBS * 8192u);
+                const uint32_t block = (quad & 63u) >> 3;
+                tables[block * 32u + (v & 31u)] = unit;
+                tables[256u + block * 32u + (v & 31u)] = unit * static_cast<float>(total_q);
+            }
+        } else {
+            static_assert(TILED || LIMBS == 1, "the row-major layout is the int8 one");
+            reinterpret_cast<uint32_t*>(q)[static_cast<uint64_t>(v) * quads_per_row + quad] = packed[0];
+            if ((quad & 7u) == 0) {
+                const uint64_t slot = static_cast<uint64_t>(quad >> 3) * ((vectors + 31u) & ~31u) + v;
+                scale[slot] = unit;
+                if (sum != nullptr) sum[slot] = total_q;
             }
         }
-        if ((quad & 7u) == 0) {
-            const uint64_t slot = static_cast<uint64_t>(quad >> 3) * ((vectors + 31u) & ~31u) + v;
-            const float unit = amax / kRange;
-            scale[slot] = unit;
-            if (sum != nullptr) sum[slot] = total_q;
-            if (xsum != nullptr) xsum[slot] = unit * static_cast<float>(total_q);
-        }
     }
+}
+
+uint32_t grid_for(uint64_t items) {
+    uint64_t blocks = (items + 255) / 256;
+    return static_cast<uint32_t>(blocks > 16384 ? 16384 : blocks);
 }
 
 }  // namespace
 
 hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t vectors,
-                                uint64_t columns, int limbs, int8_t* q, uint64_t limb_stride,
-                                float* scale, int32_t* sum, float* xsum, hipStream_t stream) {
+                                uint64_t columns, int8_t* q, float* scale, int32_t* sum,
+                                hipStream_t stream) {
     const uint64_t total = vectors * (columns >> 2);
     if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL((quantize_kernel<1, false>), dim3(grid_for(total)), dim3(256), 0, stream, x,
+                       x_row_stride, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
+                       scale, sum);
+    return hipGetLastError();
+}
+
+hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vectors, uint64_t columns,
+                          int limbs, uint8_t* tiles, hipStream_t stream) {
+    const uint64_t total = vectors * (((columns + 255) & ~255ull) >> 2);
+    if (total == 0) return hipSuccess;
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
-    uint64_t blocks = (total + 255) / 256;
-    if (blocks > 16384) blocks = 16384;
-    const dim3 grid(static_cast<uint32_t>(blocks));
+    const dim3 grid(grid_for(total));
     if (limbs == 1)
-        hipLaunchKernelGGL(quantize_kernel<1>, grid, dim3(256), 0, stream, x, x_row_stride,
-                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
-                           limb_stride, scale, sum, xsum);
+        hipLaunchKernelGGL((quantize_kernel<1, true>), grid, dim3(256), 0, stream, x, x_row_stride,
+                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns),
+                           reinterpret_cast<int8_t*>(tiles), nullptr, nullptr);
     else
-        hipLaunchKernelGGL(quantize_kernel<3>, grid, dim3(256), 0, stream, x, x_row_stride,
-                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
-                           limb_stride, scale, sum, xsum);
+        hipLaunchKernelGGL((quantize_kernel<3, true>), grid, dim3(256), 0, stream, x, x_row_stride,
+                           static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns),
+                           reinterpret_cast<int8_t*>(tiles), nullptr, nullptr);
     return hipGetLastError();
 }
 

@@ -97,7 +97,7 @@ int validate_weight(const char* operation, const TensorView& weight, int32_t cod
 // cf. linear_kernel_kind, crates/runtime-metal/src/quantized.rs:1204-1220.
 int select_kernel(et_linear_plan* plan, std::string* error) {
     plan->gather_offset = plan->gather_bytes = 0;
-    plan->q_offset = plan->scale_offset = plan->sum_offset = plan->bias_offset = 0;
+    plan->q_offset = plan->bias_offset = 0;
     plan->workspace_bytes = 0;
     plan->vectors_per_launch = 0;
     if (plan->vectors == 0 || plan->rows == 0) {
@@ -114,15 +114,10 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     cursor = align_up(plan->gather_bytes, 256);
     plan->bias_offset = cursor;  // dense copy of a strided bias
     cursor = align_up(cursor + plan->rows * 4u, 256);
-    const auto plan_matrix_core = [&](LinearKernel kernel, uint64_t limbs) {
+    const auto plan_matrix_core = [&](LinearKernel kernel, int limbs) {
         plan->kernel = kernel;
-        plan->q_offset = cursor;
-        cursor = align_up(cursor + limbs * plan->vectors * plan->columns, 256);
-        plan->scale_offset = cursor;
-        const uint64_t padded_vectors = align_up(plan->vectors, 32);  // [columns/32, padded] tables
-        cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
-        plan->sum_offset = cursor;
-        cursor = align_up(cursor + padded_vectors * (plan->columns / 32) * 4u, 256);
+        plan->q_offset = cursor;  // activation tiles, see tile_blob_bytes()
+        cursor = align_up(cursor + tile_workspace_bytes(limbs, plan->vectors, plan->columns), 256);
     };
     if (plan->activation_mode == ET_ACT_INT8) {
         if (!gemm_i8_supported(plan->codec, plan->columns))
@@ -351,16 +346,12 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
                             " bytes is smaller than the planned " +
                             std::to_string(plan.workspace_bytes));
         const int limbs = plan.kernel == LinearKernel::kGemmI8 ? 1 : 3;
-        const uint64_t limb_stride = plan.vectors * plan.columns;
-        const uint32_t table_stride = static_cast<uint32_t>(align_up(plan.vectors, 32));
-        auto* q = reinterpret_cast<int8_t*>(scratch + plan.q_offset);
-        auto* scale = reinterpret_cast<float*>(scratch + plan.scale_offset);
-        auto* xsum = reinterpret_cast<float*>(scratch + plan.sum_offset);
-        if (hipError_t status = quantize_activations(x, x_row_stride, plan.vectors, plan.columns, limbs,
-                                                     q, limb_stride, scale, nullptr, xsum, s))
+        auto* tiles = scratch + plan.q_offset;
+        if (hipError_t status =
+                quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs, tiles, s))
             return hip_failure(error, "quantized_linear", status);
-        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, q, limb_stride, scale, xsum,
-                                        table_stride, bias, y, plan.rows, plan.columns, plan.vectors, s))
+        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, bias, y, plan.rows,
+                                        plan.columns, plan.vectors, s))
             return hip_failure(error, "quantized_linear", status);
         return ET_OK;
     }

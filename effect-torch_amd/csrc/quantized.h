@@ -53,7 +53,7 @@ struct et_linear_plan {
     // workspace sections (byte offsets), all 256-byte aligned
     uint64_t gather_offset, gather_bytes;  // densified f32 input
     uint64_t bias_offset;                  // densified f32 bias
-    uint64_t q_offset, scale_offset, sum_offset;
+    uint64_t q_offset;                     // quantised activation tiles (matrix-core kernels)
     uint64_t workspace_bytes;
 };
 
