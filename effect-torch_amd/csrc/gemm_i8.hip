@@ -62,17 +62,14 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-struct __attribute__((packed, aligned(2))) Bytes16 {
-    uint32_t v[4];
-};
-
 constexpr int kStageBlocks = 8;  // 32-column blocks per stage
 
 // Packed weights one lane holds for NB consecutive blocks of its row (its 16-column half).
 template <int CODEC, int NB>
 struct StageWeights {
-    uint4 q[NB];
-    uint32_t d[NB];  // fp16 bits
+    uint4 q[NB];        // the aligned 20-byte window around the 16 quant bytes: dwords 0..3
+    uint32_t tail[NB];  // and dword 4 (dword 3 again if the window is not shifted)
+    uint32_t d[NB];     // fp16 bits
 };
 template <int NB>
 struct StageWeights<kQ4_K, NB> {
@@ -83,13 +80,12 @@ struct StageWeights<kQ4_K, NB> {
 // VMEM instructions load_stage_weights issues (for the counted wait).
 template <int CODEC, int NB>
 constexpr int weight_loads() {
-    return CODEC == kQ4_K ? 1 + NB / 2 : 2 * NB;
+    return CODEC == kQ4_K ? 1 + NB / 2 : 3 * NB;
 }
 
-// first_block: index of the first 32-column block to load; blocks: how many of the NB exist.
+// first_block: index of the first of the NB 32-column blocks to load.
 template <int CODEC, int NB>
-__device__ __forceinline__ void load_stage_weights(const uint8_t* row, uint32_t first_block,
-                                                   uint32_t blocks, uint32_t half,
+__device__ __forceinline__ void load_stage_weights(const uint8_t* row, uint32_t first_block, uint32_t half,
                                                    StageWeights<CODEC, NB>& w) {
     if constexpr (CODEC == kQ4_K) {
         const uint8_t* block = row + static_cast<uint64_t>(first_block >> 3) * 144u;
@@ -102,27 +98,45 @@ __device__ __forceinline__ void load_stage_weights(const uint8_t* row, uint32_t 
         constexpr uint32_t kBytes = CODEC == kQ8_0 ? 34u : 18u;
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            // Blocks past the end of the row re-read an existing block; they are not used.
-            const uint32_t index = b < static_cast<int>(blocks) ? first_block + b : 0u;
-            const uint8_t* block = row + static_cast<uint64_t>(index) * kBytes;
-            const uint32_t offset = CODEC == kQ8_0 ? 2u + 16u * half : 2u;
-            const Bytes16 raw = *reinterpret_cast<const Bytes16*>(block + offset);
-            w.q[b] = make_uint4(raw.v[0], raw.v[1], raw.v[2], raw.v[3]);
+            const uint8_t* block = row + static_cast<uint64_t>(first_block + b) * kBytes;
+            // The 16 quant bytes start 2 bytes into a block that is itself only 2-byte aligned.
+            // A misaligned 16-byte load is served piecemeal; instead load the aligned 20-byte
+            // window around them (4 + 1 dwords); weight_operand() shifts by the 0 or 2 odd bytes.
+            // Every dword read holds at least one byte of the block, so no read leaves the buffer's
+            // pages: the fifth dword is only fetched when the window is shifted (else the fourth
+            // again: a load under a branch would cost the compiler its count of loads in flight).
+            const uint8_t* quants = block + (CODEC == kQ8_0 ? 2u + 16u * half : 2u);
+            const uint32_t odd = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(quants)) & 3u;  // 0 or 2
+            const uint8_t* window = quants - odd;
+            w.q[b] = *reinterpret_cast<const uint4*>(window);
+            w.tail[b] = *reinterpret_cast<const uint32_t*>(window + (odd ? 16 : 12));
             w.d[b] = *reinterpret_cast<const uint16_t*>(block);
         }
     }
 }
 
 // MFMA B operand (16 int8 weights) of local block b for this lane's half.
+// The 16 quant bytes out of the aligned window (32-wide codecs).
 template <int CODEC, int NB>
-__device__ __forceinline__ v4i weight_operand(const StageWeights<CODEC, NB>& w, int b, uint32_t half) {
+__device__ __forceinline__ uint4 window_quants(const StageWeights<CODEC, NB>& w, int b, bool shifted) {
+    const uint4 low = w.q[b];
+    if (!shifted) return low;
+    return make_uint4(__builtin_amdgcn_alignbit(low.y, low.x, 16), __builtin_amdgcn_alignbit(low.z, low.y, 16),
+                      __builtin_amdgcn_alignbit(low.w, low.z, 16), __builtin_amdgcn_alignbit(w.tail[b], low.w, 16));
+}
+
+// `shifted`: the block's quant bytes start 2 bytes into their aligned window (32-wide codecs).
+template <int CODEC, int NB>
+__device__ __forceinline__ v4i weight_operand(const StageWeights<CODEC, NB>& w, int b, uint32_t half,
+                                              bool shifted) {
     if constexpr (CODEC == kQ8_0) {
-        return v4i{static_cast<int>(w.q[b].x), static_cast<int>(w.q[b].y), static_cast<int>(w.q[b].z),
-                   static_cast<int>(w.q[b].w)};
+        const uint4 q = window_quants<CODEC, NB>(w, b, shifted);
+        return v4i{static_cast<int>(q.x), static_cast<int>(q.y), static_cast<int>(q.z), static_cast<int>(q.w)};
     } else if constexpr (CODEC == kQ4_0) {
         // element j = low nibble of byte j (j < 16), element j+16 = high nibble:
         // lanes 0-31 take the low nibbles, lanes 32-63 the high ones; value = nibble - 8.
-        const uint32_t words[4] = {w.q[b].x, w.q[b].y, w.q[b].z, w.q[b].w};
+        const uint4 q = window_quants<CODEC, NB>(w, b, shifted);
+        const uint32_t words[4] = {q.x, q.y, q.z, q.w};
         v4i out;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -203,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: uniform branches
     const uint32_t tile0 = vector_group * MT;
     const uint32_t xblocks = columns >> 5;
-    const uint32_t stages = (xblocks + kStageBlocks - 1) / kStageBlocks;
+    const uint32_t stages = xblocks / kStageBlocks;  // whole: columns % 256 == 0
     // Both loops run a whole number of ring turns; the stages past the end are empty.
     const uint32_t padded_stages = (stages + S::kDepth - 1) / S::kDepth * S::kDepth;
 
@@ -254,19 +268,13 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t n = min(n0 + (lane & 31u), rows - 1u);
     const uint64_t row_bytes = static_cast<uint64_t>(columns / block_values(CODEC)) * block_bytes(CODEC);
     const uint8_t* w_row = weight + n * row_bytes;
+    const uint32_t row_parity = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(w_row));
 
-    // Blocks of stage `stage` this wave contracts: first .. first + count (count may be 0).
+    // Stages are whole (columns % 256 == 0): this wave contracts blocks first .. first + NB of each.
     const auto wave_first = [&](uint32_t stage) { return stage * kStageBlocks + wave_k * NB; };
-    const auto wave_count = [&](uint32_t stage) {
-        const uint32_t first = wave_first(stage);
-        return first < xblocks ? min(xblocks - first, static_cast<uint32_t>(NB)) : 0u;
-    };
     // Requests this lane's weights of a stage (past the end: the last stage again, unused).
     const auto request = [&](uint32_t stage, StageWeights<CODEC, NB>& w) {
-        const uint32_t s = min(stage, stages - 1u);
-        uint32_t first = wave_first(s), count = wave_count(s);
-        if (count == 0) first = 0;  // a wave with no blocks in a partial last stage: any valid address
-        load_stage_weights<CODEC, NB>(w_row, first, count, half, w);
+        load_stage_weights<CODEC, NB>(w_row, wave_first(min(stage, stages - 1u)), half, w);
     };
 
     float acc[MT][16];
@@ -288,7 +296,11 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 
     // Contracts stage `stage` from its LDS slot and the weight registers `w`.
     const auto contract = [&](uint32_t stage, const StageWeights<CODEC, NB>& w) {
-        const uint32_t stage_blocks = wave_count(stage);
+        // All NB blocks, or none in the padding of the last ring turn. Written as a count that each
+        // block tests on its own: as straight-line code the stage needs more registers than the
+        // 168 a wave of this workgroup may hold, and spills.
+        const uint32_t first_block = wave_first(stage);
+        const uint32_t stage_blocks = first_block < xblocks ? min(xblocks - first_block, static_cast<uint32_t>(NB)) : 0u;
         const uint32_t b_base = wave_k * NB;  // first block of this wave inside the stage
         const uint8_t* base = lds + (stage % S::kDepth) * S::kSlotBytes;
         float d_block = 0.f, dmin_block = 0.f;
@@ -300,7 +312,13 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         for (int bb = 0; bb < NB; bb++) {
             if (static_cast<uint32_t>(bb) < stage_blocks) {  // wave-uniform
                 const uint32_t b = b_base + bb;              // block inside the stage
-                const v4i bw = weight_operand<CODEC, NB>(w, bb, half);
+                bool shifted = false;
+                if constexpr (CODEC != kQ4_K) {
+                    // parity of the quant bytes' address, as in load_stage_weights()
+                    constexpr uint32_t kBytes = CODEC == kQ8_0 ? 34u : 18u;
+                    shifted = ((row_parity + (wave_first(stage) + bb) * kBytes + 2u) & 2u) != 0;
+                }
+                const v4i bw = weight_operand<CODEC, NB>(w, bb, half, shifted);
                 float w_scale;
                 if constexpr (CODEC == kQ4_K) {
                     float sc, mn;
@@ -309,15 +327,17 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 } else {
                     w_scale = half_bits_to_float(w.d[bb]);
                 }
-                // rank-1 operands: only the k = 0 half carries values
-                const float w_operand = half == 0 ? w_scale : 0.f;
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const uint8_t* blob = base + t * S::kBlob;
+                    // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1
+                    // product in the MFMA result layout (only the k = 0 half of the lanes carries values).
+                    // One 4-byte LDS read per lane instead of 64 bytes: LDS bandwidth is what this
+                    // kernel runs out of first.
                     const float x_scale =
                         *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
-                    const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale : 0.f, w_operand,
-                                                                         zero_f, 0, 0, 0);
+                    const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale : 0.f,
+                                                                         half == 0 ? w_scale : 0.f, zero_f, 0, 0, 0);
                     const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
                     if constexpr (LIMBS == 1) {
                         const v4i ax = *reinterpret_cast<const v4i*>(chunk);
@@ -346,7 +366,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         if constexpr (CODEC == kQ4_K) {
           if (stage_blocks > 0) {
             // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
-            // lane half h supplies sub-block 2j + h. (Q4_K stages are whole: all blocks or none.)
+            // lane half h supplies sub-block 2j + h.
 #pragma unroll
             for (int jj = 0; jj < NB / 2; jj++) {
                 const uint32_t g = b_base + 2u * jj + half;
@@ -480,9 +500,8 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
 }  // namespace
 
 bool gemm_i8_supported(int32_t codec, uint64_t columns) {
-    if (codec == kQ8_0 || codec == kQ4_0) return columns % 32 == 0 && columns > 0;
-    if (codec == kQ4_K) return columns % 256 == 0 && columns > 0;
-    return false;
+    // Whole stages of 256 columns, also for the 32-wide codecs.
+    return (codec == kQ8_0 || codec == kQ4_0 || codec == kQ4_K) && columns % 256 == 0 && columns > 0;
 }
 
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,

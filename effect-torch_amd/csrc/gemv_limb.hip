@@ -26,34 +26,10 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstdio>
-#include <cstdlib>
 
 #include "et_codecs.h"
 #include "gemv_common.h"
 #include "kernels.h"
-
-#ifdef ET_TRACE
-// Debug build only: per-wave timestamps (100 MHz wall clock), kept in registers
-// and written once at the end of the wave.
-__device__ unsigned long long* g_et_trace = nullptr;
-#define ET_STAMP_DECL unsigned long long et_stamps[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define ET_STAMP(k) et_stamps[k] = wall_clock64()
-#define ET_STAMP_FLUSH()                                                                         \
-    do {                                                                                         \
-        if (g_et_trace != nullptr && (threadIdx.x & 63u) == 0)                                   \
-            for (int k_ = 0; k_ < 8; k_++)                                                       \
-                g_et_trace[(static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + k_] = \
-                    et_stamps[k_];                                                               \
-    } while (0)
-extern "C" int et_dbg_set_trace(unsigned long long* buffer) {
-    return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(g_et_trace), &buffer, sizeof buffer));
-}
-#else
-#define ET_STAMP_DECL
-#define ET_STAMP(k) do {} while (0)
-#define ET_STAMP_FLUSH() do {} while (0)
-#endif
 
 namespace et {
 namespace {
@@ -383,8 +359,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
                     xv[m][i] = reinterpret_cast<const float4*>(x + m * x_row_stride)[quad];
             }
     };
-    ET_STAMP_DECL;
-    ET_STAMP(0);
     float4 xv[M][NI];
     load_x(0, xv);
 
@@ -433,19 +407,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
                 const uint32_t f = threadIdx.x + i * THREADS;
                 if (f < kSliceQuads) stage_quad(stage[m], xv[m][i], f);  // wave-uniform condition
             }
-        ET_STAMP(1);
         __syncthreads();
-        ET_STAMP(2);
         if (s == slice) {
 #pragma unroll
             for (int m = 0; m < M; m++) load_limbs(stage[m], lane_id, active, xr[m]);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
-#ifdef ET_TRACE
-    asm volatile("" ::"v"(xr[0].limb[2][15]), "v"(xr[0].sum[1]));
-    ET_STAMP(3);
-#endif
 
     // Writes the outputs of iteration `it` from the per-row totals.
     auto write_rows = [&](uint32_t it, const float (&total)[R][M]) {
@@ -503,10 +471,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
             fold_row(current[r], total[r]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        ET_STAMP(5);
         write_rows(0, total);
-        ET_STAMP(6);
-        ET_STAMP_FLUSH();
     } else {
         // Two R-row buffers in ping-pong. Row 0 of the first is already on its way.
         typename T::Data other[R];
@@ -525,8 +490,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
                 write_rows(it + 1, total);
             }
         }
-        ET_STAMP(6);
-        ET_STAMP_FLUSH();
     }
 }
 
@@ -542,13 +505,11 @@ hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, 
 // Picks rows per workgroup and the single-shot depth for WAVES / NK row groups.
 template <class T, int M, int WAVES, int NK>
 hipError_t launch_rows(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
-                       float* y, uint32_t rows, uint32_t columns, hipStream_t stream,
-                       uint32_t force_depth = 0) {
+                       float* y, uint32_t rows, uint32_t columns, hipStream_t stream) {
     constexpr uint32_t RG = WAVES / NK;
     // One contiguous range of rows per CU; a wave takes ceil(range / RG) of them.
     const uint32_t share = (rows + 255u) / 256u;
-    uint32_t depth = (share + RG - 1) / RG;
-    if (force_depth) depth = force_depth;
+    const uint32_t depth = (share + RG - 1) / RG;
     // Registers bound the single-shot depth: 4 rows with more than 8 waves (128 VGPRs), else 8.
     constexpr uint32_t kMaxDepth = (WAVES > 8 || M > 1) ? 4 : 8;
 #define ET_SHOT(D)                                                                               \
@@ -586,12 +547,6 @@ hipError_t launch_slices(const uint8_t* weight, const float* x, uint64_t x_row_s
                          hipStream_t stream) {
     const uint32_t slices = (columns + kSliceColumns - 1) / kSliceColumns;
     if (slices <= 1) {
-        if (M == 1 && getenv("ET_EXP")) {  // EXPERIMENT HOOK "waves,depth"
-            int w = 8, d = 0;
-            sscanf(getenv("ET_EXP"), "%d,%d", &w, &d);
-            if (w == 14) return launch_rows<T, 1, 14, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream, d);
-            if (w == 16) return launch_rows<T, 1, 16, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream, d);
-        }
         return launch_rows<T, M, 8, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream);
     }
     if (slices <= 2) return launch_rows<T, M, 8, 2>(weight, x, x_row_stride, bias, y, rows, columns, stream);

@@ -209,13 +209,11 @@ def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
 
 
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0])
-@pytest.mark.parametrize("vectors,rows,columns", [(4, 129, 256), (8, 64, 2304), (33, 1, 512), (65, 300, 1024),
+@pytest.mark.parametrize("vectors,rows,columns", [(9, 129, 256), (12, 64, 2304), (33, 1, 512), (65, 300, 1024),
                                                   (100, 130, 4096), (130, 257, 768), (200, 63, 256)])
 def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, rows, columns):
-    # four or more vectors: 3-limb activations on the matrix cores; ragged tiles on every side,
-    # one and several stages of eight blocks, a partial last stage for the 32-wide codecs
-    if codec != oracle.Q4_K:
-        columns += 32
+    # nine or more vectors: 3-limb activations on the matrix cores; ragged tiles on both sides,
+    # one and several stages of 256 columns, ring turns with padding stages
     rng = np.random.default_rng(codec * 11 + vectors + rows + columns)
     weight = synth.random_weight(codec, rows, columns, rng)
     x = synth.random_activations(vectors, columns, rng)
@@ -225,6 +223,16 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
                                   None, et.GgmlQuant(codec), (rows, columns))
     assert plan.kernel == "quantize_limbs+gemm_i8"
     got = run_linear(et, device, codec, rows, columns, x, weight, bias)
+    if codec != oracle.Q4_K:
+        # a width that is not a whole number of 256-column stages stays on the GEMV kernels
+        odd = columns + 32
+        weight_odd = synth.random_weight(codec, rows, odd, rng)
+        x_odd = synth.random_activations(vectors, odd, rng)
+        plan = et.linear_requirements(torch.zeros(vectors, odd), torch.zeros((rows, weight_odd.shape[1]), dtype=torch.uint8),
+                                      None, et.GgmlQuant(codec), (rows, odd))
+        assert plan.kernel.startswith("gemv")
+        close(run_linear(et, device, codec, rows, odd, x_odd, weight_odd, bias),
+              oracle.linear_into(codec, rows, odd, x_odd, weight_odd, bias))
     close(got, oracle.linear_into(codec, rows, columns, x, weight, bias))
     exact = x.astype(np.float64) @ oracle.decode_rows(codec, weight, columns).astype(np.float64).T
     if bias is not None:
