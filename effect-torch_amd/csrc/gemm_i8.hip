@@ -44,6 +44,10 @@
 // per load. The loaders absorb both: they wait with an explicit count, nothing else
 // depends on them, and the consumers issue no global loads at all until they store.
 //
+// The consumers run each stage as a software pipeline over its (block, tile) steps: LDS
+// reads one step ahead of the MFMAs, the f32 epilogue one step behind them, so that the
+// matrix pipe, the VALU and LDS work on three different steps at a time.
+//
 // MFMA operand roles: A = activations, B = weights. A lane of the 32x32 result holds
 // one weight row n = lane % 32 and sixteen vectors m = 8*(r/4) + 4*(lane/32) + r%4,
 // and every result register row is stored as 128 contiguous bytes of y.
@@ -264,14 +268,14 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             d_block = half_bits_to_float(header.x & 0xffffu);
             dmin_block = half_bits_to_float(header.x >> 16);
         }
+        // B operands (16 int8 weights of row n, this lane's half of the block) and block scales
+        v4i bw[NB];
+        float w_scale[NB];
 #pragma unroll
         for (int bb = 0; bb < NB; bb++) {
             const uint32_t b = b_base + bb;  // block inside the stage
-            // B operand (16 int8 weights of row n, this lane's half of the block) and its scale
-            v4i bw;
-            float w_scale;
             if constexpr (CODEC == kQ8_0) {
-                bw = *reinterpret_cast<const v4i*>(region + (wave_n * 8u + b) * 1024u + lane * 16u);
+                bw[bb] = *reinterpret_cast<const v4i*>(region + (wave_n * 8u + b) * 1024u + lane * 16u);
             } else if constexpr (CODEC == kQ4_0) {
                 // element j = low nibble of byte j (j < 16), element j+16 = high nibble:
                 // lanes 0-31 take the low nibbles, lanes 32-63 the high ones; value = nibble - 8.
@@ -282,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 for (int i = 0; i < 4; i++) {
                     const uint32_t nib = (half ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu;
                     // (nib - 8) per byte without borrows between bytes
-                    bw[i] = static_cast<int>(((nib | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+                    bw[bb][i] = static_cast<int>(((nib | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
                 }
             } else {
                 // sub-block 2p + side: low (side 0) or high (side 1) nibbles of pair p
@@ -290,52 +294,78 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    bw[i] = static_cast<int>(((b & 1u) ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu);
+                    bw[bb][i] = static_cast<int>(((b & 1u) ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu);
             }
             if constexpr (CODEC == kQ4_K) {
                 float sc, mn;
                 q4k_scale_min(header, b, sc, mn);
-                w_scale = d_block * sc;
+                w_scale[bb] = d_block * sc;
             } else {
                 const uint32_t word = *reinterpret_cast<const uint32_t*>(
                     region + W::kSmallAt + (wave_n * 4u + (b >> 1)) * 256u + ((b & 1u) * 32u + (lane & 31u)) * 4u);
-                w_scale = half_bits_to_float(word & 0xffffu);
+                w_scale[bb] = half_bits_to_float(word & 0xffffu);
             }
-#pragma unroll
-            for (int t = 0; t < MT; t++) {
-                const uint8_t* blob = slot + t * S::kBlob;
-                // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1
-                // product in the MFMA result layout (only the k = 0 half of the lanes carries values).
-                const float x_scale =
-                    *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
-                const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale : 0.f,
-                                                                     half == 0 ? w_scale : 0.f, zero_f, 0, 0, 0);
-                const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
-                if constexpr (LIMBS == 1) {
-                    const v4i ax = *reinterpret_cast<const v4i*>(chunk);
-                    const v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(ax, bw, zero_i, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[t][r] = fmaf(static_cast<float>(c[r]), sd[r], acc[t][r]);
-                } else {
-                    const v4i a0 = *reinterpret_cast<const v4i*>(chunk);
-                    const v4i a1 = *reinterpret_cast<const v4i*>(chunk + 8192u);
-                    const v4i a2 = *reinterpret_cast<const v4i*>(chunk + 16384u);
-                    const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bw, zero_i, 0, 0, 0);
-                    const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bw, zero_i, 0, 0, 0);
-                    const v16i c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a2, bw, zero_i, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        // |c0 + 256 c1| < 2^28 is exact in int32; the top limb joins in f32
-                        const float low = static_cast<float>(c0[r] + (c1[r] << 8));
-                        const float all = fmaf(65536.0f, static_cast<float>(c2[r]), low);
-                        acc[t][r] = fmaf(all, sd[r], acc[t][r]);
-                    }
-                }
-                // One tile at a time: interleaving the tiles of a block costs more registers than
-                // the 168 a wave of this 12-wave workgroup may hold.
-                if constexpr (MT > 1) __builtin_amdgcn_sched_barrier(0);
-            }
+            // rank-1 operand: only the k = 0 half of the lanes carries a value
+            w_scale[bb] = half == 0 ? w_scale[bb] : 0.f;
         }
+
+        // The NB * MT (block, tile) steps of the stage as a software pipeline. Each step reads its
+        // A operands (and the activation scales) from LDS one step ahead, issues its MFMAs, and
+        // runs the f32 epilogue of an earlier step while they execute: with one limb the previous
+        // step's (its results are double-buffered), with three limbs its own (three results of
+        // sixteen registers each leave no room for a second set).
+        constexpr int kSteps = NB * MT;
+        const auto read_step = [&](int step, v4i (&a)[LIMBS], float& x_scale) {
+            const uint32_t b = b_base + step / MT;
+            const uint8_t* blob = slot + (step % MT) * S::kBlob;
+            x_scale = *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
+            const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
+#pragma unroll
+            for (int l = 0; l < LIMBS; l++) a[l] = *reinterpret_cast<const v4i*>(chunk + l * 8192u);
+        };
+        // acc[t] += sd * (c[0] + 256 c[1] + 65536 c[2])
+        const auto epilogue = [&](int step, const v16f& sd, const v16i (&c)[LIMBS]) {
+            const int t = step % MT;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                if constexpr (LIMBS == 1) {
+                    acc[t][r] = fmaf(static_cast<float>(c[0][r]), sd[r], acc[t][r]);
+                } else {
+                    // |c0 + 256 c1| < 2^28 is exact in int32; the top limb joins in f32
+                    const float low = static_cast<float>(c[0][r] + (c[1][r] << 8));
+                    const float all = fmaf(65536.0f, static_cast<float>(c[2][r]), low);
+                    acc[t][r] = fmaf(all, sd[r], acc[t][r]);
+                }
+            }
+        };
+        v4i a_next[LIMBS];
+        float x_scale_next;
+        read_step(0, a_next, x_scale_next);
+        v16f sd_previous;
+        v16i c_previous[LIMBS];
+#pragma unroll
+        for (int step = 0; step < kSteps; step++) {
+            const int bb = step / MT;
+            // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1
+            // product in the MFMA result layout.
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale_next : 0.f, w_scale[bb],
+                                                                 zero_f, 0, 0, 0);
+            v16i c[LIMBS];
+#pragma unroll
+            for (int l = 0; l < LIMBS; l++)
+                c[l] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[l], bw[bb], zero_i, 0, 0, 0);
+            if (step + 1 < kSteps) read_step(step + 1, a_next, x_scale_next);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (LIMBS == 1) {
+                if (step > 0) epilogue(step - 1, sd_previous, c_previous);
+                sd_previous = sd;
+                c_previous[0] = c[0];
+            } else {
+                epilogue(step, sd, c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (LIMBS == 1) epilogue(kSteps - 1, sd_previous, c_previous);
         if constexpr (CODEC == kQ4_K) {
             // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
             // lane half h supplies sub-block 2j + h.
