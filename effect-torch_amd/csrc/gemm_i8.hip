@@ -116,8 +116,9 @@ template <int CODEC, int MT, int LIMBS, int AHEAD>
 struct Shape {
     using W = WeightLayout<CODEC>;
     static constexpr int kDepth = AHEAD + 1;
-    static constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);
-    static constexpr uint32_t kActivationBytes = MT * kBlob;
+    static constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);        // in memory, padded
+    static constexpr uint32_t kTile = LIMBS * 8192u + 2048u;          // in LDS: operands and both tables
+    static constexpr uint32_t kActivationBytes = MT * kTile;
     static constexpr uint32_t kSlotBytes = kActivationBytes + W::kBytes;
     // One global_load_lds moves up to 1 KiB per wave.
     static constexpr int kActivationJobs = kActivationBytes / 1024;
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 if (job >= static_cast<uint32_t>(S::kJobs)) job -= S::kJobs;
                 if (job < static_cast<uint32_t>(S::kActivationJobs)) {
                     // 1 KiB of the activation blobs, as they lie in memory
-                    const uint32_t t = job / (S::kBlob / 1024u), within = job % (S::kBlob / 1024u);
+                    const uint32_t t = job / (S::kTile / 1024u), within = job % (S::kTile / 1024u);
                     const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
                     const uint8_t* src = tiles + (static_cast<uint64_t>(s) * vector_tiles + tile) * S::kBlob +
                                          within * 1024u + lane * 16u;
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         constexpr int kSteps = NB * MT;
         const auto read_step = [&](int step, v4i (&a)[LIMBS], float& x_scale) {
             const uint32_t b = b_base + step / MT;
-            const uint8_t* blob = slot + (step % MT) * S::kBlob;
+            const uint8_t* blob = slot + (step % MT) * S::kTile;
             x_scale = *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
             const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
 #pragma unroll
@@ -378,7 +379,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const float a_operand = *reinterpret_cast<const float*>(
-                        slot + t * S::kBlob + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
+                        slot + t * S::kTile + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
                     acc_min[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc_min[t], 0, 0, 0);
                 }
             }
@@ -449,8 +450,8 @@ template <int CODEC>
 hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const float* bias,
                         float* y, uint32_t rows, uint32_t columns, uint32_t vectors,
                         hipStream_t stream) {
-    // The ring depth is what LDS allows: 28 KiB of activations per stage and 32 vectors with
-    // three limbs, 12 KiB with one; 9 to 18 KiB of weights.
+    // The ring depth is what LDS allows: 26 KiB of activations per stage and 32 vectors with
+    // three limbs, 10 KiB with one; 9 to 18 KiB of weights.
     if (limbs == 3) {
         constexpr int kAhead = CODEC == kQ8_0 ? 2 : 3;
         return launch<CODEC, 1, 3, kAhead>(weight, tiles, bias, y, rows, columns, vectors, stream);
@@ -458,8 +459,8 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
     if (vectors <= 32) return launch<CODEC, 1, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
     // Q4_K carries a second accumulator (the min term): four tiles of both do not fit in registers.
     if (vectors <= 64 || CODEC == kQ4_K)
-        return launch<CODEC, 2, 1, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    return launch<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, bias, y, rows, columns,
+        return launch<CODEC, 2, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    return launch<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 3 : 1)>(weight, tiles, bias, y, rows, columns,
                                                                             vectors, stream);
 }
 

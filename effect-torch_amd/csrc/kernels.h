@@ -72,8 +72,8 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
 // ---- gemm_i8.hip: matrix-core contraction over quantised activation tiles ---------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
 // From this many vectors on, f32-mode requests use the matrix cores (3-limb activations):
-// measured on MI355X, three launches of the 3-vector GEMV are still faster below it.
-constexpr uint32_t kGemmMinVectors = 9;
+// measured on MI355X, two launches of the 3-vector GEMV are still faster below it.
+constexpr uint32_t kGemmMinVectors = 7;
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
                    const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
                    hipStream_t stream);

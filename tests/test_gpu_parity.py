@@ -209,10 +209,10 @@ def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
 
 
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0])
-@pytest.mark.parametrize("vectors,rows,columns", [(9, 129, 256), (12, 64, 2304), (33, 1, 512), (65, 300, 1024),
+@pytest.mark.parametrize("vectors,rows,columns", [(7, 129, 256), (12, 64, 2304), (33, 1, 512), (65, 300, 1024),
                                                   (100, 130, 4096), (130, 257, 768), (200, 63, 256)])
 def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, rows, columns):
-    # nine or more vectors: 3-limb activations on the matrix cores; ragged tiles on both sides,
+    # seven or more vectors: 3-limb activations on the matrix cores; ragged tiles on both sides,
     # one and several stages of 256 columns, ring turns with padding stages
     rng = np.random.default_rng(codec * 11 + vectors + rows + columns)
     weight = synth.random_weight(codec, rows, columns, rng)
