@@ -269,6 +269,24 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             d_block = half_bits_to_float(header.x & 0xffffu);
             dmin_block = half_bits_to_float(header.x >> 16);
         }
+        if constexpr (CODEC == kQ4_K) {
+            // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
+            // lane half h supplies sub-block 2j + h. First in the stage: its LDS reads go out with
+            // the other operands' and its MFMAs run under the first steps.
+#pragma unroll
+            for (int jj = 0; jj < NB / 2; jj++) {
+                const uint32_t g = b_base + 2u * jj + half;
+                float sc, mn;
+                q4k_scale_min(header, g, sc, mn);
+                const float b_operand = dmin_block * mn;
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const float a_operand = *reinterpret_cast<const float*>(
+                        slot + t * S::kTile + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
+                    acc_min[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc_min[t], 0, 0, 0);
+                }
+            }
+        }
         // B operands (16 int8 weights of row n, this lane's half of the block) and block scales
         v4i bw[NB];
         float w_scale[NB];
@@ -367,23 +385,6 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (LIMBS == 1) epilogue(kSteps - 1, sd_previous, c_previous);
-        if constexpr (CODEC == kQ4_K) {
-            // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
-            // lane half h supplies sub-block 2j + h.
-#pragma unroll
-            for (int jj = 0; jj < NB / 2; jj++) {
-                const uint32_t g = b_base + 2u * jj + half;
-                float sc, mn;
-                q4k_scale_min(header, g, sc, mn);
-                const float b_operand = dmin_block * mn;
-#pragma unroll
-                for (int t = 0; t < MT; t++) {
-                    const float a_operand = *reinterpret_cast<const float*>(
-                        slot + t * S::kTile + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
-                    acc_min[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc_min[t], 0, 0, 0);
-                }
-            }
-        }
     }
 
     // ---- combine the K shares, add bias, store ----------------------------------
@@ -454,6 +455,7 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
     // three limbs, 10 KiB with one; 9 to 18 KiB of weights.
     if (limbs == 3) {
         constexpr int kAhead = CODEC == kQ8_0 ? 2 : 3;
+        // One 32-vector tile per workgroup: two tiles of three-limb results do not fit in registers.
         return launch<CODEC, 1, 3, kAhead>(weight, tiles, bias, y, rows, columns, vectors, stream);
     }
     if (vectors <= 32) return launch<CODEC, 1, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
