@@ -35,8 +35,8 @@
 //   weights      are gathered so that LDS holds every MFMA B operand where the lane
 //                that needs it reads one 16-byte slot at base + 16 * lane: loader lane
 //                l fetches the 16 quant bytes of row l % 32 and column half l / 32
-//                straight from the packed row (the source may be 2-byte aligned);
-//                block scales come with 4-byte copies, Q4_K headers with 16-byte ones.
+//                straight from the packed row (for the 2-byte aligned Q8_0 / Q4_0 blocks:
+//                the dword-aligned window around them, see WeightLayout).
 // Why separate waves: loads return in order and are counted per wave; a wave that
 // mixes global_load_lds with loads into registers gets a full wait (vmcnt 0) from
 // the compiler before every use of a loaded register, and a consumer wave whose
@@ -93,24 +93,34 @@ constexpr int vmcnt_only(int n) {
 }
 
 // Weight region of an LDS slot, per codec. "Quant pieces" are 1 KiB: 64 slots of 16 bytes.
-//   Q8_0  piece (g, b): slot l = quants of row 32g + l%32, block b, column half l/32.
-//         scale pieces of 256 bytes, (g, j): word l = first 4 bytes (d, 2 quants) of block 2j + l/32.
-//   Q4_0  piece (g, j): slot l = the 16 quant bytes (both nibble halves) of block 2j + l/32.
-//         scale pieces as Q8_0.
-//   Q4_K  piece (g, p): slot l = bytes 16*(l/32) .. +16 of nibble pair p.
+//   Q4_K  piece (g, p): slot l = bytes 16*(l/32) .. +16 of nibble pair p of row 32g + l%32.
 //         header pieces of 1 KiB, one per two row groups h: slot l = header of row 64h + l.
+//   Q8_0, Q4_0: blocks are only 2-byte aligned, and a gather of misaligned 16-byte pieces is
+//         served several times slower than an aligned one. So LDS receives the dword-aligned
+//         20-byte WINDOW that starts at or 2 bytes before `start` = block + 16 * half
+//         (Q8_0) or block (Q4_0): dwords 0..3 in a quant piece, dword 4 in a "tail" piece of
+//         256 bytes. The window holds start .. start + 18: the fp16 scale (half 0) and 16
+//         quant bytes at start + 2. The consumer shifts by the odd 2 bytes where needed.
+//         Q8_0 piece (g, b): slot l = window of row 32g + l%32, block b, column half l/32.
+//         Q4_0 piece (g, j): slot l = window of row 32g + l%32, block 2j + l/32 (both nibble halves).
 template <int CODEC>
 struct WeightLayout {
     static constexpr bool kSuper = CODEC == kQ4_K;
     static constexpr uint32_t kBlockBytes = CODEC == kQ8_0 ? 34u : 18u;  // 32-wide codecs
     static constexpr int kQuantPieces = CODEC == kQ8_0 ? 8 : 4;          // per row group and stage
     static constexpr int kQuantJobs = kRowGroups * kQuantPieces;
-    static constexpr int kSmallJobs = kSuper ? kRowGroups / 2 : kRowGroups * 4;  // headers / scale pieces
+    static constexpr int kSmallJobs = kSuper ? kRowGroups / 2 : kQuantJobs;  // headers / tails
     static constexpr uint32_t kSmallBytes = kSuper ? 1024u : 256u;
     static constexpr uint32_t kSmallAt = kQuantJobs * 1024u;  // offset of the small pieces
     static constexpr uint32_t kBytes = kSmallAt + kSmallJobs * kSmallBytes;
     static constexpr int kJobs = kQuantJobs + kSmallJobs;
 };
+
+// Start of the window of (row pointer, block index, column half): see WeightLayout.
+template <int CODEC>
+__device__ __forceinline__ const uint8_t* window_start(const uint8_t* row, uint64_t block, uint32_t half) {
+    return row + block * WeightLayout<CODEC>::kBlockBytes + (CODEC == kQ8_0 ? 16u * half : 0u);
+}
 
 template <int CODEC, int MT, int LIMBS, int AHEAD>
 struct Shape {
@@ -186,12 +196,14 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                     const uint32_t g = job / W::kQuantPieces, piece = job % W::kQuantPieces;
                     const uint32_t row = min(row0 + 32u * g + (lane & 31u), rows - 1u);
                     const uint8_t* src = weight + row * row_bytes;
-                    if constexpr (CODEC == kQ4_K)
+                    if constexpr (CODEC == kQ4_K) {
                         src += static_cast<uint64_t>(s) * 144u + 16u + 32u * piece + 16u * (lane >> 5);
-                    else if constexpr (CODEC == kQ8_0)
-                        src += (static_cast<uint64_t>(s) * kStageBlocks + piece) * 34u + 2u + 16u * (lane >> 5);
-                    else
-                        src += (static_cast<uint64_t>(s) * kStageBlocks + 2u * piece + (lane >> 5)) * 18u + 2u;
+                    } else {
+                        const uint64_t block = CODEC == kQ8_0 ? static_cast<uint64_t>(s) * kStageBlocks + piece
+                                                              : static_cast<uint64_t>(s) * kStageBlocks + 2u * piece + (lane >> 5);
+                        src = window_start<CODEC>(src, block, lane >> 5);
+                        src -= reinterpret_cast<uintptr_t>(src) & 2u;  // dword aligned
+                    }
                     __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                      reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
                     continue;
@@ -204,11 +216,14 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                                                      reinterpret_cast<uint4*>(region + W::kSmallAt + job * 1024u), 16,
                                                      0, 0);
                 } else {
-                    const uint32_t g = job / 4u, pair = job % 4u;
+                    // dword 4 of the same windows
+                    const uint32_t g = job / W::kQuantPieces, piece = job % W::kQuantPieces;
                     const uint32_t row = min(row0 + 32u * g + (lane & 31u), rows - 1u);
-                    const uint8_t* src = weight + row * row_bytes +
-                                         (static_cast<uint64_t>(s) * kStageBlocks + 2u * pair + (lane >> 5)) * W::kBlockBytes;
-                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src),
+                    const uint64_t block = CODEC == kQ8_0 ? static_cast<uint64_t>(s) * kStageBlocks + piece
+                                                          : static_cast<uint64_t>(s) * kStageBlocks + 2u * piece + (lane >> 5);
+                    const uint8_t* src = window_start<CODEC>(weight + row * row_bytes, block, lane >> 5);
+                    src -= reinterpret_cast<uintptr_t>(src) & 2u;
+                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src + 16),
                                                      reinterpret_cast<uint32_t*>(region + W::kSmallAt + job * 256u), 4,
                                                      0, 0);
                 }
@@ -235,6 +250,9 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t wave_k = wave / kRowGroups;  // share of the stage's blocks
     const uint32_t n0 = row0 + wave_n * 32u;
     const uint32_t m0 = tile0 * 32u;
+    // Low address bits of this lane's weight row (the loaders clamp rows the same way).
+    const uint32_t row_parity = static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>(weight + min(n0 + (lane & 31u), rows - 1u) * row_bytes));
 
     float acc[MT][16];
     v16f acc_min[MT];
@@ -293,36 +311,48 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 #pragma unroll
         for (int bb = 0; bb < NB; bb++) {
             const uint32_t b = b_base + bb;  // block inside the stage
-            if constexpr (CODEC == kQ8_0) {
-                bw[bb] = *reinterpret_cast<const v4i*>(region + (wave_n * 8u + b) * 1024u + lane * 16u);
-            } else if constexpr (CODEC == kQ4_0) {
-                // element j = low nibble of byte j (j < 16), element j+16 = high nibble:
-                // lanes 0-31 take the low nibbles, lanes 32-63 the high ones; value = nibble - 8.
-                const uint4 raw = *reinterpret_cast<const uint4*>(region + (wave_n * 4u + (b >> 1)) * 1024u +
-                                                                  ((b & 1u) * 32u + (lane & 31u)) * 16u);
-                const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t nib = (half ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu;
-                    // (nib - 8) per byte without borrows between bytes
-                    bw[bb][i] = static_cast<int>(((nib | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
-                }
-            } else {
+            if constexpr (CODEC == kQ4_K) {
                 // sub-block 2p + side: low (side 0) or high (side 1) nibbles of pair p
                 const uint4 raw = *reinterpret_cast<const uint4*>(region + (wave_n * 4u + (b >> 1)) * 1024u + lane * 16u);
                 const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     bw[bb][i] = static_cast<int>(((b & 1u) ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu);
-            }
-            if constexpr (CODEC == kQ4_K) {
                 float sc, mn;
                 q4k_scale_min(header, b, sc, mn);
                 w_scale[bb] = d_block * sc;
             } else {
-                const uint32_t word = *reinterpret_cast<const uint32_t*>(
-                    region + W::kSmallAt + (wave_n * 4u + (b >> 1)) * 256u + ((b & 1u) * 32u + (lane & 31u)) * 4u);
-                w_scale[bb] = half_bits_to_float(word & 0xffffu);
+                // This lane's window: piece and slot as the loaders filled them.
+                const uint32_t piece = CODEC == kQ8_0 ? wave_n * 8u + b : wave_n * 4u + (b >> 1);
+                const uint32_t in_piece = CODEC == kQ8_0 ? lane : (b & 1u) * 32u + (lane & 31u);
+                const uint4 low = *reinterpret_cast<const uint4*>(region + piece * 1024u + in_piece * 16u);
+                const uint32_t tail = *reinterpret_cast<const uint32_t*>(region + W::kSmallAt + piece * 256u + in_piece * 4u);
+                // The scale sits in the window of column half 0 (for Q4_0 that is this window).
+                const uint32_t scale_word =
+                    CODEC == kQ8_0 ? *reinterpret_cast<const uint32_t*>(region + piece * 1024u + (lane & 31u) * 16u) : low.x;
+                // Do the windows begin 2 bytes before their start? (same arithmetic as the loaders')
+                const uint32_t block_at = row_parity + (stage * kStageBlocks + b) * W::kBlockBytes;
+                const bool scale_shifted = (block_at & 2u) != 0;
+                const bool shifted = ((block_at + (CODEC == kQ8_0 ? 16u * half : 0u)) & 2u) != 0;
+                w_scale[bb] = half_bits_to_float(scale_shifted ? scale_word >> 16 : scale_word & 0xffffu);
+                // quant bytes: window + 4 if shifted, window + 2 if not
+                uint32_t words[4];
+                words[0] = shifted ? low.y : __builtin_amdgcn_alignbit(low.y, low.x, 16);
+                words[1] = shifted ? low.z : __builtin_amdgcn_alignbit(low.z, low.y, 16);
+                words[2] = shifted ? low.w : __builtin_amdgcn_alignbit(low.w, low.z, 16);
+                words[3] = shifted ? tail : __builtin_amdgcn_alignbit(tail, low.w, 16);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if constexpr (CODEC == kQ8_0) {
+                        bw[bb][i] = static_cast<int>(words[i]);
+                    } else {
+                        // element j = low nibble of byte j (j < 16), element j+16 = high nibble: lanes
+                        // 0-31 take the low nibbles, lanes 32-63 the high ones; value = nibble - 8,
+                        // per byte without borrows between bytes.
+                        const uint32_t nib = (half ? (words[i] >> 4) : words[i]) & 0x0f0f0f0fu;
+                        bw[bb][i] = static_cast<int>(((nib | 0x80808080u) - 0x08080808u) ^ 0x80808080u);
+                    }
+                }
             }
             // rank-1 operand: only the k = 0 half of the lanes carries a value
             w_scale[bb] = half == 0 ? w_scale[bb] : 0.f;
@@ -461,7 +491,7 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
     if (vectors <= 32) return launch<CODEC, 1, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
     // Q4_K carries a second accumulator (the min term): four tiles of both do not fit in registers.
     if (vectors <= 64 || CODEC == kQ4_K)
-        return launch<CODEC, 2, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
+        return launch<CODEC, 2, 1, (CODEC == kQ8_0 ? 2 : 3)>(weight, tiles, bias, y, rows, columns, vectors, stream);
     return launch<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 3 : 1)>(weight, tiles, bias, y, rows, columns,
                                                                             vectors, stream);
 }
