@@ -124,9 +124,14 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
     }
 }
 
-uint32_t grid_for(uint64_t items) {
-    uint64_t blocks = (items + 255) / 256;
-    return static_cast<uint32_t>(blocks > 16384 ? 16384 : blocks);
+// Small batches are latency-bound: one wave per workgroup spreads them over all CUs.
+struct Geometry {
+    uint32_t blocks, threads;
+};
+Geometry geometry_for(uint64_t items) {
+    const uint32_t threads = items <= 256u * 1024u ? 64u : 256u;
+    const uint64_t blocks = (items + threads - 1) / threads;
+    return {static_cast<uint32_t>(blocks > 16384 ? 16384 : blocks), threads};
 }
 
 }  // namespace
@@ -136,7 +141,8 @@ hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
                                 hipStream_t stream) {
     const uint64_t total = vectors * (columns >> 2);
     if (total == 0) return hipSuccess;
-    hipLaunchKernelGGL((quantize_kernel<1, false>), dim3(grid_for(total)), dim3(256), 0, stream, x,
+    const Geometry g = geometry_for(total);
+    hipLaunchKernelGGL((quantize_kernel<1, false>), dim3(g.blocks), dim3(g.threads), 0, stream, x,
                        x_row_stride, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), q,
                        scale, sum);
     return hipGetLastError();
@@ -147,13 +153,14 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
     const uint64_t total = vectors * (((columns + 255) & ~255ull) >> 2);
     if (total == 0) return hipSuccess;
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
-    const dim3 grid(grid_for(total));
+    const Geometry g = geometry_for(total);
+    const dim3 grid(g.blocks), block(g.threads);
     if (limbs == 1)
-        hipLaunchKernelGGL((quantize_kernel<1, true>), grid, dim3(256), 0, stream, x, x_row_stride,
+        hipLaunchKernelGGL((quantize_kernel<1, true>), grid, block, 0, stream, x, x_row_stride,
                            static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns),
                            reinterpret_cast<int8_t*>(tiles), nullptr, nullptr);
     else
-        hipLaunchKernelGGL((quantize_kernel<3, true>), grid, dim3(256), 0, stream, x, x_row_stride,
+        hipLaunchKernelGGL((quantize_kernel<3, true>), grid, block, 0, stream, x, x_row_stride,
                            static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns),
                            reinterpret_cast<int8_t*>(tiles), nullptr, nullptr);
     return hipGetLastError();
