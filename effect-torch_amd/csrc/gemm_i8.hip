@@ -28,21 +28,23 @@
 // MFMAs: four of them share 32 weight rows and split the eight blocks of every
 // stage between them; their accumulators meet in LDS at the end.
 //
-// Operand streams. Four more waves, the loaders, do nothing but copy the operands
-// of stage s + AHEAD into an LDS ring of AHEAD + 1 slots with global_load_lds while
-// the consumers contract stage s; one s_barrier per stage joins the two groups.
+// Operand streams. Four more waves, the loaders, do nothing but copy operands of
+// later stages into LDS rings with global_load_lds while the consumers contract
+// stage s; one s_barrier per stage joins the groups. Two loaders serve the
+// activation ring, two the weight ring: loads return in order per wave, so streams
+// with different leads must not share a wave. Activations are re-read by every
+// workgroup and come from L2: two stages of lead. Weights come from HBM, and what
+// bounds a CU's share of the bandwidth is how many bytes it keeps in flight: their
+// ring takes all the LDS that is left (up to twelve stages).
 //   activations  arrive as ready-made stage blobs (see kernels.h): a linear copy;
-//   weights      are gathered so that LDS holds every MFMA B operand where the lane
-//                that needs it reads one 16-byte slot at base + 16 * lane: loader lane
-//                l fetches the 16 quant bytes of row l % 32 and column half l / 32
-//                straight from the packed row (for the 2-byte aligned Q8_0 / Q4_0 blocks:
-//                the dword-aligned window around them, see WeightLayout).
+//   weights      the stage's bytes of the workgroup's rows, row after row as in memory
+//                (see WeightLayout for how the consumers read their operands out of them).
 // Why separate waves: loads return in order and are counted per wave; a wave that
 // mixes global_load_lds with loads into registers gets a full wait (vmcnt 0) from
 // the compiler before every use of a loaded register, and a consumer wave whose
-// lanes each read another weight row stalls in the address unit for about 64 clocks
-// per load. The loaders absorb both: they wait with an explicit count, nothing else
-// depends on them, and the consumers issue no global loads at all until they store.
+// lanes each read another weight row (what the B operand needs) stalls in the address
+// unit on every load. The loaders absorb both: they copy along rows, wait with an
+// explicit count, and the consumers issue no global loads at all until they store.
 //
 // The consumers run each stage as a software pipeline over its (block, tile) steps: LDS
 // reads one step ahead of the MFMAs, the f32 epilogue one step behind them, so that the
@@ -68,7 +70,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kStageBlocks = 8;  // 32-column blocks per stage
 constexpr int kConsumers = 8;    // waves that run the MFMAs: two per SIMD
-constexpr int kLoaders = 4;      // waves that only copy operands into LDS: one per SIMD
+constexpr int kWeightLoaders = 2;      // waves that only gather weights into LDS
+constexpr int kActivationLoaders = 2;  // waves that only copy activation blobs into LDS
+constexpr int kLoaders = kWeightLoaders + kActivationLoaders;
 constexpr int kThreads = 64 * (kConsumers + kLoaders);
 constexpr int kSplit = 4;                         // consumer waves sharing a row group
 constexpr int kRowGroups = kConsumers / kSplit;   // 32-row groups per workgroup
@@ -92,64 +96,59 @@ constexpr int vmcnt_only(int n) {
     return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
 }
 
-// Weight region of an LDS slot, per codec. "Quant pieces" are 1 KiB: 64 slots of 16 bytes.
-//   Q4_K  piece (g, p): slot l = bytes 16*(l/32) .. +16 of nibble pair p of row 32g + l%32.
-//         header pieces of 1 KiB, one per two row groups h: slot l = header of row 64h + l.
-//   Q8_0, Q4_0: blocks are only 2-byte aligned, and a gather of misaligned 16-byte pieces is
-//         served several times slower than an aligned one. So LDS receives the dword-aligned
-//         20-byte WINDOW that starts at or 2 bytes before `start` = block + 16 * half
-//         (Q8_0) or block (Q4_0): dwords 0..3 in a quant piece, dword 4 in a "tail" piece of
-//         256 bytes. The window holds start .. start + 18: the fp16 scale (half 0) and 16
-//         quant bytes at start + 2. The consumer shifts by the odd 2 bytes where needed.
-//         Q8_0 piece (g, b): slot l = window of row 32g + l%32, block b, column half l/32.
-//         Q4_0 piece (g, j): slot l = window of row 32g + l%32, block 2j + l/32 (both nibble halves).
+// Weight slot in LDS: the stage's bytes of the workgroup's 64 rows, row after row exactly as in
+// memory (a row's stage is 144 bytes for Q4_K and Q4_0, 272 for Q8_0: whole 16-byte chunks), so a
+// copy instruction's 64 lanes walk along rows and touch about fifteen cache lines. (Gathering one
+// chunk per row instead, ready in operand order, touches 32 to 64 lines per instruction and made
+// the loaders' issue rate the bound of the whole kernel.) The consumers pick their operands out
+// of the rows:
+//   Q4_K  16-byte reads at row*144 + {0 (header), 16 + 32*pair + 16*half}: the 144-byte pitch
+//         spreads eight consecutive rows over all banks.
+//   Q8_0, Q4_0: blocks are 2-byte aligned. A lane reads the five dwords around its block start
+//         (+ 16*half for Q8_0): they hold the fp16 scale and the 16 quant bytes behind it, to be
+//         shifted by 16 bits for even blocks (block starts alternate between 0 and 2 mod 4).
 template <int CODEC>
 struct WeightLayout {
-    static constexpr bool kSuper = CODEC == kQ4_K;
-    static constexpr uint32_t kBlockBytes = CODEC == kQ8_0 ? 34u : 18u;  // 32-wide codecs
-    static constexpr int kQuantPieces = CODEC == kQ8_0 ? 8 : 4;          // per row group and stage
-    static constexpr int kQuantJobs = kRowGroups * kQuantPieces;
-    static constexpr int kSmallJobs = kSuper ? kRowGroups / 2 : kQuantJobs;  // headers / tails
-    static constexpr uint32_t kSmallBytes = kSuper ? 1024u : 256u;
-    static constexpr uint32_t kSmallAt = kQuantJobs * 1024u;  // offset of the small pieces
-    static constexpr uint32_t kBytes = kSmallAt + kSmallJobs * kSmallBytes;
-    static constexpr int kJobs = kQuantJobs + kSmallJobs;
+    static constexpr uint32_t kBlockBytes = CODEC == kQ8_0 ? 34u : 18u;      // 32-wide codecs
+    static constexpr uint32_t kRowBytes = CODEC == kQ8_0 ? 272u : 144u;      // one row's stage
+    static constexpr uint32_t kBytes = kRows * kRowBytes;
+    static constexpr int kJobs = kBytes / 1024;
+    static_assert(kBytes % 1024 == 0, "whole copy instructions");
 };
 
-// Start of the window of (row pointer, block index, column half): see WeightLayout.
-template <int CODEC>
-__device__ __forceinline__ const uint8_t* window_start(const uint8_t* row, uint64_t block, uint32_t half) {
-    return row + block * WeightLayout<CODEC>::kBlockBytes + (CODEC == kQ8_0 ? 16u * half : 0u);
-}
-
-template <int CODEC, int MT, int LIMBS, int AHEAD>
+// AX / AW: how many stages the activation / weight stream runs ahead of the MFMAs.
+template <int CODEC, int MT, int LIMBS, int AX, int AW>
 struct Shape {
     using W = WeightLayout<CODEC>;
-    static constexpr int kDepth = AHEAD + 1;
     static constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);        // in memory, padded
     static constexpr uint32_t kTile = LIMBS * 8192u + 2048u;          // in LDS: operands and both tables
-    static constexpr uint32_t kActivationBytes = MT * kTile;
-    static constexpr uint32_t kSlotBytes = kActivationBytes + W::kBytes;
-    // One global_load_lds moves up to 1 KiB per wave.
+    // Two rings: activations come from L2 (every workgroup reads the same blobs) and need little
+    // lead; weights come from HBM and need as much as LDS allows.
+    static constexpr int kActivationDepth = AX + 1, kWeightDepth = AW + 1;
+    static constexpr uint32_t kActivationBytes = MT * kTile;            // per slot
+    static constexpr uint32_t kWeightRingAt = kActivationDepth * kActivationBytes;
+    static constexpr uint32_t kRingBytes = kWeightRingAt + kWeightDepth * W::kBytes;
+    // One global_load_lds moves up to 1 KiB per wave. Every loader of a stream issues the same
+    // number of copies per stage (for its counted wait): jobs are dealt round-robin and the last
+    // round wraps around to the first jobs, copied twice.
     static constexpr int kActivationJobs = kActivationBytes / 1024;
-    static constexpr int kJobs = kActivationJobs + W::kJobs;
-    // Every loader issues the same number of copies per stage (for its counted wait): jobs are
-    // dealt round-robin and the last round wraps around to the first jobs, copied twice.
-    static constexpr int kRounds = (kJobs + kLoaders - 1) / kLoaders;
-    static_assert(kJobs >= kLoaders, "the wrap-around of the last round needs a full first round");
+    static constexpr int kActivationRounds = (kActivationJobs + kActivationLoaders - 1) / kActivationLoaders;
+    static constexpr int kWeightRounds = (W::kJobs + kWeightLoaders - 1) / kWeightLoaders;
+    static_assert(kActivationJobs >= kActivationLoaders && W::kJobs >= kWeightLoaders,
+                  "the wrap-around of the last round needs a full first round");
     // vmcnt is a 6-bit counter: a smaller bound only waits for more than necessary.
-    static constexpr int kLoaderWait = (AHEAD - 1) * kRounds < 63 ? (AHEAD - 1) * kRounds : 63;
+    static constexpr int kActivationWait = (AX - 1) * kActivationRounds < 63 ? (AX - 1) * kActivationRounds : 63;
+    static constexpr int kWeightWait = (AW - 1) * kWeightRounds < 63 ? (AW - 1) * kWeightRounds : 63;
     static constexpr uint32_t kExchangeBytes = (kSplit - 1) * kRowGroups * MT * 16 * 64 * 4;
-    static constexpr uint32_t kLdsBytes =
-        kDepth * kSlotBytes > kExchangeBytes ? kDepth * kSlotBytes : kExchangeBytes;
+    static constexpr uint32_t kLdsBytes = kRingBytes > kExchangeBytes ? kRingBytes : kExchangeBytes;
 };
 
-template <int CODEC, int MT, int LIMBS, int AHEAD>
+template <int CODEC, int MT, int LIMBS, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint8_t* __restrict__ weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
     uint32_t vectors, uint32_t row_tiles, uint32_t vector_groups) {
-    using S = Shape<CODEC, MT, LIMBS, AHEAD>;
+    using S = Shape<CODEC, MT, LIMBS, AX, AW>;
     using W = WeightLayout<CODEC>;
     constexpr int NB = kBlocksPerWave;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -165,81 +164,66 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: uniform branches
     const uint32_t tile0 = vector_group * MT;
     const uint32_t stages = columns / 256u;  // whole: columns % 256 == 0
-    // Both loops run a whole number of ring turns; the stages past the end are empty.
-    const uint32_t padded_stages = (stages + S::kDepth - 1) / S::kDepth * S::kDepth;
     const uint64_t row_bytes = static_cast<uint64_t>(columns / block_values(CODEC)) * block_bytes(CODEC);
     const uint32_t row0 = row_tile * kRows;
 
-    if (wave >= static_cast<uint32_t>(kConsumers)) {
-        // ---- loader waves ---------------------------------------------------------
-        const uint32_t loader = wave - kConsumers;
+    if (wave >= static_cast<uint32_t>(kConsumers + kWeightLoaders)) {
+        // ---- activation loaders -----------------------------------------------------
+        const uint32_t loader = wave - (kConsumers + kWeightLoaders);
         const auto request = [&](uint32_t stage) {
             const uint32_t s = min(stage, stages - 1u);  // past the end: a copy nobody reads
-            uint8_t* slot = lds + (stage % S::kDepth) * S::kSlotBytes;
+            uint8_t* slot = lds + (stage % S::kActivationDepth) * S::kActivationBytes;
 #pragma unroll
-            for (int i = 0; i < S::kRounds; i++) {
-                uint32_t job = i * kLoaders + loader;
-                if (job >= static_cast<uint32_t>(S::kJobs)) job -= S::kJobs;
-                if (job < static_cast<uint32_t>(S::kActivationJobs)) {
-                    // 1 KiB of the activation blobs, as they lie in memory
-                    const uint32_t t = job / (S::kTile / 1024u), within = job % (S::kTile / 1024u);
-                    const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
-                    const uint8_t* src = tiles + (static_cast<uint64_t>(s) * vector_tiles + tile) * S::kBlob +
-                                         within * 1024u + lane * 16u;
-                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
-                                                     reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
-                    continue;
-                }
-                job -= S::kActivationJobs;
-                uint8_t* region = slot + S::kActivationBytes;
-                if (job < static_cast<uint32_t>(W::kQuantJobs)) {
-                    const uint32_t g = job / W::kQuantPieces, piece = job % W::kQuantPieces;
-                    const uint32_t row = min(row0 + 32u * g + (lane & 31u), rows - 1u);
-                    const uint8_t* src = weight + row * row_bytes;
-                    if constexpr (CODEC == kQ4_K) {
-                        src += static_cast<uint64_t>(s) * 144u + 16u + 32u * piece + 16u * (lane >> 5);
-                    } else {
-                        const uint64_t block = CODEC == kQ8_0 ? static_cast<uint64_t>(s) * kStageBlocks + piece
-                                                              : static_cast<uint64_t>(s) * kStageBlocks + 2u * piece + (lane >> 5);
-                        src = window_start<CODEC>(src, block, lane >> 5);
-                        src -= reinterpret_cast<uintptr_t>(src) & 2u;  // dword aligned
-                    }
-                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
-                                                     reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
-                    continue;
-                }
-                job -= W::kQuantJobs;
-                if constexpr (CODEC == kQ4_K) {
-                    const uint32_t row = min(row0 + 64u * job + lane, rows - 1u);
-                    const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(s) * 144u;
-                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
-                                                     reinterpret_cast<uint4*>(region + W::kSmallAt + job * 1024u), 16,
-                                                     0, 0);
-                } else {
-                    // dword 4 of the same windows
-                    const uint32_t g = job / W::kQuantPieces, piece = job % W::kQuantPieces;
-                    const uint32_t row = min(row0 + 32u * g + (lane & 31u), rows - 1u);
-                    const uint64_t block = CODEC == kQ8_0 ? static_cast<uint64_t>(s) * kStageBlocks + piece
-                                                          : static_cast<uint64_t>(s) * kStageBlocks + 2u * piece + (lane >> 5);
-                    const uint8_t* src = window_start<CODEC>(weight + row * row_bytes, block, lane >> 5);
-                    src -= reinterpret_cast<uintptr_t>(src) & 2u;
-                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(src + 16),
-                                                     reinterpret_cast<uint32_t*>(region + W::kSmallAt + job * 256u), 4,
-                                                     0, 0);
-                }
+            for (int i = 0; i < S::kActivationRounds; i++) {
+                uint32_t job = i * kActivationLoaders + loader;  // 1 KiB of the blobs, as they lie in memory
+                if (job >= static_cast<uint32_t>(S::kActivationJobs)) job -= S::kActivationJobs;
+                const uint32_t t = job / (S::kTile / 1024u), within = job % (S::kTile / 1024u);
+                const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
+                const uint8_t* src = tiles + (static_cast<uint64_t>(s) * vector_tiles + tile) * S::kBlob +
+                                     within * 1024u + lane * 16u;
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
+                                                 reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
             }
         };
-        for (uint32_t a = 0; a < static_cast<uint32_t>(AHEAD); a++) request(a);
-        for (uint32_t stage = 0; stage < padded_stages; stage++) {
-            // Loads return in order: all but the newest AHEAD - 1 requests have landed.
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kLoaderWait));
-            // Passing the barrier says "stage is in LDS" to the consumers and "the slot of
-            // stage - 1 is free" to the loaders.
+        for (uint32_t a = 0; a < static_cast<uint32_t>(AX); a++) request(a);
+        for (uint32_t stage = 0; stage < stages; stage++) {
+            // Loads return in order: all but the newest AX - 1 requests have landed.
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kActivationWait));
+            // Passing the barrier says "stage is in LDS" to the consumers and "the slots of
+            // stage - 1 are free" to the loaders.
             __builtin_amdgcn_s_barrier();
-            request(stage + AHEAD);
+            request(stage + AX);
         }
         __builtin_amdgcn_s_waitcnt(vmcnt_only(0));  // nothing may still write the ring
         __builtin_amdgcn_s_barrier();               // the consumers' two exchange barriers
+        __builtin_amdgcn_s_barrier();
+        return;
+    }
+    if (wave >= static_cast<uint32_t>(kConsumers)) {
+        // ---- weight loaders ---------------------------------------------------------
+        const uint32_t loader = wave - kConsumers;
+        const auto request = [&](uint32_t stage) {
+            const uint32_t s = min(stage, stages - 1u);
+            uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * W::kBytes;
+#pragma unroll
+            for (int i = 0; i < S::kWeightRounds; i++) {
+                uint32_t job = i * kWeightLoaders + loader;
+                if (job >= static_cast<uint32_t>(W::kJobs)) job -= W::kJobs;
+                const uint32_t at = job * 1024u + lane * 16u;  // byte of the slot this lane fills
+                const uint32_t row = min(row0 + at / W::kRowBytes, rows - 1u);
+                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(s) * W::kRowBytes + at % W::kRowBytes;
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
+                                                 reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
+            }
+        };
+        for (uint32_t a = 0; a < static_cast<uint32_t>(AW); a++) request(a);
+        for (uint32_t stage = 0; stage < stages; stage++) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kWeightWait));
+            __builtin_amdgcn_s_barrier();
+            request(stage + AW);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_s_barrier();
         return;
     }
@@ -250,10 +234,6 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t wave_k = wave / kRowGroups;  // share of the stage's blocks
     const uint32_t n0 = row0 + wave_n * 32u;
     const uint32_t m0 = tile0 * 32u;
-    // Low address bits of this lane's weight row (the loaders clamp rows the same way).
-    const uint32_t row_parity = static_cast<uint32_t>(
-        reinterpret_cast<uintptr_t>(weight + min(n0 + (lane & 31u), rows - 1u) * row_bytes));
-
     float acc[MT][16];
     v16f acc_min[MT];
 #pragma unroll
@@ -271,19 +251,18 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         zero_f[r] = 0.f;
     }
 
-    for (uint32_t stage = 0; stage < padded_stages; stage++) {
+    for (uint32_t stage = 0; stage < stages; stage++) {
         // A plain s_barrier: __syncthreads() would add a fence the loop does not need.
         __builtin_amdgcn_s_barrier();
-        if (stage >= stages) continue;  // padding of the last ring turn
-        const uint8_t* slot = lds + (stage % S::kDepth) * S::kSlotBytes;
-        const uint8_t* region = slot + S::kActivationBytes;
+        const uint8_t* slot = lds + (stage % S::kActivationDepth) * S::kActivationBytes;
+        const uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * W::kBytes;
         const uint32_t b_base = wave_k * NB;  // first block of this wave inside the stage
+        const uint8_t* row_in_slot = region + (wave_n * 32u + (lane & 31u)) * W::kRowBytes;  // this lane's row
 
         uint4 header = make_uint4(0u, 0u, 0u, 0u);
         float d_block = 0.f, dmin_block = 0.f;
         if constexpr (CODEC == kQ4_K) {
-            header = *reinterpret_cast<const uint4*>(region + W::kSmallAt + (wave_n >> 1) * 1024u +
-                                                    ((wave_n & 1u) * 32u + (lane & 31u)) * 16u);
+            header = *reinterpret_cast<const uint4*>(row_in_slot);
             d_block = half_bits_to_float(header.x & 0xffffu);
             dmin_block = half_bits_to_float(header.x >> 16);
         }
@@ -313,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             const uint32_t b = b_base + bb;  // block inside the stage
             if constexpr (CODEC == kQ4_K) {
                 // sub-block 2p + side: low (side 0) or high (side 1) nibbles of pair p
-                const uint4 raw = *reinterpret_cast<const uint4*>(region + (wave_n * 4u + (b >> 1)) * 1024u + lane * 16u);
+                const uint4 raw = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 32u * (b >> 1) + 16u * half);
                 const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int i = 0; i < 4; i++)
@@ -322,25 +301,22 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 q4k_scale_min(header, b, sc, mn);
                 w_scale[bb] = d_block * sc;
             } else {
-                // This lane's window: piece and slot as the loaders filled them.
-                const uint32_t piece = CODEC == kQ8_0 ? wave_n * 8u + b : wave_n * 4u + (b >> 1);
-                const uint32_t in_piece = CODEC == kQ8_0 ? lane : (b & 1u) * 32u + (lane & 31u);
-                const uint4 low = *reinterpret_cast<const uint4*>(region + piece * 1024u + in_piece * 16u);
-                const uint32_t tail = *reinterpret_cast<const uint32_t*>(region + W::kSmallAt + piece * 256u + in_piece * 4u);
-                // The scale sits in the window of column half 0 (for Q4_0 that is this window).
+                // Five dwords from the dword at or 2 bytes before the block start (+ 16 for the
+                // second column half of Q8_0): scale and quants of even blocks start in the low
+                // half of the first dword, those of odd blocks in its high half.
+                const uint32_t start = b * W::kBlockBytes + (CODEC == kQ8_0 ? 16u * half : 0u);
+                const uint32_t* window = reinterpret_cast<const uint32_t*>(row_in_slot + (start & ~3u));
+                const uint32_t d0 = window[0], d1 = window[1], d2 = window[2], d3 = window[3], d4 = window[4];
+                const bool odd = (b & 1u) != 0;  // (row * pitch + b * 34 or 18) & 2, pitch % 4 == 0
+                // The scale sits at the block start: for the second half of Q8_0 in another dword.
                 const uint32_t scale_word =
-                    CODEC == kQ8_0 ? *reinterpret_cast<const uint32_t*>(region + piece * 1024u + (lane & 31u) * 16u) : low.x;
-                // Do the windows begin 2 bytes before their start? (same arithmetic as the loaders')
-                const uint32_t block_at = row_parity + (stage * kStageBlocks + b) * W::kBlockBytes;
-                const bool scale_shifted = (block_at & 2u) != 0;
-                const bool shifted = ((block_at + (CODEC == kQ8_0 ? 16u * half : 0u)) & 2u) != 0;
-                w_scale[bb] = half_bits_to_float(scale_shifted ? scale_word >> 16 : scale_word & 0xffffu);
-                // quant bytes: window + 4 if shifted, window + 2 if not
+                    CODEC == kQ8_0 ? *reinterpret_cast<const uint32_t*>(row_in_slot + ((b * W::kBlockBytes) & ~3u)) : d0;
+                w_scale[bb] = half_bits_to_float(odd ? scale_word >> 16 : scale_word & 0xffffu);
                 uint32_t words[4];
-                words[0] = shifted ? low.y : __builtin_amdgcn_alignbit(low.y, low.x, 16);
-                words[1] = shifted ? low.z : __builtin_amdgcn_alignbit(low.z, low.y, 16);
-                words[2] = shifted ? low.w : __builtin_amdgcn_alignbit(low.w, low.z, 16);
-                words[3] = shifted ? tail : __builtin_amdgcn_alignbit(tail, low.w, 16);
+                words[0] = odd ? d1 : __builtin_amdgcn_alignbit(d1, d0, 16);
+                words[1] = odd ? d2 : __builtin_amdgcn_alignbit(d2, d1, 16);
+                words[2] = odd ? d3 : __builtin_amdgcn_alignbit(d3, d2, 16);
+                words[3] = odd ? d4 : __builtin_amdgcn_alignbit(d4, d3, 16);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     if constexpr (CODEC == kQ8_0) {
@@ -448,12 +424,12 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     }
 }
 
-template <int CODEC, int MT, int LIMBS, int AHEAD>
+template <int CODEC, int MT, int LIMBS, int AX, int AW>
 hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
                   uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
-    using S = Shape<CODEC, MT, LIMBS, AHEAD>;
-    static_assert(S::kLdsBytes <= 160 * 1024, "LDS of a gfx950 CU");
-    const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, AHEAD>;
+    using S = Shape<CODEC, MT, LIMBS, AX, AW>;
+    static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
+    const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, AX, AW>;
     // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
     static bool allowed[64] = {};
     int device = 0;
@@ -477,23 +453,40 @@ hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias
     return hipGetLastError();
 }
 
+// Weight lead (stages) that fills what the activation ring leaves of LDS.
+template <int CODEC, int MT, int LIMBS, int AX>
+constexpr int weight_lead() {
+    constexpr uint32_t tile = LIMBS * 8192u + 2048u;
+    constexpr uint32_t left = 156u * 1024u - (AX + 1) * MT * tile;
+    constexpr int depth = static_cast<int>(left / WeightLayout<CODEC>::kBytes);
+    // the counted wait holds at most 63 copies: (lead - 1) * rounds of a weight loader
+    constexpr int rounds = (WeightLayout<CODEC>::kJobs + kWeightLoaders - 1) / kWeightLoaders;
+    constexpr int by_counter = 63 / rounds + 1;
+    return (depth - 1 < by_counter ? depth - 1 : by_counter) < 12 ? (depth - 1 < by_counter ? depth - 1 : by_counter) : 12;
+}
+
+template <int CODEC, int MT, int LIMBS, int AX>
+hipError_t launch_shape(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
+                        uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+    constexpr int kWeightLead = weight_lead<CODEC, MT, LIMBS, AX>();
+    static_assert(kWeightLead >= 1, "no room for a weight ring");
+    return launch<CODEC, MT, LIMBS, AX, kWeightLead>(weight, tiles, bias, y, rows, columns, vectors, stream);
+}
+
 template <int CODEC>
 hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const float* bias,
                         float* y, uint32_t rows, uint32_t columns, uint32_t vectors,
                         hipStream_t stream) {
-    // The ring depth is what LDS allows: 26 KiB of activations per stage and 32 vectors with
-    // three limbs, 10 KiB with one; 9 to 18 KiB of weights.
-    if (limbs == 3) {
-        constexpr int kAhead = CODEC == kQ8_0 ? 2 : 3;
-        // One 32-vector tile per workgroup: two tiles of three-limb results do not fit in registers.
-        return launch<CODEC, 1, 3, kAhead>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    }
-    if (vectors <= 32) return launch<CODEC, 1, 1, 3>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    // Q4_K carries a second accumulator (the min term): four tiles of both do not fit in registers.
+    // Activations: 26 KiB per stage and 32-vector tile with three limbs, 10 KiB with one; two
+    // stages of lead. The weight ring (9 to 20 KiB per stage) takes the rest of LDS.
+    // One 32-vector tile per workgroup with three limbs: two tiles of three-limb results do not
+    // fit in registers. Q4_K carries a second accumulator (the min term): at most two tiles.
+    if (limbs == 3) return launch_shape<CODEC, 1, 3, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    if (vectors <= 32) return launch_shape<CODEC, 1, 1, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
     if (vectors <= 64 || CODEC == kQ4_K)
-        return launch<CODEC, 2, 1, (CODEC == kQ8_0 ? 2 : 3)>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    return launch<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 3 : 1)>(weight, tiles, bias, y, rows, columns,
-                                                                            vectors, stream);
+        return launch_shape<CODEC, 2, 1, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, bias, y, rows,
+                                                                                columns, vectors, stream);
 }
 
 }  // namespace
