@@ -35,7 +35,7 @@
 // with different leads must not share a wave. Activations are re-read by every
 // workgroup and come from L2: two stages of lead. Weights come from HBM, and what
 // bounds a CU's share of the bandwidth is how many bytes it keeps in flight: their
-// ring takes all the LDS that is left (up to twelve stages).
+// ring gets up to three stages of lead.
 //   activations  arrive as ready-made stage blobs (see kernels.h): a linear copy;
 //   weights      the stage's bytes of the workgroup's rows, row after row as in memory
 //                (see WeightLayout for how the consumers read their operands out of them).
@@ -462,7 +462,10 @@ constexpr int weight_lead() {
     // the counted wait holds at most 63 copies: (lead - 1) * rounds of a weight loader
     constexpr int rounds = (WeightLayout<CODEC>::kJobs + kWeightLoaders - 1) / kWeightLoaders;
     constexpr int by_counter = 63 / rounds + 1;
-    return (depth - 1 < by_counter ? depth - 1 : by_counter) < 12 ? (depth - 1 < by_counter ? depth - 1 : by_counter) : 12;
+    // More than three stages of lead gained nothing in measurements (a small batch waits for the
+    // copies' issue time, not their latency) and only delays the first stage.
+    constexpr int fits = depth - 1 < by_counter ? depth - 1 : by_counter;
+    return fits < 3 ? fits : 3;
 }
 
 template <int CODEC, int MT, int LIMBS, int AX>
