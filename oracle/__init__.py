@@ -78,6 +78,11 @@ def lib() -> ctypes.CDLL:
         L.et_oracle_quantize_q8.argtypes = [sz, sz, vp, vp, vp, vp]
         L.et_oracle_linear_q8_rows.restype = ci
         L.et_oracle_linear_q8_rows.argtypes = [ci, sz, sz, sz, vp, vp, vp, vp, vp, vp, sz, sz]
+        L.et_oracle_f32_to_fp16.restype = ctypes.c_uint16
+        L.et_oracle_f32_to_fp16.argtypes = [ctypes.c_float]
+        L.et_oracle_kv_attention.restype = ci
+        L.et_oracle_kv_attention.argtypes = [ci, vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, sz, sz, sz,
+                                             vp, vp, vp, ctypes.c_double, sz, vp, ctypes.c_char_p, sz]
         _lib = L
     return _lib
 
@@ -238,3 +243,37 @@ def linear_q8_rows(codec, rows, columns, q, scale, total, weight, bias=None, row
     if rc != 0:
         raise OracleError("et_oracle_linear_q8_rows: invalid geometry or codec")
     return y
+
+
+def f32_to_fp16_bits(value) -> int:
+    """binary32 -> binary16 bits, round to nearest even (et_oracle_f32_to_fp16)."""
+    return int(lib().et_oracle_f32_to_fp16(ctypes.c_float(float(np.float32(value)))))
+
+
+def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_table: np.ndarray,
+                 cursors, advances, q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float,
+                 window: int = 0, active_batch=None) -> np.ndarray:
+    """Paged KV attention (et_oracle_kv_attention): writes the new rows of ``k`` / ``v`` into the
+    slabs IN PLACE (float32 or float16 ``[max_tokens, kv_heads, width]``), then attends.
+    ``q`` is ``[batch, query_heads, tokens, width]``; returns the output of the same shape."""
+    assert k_slab.dtype == v_slab.dtype and k_slab.dtype in (np.float32, np.float16)
+    assert k_slab.flags.c_contiguous and v_slab.flags.c_contiguous and k_slab.shape == v_slab.shape
+    max_tokens, kv_heads, width = k_slab.shape
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    batch, query_heads, tokens, _ = q.shape
+    assert k.shape == (batch, kv_heads, tokens, width) and v.shape == k.shape
+    table = np.ascontiguousarray(block_table, dtype=np.uint32).reshape(batch, -1)
+    cursors = np.ascontiguousarray(cursors, dtype=np.uint32)
+    advances = np.ascontiguousarray(advances, dtype=np.uint32)
+    out = np.zeros_like(q)
+    err = ctypes.create_string_buffer(256)
+    rc = lib().et_oracle_kv_attention(0 if k_slab.dtype == np.float32 else 3, _ptr(k_slab), _ptr(v_slab),
+                                      max_tokens, kv_heads, width, block_size, _ptr(table), table.shape[1],
+                                      _ptr(cursors), _ptr(advances), batch,
+                                      batch if active_batch is None else active_batch, query_heads, tokens,
+                                      _ptr(q), _ptr(k), _ptr(v), float(scale), window, _ptr(out), err, 256)
+    if rc != 0:
+        raise OracleError(err.value.decode())
+    return out
