@@ -25,3 +25,10 @@ from .quantized import (  # noqa: F401
     quantize_activations,
     quantized_linear,
 )
+from .kv_cache import (  # noqa: F401
+    KvLayer,
+    kv_attention_into,
+    kv_attention_kernel,
+    kv_attention_status_check,
+    kv_attention_workspace_bytes,
+)

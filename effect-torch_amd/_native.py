@@ -34,10 +34,33 @@ class EtTensor(ctypes.Structure):
     ]
 
 
+class EtKvLayer(ctypes.Structure):
+    """``et_kv_layer`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("k_slab", ctypes.c_void_p),
+        ("v_slab", ctypes.c_void_p),
+        ("slab_dtype", ctypes.c_int32),
+        ("max_tokens", ctypes.c_uint64),
+        ("kv_heads", ctypes.c_uint64),
+        ("head_dim", ctypes.c_uint64),
+        ("block_size", ctypes.c_uint64),
+        ("block_table", ctypes.c_void_p),
+        ("table_stride", ctypes.c_uint64),
+        ("cursors", ctypes.c_void_p),
+        ("advances", ctypes.c_void_p),
+        ("slots", ctypes.c_uint64),
+        ("active_batch", ctypes.c_uint64),
+        ("context_window", ctypes.c_uint64),
+        ("max_context", ctypes.c_uint64),
+    ]
+
+
 # Every symbol include/et_hip.h declares: name -> (restype, argtypes).
 _vp, _u64, _i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32
 _T = ctypes.POINTER(EtTensor)
 _PP = ctypes.POINTER(ctypes.c_void_p)
+_KV = ctypes.POINTER(EtKvLayer)
 SIGNATURES = {
     "et_hip_is_available": (ctypes.c_int, []),
     "et_hip_codec_name": (ctypes.c_char_p, [_i32]),
@@ -64,6 +87,10 @@ SIGNATURES = {
     "et_hip_embedding_into": (ctypes.c_int, [_vp, _T, _T, _T, _vp, _vp, _vp]),
     "et_hip_embedding_status_check": (ctypes.c_int, [_vp, _vp]),
     "et_hip_dequantize_rows": (ctypes.c_int, [_i32, _u64, _u64, _vp, _vp, _vp]),
+    "et_hip_kv_attention_workspace_bytes": (_u64, [_KV, _u64, _u64]),
+    "et_hip_kv_attention_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp, _vp]),
+    "et_hip_kv_attention_status_check": (ctypes.c_int, [_KV, _u64, _vp]),
+    "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),

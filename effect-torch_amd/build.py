@@ -31,8 +31,10 @@ SOURCES = {
     "gemv_generic.hip": [],
     "quantize_act.hip": ["-ffp-contract=off"],
     "gemm_i8.hip": [],
+    "kv_attention.hip": [],
     "calibrate.hip": [],
     "quantized.cpp": [],
+    "kv_cache.cpp": [],
     "c_api.cpp": [],
 }
 

@@ -11,6 +11,7 @@
 #include "et_codecs.h"
 #include "et_hip.h"
 #include "kernels.h"
+#include "kv_cache.h"
 #include "quantized.h"
 
 namespace {
@@ -270,6 +271,53 @@ int et_hip_dequantize_rows(int32_t codec, uint64_t rows, uint64_t columns, const
             return ET_ERR_EXECUTION;
         }
         return ET_OK;
+    });
+}
+
+uint64_t et_hip_kv_attention_workspace_bytes(const et_kv_layer* layer, uint64_t query_heads,
+                                             uint64_t tokens) {
+    uint64_t bytes = 0;
+    guarded([&](std::string* error) -> int {
+        if (layer == nullptr) {
+            *error = "kv attention: layer is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::kv::workspace_bytes(*layer, query_heads, tokens, &bytes, error);
+    });
+    return bytes;
+}
+
+const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_heads, uint64_t tokens) {
+    return layer ? et::kv::kernel_name(*layer, query_heads, tokens) : "";
+}
+
+int et_hip_kv_attention_into(const et_kv_layer* layer, const et_tensor* q, const et_tensor* k,
+                             const et_tensor* v, double scale, uint64_t window,
+                             const et_tensor* destination, void* workspace, uint64_t workspace_bytes,
+                             void* status, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (layer == nullptr) {
+            *error = "kv attention: layer is NULL";
+            return ET_ERR_INVALID;
+        }
+        TensorView qv, kv, vv, dst;
+        if (!TensorView::from_c(q, &qv, error) || !TensorView::from_c(k, &kv, error) ||
+            !TensorView::from_c(v, &vv, error) || !TensorView::from_c(destination, &dst, error)) {
+            *error = "kv attention: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::kv::attention_into(*layer, qv, kv, vv, scale, window, dst, workspace, workspace_bytes,
+                                      status, stream, cancel, error);
+    });
+}
+
+int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens, const void* status_host) {
+    return guarded([&](std::string* error) -> int {
+        if (layer == nullptr || status_host == nullptr) {
+            *error = "kv attention: layer or status is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::kv::status_check(*layer, tokens, status_host, error);
     });
 }
 

@@ -78,6 +78,46 @@ hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_
                    const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
                    hipStream_t stream);
 
+// ---- kv_attention.hip: paged key/value-cache attention ---------------------------
+constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch
+constexpr int kKvAnyWidthPerLane = 8;     // the any-width kernel covers head widths up to 64 * 8
+// Codes of the device status word (slot << 40 | code << 32 | value; ~0 = nothing to report).
+enum : uint32_t {
+    kKvBadAdvance = 1,    // value = the advance
+    kKvOverCapacity = 2,  // value = live context
+    kKvShortTable = 3,    // value = cursor + advance
+    kKvOverDeclared = 4,  // value = cursor + advance, above the caller's max_context
+    kKvBlockOutside = 5,  // value = physical row
+};
+struct KvAttention {
+    void* k_slab;
+    void* v_slab;
+    bool slab_is_f16;
+    uint32_t max_tokens, kv_heads, width, block_size;
+    const uint32_t* block_table;  // [batch, table_stride]
+    uint32_t table_stride;
+    const uint32_t* cursors;      // [batch]
+    const uint32_t* advances;     // [batch]
+    uint32_t batch, active_batch, query_heads, tokens;
+    uint32_t context_window, window, max_context;
+    const float* q;               // [batch, query_heads, tokens, width]
+    const float* k;               // [batch, kv_heads, tokens, width]
+    const float* v;
+    double scale;
+    float* out;                   // like q
+    void* status;                 // 16 bytes, initialised with kv_status_init
+};
+struct KvLaunchShape {
+    bool streaming;
+    uint32_t splits;
+    uint64_t workgroups;
+    uint64_t workspace_bytes;
+};
+KvLaunchShape kv_attention_shape(const KvAttention& p);
+hipError_t kv_status_init(void* status, hipStream_t stream);
+// Writes the new rows, attends, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
+hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream);
+
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
 // sink must hold 4 * `workgroups` words; bytes < 2^36.
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,

@@ -1,0 +1,198 @@
+#include "kv_cache.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+
+#include "kernels.h"
+
+namespace et {
+namespace kv {
+namespace {
+
+int fail(std::string* error, int status, const std::string& message) {
+    *error = message;
+    return status;
+}
+
+constexpr uint64_t kLimit = 0xffffffffull;
+
+// Geometry of the layer alone; `p` receives what the kernels need of it.
+int layer_geometry(const et_kv_layer& layer, KvAttention* p, std::string* error) {
+    if (layer.slab_dtype != ET_DTYPE_F32 && layer.slab_dtype != ET_DTYPE_F16)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: slabs must be f32 or f16");
+    if (layer.kv_heads == 0 || layer.head_dim == 0 || layer.block_size == 0 || layer.max_tokens == 0)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: empty pool geometry");
+    if (layer.max_tokens > kLimit || layer.kv_heads > kLimit || layer.head_dim > kLimit ||
+        layer.block_size > kLimit || layer.table_stride > kLimit || layer.slots >= (1ull << 24) ||
+        layer.max_context > kLimit || layer.context_window > kLimit)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: geometry exceeds 32-bit positions");
+    if (layer.block_size > layer.max_tokens)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: pool smaller than one block");
+    if (layer.active_batch > layer.slots)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: active batch " + std::to_string(layer.active_batch) +
+                                                   " exceeds " + std::to_string(layer.slots) + " kv slots");
+    p->slab_is_f16 = layer.slab_dtype == ET_DTYPE_F16;
+    p->max_tokens = static_cast<uint32_t>(layer.max_tokens);
+    p->kv_heads = static_cast<uint32_t>(layer.kv_heads);
+    p->width = static_cast<uint32_t>(layer.head_dim);
+    p->block_size = static_cast<uint32_t>(layer.block_size);
+    p->table_stride = static_cast<uint32_t>(layer.table_stride);
+    p->batch = static_cast<uint32_t>(layer.slots);
+    p->active_batch = static_cast<uint32_t>(layer.active_batch);
+    p->context_window = static_cast<uint32_t>(layer.context_window);
+    p->max_context = static_cast<uint32_t>(layer.max_context);
+    return ET_OK;
+}
+
+int query_geometry(uint64_t query_heads, uint64_t tokens, KvAttention* p, std::string* error) {
+    if (p->kv_heads == 0 || query_heads % p->kv_heads != 0 || query_heads == 0)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: incompatible grouped-query q/k/v shapes");
+    if (query_heads > kLimit || tokens > kLimit || tokens == 0)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: geometry exceeds 32-bit positions");
+    if (p->width > 64u * kKvAnyWidthPerLane)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "kv attention: head width " + std::to_string(p->width) + " is above " +
+                        std::to_string(64 * kKvAnyWidthPerLane));
+    p->query_heads = static_cast<uint32_t>(query_heads);
+    p->tokens = static_cast<uint32_t>(tokens);
+    return ET_OK;
+}
+
+uint64_t product(const std::vector<uint64_t>& shape, size_t from, size_t to) {
+    uint64_t total = 1;
+    for (size_t d = from; d < to; d++) total *= shape[d];
+    return total;
+}
+
+}  // namespace
+
+int workspace_bytes(const et_kv_layer& layer, uint64_t query_heads, uint64_t tokens, uint64_t* bytes,
+                    std::string* error) {
+    KvAttention p{};
+    int status = layer_geometry(layer, &p, error);
+    if (status == ET_OK) status = query_geometry(query_heads, tokens, &p, error);
+    if (status != ET_OK) return status;
+    *bytes = kv_attention_shape(p).workspace_bytes;
+    return ET_OK;
+}
+
+const char* kernel_name(const et_kv_layer& layer, uint64_t query_heads, uint64_t tokens) {
+    KvAttention p{};
+    std::string error;
+    if (layer_geometry(layer, &p, &error) != ET_OK || query_geometry(query_heads, tokens, &p, &error) != ET_OK)
+        return "";
+    const KvLaunchShape shape = kv_attention_shape(p);
+    if (shape.streaming) return shape.splits > 1 ? "kv_write+kv_attend+kv_merge" : "kv_write+kv_attend";
+    return shape.splits > 1 ? "kv_write+kv_attend_any+kv_merge" : "kv_write+kv_attend_any";
+}
+
+int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, const quantized::TensorView& k,
+                   const quantized::TensorView& v, double scale, uint64_t window,
+                   const quantized::TensorView& destination, void* workspace, uint64_t workspace_bytes,
+                   void* status, void* stream, const volatile int32_t* cancel, std::string* error) {
+    // napi/mod.rs:3331-3344
+    const size_t rank = q.shape.size();
+    if (rank < 4 || q.dtype != ET_DTYPE_F32 || k.dtype != ET_DTYPE_F32 || v.dtype != ET_DTYPE_F32 ||
+        k.shape.size() != rank || v.shape.size() != rank || destination.shape != q.shape ||
+        destination.dtype != ET_DTYPE_F32)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: expected matching rank-4-or-higher f32 tensors");
+    const uint64_t batch = product(q.shape, 0, rank - 3);
+    const uint64_t query_heads = q.shape[rank - 3], tokens = q.shape[rank - 2], width = q.shape[rank - 1];
+    const uint64_t kv_heads = k.shape[rank - 3];
+    // :3353-3365
+    bool compatible = v.shape[rank - 3] == kv_heads && kv_heads != 0 && query_heads % kv_heads == 0 &&
+                      k.shape[rank - 2] == tokens && v.shape[rank - 2] == tokens &&
+                      k.shape[rank - 1] == width && v.shape[rank - 1] == width;
+    for (size_t d = 0; d + 3 < rank; d++)
+        compatible = compatible && k.shape[d] == q.shape[d] && v.shape[d] == q.shape[d];
+    if (!compatible) return fail(error, ET_ERR_UNSUPPORTED, "kv attention: incompatible grouped-query q/k/v shapes");
+    // :3366-3371
+    if (batch != layer.slots)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: batch " + std::to_string(batch) +
+                                                   " does not match " + std::to_string(layer.slots) + " kv slots");
+    // kv_prepare, :3583-3588
+    if (kv_heads != layer.kv_heads || width != layer.head_dim)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "kv attention: layer shape [" + std::to_string(kv_heads) + ", " + std::to_string(width) +
+                        "] does not match pool geometry [" + std::to_string(layer.kv_heads) + ", " +
+                        std::to_string(layer.head_dim) + "]");
+    KvAttention p{};
+    int code = layer_geometry(layer, &p, error);
+    if (code == ET_OK) code = query_geometry(query_heads, tokens, &p, error);
+    if (code != ET_OK) return code;
+    if (window > kLimit) return fail(error, ET_ERR_UNSUPPORTED, "kv attention: geometry exceeds 32-bit positions");
+    if (!q.is_contiguous() || !k.is_contiguous() || !v.is_contiguous() || !destination.is_contiguous())
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: q, k, v and the destination must be contiguous");
+    if (batch == 0) return ET_OK;
+    if (status == nullptr) return fail(error, ET_ERR_INVALID, "kv attention: status block is NULL");
+    if (layer.k_slab == nullptr || layer.v_slab == nullptr || layer.block_table == nullptr ||
+        layer.cursors == nullptr || layer.advances == nullptr || q.data == nullptr || k.data == nullptr ||
+        v.data == nullptr || destination.data == nullptr)
+        return fail(error, ET_ERR_INVALID, "kv attention: NULL device pointer");
+    p.k_slab = layer.k_slab;
+    p.v_slab = layer.v_slab;
+    p.block_table = layer.block_table;
+    p.cursors = layer.cursors;
+    p.advances = layer.advances;
+    p.window = static_cast<uint32_t>(window);
+    p.q = static_cast<const float*>(q.data) + q.offset;
+    p.k = static_cast<const float*>(k.data) + k.offset;
+    p.v = static_cast<const float*>(v.data) + v.offset;
+    p.out = const_cast<float*>(static_cast<const float*>(destination.data)) + destination.offset;
+    p.scale = scale;
+    p.status = status;
+    const KvLaunchShape shape = kv_attention_shape(p);
+    if (shape.streaming) {
+        // the streaming kernel moves 16 bytes per lane
+        const auto misaligned = [](const void* pointer) { return reinterpret_cast<uintptr_t>(pointer) % 16 != 0; };
+        if (misaligned(p.k_slab) || misaligned(p.v_slab))
+            return fail(error, ET_ERR_INVALID, "kv attention: slabs must be 16-byte aligned");
+    }
+    if (shape.workgroups > 0x7fffffffull)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: launch exceeds the grid limit");
+    if (workspace_bytes < shape.workspace_bytes || (shape.workspace_bytes != 0 && workspace == nullptr))
+        return fail(error, ET_ERR_EXECUTION,
+                    "kv attention: workspace of " + std::to_string(workspace_bytes) + " bytes is smaller than the " +
+                        std::to_string(shape.workspace_bytes) + " required");
+    if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    hipError_t launched = kv_status_init(status, static_cast<hipStream_t>(stream));
+    if (launched == hipSuccess) launched = kv_attention(p, workspace, static_cast<hipStream_t>(stream));
+    if (launched != hipSuccess)
+        return fail(error, ET_ERR_EXECUTION, std::string("kv attention: HIP error: ") + hipGetErrorString(launched));
+    return ET_OK;
+}
+
+int status_check(const et_kv_layer& layer, uint64_t tokens, const void* status_host, std::string* error) {
+    unsigned long long word;
+    std::memcpy(&word, status_host, sizeof word);
+    if (word == ~0ull) return ET_OK;
+    const uint64_t slot = word >> 40, code = (word >> 32) & 0xff, value = word & 0xffffffffull;
+    switch (code) {
+        case kKvBadAdvance:  // napi/mod.rs:3590-3594
+            return fail(error, ET_ERR_EXECUTION,
+                        "kv attention: advance " + std::to_string(value) + " out of range for chunk length " +
+                            std::to_string(tokens));
+        case kKvOverCapacity:  // :3597-3603
+            return fail(error, ET_ERR_EXECUTION,
+                        "kv attention: live context " + std::to_string(value) + " exceeds pool capacity " +
+                            std::to_string(layer.max_tokens));
+        case kKvShortTable:
+            return fail(error, ET_ERR_EXECUTION,
+                        "kv attention: block table of slot " + std::to_string(slot) + " does not cover " +
+                            std::to_string(value) + " tokens");
+        case kKvOverDeclared:
+            return fail(error, ET_ERR_EXECUTION,
+                        "kv attention: slot " + std::to_string(slot) + " needs " + std::to_string(value) +
+                            " tokens, above the declared max_context " + std::to_string(layer.max_context));
+        case kKvBlockOutside:
+            return fail(error, ET_ERR_EXECUTION,
+                        "kv attention: slot " + std::to_string(slot) + " maps to row " + std::to_string(value) +
+                            " outside the pool of " + std::to_string(layer.max_tokens));
+        default:
+            return fail(error, ET_ERR_EXECUTION, "kv attention: unknown device status " + std::to_string(word));
+    }
+}
+
+}  // namespace kv
+}  // namespace et

@@ -195,6 +195,68 @@ int et_hip_embedding_status_check(const et_embedding_plan* plan, const void* sta
 int et_hip_dequantize_rows(int32_t codec, uint64_t rows, uint64_t columns, const uint8_t* weight,
                            float* out, void* stream);
 
+/* ---- paged key/value-cache attention ---------------------------------------
+ *
+ * The decode neighbour of quantized_linear: kv_attention_into
+ * (crates/runtime-cpu/src/napi/mod.rs:3320-3544). The caller keeps what the
+ * reference keeps on the host - block allocation, eviction, the cursors'
+ * advance between steps (kv_prepare / kv_evict, :3568-3627) - and hands over
+ * the state of one layer as device arrays. */
+
+/* One layer of a KvContext (napi/mod.rs:2656-2664) over its pool (PoolInner,
+ * :2501-2513; slabs crates/runtime-cpu/src/pool.rs). All pointers are device
+ * pointers. */
+typedef struct {
+    void* k_slab;                /* [max_tokens, kv_heads, head_dim], f32 or f16; written and read */
+    void* v_slab;
+    int32_t slab_dtype;          /* ET_DTYPE_F32 or ET_DTYPE_F16 (the reference's int8 tier is not covered) */
+    uint64_t max_tokens;         /* pool.max_tokens */
+    uint64_t kv_heads;           /* pool.kv_heads */
+    uint64_t head_dim;           /* pool.head_dim */
+    uint64_t block_size;         /* pool.block_size */
+    const uint32_t* block_table; /* [slots, table_stride]: SeqState.blocks of every slot, already
+                                    grown to cover cursor + advance */
+    uint64_t table_stride;
+    const uint32_t* cursors;     /* [slots] SeqState.cursor */
+    const uint32_t* advances;    /* [slots] SeqState.advance */
+    uint64_t slots;              /* context.slots.len() = the batch of q */
+    uint64_t active_batch;       /* context.active_batch: slots beyond it get zeros */
+    uint64_t context_window;     /* context.window, 0 = none */
+    uint64_t max_context;        /* host-side upper bound of cursor + advance over the active slots;
+                                    it sizes the launch and the workspace */
+} et_kv_layer;
+
+/* Device scratch et_hip_kv_attention_into needs for these sizes (partial results
+ * of the context splits); may be 0. */
+uint64_t et_hip_kv_attention_workspace_bytes(const et_kv_layer* layer, uint64_t query_heads,
+                                             uint64_t tokens);
+
+/* = kv_attention_into (napi/mod.rs:3320-3544): appends `advance` rows of k / v
+ * per active slot to the slabs, then attends causally over each slot's cached
+ * context (grouped-query: query head h reads kv head h / (query_heads /
+ * kv_heads)) with softmax(q.k * scale) in f32 (the reference accumulates in
+ * f64; results agree to 1e-4).
+ *   q [.., query_heads, tokens, head_dim], k and v [.., kv_heads, tokens, head_dim],
+ *   destination like q: f32, rank >= 4, contiguous; the leading dims multiply to `slots`.
+ *   window: the operator's own sliding window, 0 = none.
+ * The cursors live on the device, so the checks of kv_prepare that depend on
+ * them cannot fail this call: a slot that fails one is skipped and the device
+ * `status` block (ET_HIP_STATUS_BYTES, initialised by this call on `stream`)
+ * records it for et_hip_kv_attention_status_check. */
+int et_hip_kv_attention_into(const et_kv_layer* layer, const et_tensor* q, const et_tensor* k,
+                             const et_tensor* v, double scale, uint64_t window,
+                             const et_tensor* destination, void* workspace,
+                             uint64_t workspace_bytes, void* status, void* stream,
+                             const volatile int32_t* cancel);
+/* After the stream has completed and `status` has been copied to the host: 0, or
+ * ET_ERR_EXECUTION with the reference's message, e.g. "kv attention: advance {a}
+ * out of range for chunk length {tokens}" (napi/mod.rs:3590-3594). */
+int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
+                                     const void* status_host);
+/* Name of the kernel variant these sizes select, for profiles and diagnostics. */
+const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_heads,
+                                       uint64_t tokens);
+
 /* ---- int8 activation quantiser (stage 1 of ET_ACT_INT8) ------------------- */
 
 /* The activation quantiser on its own, exposed so that tests can check the

@@ -82,7 +82,7 @@ def lib() -> ctypes.CDLL:
         L.et_oracle_f32_to_fp16.argtypes = [ctypes.c_float]
         L.et_oracle_kv_attention.restype = ci
         L.et_oracle_kv_attention.argtypes = [ci, vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, sz, sz, sz,
-                                             vp, vp, vp, ctypes.c_double, sz, vp, ctypes.c_char_p, sz]
+                                             vp, vp, vp, ctypes.c_double, sz, sz, vp, ctypes.c_char_p, sz]
         _lib = L
     return _lib
 
@@ -252,7 +252,7 @@ def f32_to_fp16_bits(value) -> int:
 
 def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_table: np.ndarray,
                  cursors, advances, q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float,
-                 window: int = 0, active_batch=None) -> np.ndarray:
+                 window: int = 0, active_batch=None, context_window: int = 0) -> np.ndarray:
     """Paged KV attention (et_oracle_kv_attention): writes the new rows of ``k`` / ``v`` into the
     slabs IN PLACE (float32 or float16 ``[max_tokens, kv_heads, width]``), then attends.
     ``q`` is ``[batch, query_heads, tokens, width]``; returns the output of the same shape."""
@@ -269,11 +269,11 @@ def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_
     advances = np.ascontiguousarray(advances, dtype=np.uint32)
     out = np.zeros_like(q)
     err = ctypes.create_string_buffer(256)
-    rc = lib().et_oracle_kv_attention(0 if k_slab.dtype == np.float32 else 3, _ptr(k_slab), _ptr(v_slab),
+    rc = lib().et_oracle_kv_attention(0 if k_slab.dtype == np.float32 else 2, _ptr(k_slab), _ptr(v_slab),
                                       max_tokens, kv_heads, width, block_size, _ptr(table), table.shape[1],
                                       _ptr(cursors), _ptr(advances), batch,
                                       batch if active_batch is None else active_batch, query_heads, tokens,
-                                      _ptr(q), _ptr(k), _ptr(v), float(scale), window, _ptr(out), err, 256)
+                                      _ptr(q), _ptr(k), _ptr(v), float(scale), context_window, window, _ptr(out), err, 256)
     if rc != 0:
         raise OracleError(err.value.decode())
     return out

@@ -61,9 +61,9 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
                            const uint32_t* block_table, size_t table_stride,
                            const uint32_t* cursors, const uint32_t* advances, size_t batch,
                            size_t active_batch, size_t query_heads, size_t tokens, const float* q,
-                           const float* k, const float* v, double scale, size_t window, float* out,
-                           char* err, size_t err_len) {
-    if (slab_dtype != 0 && slab_dtype != 3) return fail(err, err_len, "kv attention: unsupported slab dtype");
+                           const float* k, const float* v, double scale, size_t context_window, size_t window,
+                           float* out, char* err, size_t err_len) {
+    if (slab_dtype != 0 && slab_dtype != 2) return fail(err, err_len, "kv attention: unsupported slab dtype");
     /* napi/mod.rs:3347-3360 */
     if (kv_heads == 0 || query_heads % kv_heads != 0)
         return fail(err, err_len, "kv attention: incompatible grouped-query q/k/v shapes");
@@ -81,7 +81,7 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
             { free(weights); return fail(err, err_len, message); }
         }
         const size_t needed = cursor + advance;
-        const size_t start = window != 0 ? (needed > window ? needed - window : 0) : 0;
+        const size_t start = context_window != 0 ? (needed > context_window ? needed - context_window : 0) : 0;
         if (needed - start > max_tokens) { free(weights); return fail(err, err_len, "kv attention: live context exceeds pool capacity"); }
         if ((needed + block_size - 1) / block_size > table_stride)
             { free(weights); return fail(err, err_len, "kv attention: block table too short"); }

@@ -32,18 +32,19 @@ extern "C" {
 /* binary32 -> binary16 bits, round to nearest even (pool.rs:72-79 stores through f16::from_f32). */
 uint16_t et_oracle_f32_to_fp16(float value);
 
-/* slab_dtype: 0 = f32, 3 = f16 (the et_dtype codes). Slabs are [max_tokens, kv_heads, width].
+/* slab_dtype: 0 = f32, 2 = f16 (the DType order of crates/runtime/src/dtype.rs:13-21). Slabs are [max_tokens, kv_heads, width].
  * block_table[slot * table_stride + i] = physical block of logical block i of that slot.
  * q is [batch, query_heads, tokens, width], k and v [batch, kv_heads, tokens, width], all f32,
- * out like q. window = 0 means no sliding window. Writes the new rows first, then attends.
+ * out like q. context_window is the pool's sliding window (kv_prepare's `start`, :3599), window
+ * the operator's own (:3482-3483); 0 means none for either. Writes the new rows first, then attends.
  * Returns 0, or -1 with a message in err. */
 int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t max_tokens,
                            size_t kv_heads, size_t width, size_t block_size,
                            const uint32_t* block_table, size_t table_stride,
                            const uint32_t* cursors, const uint32_t* advances, size_t batch,
                            size_t active_batch, size_t query_heads, size_t tokens, const float* q,
-                           const float* k, const float* v, double scale, size_t window, float* out,
-                           char* err, size_t err_len);
+                           const float* k, const float* v, double scale, size_t context_window, size_t window,
+                           float* out, char* err, size_t err_len);
 
 #ifdef __cplusplus
 }

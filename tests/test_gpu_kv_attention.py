@@ -1,0 +1,217 @@
+"""Paged key/value-cache attention on the GPU against the CPU oracle (oracle/et_oracle_kv.c).
+
+Bars: slabs after the call are bit-identical to the oracle's (f32 copies, f16 round-to-nearest-even);
+outputs agree to 1e-4 (f32 online softmax against the oracle's f64 three passes).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 1e-4
+
+
+def make_case(rng, *, slots, query_heads, kv_heads, width, block_size, contexts, tokens, advances, dtype,
+              spare_blocks=3):
+    """Random slabs with `contexts[b]` cached positions per slot behind a shuffled block table."""
+    contexts = np.asarray(contexts, dtype=np.int64)
+    advances = np.asarray(advances, dtype=np.int64)
+    blocks_per_slot = int(max(1, -(-int((contexts + tokens).max()) // block_size)))
+    total_blocks = slots * blocks_per_slot + spare_blocks
+    max_tokens = total_blocks * block_size
+    table = rng.permutation(total_blocks)[: slots * blocks_per_slot].reshape(slots, blocks_per_slot).astype(np.uint32)
+    k_slab = rng.standard_normal((max_tokens, kv_heads, width)).astype(np.float32).astype(dtype)
+    v_slab = rng.standard_normal((max_tokens, kv_heads, width)).astype(np.float32).astype(dtype)
+    q = rng.standard_normal((slots, query_heads, tokens, width)).astype(np.float32)
+    k = rng.standard_normal((slots, kv_heads, tokens, width)).astype(np.float32)
+    v = rng.standard_normal((slots, kv_heads, tokens, width)).astype(np.float32)
+    return dict(k_slab=k_slab, v_slab=v_slab, table=table, cursors=contexts.astype(np.uint32),
+                advances=advances.astype(np.uint32), q=q, k=k, v=v, block_size=block_size,
+                max_context=int((contexts + advances).max()))
+
+
+def run_gpu(et, device, case, scale, *, window=0, context_window=0, active_batch=None, max_context=None):
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+    layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)),
+                       dev(case["cursors"].view(np.int32)), dev(case["advances"].view(np.int32)),
+                       case["max_context"] if max_context is None else max_context,
+                       active_batch=active_batch, context_window=context_window)
+    q = dev(case["q"])
+    out = torch.full_like(q, float("nan"))
+    et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, window, out)
+    return out.cpu().numpy(), k_slab.cpu().numpy(), v_slab.cpu().numpy(), layer
+
+
+def run_oracle(case, scale, *, window=0, context_window=0, active_batch=None):
+    k_slab, v_slab = case["k_slab"].copy(), case["v_slab"].copy()
+    out = oracle.kv_attention(k_slab, v_slab, case["block_size"], case["table"], case["cursors"], case["advances"],
+                              case["q"], case["k"], case["v"], scale, window=window,
+                              context_window=context_window, active_batch=active_batch)
+    return out, k_slab, v_slab
+
+
+def compare(got, want):
+    out, k_slab, v_slab = got[:3]
+    ref_out, ref_k, ref_v = want
+    assert np.array_equal(k_slab.view(np.uint8), ref_k.view(np.uint8)), "K slab differs"
+    assert np.array_equal(v_slab.view(np.uint8), ref_v.view(np.uint8)), "V slab differs"
+    assert np.isfinite(out).all()
+    error = np.abs(out - ref_out).max()
+    assert error <= OUT_TOL, f"max |out - oracle| = {error}"
+
+
+def test_the_reference_test_case(et, device):
+    # napi/mod.rs:4963-5051
+    q = np.arange(48, dtype=np.float32).reshape(1, 4, 3, 4)
+    k = (np.arange(24, 48).astype(np.float32) * np.float32(0.01)).reshape(1, 2, 3, 4)
+    v = (np.arange(48, 72).astype(np.float32) * np.float32(0.01)).reshape(1, 2, 3, 4)
+    case = dict(k_slab=np.zeros((8, 2, 4), np.float32), v_slab=np.zeros((8, 2, 4), np.float32),
+                table=np.array([[1, 0]], np.uint32), cursors=np.array([0], np.uint32),
+                advances=np.array([3], np.uint32), q=q, k=k, v=v, block_size=4, max_context=3)
+    got = run_gpu(et, device, case, 0.5)
+    assert et.kv_attention_kernel(got[3], 4, 3).startswith("kv_write+kv_attend_any")
+    compare(got, run_oracle(case, 0.5))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("lanes", [8, 16, 32])
+@pytest.mark.parametrize("group,kv_heads", [(1, 3), (2, 2), (4, 2), (8, 1), (3, 2), (12, 1)])
+def test_streaming_kernel_shapes(et, device, dtype, lanes, group, kv_heads):
+    width = lanes * (4 if dtype == np.float32 else 8)
+    rng = np.random.default_rng(1000 * lanes + 10 * group + kv_heads)
+    case = make_case(rng, slots=3, query_heads=group * kv_heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=[0, 37, 200], tokens=1, advances=[1, 1, 1], dtype=dtype)
+    scale = 1.0 / np.sqrt(width)
+    got = run_gpu(et, device, case, scale)
+    assert et.kv_attention_kernel(got[3], group * kv_heads, 1).startswith("kv_write+kv_attend+")  or \
+        et.kv_attention_kernel(got[3], group * kv_heads, 1) == "kv_write+kv_attend"
+    compare(got, run_oracle(case, scale))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("block_size", [1, 5, 16, 64])
+@pytest.mark.parametrize("tokens,advances", [(1, [1, 1, 1, 1]), (4, [4, 1, 3, 2])])
+def test_paging_chunks_and_ragged_advances(et, device, dtype, block_size, tokens, advances):
+    rng = np.random.default_rng(block_size * 7 + tokens)
+    case = make_case(rng, slots=4, query_heads=8, kv_heads=2, width=128, block_size=block_size,
+                     contexts=[0, 1, 63, 129], tokens=tokens, advances=advances, dtype=dtype)
+    got = run_gpu(et, device, case, 0.09)
+    compare(got, run_oracle(case, 0.09))
+
+
+@pytest.mark.parametrize("width,dtype", [(4, np.float16), (20, np.float32), (96, np.float16), (200, np.float32)])
+def test_any_width_kernel(et, device, width, dtype):
+    rng = np.random.default_rng(width)
+    case = make_case(rng, slots=2, query_heads=6, kv_heads=3, width=width, block_size=8,
+                     contexts=[5, 300], tokens=2, advances=[2, 1], dtype=dtype)
+    got = run_gpu(et, device, case, 0.2)
+    assert "kv_attend_any" in et.kv_attention_kernel(got[3], 6, 2)
+    compare(got, run_oracle(case, 0.2))
+
+
+@pytest.mark.parametrize("context_window,window", [(0, 50), (70, 0), (100, 33), (40, 90), (0, 1)])
+@pytest.mark.parametrize("width", [128, 24])
+def test_sliding_windows(et, device, context_window, window, width):
+    rng = np.random.default_rng(context_window + window + width)
+    case = make_case(rng, slots=3, query_heads=4, kv_heads=2, width=width, block_size=16,
+                     contexts=[3, 64, 250], tokens=2, advances=[2, 2, 1], dtype=np.float16)
+    got = run_gpu(et, device, case, 0.1, window=window, context_window=context_window)
+    compare(got, run_oracle(case, 0.1, window=window, context_window=context_window))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_long_context_is_split(et, device, dtype):
+    rng = np.random.default_rng(77)
+    case = make_case(rng, slots=2, query_heads=8, kv_heads=2, width=128, block_size=16,
+                     contexts=[5000, 777], tokens=1, advances=[1, 1], dtype=dtype)
+    scale = 1.0 / np.sqrt(128)
+    got = run_gpu(et, device, case, scale)
+    assert et.kv_attention_kernel(got[3], 8, 1).endswith("+kv_merge")
+    assert et.kv_attention_workspace_bytes(got[3], 8, 1) > 0
+    compare(got, run_oracle(case, scale))
+    # a generous bound changes the launch, not the result
+    again = run_gpu(et, device, case, scale, max_context=100000)
+    compare(again, run_oracle(case, scale))
+
+
+def test_inactive_slots_are_zero_and_untouched(et, device):
+    rng = np.random.default_rng(3)
+    case = make_case(rng, slots=4, query_heads=8, kv_heads=2, width=128, block_size=16,
+                     contexts=[10, 20, 30, 40], tokens=1, advances=[1, 1, 1, 1], dtype=np.float16)
+    got = run_gpu(et, device, case, 0.1, active_batch=2)
+    assert np.all(got[0][2:] == 0)
+    compare(got, run_oracle(case, 0.1, active_batch=2))
+
+
+def test_decode_steps_advance_the_cache(et, device):
+    # three decode steps through one layer object: what a step writes, the next reads
+    rng = np.random.default_rng(8)
+    case = make_case(rng, slots=2, query_heads=8, kv_heads=2, width=128, block_size=16,
+                     contexts=[14, 28], tokens=1, advances=[1, 1], dtype=np.float16, spare_blocks=0)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+    cursors = dev(case["cursors"].view(np.int32))
+    layer = et.KvLayer(k_slab, v_slab, 16, dev(case["table"].view(np.int32)), cursors,
+                       dev(case["advances"].view(np.int32)), 40)
+    ref_k, ref_v = case["k_slab"].copy(), case["v_slab"].copy()
+    ref_cursors = case["cursors"].copy()
+    for step in range(3):
+        q = rng.standard_normal((2, 8, 1, 128)).astype(np.float32)
+        k = rng.standard_normal((2, 2, 1, 128)).astype(np.float32)
+        v = rng.standard_normal((2, 2, 1, 128)).astype(np.float32)
+        out = torch.empty(2, 8, 1, 128, device=device)
+        et.kv_attention_into(layer, dev(q), dev(k), dev(v), 0.1, None, out)
+        want = oracle.kv_attention(ref_k, ref_v, 16, case["table"], ref_cursors, case["advances"], q, k, v, 0.1)
+        assert np.abs(out.cpu().numpy() - want).max() <= OUT_TOL
+        cursors += 1
+        ref_cursors += 1
+    assert np.array_equal(k_slab.cpu().numpy().view(np.uint8), ref_k.view(np.uint8))
+
+
+def test_device_side_checks_report_the_reference_errors(et, device):
+    rng = np.random.default_rng(4)
+    base = dict(slots=2, query_heads=4, kv_heads=2, width=128, block_size=16, contexts=[10, 20], tokens=2,
+                dtype=np.float16)
+    case = make_case(rng, advances=[2, 3], **base)
+    with pytest.raises(et.QuantizedError, match="kv attention: advance 3 out of range for chunk length 2"):
+        run_gpu(et, device, case, 0.1, max_context=64)
+    case = make_case(rng, advances=[0, 3], **base)
+    with pytest.raises(et.QuantizedError, match="kv attention: advance 0 out of range for chunk length 2"):
+        run_gpu(et, device, case, 0.1, max_context=64)
+    case = make_case(rng, advances=[1, 1], **base)
+    case["cursors"][1] = 40  # the table covers 2 blocks = 32 positions
+    with pytest.raises(et.QuantizedError, match="block table of slot 1 does not cover 41 tokens"):
+        run_gpu(et, device, case, 0.1, max_context=64)
+    case = make_case(rng, advances=[1, 1], **base)
+    with pytest.raises(et.QuantizedError, match="above the declared max_context 5"):
+        run_gpu(et, device, case, 0.1, max_context=5)
+    case = make_case(rng, advances=[1, 1], **base)
+    case["table"][0, 0] = 1000
+    with pytest.raises(et.QuantizedError, match="outside the pool"):
+        run_gpu(et, device, case, 0.1)
+
+
+@pytest.mark.parametrize("dtype", [np.float16])
+def test_decode_batch_at_full_size(et, device, dtype):
+    # 32 slots x 32 query heads over 8 kv heads of width 128, contexts around 2048, block size 16
+    rng = np.random.default_rng(2048)
+    contexts = rng.integers(1900, 2048, 32)
+    case = make_case(rng, slots=32, query_heads=32, kv_heads=8, width=128, block_size=16, contexts=contexts,
+                     tokens=1, advances=[1] * 32, dtype=dtype, spare_blocks=7)
+    scale = 1.0 / np.sqrt(128)
+    got = run_gpu(et, device, case, scale)
+    compare(got, run_oracle(case, scale))
+    # size-independent property: with every key zero all scores are equal, the output is the mean of V
+    case["k_slab"][:] = 0
+    case["k"][:] = 0
+    out = run_gpu(et, device, case, scale)[0]
+    for b in (0, 31):
+        rows = [case["table"][b, p // 16] * 16 + p % 16 for p in range(contexts[b])]
+        values = np.concatenate([case["v_slab"][rows].astype(np.float64),
+                                 case["v"][b].astype(dtype).astype(np.float64).transpose(1, 0, 2)])
+        mean = values.mean(axis=0)  # [kv_heads, width]
+        assert np.abs(out[b, :, 0] - np.repeat(mean, 4, axis=0)).max() <= OUT_TOL

@@ -155,3 +155,69 @@ def test_embedding_status_wording(et):
         bad = ctypes.create_string_buffer(struct.pack("<Qq", 0, value), 16)
         assert N.lib().et_hip_embedding_status_check(plan._handle, bad) == N.ERR_EXECUTION
         assert N.last_error() == f"quantized_embedding: index {value} is outside 0..1"
+
+
+def _kv_layer(et, torch, *, slots=2, kv_heads=2, width=8, max_tokens=32, block_size=4, dtype=None, **kw):
+    dtype = dtype or torch.float32
+    slab = torch.zeros(max_tokens, kv_heads, width, dtype=dtype)
+    table = torch.zeros(slots, 4, dtype=torch.int32)
+    zeros = torch.zeros(slots, dtype=torch.int32)
+    return et.KvLayer(slab, slab.clone(), block_size, table, zeros, zeros.clone(), kw.pop("max_context", 16), **kw)
+
+
+def test_kv_attention_validation_follows_the_reference(et):
+    import torch
+    layer = _kv_layer(et, torch)
+    q = torch.zeros(2, 4, 3, 8)
+    kv = torch.zeros(2, 2, 3, 8)
+    out = torch.zeros_like(q)
+
+    def fails(message, *args):
+        with pytest.raises(et.QuantizedError, match=message):
+            et.kv_attention_into(layer, *args, stream=0)
+
+    fails("expected matching rank-4-or-higher f32 tensors", q[0], kv[0], kv[0], 1.0, None, out[0])
+    fails("expected matching rank-4-or-higher f32 tensors", q.double(), kv, kv, 1.0, None, out)
+    fails("expected matching rank-4-or-higher f32 tensors", q, kv, kv, 1.0, None, out[:, :2])
+    fails("incompatible grouped-query q/k/v shapes", q, kv[:, :, :2], kv, 1.0, None, out)
+    fails("incompatible grouped-query q/k/v shapes", q, torch.zeros(2, 3, 3, 8), torch.zeros(2, 3, 3, 8), 1.0, None, out)
+    fails("incompatible grouped-query q/k/v shapes", q[:1], kv, kv, 1.0, None, out[:1])
+    fails("batch 3 does not match 2 kv slots", torch.zeros(3, 4, 3, 8), torch.zeros(3, 2, 3, 8),
+          torch.zeros(3, 2, 3, 8), 1.0, None, torch.zeros(3, 4, 3, 8))
+    fails(r"layer shape \[1, 8\] does not match pool geometry \[2, 8\]", q, kv[:, :1], kv[:, :1], 1.0, None, out)
+    fails("must be contiguous", q.transpose(0, 1).contiguous().transpose(0, 1), kv, kv, 1.0, None, out)
+    flag = et.CancellationFlag()
+    flag.cancel()
+    with pytest.raises(et.Cancelled, match="operation aborted"):
+        et.kv_attention_into(layer, q, kv, kv, 1.0, None, out, cancelled=flag, stream=0)
+    with pytest.raises(et.QuantizedError, match="slabs must be f32 or f16"):
+        _kv_layer(et, torch, dtype=torch.bfloat16)
+
+
+def test_kv_attention_launch_shapes_and_status_wording(et):
+    import ctypes
+    import struct
+    import torch
+    from effect_torch_amd import _native
+    decode = _kv_layer(et, torch, slots=32, kv_heads=8, width=128, max_tokens=32 * 2048, block_size=16,
+                       dtype=torch.float16, max_context=2048)
+    assert et.kv_attention_kernel(decode, 32, 1) == "kv_write+kv_attend+kv_merge"
+    assert et.kv_attention_workspace_bytes(decode, 32, 1) % (32 * 32 * 130 * 4) == 0
+    short = _kv_layer(et, torch, slots=512, kv_heads=8, width=128, max_tokens=4096, block_size=16,
+                      dtype=torch.float16, max_context=8)
+    assert et.kv_attention_kernel(short, 32, 1) == "kv_write+kv_attend"
+    assert et.kv_attention_workspace_bytes(short, 32, 1) == 0
+    odd = _kv_layer(et, torch, width=12)
+    assert et.kv_attention_kernel(odd, 4, 1).startswith("kv_write+kv_attend_any")
+    assert et.kv_attention_kernel(odd, 3, 1) == ""  # 3 query heads over 2 kv heads
+
+    def message(word):
+        layer = decode.struct()
+        buf = ctypes.create_string_buffer(struct.pack("<QQ", word, 0), 16)
+        status = _native.lib().et_hip_kv_attention_status_check(ctypes.byref(layer), 7, buf)
+        return status, _native.last_error()
+
+    assert message(2**64 - 1)[0] == 0
+    assert message((3 << 40) | (1 << 32) | 9) == (2, "kv attention: advance 9 out of range for chunk length 7")
+    assert message((1 << 32) | 0) == (2, "kv attention: advance 0 out of range for chunk length 7")
+    assert message((2 << 32) | 70000) == (2, "kv attention: live context 70000 exceeds pool capacity 65536")

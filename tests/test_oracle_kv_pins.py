@@ -97,13 +97,14 @@ def test_closed_forms_and_paging(dtype):
     again = oracle.kv_attention(k2, v2, bs, table2, context, advances, q, k_new, v_new, 0.35)
     assert np.array_equal(got, again)
     # windowed: the last 5 positions only
-    k3, v3 = k2.copy(), v2.copy()
-    windowed = oracle.kv_attention(k3, v3, bs, table2, context, advances, q, k_new, v_new, 0.35, window=5)
-    start = np.maximum(needed - 5, 0)
-    want_w = dense_attention(q, k_seen, v_seen, 0.35,
-                             lambda b, t: max(min(context[b] + t + 1, needed[b]) - 5, start[b], 0),
-                             lambda b, t: min(context[b] + t + 1, needed[b]))
-    assert np.allclose(windowed, want_w, rtol=0, atol=2e-6)
+    for context_window, window in ((0, 5), (5, 0), (6, 3), (3, 6)):
+        windowed = oracle.kv_attention(k2.copy(), v2.copy(), bs, table2, context, advances, q, k_new, v_new,
+                                       0.35, window=window, context_window=context_window)
+        start = np.maximum(needed - context_window, 0) if context_window else np.zeros_like(needed)
+        end = lambda b, t: min(context[b] + t + 1, needed[b])
+        begin = lambda b, t: max(end(b, t) - window, start[b], 0) if window else start[b]
+        want_w = dense_attention(q, k_seen, v_seen, 0.35, begin, end)
+        assert np.allclose(windowed, want_w, rtol=0, atol=2e-6)
     # inactive slots stay zero
     part = oracle.kv_attention(k2.copy(), v2.copy(), bs, table2, context, advances, q, k_new, v_new, 0.35,
                                active_batch=1)
