@@ -45,9 +45,10 @@ def parse_args():
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--workload", default="q4_k_gemv_14336x4096",
-                   help="one of effect_torch_amd.synth.CONFIGS")
+                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
+    p.add_argument("--context", type=int, default=2048, help="kv_attention_decode: positions per slot")
     p.add_argument("--hot", action="store_true", help="reuse one weight buffer (cache-resident; not the headline)")
     p.add_argument("--no-graph", action="store_true", help="enqueue the steps one by one instead of replaying a HIP graph")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -163,6 +164,107 @@ def calibrate(args, et):
     }))
 
 
+def kv_decode(args, et):
+    """Workload ``kv_attention_decode``: one decode step of paged key/value-cache attention for a
+    Llama-3-8B-shaped layer - 32 slots, 32 query heads over 8 kv heads of width 128, f16 slabs in
+    blocks of 16 tokens, 2047 cached positions plus the new one per slot. A step appends the new
+    K / V rows and attends (write + attend + merge kernels); the K and V rows every slot reads
+    are the algorithmic bytes. Two layers' slabs (2 x 268 MB) alternate so that no step finds its
+    rows in the 256 MB Infinity Cache."""
+    import numpy as np
+    import torch
+
+    device = torch.device("cuda:0")
+    slots, query_heads, kv_heads, width, block, context = 32, 32, 8, 128, 16, args.context
+    layers = 1 if args.hot else 2
+    rng = np.random.default_rng(7)
+    blocks_per_slot = -(-context // block)
+    total_blocks = slots * blocks_per_slot
+    max_tokens = total_blocks * block
+    table_host = rng.permutation(total_blocks).reshape(slots, blocks_per_slot).astype(np.int32)
+    cursors_host = np.full(slots, context - 1, dtype=np.int32)
+    advances_host = np.ones(slots, dtype=np.int32)
+    q_host = rng.standard_normal((slots, query_heads, 1, width)).astype(np.float32)
+    k_host = rng.standard_normal((slots, kv_heads, 1, width)).astype(np.float32)
+    v_host = rng.standard_normal((slots, kv_heads, 1, width)).astype(np.float32)
+    scale = 1.0 / float(np.sqrt(width))
+    table = torch.from_numpy(table_host).to(device)
+    cursors, advances = torch.from_numpy(cursors_host).to(device), torch.from_numpy(advances_host).to(device)
+    q, k, v = (torch.from_numpy(a).to(device) for a in (q_host, k_host, v_host))
+    states = []
+    for _ in range(layers):
+        k_slab = torch.randn(max_tokens, kv_heads, width, device=device, dtype=torch.float16)
+        v_slab = torch.randn(max_tokens, kv_heads, width, device=device, dtype=torch.float16)
+        states.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context))
+    out = torch.empty_like(q)
+    need = et.kv_attention_workspace_bytes(states[0], query_heads, 1)
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    statuses = []
+
+    def step(i):
+        statuses.append(et.kv_attention_into(states[i % layers], q, k, v, scale, None, out, workspace=workspace,
+                                             synchronize=False))
+        if len(statuses) > 4:
+            statuses.pop(0)
+
+    # Parity gate before any timing: the first slots against the CPU oracle.
+    import oracle
+    step(0)
+    torch.cuda.synchronize()
+    et.kv_attention_status_check(states[0], 1, statuses[-1])
+    check = 2
+    k_ref, v_ref = states[0].k_slab.cpu().numpy(), states[0].v_slab.cpu().numpy()
+    want = oracle.kv_attention(k_ref, v_ref, block, table_host[:check].view(np.uint32),
+                               cursors_host[:check].view(np.uint32), advances_host[:check].view(np.uint32),
+                               q_host[:check], k_host[:check], v_host[:check], scale)
+    err = float(np.abs(out.cpu().numpy()[:check] - want).max())
+    assert err <= 1e-4, f"parity gate failed: max |err| {err:.4g}"
+
+    ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    seconds = ms * 1e-3
+    slab_bytes = 2 * slots * context * kv_heads * width * 2           # K and V rows read
+    small = 4 * (2 * q.numel() + 2 * k.numel()) + 2 * 2 * k.numel()  # q, out, new k / v in, new rows out
+    algorithmic = slab_bytes + small
+    gbs = algorithmic / seconds / 1e9
+    tokens_per_s = slots / seconds
+    result = {
+        "metric": "kv_attention_decode GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 slabs, f32 arithmetic", "data": "synthetic",
+        "config": {
+            "workload": f"kv_attention_decode: {slots} slots x {query_heads} query heads / {kv_heads} kv heads x "
+                        f"width {width}, context {context}, f16 slabs, block {block}",
+            "slabs": "hot: one layer" if args.hot else f"cold: alternating over {layers} layers "
+                                                       f"({layers * slab_bytes >> 20} MiB)",
+            "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues",
+            "layer_steps_per_s": round(1.0 / seconds, 1),
+            "slot_tokens_per_s_per_layer": round(tokens_per_s, 1),
+            "host_wall_ms": round(wall * 1e3, 3),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(("kv_attention_decode", context)),
+                     "kernel": et.kv_attention_kernel(states[0], query_heads, 1),
+                     "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
+    }
+    if not args.no_cpu:
+        calls, t0 = 0, time.perf_counter()
+        sample = 4
+        while time.perf_counter() - t0 < args.cpu_seconds or calls == 0:
+            oracle.kv_attention(k_ref, v_ref, block, table_host[:sample].view(np.uint32),
+                                cursors_host[:sample].view(np.uint32), advances_host[:sample].view(np.uint32),
+                                q_host[:sample], k_host[:sample], v_host[:sample], scale)
+            calls += 1
+        elapsed = time.perf_counter() - t0
+        per_step = elapsed / calls * (slots / sample)
+        result["cpu_baseline"] = {
+            "value": round(algorithmic / per_step / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{calls} call(s) over {sample} of the {slots} slots, scaled by {slots // sample}; "
+                      f"{elapsed:.1f} s of CPU work; scalar C restatement of the reference's f64 three-pass loop "
+                      f"({per_step * 1e3:.0f} ms per step)"}
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -179,9 +281,12 @@ def main():
 
     if args.workload in ("calibrate_read", "calibrate_copy"):
         return calibrate(args, et)
+    if args.workload == "kv_attention_decode":
+        assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
+        return kv_decode(args, et)
     if args.workload not in synth.CONFIGS:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
-                 "or calibrate_read / calibrate_copy")
+                 "or calibrate_read / calibrate_copy / kv_attention_decode")
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")

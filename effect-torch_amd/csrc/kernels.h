@@ -81,7 +81,7 @@ hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch
 constexpr int kKvAnyWidthPerLane = 8;     // the any-width kernel covers head widths up to 64 * 8
-// Codes of the device status word (slot << 40 | code << 32 | value; ~0 = nothing to report).
+// The device status block holds one word per slot: 0, or code << 32 | value.
 enum : uint32_t {
     kKvBadAdvance = 1,    // value = the advance
     kKvOverCapacity = 2,  // value = live context
@@ -105,7 +105,7 @@ struct KvAttention {
     const float* v;
     double scale;
     float* out;                   // like q
-    void* status;                 // 16 bytes, initialised with kv_status_init
+    void* status;                 // 8 bytes per slot, written by the call
 };
 struct KvLaunchShape {
     bool streaming;
@@ -114,8 +114,7 @@ struct KvLaunchShape {
     uint64_t workspace_bytes;
 };
 KvLaunchShape kv_attention_shape(const KvAttention& p);
-hipError_t kv_status_init(void* status, hipStream_t stream);
-// Writes the new rows, attends, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
+// Attends and appends the new rows, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
 hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream);
 
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------

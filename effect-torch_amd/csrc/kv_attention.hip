@@ -3,14 +3,18 @@
 // with the cursor arithmetic of kv_prepare (:3568-3603); block allocation stays with the
 // caller, which hands over the block table already sized.
 //
-//   1. kv_write_kernel     new K / V rows -> slabs (f32, or f16 rounded to nearest even as
-//                          SlabWriter::set_f32 does, crates/runtime-cpu/src/pool.rs:72-79)
-//   2. kv_attend_kernel    one workgroup per (slot, query token, kv head, context split):
-//                          streams the split's K and V rows once for all query heads of the
-//                          group, online softmax in f32; writes the output, or (m, l, acc)
-//                          partials when the context is split
+//   1. kv_attend_kernel    one workgroup per (slot, query token, kv head, context split):
+//                          streams the split's cached K and V rows once for all query heads
+//                          of the group, takes the new rows straight from the k / v inputs
+//                          (rounded as the slab stores them) and appends them to the slabs
+//                          (f32, or f16 rounded to nearest even as SlabWriter::set_f32 does,
+//                          crates/runtime-cpu/src/pool.rs:72-79); online softmax in f32;
+//                          writes the output, or (m, l, acc) partials when the context is split
 //      kv_attend_any_kernel  the same for widths / groups the streaming kernel does not cover
-//   3. kv_merge_kernel     combines the partials of the splits
+//   2. kv_merge_kernel     combines the partials of the splits
+//
+// The reference writes the new rows first and attends afterwards (napi/mod.rs:3393-3544); here
+// no workgroup reads a new row back from the slab, so one launch does both.
 //
 // Slabs are [max_tokens, kv_heads, width]; the row of logical position p of a slot is
 // table[slot][p / block_size] * block_size + p % block_size.
@@ -26,6 +30,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
+constexpr uint32_t kNoBlock = 0xffffffffu;
 constexpr float kLowest = -1.0e30f;  // "no score yet": finite, so that exp2(kLowest - m) = 0 without NaN
 
 struct KvArgs {
@@ -47,39 +52,35 @@ struct KvArgs {
     float scale_log2;  // scale * log2(e)
 };
 
-// status word: (slot << 40 | code << 32 | value); the smallest key wins, which is the first
-// failing slot in the reference's iteration order and, inside it, the first check that fails.
-__device__ void report(unsigned long long* status, uint32_t slot, uint32_t code, uint32_t value) {
-    atomicMin(status, (static_cast<unsigned long long>(slot) << 40) |
-                          (static_cast<unsigned long long>(code) << 32) | value);
-}
-
 struct Span {
     uint32_t cursor, advance, needed, start;
+    uint32_t code, value;  // the first check of kv_prepare that fails, 0 = none
     bool ok;
 };
 
 // kv_prepare (napi/mod.rs:3588-3609) on device-resident cursors.
-__device__ Span slot_span(const KvArgs& a, uint32_t slot, bool reporter) {
+__device__ Span slot_span(const KvArgs& a, uint32_t slot) {
     Span s;
     s.cursor = a.cursors[slot];
     s.advance = a.advances[slot];
     s.needed = s.cursor + s.advance;
     s.start = a.context_window != 0 && s.needed > a.context_window ? s.needed - a.context_window : 0;
-    s.ok = true;
+    s.code = 0;
+    s.value = 0;
     if (s.advance == 0 || s.advance > a.tokens) {
-        if (reporter) report(a.status, slot, kKvBadAdvance, s.advance);
-        s.ok = false;
+        s.code = kKvBadAdvance;
+        s.value = s.advance;
     } else if (s.needed - s.start > a.max_tokens) {
-        if (reporter) report(a.status, slot, kKvOverCapacity, s.needed - s.start);
-        s.ok = false;
+        s.code = kKvOverCapacity;
+        s.value = s.needed - s.start;
     } else if ((static_cast<uint64_t>(s.needed) + a.block_size - 1) / a.block_size > a.table_stride) {
-        if (reporter) report(a.status, slot, kKvShortTable, s.needed);
-        s.ok = false;
+        s.code = kKvShortTable;
+        s.value = s.needed;
     } else if (s.needed > a.max_context) {
-        if (reporter) report(a.status, slot, kKvOverDeclared, s.needed);
-        s.ok = false;
+        s.code = kKvOverDeclared;
+        s.value = s.needed;
     }
+    s.ok = s.code == 0;
     return s;
 }
 
@@ -94,45 +95,40 @@ __device__ __forceinline__ void slab_store(float* slab, uint64_t at, float value
 __device__ __forceinline__ void slab_store(__half* slab, uint64_t at, float value) {
     slab[at] = __float2half_rn(value);
 }
+// the value a slab of this type holds after storing `value`
+__device__ __forceinline__ float slab_round(const float*, float value) { return value; }
+__device__ __forceinline__ float slab_round(const __half*, float value) {
+    return __half2float(__float2half_rn(value));
+}
 __device__ __forceinline__ float slab_load(const float* slab, uint64_t at) { return slab[at]; }
 __device__ __forceinline__ float slab_load(const __half* slab, uint64_t at) { return __half2float(slab[at]); }
 
-__global__ void kv_status_init_kernel(unsigned long long* status) {
-    if (threadIdx.x == 0) {
-        status[0] = ~0ull;
-        status[1] = 0;
-    }
-}
-
-__global__ void kv_zero_kernel(float* out, uint64_t count) {
+__global__ void kv_zero_kernel(float* out, uint64_t count, unsigned long long* status, uint32_t slots) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < count) out[i] = 0.f;
+    if (i < slots) status[i] = 0;
 }
 
-// Workgroup = (slot, token, kv head); threads run over the width.
-template <typename T>
-__global__ void kv_write_kernel(const KvArgs a) {
-    uint32_t index = blockIdx.x;
-    const uint32_t head = index % a.kv_heads;
-    index /= a.kv_heads;
-    const uint32_t token = index % a.tokens;
-    const uint32_t slot = index / a.tokens;
-    const Span s = slot_span(a, slot, token == 0 && head == 0 && threadIdx.x == 0);
-    if (!s.ok || token >= s.advance) return;
-    const uint32_t position = s.cursor + token;
-    const uint64_t row = static_cast<uint64_t>(a.table[static_cast<uint64_t>(slot) * a.table_stride +
-                                                       block_of(a, position)]) * a.block_size +
-                         within_block(a, position);
-    if (row >= a.max_tokens) {
-        if (threadIdx.x == 0) report(a.status, slot, kKvBlockOutside, static_cast<uint32_t>(row));
-        return;
+// The status word of a slot: 0, or code << 32 | value. Written by one wave per slot, which also
+// checks that the rows of the new positions lie inside the pool.
+__device__ void write_slot_status(const KvArgs& a, uint32_t slot, const Span& s, int lane) {
+    uint32_t code = s.code, value = s.value;
+    if (s.ok) {
+        uint32_t worst = 0;
+        for (uint32_t token = lane; token < s.advance; token += 64) {
+            const uint32_t position = s.cursor + token;
+            const uint64_t row = static_cast<uint64_t>(a.table[static_cast<uint64_t>(slot) * a.table_stride +
+                                                               block_of(a, position)]) * a.block_size +
+                                 within_block(a, position);
+            if (row >= a.max_tokens) worst = max(worst, static_cast<uint32_t>(min(row, uint64_t{0xffffffffu})));
+        }
+        for (int offset = 32; offset > 0; offset >>= 1) worst = max(worst, __shfl_xor(worst, offset));
+        if (worst != 0) {
+            code = kKvBlockOutside;
+            value = worst;
+        }
     }
-    const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + head) * a.tokens + token) * a.width;
-    const uint64_t target = (row * a.kv_heads + head) * a.width;
-    for (uint32_t column = threadIdx.x; column < a.width; column += blockDim.x) {
-        slab_store(static_cast<T*>(a.k_slab), target + column, a.k[source + column]);
-        slab_store(static_cast<T*>(a.v_slab), target + column, a.v[source + column]);
-    }
+    if (lane == 0) a.status[slot] = (static_cast<unsigned long long>(code) << 32) | value;
 }
 
 // Positions a query attends to (napi/mod.rs:3481-3483).
@@ -172,6 +168,10 @@ struct Piece<float> {
         const uint32_t w = i == 0 ? raw.x : i == 1 ? raw.y : i == 2 ? raw.z : raw.w;
         return __uint_as_float(w);
     }
+    // what the slab would hold for these input values
+    __device__ __forceinline__ void from_input(const float* source) {
+        raw = *reinterpret_cast<const uint4*>(source);
+    }
 };
 template <>
 struct Piece<__half> {
@@ -181,7 +181,59 @@ struct Piece<__half> {
         const uint32_t w = (i >> 1) == 0 ? raw.x : (i >> 1) == 1 ? raw.y : (i >> 1) == 2 ? raw.z : raw.w;
         return __half2float(__ushort_as_half(static_cast<unsigned short>((i & 1) ? (w >> 16) : (w & 0xffffu))));
     }
+    __device__ __forceinline__ void from_input(const float* source) {
+        const float4 low = *reinterpret_cast<const float4*>(source);
+        const float4 high = *reinterpret_cast<const float4*>(source + 4);
+        const auto pack = [](float x, float y) {
+            return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(x))) |
+                   (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y))) << 16);
+        };
+        raw = make_uint4(pack(low.x, low.y), pack(low.z, low.w), pack(high.x, high.y), pack(high.z, high.w));
+    }
 };
+
+// One step of the online softmax over U positions per lane group: scores of the G query heads
+// against kp[], then the running maximum, denominator and value sums.
+template <typename T, int LPT, int G, int U>
+__device__ __forceinline__ void attend_step(const float (&q)[G][Piece<T>::kDims], const Piece<T> (&kp)[U],
+                                            const Piece<T> (&vp)[U], const bool (&live)[U], float (&m)[G],
+                                            float (&l)[G], float (&acc)[G][Piece<T>::kDims]) {
+    constexpr int DPL = Piece<T>::kDims;
+    float score[G][U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float part = 0.f;
+#pragma unroll
+            for (int d = 0; d < DPL; d++) part = fmaf(q[g][d], kp[u].get(d), part);
+            part = group_sum<LPT>(part);
+            score[g][u] = live[u] ? part : -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        float top = m[g];
+#pragma unroll
+        for (int u = 0; u < U; u++) top = fmaxf(top, score[g][u]);
+        const float keep = __builtin_amdgcn_exp2f(m[g] - top);
+        float p[U], total = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            p[u] = __builtin_amdgcn_exp2f(score[g][u] - top);
+            total += p[u];
+        }
+        m[g] = top;
+        l[g] = fmaf(l[g], keep, total);
+#pragma unroll
+        for (int d = 0; d < DPL; d++) {
+            float value = acc[g][d] * keep;
+#pragma unroll
+            for (int u = 0; u < U; u++) value = fmaf(p[u], vp[u].get(d), value);
+            acc[g][d] = value;
+        }
+    }
+}
 
 // Streaming kernel. LPT lanes share one position (each holds Piece<T>::kDims of the width,
 // width == LPT * kDims), so a wave covers 64 / LPT positions per load and the workgroup
@@ -213,7 +265,8 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane % LPT, group = wave * PPW + lane / LPT;
 
-    const Span s = slot_span(a, slot, false);
+    const Span s = slot_span(a, slot);
+    if (token == 0 && kv_head == 0 && chunk == 0 && split == 0 && wave == 0) write_slot_status(a, slot, s, lane);
     uint32_t begin, end;
     query_range(a, s, token, begin, end);
     // This split's share, in whole steps.
@@ -222,6 +275,8 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
     share = (share + PPG * U - 1) / (PPG * U) * (PPG * U);
     const uint32_t my_begin = min(begin + split * share, end);
     const uint32_t my_end = s.ok ? min(my_begin + share, end) : my_begin;
+    // Positions below the cursor are cached rows; the others arrive with this call.
+    const uint32_t cached_end = min(my_end, max(my_begin, s.cursor));
 
     // Physical first rows of the blocks this split touches.
     const uint32_t first_block = block_of(a, my_begin);
@@ -230,11 +285,8 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
         for (uint32_t i = threadIdx.x; i < blocks && i < kKvTableEntries; i += kThreads) {
             uint64_t row = static_cast<uint64_t>(a.table[static_cast<uint64_t>(slot) * a.table_stride +
                                                          first_block + i]) * a.block_size;
-            if (row + a.block_size > a.max_tokens) {
-                // the last block may be cut by the pool's end; positions beyond it are the writer's to report
-                if (row >= a.max_tokens) row = 0;
-            }
-            rows_of_block[i] = static_cast<uint32_t>(row);
+            // a block outside the pool is reported by the slot's status; it is neither read nor written
+            rows_of_block[i] = row >= a.max_tokens ? kNoBlock : static_cast<uint32_t>(row);
         }
     }
     __syncthreads();
@@ -258,64 +310,33 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
 
     const uint64_t row_bytes = static_cast<uint64_t>(a.kv_heads) * a.width * sizeof(T);
     const uint64_t lane_offset = (static_cast<uint64_t>(kv_head) * a.width + sub * DPL) * sizeof(T);
-    const char* k_base = static_cast<const char*>(a.k_slab) + lane_offset;
-    const char* v_base = static_cast<const char*>(a.v_slab) + lane_offset;
-
-    auto fetch = [&](uint32_t step_begin, Piece<T> (&kp)[U], Piece<T> (&vp)[U]) {
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            // positions past the split's end read its last row again and are masked out below
-            const uint32_t position = min(step_begin + u * PPG + group, my_end - 1);
-            uint32_t row = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)] +
-                           within_block(a, position);
-            row = min(row, a.max_tokens - 1);
-            kp[u].raw = *reinterpret_cast<const uint4*>(k_base + row * row_bytes);
-            vp[u].raw = *reinterpret_cast<const uint4*>(v_base + row * row_bytes);
-        }
+    char* k_base = static_cast<char*>(a.k_slab) + lane_offset;
+    char* v_base = static_cast<char*>(a.v_slab) + lane_offset;
+    const auto row_of = [&](uint32_t position) {
+        const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
+        return base == kNoBlock ? 0u : min(base + within_block(a, position), a.max_tokens - 1);
     };
 
-    if (my_end > my_begin) {
-        Piece<T> kp[U], vp[U];
-        fetch(my_begin, kp, vp);
-        for (uint32_t step = my_begin; step < my_end; step += PPG * U) {
-            Piece<T> kn[U], vn[U];
-            const bool more = step + PPG * U < my_end;
-            if (more) fetch(step + PPG * U, kn, vn);
-            float score[G][U];
+    if (cached_end > my_begin) {
+        const auto fetch = [&](uint32_t step_begin, Piece<T> (&kp)[U], Piece<T> (&vp)[U]) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const bool live = step + u * PPG + group < my_end;
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    float part = 0.f;
-#pragma unroll
-                    for (int d = 0; d < DPL; d++) part = fmaf(q[g][d], kp[u].get(d), part);
-                    part = group_sum<LPT>(part);
-                    score[g][u] = live ? part : -INFINITY;
-                }
+                // positions past the end read the last cached row again and are masked out below
+                const uint32_t row = row_of(min(step_begin + u * PPG + group, cached_end - 1));
+                kp[u].raw = *reinterpret_cast<const uint4*>(k_base + row * row_bytes);
+                vp[u].raw = *reinterpret_cast<const uint4*>(v_base + row * row_bytes);
             }
+        };
+        Piece<T> kp[U], vp[U];
+        fetch(my_begin, kp, vp);
+        for (uint32_t step = my_begin; step < cached_end; step += PPG * U) {
+            Piece<T> kn[U], vn[U];
+            const bool more = step + PPG * U < cached_end;
+            if (more) fetch(step + PPG * U, kn, vn);
+            bool live[U];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                float top = m[g];
-#pragma unroll
-                for (int u = 0; u < U; u++) top = fmaxf(top, score[g][u]);
-                const float keep = __builtin_amdgcn_exp2f(m[g] - top);
-                float p[U], total = 0.f;
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    p[u] = __builtin_amdgcn_exp2f(score[g][u] - top);
-                    total += p[u];
-                }
-                m[g] = top;
-                l[g] = fmaf(l[g], keep, total);
-#pragma unroll
-                for (int d = 0; d < DPL; d++) {
-                    float value = acc[g][d] * keep;
-#pragma unroll
-                    for (int u = 0; u < U; u++) value = fmaf(p[u], vp[u].get(d), value);
-                    acc[g][d] = value;
-                }
-            }
+            for (int u = 0; u < U; u++) live[u] = step + u * PPG + group < cached_end;
+            attend_step<T, LPT, G, U>(q, kp, vp, live, m, l, acc);
             if (more) {
 #pragma unroll
                 for (int u = 0; u < U; u++) {
@@ -324,6 +345,27 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
                 }
             }
         }
+    }
+    // The new positions of this split: from the inputs, as the slab will hold them. The workgroup
+    // whose query token is the new position itself (chunk 0) appends the row to the slabs.
+    for (uint32_t step = cached_end; step < my_end; step += PPG) {
+        const uint32_t position = step + group;
+        const bool live[1] = {position < my_end};
+        const uint32_t arrival = min(position, my_end - 1) - s.cursor;
+        const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + kv_head) * a.tokens + arrival) *
+                                    a.width + sub * DPL;
+        Piece<T> kp[1], vp[1];
+        kp[0].from_input(a.k + source);
+        vp[0].from_input(a.v + source);
+        if (live[0] && arrival == token && chunk == 0) {
+            const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
+            const uint32_t row = base + within_block(a, position);
+            if (base != kNoBlock && row < a.max_tokens) {
+                *reinterpret_cast<uint4*>(k_base + row * row_bytes) = kp[0].raw;
+                *reinterpret_cast<uint4*>(v_base + row * row_bytes) = vp[0].raw;
+            }
+        }
+        attend_step<T, LPT, G, 1>(q, kp, vp, live, m, l, acc);
     }
 
     // Combine the workgroup's softmax states.
@@ -373,10 +415,12 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
     index /= a.tokens;
     const uint32_t head = index % a.query_heads;
     const uint32_t slot = index / a.query_heads;
-    const uint32_t kv_head = head / (a.query_heads / a.kv_heads);
+    const uint32_t group_size = a.query_heads / a.kv_heads;
+    const uint32_t kv_head = head / group_size;
     const int lane = threadIdx.x;
 
-    const Span s = slot_span(a, slot, false);
+    const Span s = slot_span(a, slot);
+    if (token == 0 && head == 0 && split == 0) write_slot_status(a, slot, s, lane);
     uint32_t begin, end;
     query_range(a, s, token, begin, end);
     const uint32_t length = s.ok ? end - begin : 0;
@@ -393,19 +437,41 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
         acc[i] = 0.f;
     }
     float m = kLowest, l = 0.f;
-    const T* keys = static_cast<const T*>(a.k_slab);
-    const T* values = static_cast<const T*>(a.v_slab);
+    T* keys = static_cast<T*>(a.k_slab);
+    T* values = static_cast<T*>(a.v_slab);
     for (uint32_t position = my_begin; position < my_end; position++) {
         uint64_t row = static_cast<uint64_t>(a.table[static_cast<uint64_t>(slot) * a.table_stride +
                                                      block_of(a, position)]) * a.block_size +
                        within_block(a, position);
+        const bool inside = row < a.max_tokens;
         row = min(row, static_cast<uint64_t>(a.max_tokens - 1));
         const uint64_t at = (row * a.kv_heads + kv_head) * a.width;
+        // A new position comes from the inputs, rounded as the slab stores it; the first query head
+        // of the group whose token is that position appends it.
+        const bool arriving = position >= s.cursor;
+        const uint32_t arrival = arriving ? position - s.cursor : 0;
+        const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + kv_head) * a.tokens + arrival) * a.width;
+        const bool appends = arriving && arrival == token && head % group_size == 0 && inside;
+        float key[kKvAnyWidthPerLane], value[kKvAnyWidthPerLane];
         float part = 0.f;
 #pragma unroll
         for (int i = 0; i < kKvAnyWidthPerLane; i++) {
             const uint32_t column = lane + 64 * i;
-            if (column < a.width) part = fmaf(q[i], slab_load(keys, at + column), part);
+            key[i] = value[i] = 0.f;
+            if (column < a.width) {
+                if (arriving) {
+                    key[i] = slab_round(keys, a.k[source + column]);
+                    value[i] = slab_round(values, a.v[source + column]);
+                    if (appends) {
+                        slab_store(keys, at + column, a.k[source + column]);
+                        slab_store(values, at + column, a.v[source + column]);
+                    }
+                } else {
+                    key[i] = slab_load(keys, at + column);
+                    value[i] = slab_load(values, at + column);
+                }
+                part = fmaf(q[i], key[i], part);
+            }
         }
         const float score = group_sum<64>(part);
         const float top = fmaxf(m, score);
@@ -413,10 +479,7 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
         m = top;
         l = fmaf(l, keep, p);
 #pragma unroll
-        for (int i = 0; i < kKvAnyWidthPerLane; i++) {
-            const uint32_t column = lane + 64 * i;
-            if (column < a.width) acc[i] = fmaf(p, slab_load(values, at + column), acc[i] * keep);
-        }
+        for (int i = 0; i < kKvAnyWidthPerLane; i++) acc[i] = fmaf(p, value[i], acc[i] * keep);
     }
 #pragma unroll
     for (int i = 0; i < kKvAnyWidthPerLane; i++) {
@@ -435,23 +498,25 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
     }
 }
 
-// out[query, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp2(m_s - max m); one wave per query row.
-__global__ __launch_bounds__(64) void kv_merge_kernel(const KvArgs a) {
+// out[query, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp2(m_s - max m); a workgroup per
+// query row, a thread per column.
+__global__ void kv_merge_kernel(const KvArgs a) {
     const uint64_t query = blockIdx.x;
     const uint32_t slot = static_cast<uint32_t>(query / (static_cast<uint64_t>(a.query_heads) * a.tokens));
-    const Span s = slot_span(a, slot, false);
-    if (!s.ok) return;
-    const float* records = a.partial + query * a.splits * (a.width + 2);
-    float top = kLowest;
-    for (uint32_t i = 0; i < a.splits; i++) top = fmaxf(top, records[i * (a.width + 2)]);
-    float total = 0.f;
-    for (uint32_t i = 0; i < a.splits; i++)
-        total = fmaf(__builtin_amdgcn_exp2f(records[i * (a.width + 2)] - top), records[i * (a.width + 2) + 1], total);
-    for (uint32_t column = threadIdx.x; column < a.width; column += 64) {
-        float value = 0.f;
-        for (uint32_t i = 0; i < a.splits; i++)
-            value = fmaf(__builtin_amdgcn_exp2f(records[i * (a.width + 2)] - top),
-                         records[i * (a.width + 2) + 2 + column], value);
+    if (!slot_span(a, slot).ok) return;
+    const uint32_t stride = a.width + 2;
+    const float* records = a.partial + query * a.splits * stride;
+    for (uint32_t column = threadIdx.x; column < a.width; column += blockDim.x) {
+        float top = kLowest, total = 0.f, value = 0.f;
+#pragma unroll 4
+        for (uint32_t i = 0; i < a.splits; i++) {
+            const float m = records[i * stride], l = records[i * stride + 1], part = records[i * stride + 2 + column];
+            const float next = fmaxf(top, m);
+            const float keep = __builtin_amdgcn_exp2f(top - next), weight = __builtin_amdgcn_exp2f(m - next);
+            total = fmaf(total, keep, weight * l);
+            value = fmaf(value, keep, weight * part);
+            top = next;
+        }
         a.out[query * a.width + column] = value / total;
     }
 }
@@ -512,7 +577,7 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     const uint64_t context = p.max_context == 0 ? 1 : p.max_context;
     const uint64_t step = shape.streaming ? positions_per_step(p, g) : 64;
     uint64_t splits = 1;
-    const uint64_t wanted = shape.streaming ? 2048 : 4096;
+    const uint64_t wanted = shape.streaming ? 1024 : 4096;
     if (rows < wanted) splits = (wanted + rows - 1) / (rows == 0 ? 1 : rows);
     const uint64_t most = (context + 2 * step - 1) / (2 * step);
     if (splits > most) splits = most;
@@ -529,12 +594,6 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     const uint64_t queries = static_cast<uint64_t>(p.active_batch) * p.query_heads * p.tokens;
     shape.workspace_bytes = splits > 1 ? queries * splits * (p.width + 2) * sizeof(float) : 0;
     return shape;
-}
-
-hipError_t kv_status_init(void* status, hipStream_t stream) {
-    hipLaunchKernelGGL(kv_status_init_kernel, dim3(1), dim3(64), 0, stream,
-                       static_cast<unsigned long long*>(status));
-    return hipGetLastError();
 }
 
 hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream) {
@@ -568,24 +627,17 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     const KvLaunchShape shape = kv_attention_shape(p);
     a.splits = shape.splits;
 
-    // out.fill(0.0) for the slots that are not active (napi/mod.rs:3371).
+    // out.fill(0.0) for the slots that are not active (napi/mod.rs:3371); their status words too.
     const uint64_t per_slot = static_cast<uint64_t>(p.query_heads) * p.tokens * p.width;
     if (p.active_batch < p.batch) {
         const uint64_t count = (p.batch - p.active_batch) * per_slot;
         hipLaunchKernelGGL(kv_zero_kernel, dim3(static_cast<uint32_t>((count + 255) / 256)), dim3(256), 0, stream,
-                           p.out + p.active_batch * per_slot, count);
+                           p.out + p.active_batch * per_slot, count, a.status + p.active_batch,
+                           p.batch - p.active_batch);
     }
     if (p.active_batch == 0) return hipGetLastError();
 
-    const uint32_t writers = p.active_batch * p.tokens * p.kv_heads;
-    const uint32_t writer_threads = p.width >= 256 ? 256 : p.width > 64 ? 128 : 64;
-    if (p.slab_is_f16)
-        hipLaunchKernelGGL(kv_write_kernel<__half>, dim3(writers), dim3(writer_threads), 0, stream, a);
-    else
-        hipLaunchKernelGGL(kv_write_kernel<float>, dim3(writers), dim3(writer_threads), 0, stream, a);
-    hipError_t error = hipGetLastError();
-    if (error != hipSuccess) return error;
-
+    hipError_t error;
     if (shape.streaming) {
         const int g = streaming_group(p);
         error = p.slab_is_f16
@@ -603,7 +655,8 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     if (error != hipSuccess) return error;
     if (shape.splits > 1) {
         const uint64_t queries = static_cast<uint64_t>(p.active_batch) * p.query_heads * p.tokens;
-        hipLaunchKernelGGL(kv_merge_kernel, dim3(static_cast<uint32_t>(queries)), dim3(64), 0, stream, a);
+        const uint32_t threads = p.width > 128 ? 256 : p.width > 64 ? 128 : 64;
+        hipLaunchKernelGGL(kv_merge_kernel, dim3(static_cast<uint32_t>(queries)), dim3(threads), 0, stream, a);
         error = hipGetLastError();
     }
     return error;

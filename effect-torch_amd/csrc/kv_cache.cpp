@@ -83,8 +83,8 @@ const char* kernel_name(const et_kv_layer& layer, uint64_t query_heads, uint64_t
     if (layer_geometry(layer, &p, &error) != ET_OK || query_geometry(query_heads, tokens, &p, &error) != ET_OK)
         return "";
     const KvLaunchShape shape = kv_attention_shape(p);
-    if (shape.streaming) return shape.splits > 1 ? "kv_write+kv_attend+kv_merge" : "kv_write+kv_attend";
-    return shape.splits > 1 ? "kv_write+kv_attend_any+kv_merge" : "kv_write+kv_attend_any";
+    if (shape.streaming) return shape.splits > 1 ? "kv_attend+kv_merge" : "kv_attend";
+    return shape.splits > 1 ? "kv_attend_any+kv_merge" : "kv_attend_any";
 }
 
 int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, const quantized::TensorView& k,
@@ -156,18 +156,21 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
                     "kv attention: workspace of " + std::to_string(workspace_bytes) + " bytes is smaller than the " +
                         std::to_string(shape.workspace_bytes) + " required");
     if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
-    hipError_t launched = kv_status_init(status, static_cast<hipStream_t>(stream));
-    if (launched == hipSuccess) launched = kv_attention(p, workspace, static_cast<hipStream_t>(stream));
+    const hipError_t launched = kv_attention(p, workspace, static_cast<hipStream_t>(stream));
     if (launched != hipSuccess)
         return fail(error, ET_ERR_EXECUTION, std::string("kv attention: HIP error: ") + hipGetErrorString(launched));
     return ET_OK;
 }
 
 int status_check(const et_kv_layer& layer, uint64_t tokens, const void* status_host, std::string* error) {
-    unsigned long long word;
-    std::memcpy(&word, status_host, sizeof word);
-    if (word == ~0ull) return ET_OK;
-    const uint64_t slot = word >> 40, code = (word >> 32) & 0xff, value = word & 0xffffffffull;
+    // the first failing slot, as the reference's loop over the slots would meet it
+    unsigned long long word = 0;
+    uint64_t slot = 0;
+    for (; slot < layer.slots && word == 0; slot++)
+        std::memcpy(&word, static_cast<const char*>(status_host) + 8 * slot, sizeof word);
+    if (word == 0) return ET_OK;
+    slot -= 1;
+    const uint64_t code = word >> 32, value = word & 0xffffffffull;
     switch (code) {
         case kKvBadAdvance:  // napi/mod.rs:3590-3594
             return fail(error, ET_ERR_EXECUTION,

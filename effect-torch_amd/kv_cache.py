@@ -63,7 +63,7 @@ def kv_attention_kernel(layer: KvLayer, query_heads: int, tokens: int) -> str:
 
 def kv_attention_status_check(layer: KvLayer, tokens: int, status: torch.Tensor) -> None:
     host = status.cpu().numpy().tobytes()  # synchronises with the producing stream
-    buf = ctypes.create_string_buffer(host, N.STATUS_BYTES)
+    buf = ctypes.create_string_buffer(host, len(host))
     _check(N.lib().et_hip_kv_attention_status_check(ctypes.byref(layer.struct()), tokens, buf))
 
 
@@ -83,7 +83,7 @@ def kv_attention_into(layer: KvLayer, q: torch.Tensor, k: torch.Tensor, v: torch
         if q.dim() >= 4 and heads and tokens:
             need = int(N.lib().et_hip_kv_attention_workspace_bytes(ctypes.byref(struct), heads, tokens))
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=destination.device)
-    status = torch.empty(N.STATUS_BYTES, dtype=torch.uint8, device=destination.device)
+    status = torch.empty(8 * max(layer.cursors.numel(), 1), dtype=torch.uint8, device=destination.device)
     descs = (_desc(q), _desc(k), _desc(v), _desc(destination))
     _check(N.lib().et_hip_kv_attention_into(ctypes.byref(struct), _ref(descs[0]), _ref(descs[1]), _ref(descs[2]),
                                             float(scale), int(window or 0), _ref(descs[3]),

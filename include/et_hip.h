@@ -241,16 +241,18 @@ uint64_t et_hip_kv_attention_workspace_bytes(const et_kv_layer* layer, uint64_t 
  *   window: the operator's own sliding window, 0 = none.
  * The cursors live on the device, so the checks of kv_prepare that depend on
  * them cannot fail this call: a slot that fails one is skipped and the device
- * `status` block (ET_HIP_STATUS_BYTES, initialised by this call on `stream`)
- * records it for et_hip_kv_attention_status_check. */
+ * `status` block (8 bytes per slot, every word written by this call) records it
+ * for et_hip_kv_attention_status_check. */
+#define ET_HIP_KV_STATUS_BYTES(slots) (8 * (uint64_t)(slots))
 int et_hip_kv_attention_into(const et_kv_layer* layer, const et_tensor* q, const et_tensor* k,
                              const et_tensor* v, double scale, uint64_t window,
                              const et_tensor* destination, void* workspace,
                              uint64_t workspace_bytes, void* status, void* stream,
                              const volatile int32_t* cancel);
 /* After the stream has completed and `status` has been copied to the host: 0, or
- * ET_ERR_EXECUTION with the reference's message, e.g. "kv attention: advance {a}
- * out of range for chunk length {tokens}" (napi/mod.rs:3590-3594). */
+ * ET_ERR_EXECUTION with the reference's message for the first failing slot, e.g.
+ * "kv attention: advance {a} out of range for chunk length {tokens}"
+ * (napi/mod.rs:3590-3594). */
 int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
                                      const void* status_host);
 /* Name of the kernel variant these sizes select, for profiles and diagnostics. */

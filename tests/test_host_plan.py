@@ -201,23 +201,29 @@ def test_kv_attention_launch_shapes_and_status_wording(et):
     from effect_torch_amd import _native
     decode = _kv_layer(et, torch, slots=32, kv_heads=8, width=128, max_tokens=32 * 2048, block_size=16,
                        dtype=torch.float16, max_context=2048)
-    assert et.kv_attention_kernel(decode, 32, 1) == "kv_write+kv_attend+kv_merge"
+    assert et.kv_attention_kernel(decode, 32, 1) == "kv_attend+kv_merge"
     assert et.kv_attention_workspace_bytes(decode, 32, 1) % (32 * 32 * 130 * 4) == 0
     short = _kv_layer(et, torch, slots=512, kv_heads=8, width=128, max_tokens=4096, block_size=16,
                       dtype=torch.float16, max_context=8)
-    assert et.kv_attention_kernel(short, 32, 1) == "kv_write+kv_attend"
+    assert et.kv_attention_kernel(short, 32, 1) == "kv_attend"
     assert et.kv_attention_workspace_bytes(short, 32, 1) == 0
     odd = _kv_layer(et, torch, width=12)
-    assert et.kv_attention_kernel(odd, 4, 1).startswith("kv_write+kv_attend_any")
+    assert et.kv_attention_kernel(odd, 4, 1).startswith("kv_attend_any")
     assert et.kv_attention_kernel(odd, 3, 1) == ""  # 3 query heads over 2 kv heads
 
-    def message(word):
+    def message(word, slot=0):
         layer = decode.struct()
-        buf = ctypes.create_string_buffer(struct.pack("<QQ", word, 0), 16)
+        words = [0] * 32
+        words[slot] = word
+        words[-1] = (3 << 32) | 5  # a later slot's failure is not the one reported
+        buf = ctypes.create_string_buffer(struct.pack("<32Q", *words), 256)
         status = _native.lib().et_hip_kv_attention_status_check(ctypes.byref(layer), 7, buf)
         return status, _native.last_error()
 
-    assert message(2**64 - 1)[0] == 0
-    assert message((3 << 40) | (1 << 32) | 9) == (2, "kv attention: advance 9 out of range for chunk length 7")
+    layer = decode.struct()
+    clean = ctypes.create_string_buffer(256)
+    assert _native.lib().et_hip_kv_attention_status_check(ctypes.byref(layer), 7, clean) == 0
+    assert message((1 << 32) | 9, slot=3) == (2, "kv attention: advance 9 out of range for chunk length 7")
     assert message((1 << 32) | 0) == (2, "kv attention: advance 0 out of range for chunk length 7")
     assert message((2 << 32) | 70000) == (2, "kv attention: live context 70000 exceeds pool capacity 65536")
+    assert message((3 << 32) | 41, slot=30) == (2, "kv attention: block table of slot 30 does not cover 41 tokens")
