@@ -197,8 +197,7 @@ def kv_decode(args, et):
         v_slab = torch.randn(max_tokens, kv_heads, width, device=device, dtype=torch.float16)
         states.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context))
     out = torch.empty_like(q)
-    need = et.kv_attention_workspace_bytes(states[0], query_heads, 1)
-    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    workspace = et.kv_attention_workspace(states[0], query_heads, 1)
     statuses = []
 
     def step(i):

@@ -114,7 +114,7 @@ struct KvLaunchShape {
     uint64_t workspace_bytes;
 };
 KvLaunchShape kv_attention_shape(const KvAttention& p);
-// Attends and appends the new rows, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
+// Attends, appends the new rows, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
 hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream);
 
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------

@@ -12,6 +12,8 @@
 //                          writes the output, or (m, l, acc) partials when the context is split
 //      kv_attend_any_kernel  the same for widths / groups the streaming kernel does not cover
 //   2. kv_merge_kernel     combines the partials of the splits
+//      (Letting the last split to finish combine them inside the attend kernel was measured: the
+//      device-wide fences it needs cost far more than this second launch.)
 //
 // The reference writes the new rows first and attends afterwards (napi/mod.rs:3393-3544); here
 // no workgroup reads a new row back from the slab, so one launch does both.
@@ -235,6 +237,123 @@ __device__ __forceinline__ void attend_step(const float (&q)[G][Piece<T>::kDims]
     }
 }
 
+// Softmax state of the scatter step: the lanes r = sub % 16 of a 16-lane row with
+// r / (16 / G) == g hold the running maximum and denominator of query head g.
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) { return fmaxf(v, dpp_f32<CTRL>(v)); }
+
+template <int LANES>
+__device__ __forceinline__ float block_max(float v) {
+    if constexpr (LANES >= 2) v = dpp_max<0xB1>(v);
+    if constexpr (LANES >= 4) v = dpp_max<0x4E>(v);
+    if constexpr (LANES >= 8) v = dpp_max<0x141>(v);
+    if constexpr (LANES >= 16) v = dpp_max<0x140>(v);
+    return v;
+}
+
+__device__ __forceinline__ float from_lane(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(lane << 2, __float_as_int(v)));
+}
+
+// One stage of the reduce-scatter over a 16-lane row: partners (DPP pattern CTRL) differ in
+// bit BIT of the lane number; each keeps the half of the values whose index has its own bit
+// and adds the partner's copy of that half. With one value left the stage is a plain sum.
+template <int CTRL, int BIT, int N>
+__device__ __forceinline__ void scatter_stage(float (&w)[16], int r) {
+    if constexpr (N > 1) {
+        const bool upper = (r >> BIT) & 1;
+#pragma unroll
+        for (int k = 0; k < N / 2; k++) {
+            const float mine = upper ? w[N / 2 + k] : w[k];
+            const float theirs = upper ? w[k] : w[N / 2 + k];
+            w[k] = mine + dpp_f32<CTRL>(theirs);
+        }
+    } else {
+        w[0] += dpp_f32<CTRL>(w[0]);
+    }
+}
+
+// The same step as attend_step for LPT >= 16, with less arithmetic: the G * U partial scores are
+// reduce-scattered over the 16 lanes of a row (lane r ends with the total of pair r / R,
+// R = 16 / (G * U)), every lane does the softmax arithmetic of its own pair only, and the
+// weights come back to all lanes through the LDS crossbar. `first` is the position of u = 0.
+template <typename T, int LPT, int G, int U>
+__device__ __forceinline__ void attend_step_scatter(const float (&q)[G][Piece<T>::kDims], const Piece<T> (&kp)[U],
+                                                    const Piece<T> (&vp)[U], uint32_t first, uint32_t stride,
+                                                    uint32_t end, int lane, float& m, float& l,
+                                                    float (&acc)[G][Piece<T>::kDims]) {
+    constexpr int DPL = Piece<T>::kDims;
+    constexpr int N = G * U;       // pairs (query head, position)
+    constexpr int R = 16 / N;      // lanes holding the same pair
+    constexpr int BLOCK = 16 / G;  // lanes of one query head
+    static_assert(N <= 16 && LPT >= 16, "scatter step: at most 16 pairs over rows of 16 lanes");
+    const int r = lane & 15;
+    float w[16];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float part = 0.f;
+#pragma unroll
+            for (int d = 0; d < DPL; d++) part = fmaf(q[g][d], kp[u].get(d), part);
+            if constexpr (LPT >= 32) part += from_lane(part, lane ^ 16);
+            w[g * U + u] = part;
+        }
+    }
+    scatter_stage<0x140, 3, N>(w, r);
+    scatter_stage<0x141, 2, (N > 1 ? N / 2 : 1)>(w, r);
+    scatter_stage<0x4E, 1, (N > 2 ? N / 4 : 1)>(w, r);
+    scatter_stage<0xB1, 0, (N > 4 ? N / 8 : 1)>(w, r);
+    const int u = (r / R) % U;
+    const float score = first + u * stride < end ? w[0] : -INFINITY;
+    const float top = fmaxf(m, block_max<BLOCK>(score));
+    const float keep = __builtin_amdgcn_exp2f(m - top);
+    const float p = __builtin_amdgcn_exp2f(score - top);
+    float total = p;
+    if constexpr (BLOCK >= 2) total += dpp_f32<0xB1>(total);
+    if constexpr (BLOCK >= 4) total += dpp_f32<0x4E>(total);
+    if constexpr (BLOCK >= 8) total += dpp_f32<0x141>(total);
+    if constexpr (BLOCK >= 16) total += dpp_f32<0x140>(total);
+    l = fmaf(l, keep, total * (1.0f / R));
+    m = top;
+    const int row = lane & ~15;
+    if (__builtin_amdgcn_ballot_w64(keep != 1.0f) != 0) {  // some maximum moved: rescale the sums
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float factor = from_lane(keep, row + g * BLOCK);
+#pragma unroll
+            for (int d = 0; d < DPL; d++) acc[g][d] *= factor;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int uu = 0; uu < U; uu++) {
+            const float weight = from_lane(p, row + (g * U + uu) * R);
+#pragma unroll
+            for (int d = 0; d < DPL; d++) acc[g][d] = fmaf(weight, vp[uu].get(d), acc[g][d]);
+        }
+    }
+}
+
+// out[query, column] = sum_i w_i acc_i / sum_i w_i l_i with w_i = exp2(m_i - max m) over the
+// partial records of the context splits.
+__device__ __forceinline__ void merge_splits(const KvArgs& a, uint64_t query, uint32_t column) {
+    const uint32_t stride = a.width + 2;
+    const float* records = a.partial + query * a.splits * stride;
+    float top = kLowest, total = 0.f, value = 0.f;
+#pragma unroll 4
+    for (uint32_t i = 0; i < a.splits; i++) {
+        const float m = records[i * stride], l = records[i * stride + 1], part = records[i * stride + 2 + column];
+        const float next = fmaxf(top, m);
+        const float keep = __builtin_amdgcn_exp2f(top - next), weight = __builtin_amdgcn_exp2f(m - next);
+        total = fmaf(total, keep, weight * l);
+        value = fmaf(value, keep, weight * part);
+        top = next;
+    }
+    a.out[query * a.width + column] = value / total;
+}
+
 // Streaming kernel. LPT lanes share one position (each holds Piece<T>::kDims of the width,
 // width == LPT * kDims), so a wave covers 64 / LPT positions per load and the workgroup
 // 4 * 64 / LPT; U such loads are in flight per step. G query heads of one kv head are
@@ -299,6 +418,9 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
 #pragma unroll
         for (int d = 0; d < DPL; d++) q[g][d] = source[d] * a.scale_log2;
     }
+    // Softmax state: per query head in every lane (rows of 8 lanes), or spread over the 16 lanes of a
+    // row, lane r holding head r / (16 / G) (see attend_step_scatter).
+    constexpr bool kScatter = LPT >= 16;
     float m[G], l[G], acc[G][DPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
@@ -327,23 +449,26 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
                 vp[u].raw = *reinterpret_cast<const uint4*>(v_base + row * row_bytes);
             }
         };
-        Piece<T> kp[U], vp[U];
-        fetch(my_begin, kp, vp);
-        for (uint32_t step = my_begin; step < cached_end; step += PPG * U) {
-            Piece<T> kn[U], vn[U];
-            const bool more = step + PPG * U < cached_end;
-            if (more) fetch(step + PPG * U, kn, vn);
-            bool live[U];
+        const auto consume = [&](uint32_t step, const Piece<T> (&kp)[U], const Piece<T> (&vp)[U]) {
+            if constexpr (kScatter) {
+                attend_step_scatter<T, LPT, G, U>(q, kp, vp, step + group, PPG, cached_end, lane, m[0], l[0], acc);
+            } else {
+                bool live[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) live[u] = step + u * PPG + group < cached_end;
-            attend_step<T, LPT, G, U>(q, kp, vp, live, m, l, acc);
-            if (more) {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    kp[u] = kn[u];
-                    vp[u] = vn[u];
-                }
+                for (int u = 0; u < U; u++) live[u] = step + u * PPG + group < cached_end;
+                attend_step<T, LPT, G, U>(q, kp, vp, live, m, l, acc);
             }
+        };
+        // two register sets take turns: one is consumed while the other one's loads are in flight
+        constexpr uint32_t kStep = PPG * U;
+        Piece<T> ka[U], va[U], kb[U], vb[U];
+        fetch(my_begin, ka, va);
+        for (uint32_t step = my_begin; step < cached_end; step += 2 * kStep) {
+            if (step + kStep < cached_end) fetch(step + kStep, kb, vb);
+            consume(step, ka, va);
+            if (step + kStep >= cached_end) break;
+            if (step + 2 * kStep < cached_end) fetch(step + 2 * kStep, ka, va);
+            consume(step + kStep, kb, vb);
         }
     }
     // The new positions of this split: from the inputs, as the slab will hold them. The workgroup
@@ -365,13 +490,21 @@ __global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
                 *reinterpret_cast<uint4*>(v_base + row * row_bytes) = vp[0].raw;
             }
         }
-        attend_step<T, LPT, G, 1>(q, kp, vp, live, m, l, acc);
+        if constexpr (kScatter)
+            attend_step_scatter<T, LPT, G, 1>(q, kp, vp, position, PPG, my_end, lane, m[0], l[0], acc);
+        else
+            attend_step<T, LPT, G, 1>(q, kp, vp, live, m, l, acc);
     }
 
     // Combine the workgroup's softmax states.
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        if (sub == 0) {
+        if constexpr (kScatter) {
+            if (sub == g * (16 / G)) {
+                merge_m[group][g] = m[0];
+                merge_l[group][g] = l[0];
+            }
+        } else if (sub == 0) {
             merge_m[group][g] = m[g];
             merge_l[group][g] = l[g];
         }
@@ -498,27 +631,12 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
     }
 }
 
-// out[query, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp2(m_s - max m); a workgroup per
-// query row, a thread per column.
+// Combines the partial records of the context splits: a workgroup per query row, a thread per column.
 __global__ void kv_merge_kernel(const KvArgs a) {
     const uint64_t query = blockIdx.x;
     const uint32_t slot = static_cast<uint32_t>(query / (static_cast<uint64_t>(a.query_heads) * a.tokens));
     if (!slot_span(a, slot).ok) return;
-    const uint32_t stride = a.width + 2;
-    const float* records = a.partial + query * a.splits * stride;
-    for (uint32_t column = threadIdx.x; column < a.width; column += blockDim.x) {
-        float top = kLowest, total = 0.f, value = 0.f;
-#pragma unroll 4
-        for (uint32_t i = 0; i < a.splits; i++) {
-            const float m = records[i * stride], l = records[i * stride + 1], part = records[i * stride + 2 + column];
-            const float next = fmaxf(top, m);
-            const float keep = __builtin_amdgcn_exp2f(top - next), weight = __builtin_amdgcn_exp2f(m - next);
-            total = fmaf(total, keep, weight * l);
-            value = fmaf(value, keep, weight * part);
-            top = next;
-        }
-        a.out[query * a.width + column] = value / total;
-    }
+    for (uint32_t column = threadIdx.x; column < a.width; column += blockDim.x) merge_splits(a, query, column);
 }
 
 template <typename T, int LPT, int G>
@@ -577,8 +695,11 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     const uint64_t context = p.max_context == 0 ? 1 : p.max_context;
     const uint64_t step = shape.streaming ? positions_per_step(p, g) : 64;
     uint64_t splits = 1;
-    const uint64_t wanted = shape.streaming ? 1024 : 4096;
-    if (rows < wanted) splits = (wanted + rows - 1) / (rows == 0 ? 1 : rows);
+    // The streaming kernel keeps two workgroups per compute unit resident; with all of them
+    // resident at once no workgroup waits for a second round (measured: 512 beat 1024 and 2048).
+    const uint64_t wanted = shape.streaming ? 512 : 4096;
+    if (rows < wanted) splits = shape.streaming ? wanted / (rows == 0 ? 1 : rows)
+                                                : (wanted + rows - 1) / (rows == 0 ? 1 : rows);
     const uint64_t most = (context + 2 * step - 1) / (2 * step);
     if (splits > most) splits = most;
     if (shape.streaming) {
@@ -607,7 +728,6 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     a.k = p.k;
     a.v = p.v;
     a.out = p.out;
-    a.partial = static_cast<float*>(workspace);
     a.status = static_cast<unsigned long long*>(p.status);
     a.max_tokens = p.max_tokens;
     a.kv_heads = p.kv_heads;
@@ -626,6 +746,7 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     a.max_context = p.max_context;
     const KvLaunchShape shape = kv_attention_shape(p);
     a.splits = shape.splits;
+    a.partial = static_cast<float*>(workspace);
 
     // out.fill(0.0) for the slots that are not active (napi/mod.rs:3371); their status words too.
     const uint64_t per_slot = static_cast<uint64_t>(p.query_heads) * p.tokens * p.width;

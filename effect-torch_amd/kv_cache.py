@@ -57,6 +57,12 @@ def kv_attention_workspace_bytes(layer: KvLayer, query_heads: int, tokens: int) 
     return int(N.lib().et_hip_kv_attention_workspace_bytes(ctypes.byref(layer.struct()), query_heads, tokens))
 
 
+def kv_attention_workspace(layer: KvLayer, query_heads: int, tokens: int, device=None) -> torch.Tensor:
+    """A workspace for these sizes; it can serve any number of calls that do not overlap in time."""
+    need = kv_attention_workspace_bytes(layer, query_heads, tokens)
+    return torch.empty(max(need, 16), dtype=torch.uint8, device=device or layer.k_slab.device)
+
+
 def kv_attention_kernel(layer: KvLayer, query_heads: int, tokens: int) -> str:
     return N.lib().et_hip_kv_attention_kernel(ctypes.byref(layer.struct()), query_heads, tokens).decode()
 

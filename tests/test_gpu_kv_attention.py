@@ -33,7 +33,8 @@ def make_case(rng, *, slots, query_heads, kv_heads, width, block_size, contexts,
                 max_context=int((contexts + advances).max()))
 
 
-def run_gpu(et, device, case, scale, *, window=0, context_window=0, active_batch=None, max_context=None):
+def run_gpu(et, device, case, scale, *, window=0, context_window=0, active_batch=None, max_context=None,
+            workspace=None):
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
     k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
     layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)),
@@ -42,7 +43,7 @@ def run_gpu(et, device, case, scale, *, window=0, context_window=0, active_batch
                        active_batch=active_batch, context_window=context_window)
     q = dev(case["q"])
     out = torch.full_like(q, float("nan"))
-    et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, window, out)
+    et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, window, out, workspace=workspace)
     return out.cpu().numpy(), k_slab.cpu().numpy(), v_slab.cpu().numpy(), layer
 
 
@@ -135,6 +136,19 @@ def test_long_context_is_split(et, device, dtype):
     # a generous bound changes the launch, not the result
     again = run_gpu(et, device, case, scale, max_context=100000)
     compare(again, run_oracle(case, scale))
+
+
+def test_one_workspace_serves_calls_of_any_geometry(et, device):
+    workspace = torch.full((64 << 20,), 255, dtype=torch.uint8, device=device)
+    rng = np.random.default_rng(11)
+    for slots, heads, kv_heads, width, contexts, dtype in (
+            (2, 8, 2, 128, [5000, 777], np.float16), (5, 4, 4, 64, [900, 30, 2000, 1, 64], np.float32),
+            (1, 6, 3, 20, [700], np.float16), (2, 8, 2, 128, [4000, 4100], np.float16),
+            (3, 16, 2, 128, [300, 1200, 40], np.float16)):
+        case = make_case(rng, slots=slots, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                         contexts=contexts, tokens=1, advances=[1] * slots, dtype=dtype)
+        for _ in range(2):
+            compare(run_gpu(et, device, case, 0.1, workspace=workspace), run_oracle(case, 0.1))
 
 
 def test_inactive_slots_are_zero_and_untouched(et, device):
