@@ -36,7 +36,9 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
 # counters' reading for a plain copy of known size. These cannot be collected from inside this
 # script; the runs and their figures are in profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md.
-MEASURED_TRAFFIC = {("q4_k_gemv_14336x4096", 1, "f32"): 33338900}
+MEASURED_TRAFFIC = {("q4_k_gemv_14336x4096", 1, "f32"): 33338900,
+                    # attend kernel; profiles/kv_attend_decode_32slots_ctx2048_f16.md
+                    ("kv_attention_decode", 2048): 271028400}
 
 
 def parse_args():
