@@ -78,6 +78,17 @@ def lib() -> ctypes.CDLL:
         L.et_oracle_quantize_q8.argtypes = [sz, sz, vp, vp, vp, vp]
         L.et_oracle_linear_q8_rows.restype = ci
         L.et_oracle_linear_q8_rows.argtypes = [ci, sz, sz, sz, vp, vp, vp, vp, vp, vp, sz, sz]
+        L.et_oracle_rms_norm.restype = None
+        L.et_oracle_rms_norm.argtypes = [vp, vp, ctypes.c_double, vp, sz, sz]
+        L.et_oracle_rotary.restype = ci
+        L.et_oracle_rotary.argtypes = [vp, vp, sz, ctypes.c_double, ctypes.c_double, ci, vp, sz, sz, sz, sz,
+                                       ctypes.c_char_p, sz]
+        L.et_oracle_silu_mul.restype = None
+        L.et_oracle_silu_mul.argtypes = [vp, vp, vp, sz]
+        L.et_oracle_argmax.restype = ci
+        L.et_oracle_argmax.argtypes = [vp, sz, sz, vp, ctypes.c_char_p, sz]
+        L.et_oracle_gather_rows.restype = ci
+        L.et_oracle_gather_rows.argtypes = [vp, sz, sz, vp, sz, vp, ctypes.c_char_p, sz]
         L.et_oracle_f32_to_fp16.restype = ctypes.c_uint16
         L.et_oracle_f32_to_fp16.argtypes = [ctypes.c_float]
         L.et_oracle_kv_attention.restype = ci
@@ -275,5 +286,62 @@ def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_
                                       batch if active_batch is None else active_batch, query_heads, tokens,
                                       _ptr(q), _ptr(k), _ptr(v), float(scale), context_window, window, _ptr(out), err, 256)
     if rc != 0:
+        raise OracleError(err.value.decode())
+    return out
+
+
+def rms_norm(x: np.ndarray, weight, eps: float) -> np.ndarray:
+    """et_oracle_rms_norm over the last dimension of a float32 array."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().et_oracle_rms_norm(_ptr(x), None if w is None else _ptr(w), float(eps), _ptr(out),
+                             x.size // x.shape[-1], x.shape[-1])
+    return out
+
+
+def rotary(x: np.ndarray, offsets, theta: float, sign: float = 1.0, interleaved: bool = False) -> np.ndarray:
+    """et_oracle_rotary for ``[..., steps, head_dim]``; the batch is the first dimension (1 for rank 2)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    offsets = np.ascontiguousarray(offsets, dtype=np.uint32)
+    batch = 1 if x.ndim == 2 else x.shape[0]
+    steps, head_dim = x.shape[-2], x.shape[-1]
+    rows = x.size // (steps * head_dim) if steps * head_dim else 0
+    out = np.empty_like(x)
+    err = ctypes.create_string_buffer(256)
+    rc = lib().et_oracle_rotary(_ptr(x), _ptr(offsets), offsets.size, float(theta), float(sign),
+                                1 if interleaved else 0, _ptr(out), batch, rows, steps, head_dim, err, 256)
+    if rc != 0:
+        raise OracleError(err.value.decode())
+    return out
+
+
+def silu_mul(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    gate = np.ascontiguousarray(gate, dtype=np.float32)
+    up = np.ascontiguousarray(up, dtype=np.float32)
+    assert gate.shape == up.shape
+    out = np.empty_like(gate)
+    lib().et_oracle_silu_mul(_ptr(gate), _ptr(up), _ptr(out), gate.size)
+    return out
+
+
+def argmax_rows(logits: np.ndarray) -> np.ndarray:
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    rows = logits.size // logits.shape[-1] if logits.shape[-1] else 0
+    out = np.empty(rows, dtype=np.uint32)
+    err = ctypes.create_string_buffer(256)
+    if lib().et_oracle_argmax(_ptr(logits), rows, logits.shape[-1], _ptr(out), err, 256) != 0:
+        raise OracleError(err.value.decode())
+    return out.reshape(logits.shape[:-1])
+
+
+def gather_rows(table: np.ndarray, indexes) -> np.ndarray:
+    table = np.ascontiguousarray(table)
+    indexes = np.ascontiguousarray(indexes, dtype=np.int64)
+    out = np.empty(indexes.shape + table.shape[1:], dtype=table.dtype)
+    err = ctypes.create_string_buffer(256)
+    row_bytes = table.dtype.itemsize * int(np.prod(table.shape[1:], dtype=np.int64))
+    if lib().et_oracle_gather_rows(_ptr(table), table.shape[0], row_bytes, _ptr(indexes), indexes.size,
+                                   _ptr(out), err, 256) != 0:
         raise OracleError(err.value.decode())
     return out
