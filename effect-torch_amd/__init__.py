@@ -33,3 +33,13 @@ from .kv_cache import (  # noqa: F401
     kv_attention_workspace,
     kv_attention_workspace_bytes,
 )
+from .decode_ops import (  # noqa: F401
+    RotaryLayout,
+    gather_rows_into,
+    gather_rows_status_check,
+    greedy_status_check,
+    greedy_tokens,
+    rms_norm_into,
+    rotary_into,
+    silu_mul_into,
+)

@@ -91,6 +91,13 @@ SIGNATURES = {
     "et_hip_kv_attention_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp, _vp]),
     "et_hip_kv_attention_status_check": (ctypes.c_int, [_KV, _u64, _vp]),
     "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
+    "et_hip_rms_norm_into": (ctypes.c_int, [_T, _T, ctypes.c_double, _T, _vp]),
+    "et_hip_rotary_into": (ctypes.c_int, [_T, _vp, _u64, ctypes.c_double, ctypes.c_double, _i32, _T, _vp]),
+    "et_hip_silu_mul_into": (ctypes.c_int, [_T, _T, _T, _vp]),
+    "et_hip_greedy_tokens_into": (ctypes.c_int, [_T, _vp, _vp, _vp]),
+    "et_hip_greedy_status_check": (ctypes.c_int, [_u64, _vp]),
+    "et_hip_gather_rows_into": (ctypes.c_int, [_T, _T, _T, _vp, _vp]),
+    "et_hip_gather_rows_status_check": (ctypes.c_int, [_u64, _u64, _vp]),
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),

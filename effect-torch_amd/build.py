@@ -32,9 +32,11 @@ SOURCES = {
     "quantize_act.hip": ["-ffp-contract=off"],
     "gemm_i8.hip": [],
     "kv_attention.hip": [],
+    "decode_ops.hip": ["-ffp-contract=off"],
     "calibrate.hip": [],
     "quantized.cpp": [],
     "kv_cache.cpp": [],
+    "decode_host.cpp": [],
     "c_api.cpp": [],
 }
 

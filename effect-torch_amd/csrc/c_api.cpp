@@ -11,6 +11,7 @@
 #include "et_codecs.h"
 #include "et_hip.h"
 #include "kernels.h"
+#include "decode_host.h"
 #include "kv_cache.h"
 #include "quantized.h"
 
@@ -318,6 +319,87 @@ int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens, 
             return ET_ERR_INVALID;
         }
         return et::kv::status_check(*layer, tokens, status_host, error);
+    });
+}
+
+int et_hip_rms_norm_into(const et_tensor* x, const et_tensor* weight, double eps, const et_tensor* destination,
+                         void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView xv, wv, dst;
+        if (!TensorView::from_c(x, &xv, error) || (weight != nullptr && !TensorView::from_c(weight, &wv, error)) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "rms_norm: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::rms_norm_into(xv, weight ? &wv : nullptr, eps, dst, stream, error);
+    });
+}
+
+int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t offsets_len, double theta,
+                       double sign, int32_t layout, const et_tensor* destination, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView xv, dst;
+        if (!TensorView::from_c(x, &xv, error) || !TensorView::from_c(destination, &dst, error)) {
+            *error = "rotary: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::rotary_into(xv, offsets, offsets_len, theta, sign, layout, dst, stream, error);
+    });
+}
+
+int et_hip_silu_mul_into(const et_tensor* gate, const et_tensor* up, const et_tensor* destination, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView gv, uv, dst;
+        if (!TensorView::from_c(gate, &gv, error) || !TensorView::from_c(up, &uv, error) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "silu_mul: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::silu_mul_into(gv, uv, dst, stream, error);
+    });
+}
+
+int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* status, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView lv;
+        if (!TensorView::from_c(logits, &lv, error)) {
+            *error = "sample: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::greedy_tokens_into(lv, tokens, status, stream, error);
+    });
+}
+
+int et_hip_greedy_status_check(uint64_t rows, const void* status_host) {
+    return guarded([&](std::string* error) -> int {
+        if (status_host == nullptr && rows != 0) {
+            *error = "sample: status is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::decode::greedy_status_check(rows, status_host, error);
+    });
+}
+
+int et_hip_gather_rows_into(const et_tensor* table, const et_tensor* indexes, const et_tensor* destination,
+                            void* status, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView tv, iv, dst;
+        if (!TensorView::from_c(table, &tv, error) || !TensorView::from_c(indexes, &iv, error) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "index_select: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::gather_rows_into(tv, iv, dst, status, stream, error);
+    });
+}
+
+int et_hip_gather_rows_status_check(uint64_t table_rows, uint64_t count, const void* status_host) {
+    return guarded([&](std::string* error) -> int {
+        if (status_host == nullptr && count != 0) {
+            *error = "index_select: status is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::decode::gather_rows_status_check(table_rows, count, status_host, error);
     });
 }
 

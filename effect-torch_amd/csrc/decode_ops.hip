@@ -1,0 +1,208 @@
+// The small operators on the decode critical path next to the quantized contraction, for
+// gfx950. Each is a plain streaming kernel: the data of a decode step is a few hundred KB, so
+// what matters is one launch per operator and full-width loads.
+//
+//   rms_norm_kernel     rms_norm_forward_into_impl (crates/runtime-cpu/src/composed.rs:1457-1487)
+//   rotary_kernel       rotary_forward_into_impl (composed.rs:2683-2729)
+//   silu_mul_kernel     Tensor.silu (packages/core/src/Tensor.ts:1537-1540) times the up projection
+//   argmax_kernel       sample_logits with temperature 0 (crates/runtime/src/sampling.rs:86-103)
+//   gather_rows_kernel  index_select along dimension 0 (crates/runtime-cpu/src/indexing.rs:152-187)
+//
+// The reference computes the first two in f64 and rounds once; so do these kernels (the rows
+// are short, f64 costs nothing that shows), which keeps them within one f32 rounding of it.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "kernels.h"
+
+namespace et {
+namespace {
+
+__device__ __forceinline__ double wave_sum(double v) {
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset);
+    return v;
+}
+
+// One workgroup of 256 per row.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                       double eps, float* __restrict__ out, uint32_t columns) {
+    __shared__ double partial[4];
+    const float* in = x + static_cast<uint64_t>(blockIdx.x) * columns;
+    float* row = out + static_cast<uint64_t>(blockIdx.x) * columns;
+    double sum = 0.0;
+    for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
+    const double scale = 1.0 / sqrt(mean_square + eps);
+    for (uint32_t i = threadIdx.x; i < columns; i += 256) {
+        const double w = weight != nullptr ? static_cast<double>(weight[i]) : 1.0;
+        row[i] = static_cast<float>(static_cast<double>(in[i]) * scale * w);
+    }
+}
+
+// One thread per (row, step, pair).
+__global__ __launch_bounds__(256) void rotary_kernel(const float* __restrict__ x, const uint32_t* __restrict__ offsets,
+                                                     uint32_t offsets_len, double theta, double sign, int interleaved,
+                                                     float* __restrict__ out, uint32_t rows_per_batch, uint32_t steps,
+                                                     uint32_t head_dim, uint64_t pairs) {
+    const uint64_t item = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= pairs) return;
+    const uint32_t half = head_dim / 2;
+    const uint32_t index = static_cast<uint32_t>(item % half);
+    const uint64_t row_step = item / half;
+    const uint32_t step = static_cast<uint32_t>(row_step % steps);
+    const uint64_t row = row_step / steps;
+    const uint32_t offset = offsets_len == 1 ? offsets[0] : offsets[row / rows_per_batch];
+    const double angle = sign * static_cast<double>(static_cast<uint64_t>(offset) + step) *
+                         pow(theta, -2.0 * static_cast<double>(index) / static_cast<double>(head_dim));
+    double s, c;
+    sincos(angle, &s, &c);
+    const uint64_t base = row_step * head_dim;
+    const uint64_t first = interleaved ? base + 2 * index : base + index;
+    const uint64_t second = interleaved ? base + 2 * index + 1 : base + half + index;
+    const double a = x[first], b = x[second];
+    out[first] = static_cast<float>(a * c - b * s);
+    out[second] = static_cast<float>(b * c + a * s);
+}
+
+__device__ __forceinline__ float silu_mul_one(float gate, float up) {
+    // Tensor.sigmoid: tanh(x / 2) / 2 + 1 / 2, every step rounded to f32 (Tensor.ts:1240-1245)
+    const float sigmoid = tanhf(gate * 0.5f) * 0.5f + 0.5f;
+    return (gate * sigmoid) * up;
+}
+
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       float* __restrict__ out, uint64_t count, int vectorised) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (vectorised) {
+        if (4 * i >= count) return;
+        const float4 g = reinterpret_cast<const float4*>(gate)[i], u = reinterpret_cast<const float4*>(up)[i];
+        reinterpret_cast<float4*>(out)[i] = make_float4(silu_mul_one(g.x, u.x), silu_mul_one(g.y, u.y),
+                                                        silu_mul_one(g.z, u.z), silu_mul_one(g.w, u.w));
+    } else if (i < count) {
+        out[i] = silu_mul_one(gate[i], up[i]);
+    }
+}
+
+// One workgroup of 256 per row of logits: the largest value, the lowest token among equals, and
+// the first token that is not finite (status[row] = token + 1, 0 = none).
+__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, uint32_t columns,
+                                                     uint32_t* __restrict__ out, uint32_t* __restrict__ status) {
+    __shared__ float best_value[4];
+    __shared__ uint32_t best_token[4], bad_token[4];
+    const float* row = logits + static_cast<uint64_t>(blockIdx.x) * columns;
+    float best = -INFINITY;
+    uint32_t token = 0xffffffffu, bad = 0xffffffffu;
+    for (uint32_t i = threadIdx.x; i < columns; i += 256) {
+        const float value = row[i];
+        if (!isfinite(value)) bad = min(bad, i);
+        if (value > best) {
+            best = value;
+            token = i;
+        }
+    }
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        const float other = __shfl_xor(best, offset);
+        const uint32_t other_token = __shfl_xor(token, offset);
+        if (other > best || (other == best && other_token < token)) {
+            best = other;
+            token = other_token;
+        }
+        bad = min(bad, __shfl_xor(bad, offset));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        best_value[threadIdx.x >> 6] = best;
+        best_token[threadIdx.x >> 6] = token;
+        bad_token[threadIdx.x >> 6] = bad;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) {
+            if (best_value[w] > best || (best_value[w] == best && best_token[w] < token)) {
+                best = best_value[w];
+                token = best_token[w];
+            }
+            bad = min(bad, bad_token[w]);
+        }
+        // a row of -inf only (not finite) never selects a token: report token 0 as the CPU loop does
+        out[blockIdx.x] = token == 0xffffffffu ? 0u : token;
+        status[blockIdx.x] = bad == 0xffffffffu ? 0u : bad + 1;
+    }
+}
+
+// One workgroup per gathered row; rows are copied as bytes. status[p] = 0, or the offending
+// index + 1 (saturated) when it lies outside the table, in which case the row is left alone.
+template <typename Word>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const Word* __restrict__ table, uint64_t table_rows,
+                                                          uint64_t row_words, const void* __restrict__ indexes,
+                                                          int index_is_i64, Word* __restrict__ out,
+                                                          unsigned long long* __restrict__ status) {
+    const uint64_t p = blockIdx.x;
+    const long long id = index_is_i64 ? static_cast<const long long*>(indexes)[p]
+                                      : static_cast<long long>(static_cast<const uint32_t*>(indexes)[p]);
+    const bool inside = id >= 0 && static_cast<uint64_t>(id) < table_rows;
+    if (threadIdx.x == 0) status[p] = inside ? 0ull : (1ull << 63) | (static_cast<unsigned long long>(id) & ~(1ull << 63));
+    if (!inside) return;
+    const Word* source = table + static_cast<uint64_t>(id) * row_words;
+    Word* target = out + p * row_words;
+    for (uint64_t i = threadIdx.x; i < row_words; i += 256) target[i] = source[i];
+}
+
+}  // namespace
+
+hipError_t rms_norm(const float* x, const float* weight, double eps, float* out, uint64_t rows, uint64_t columns,
+                    hipStream_t stream) {
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps, out,
+                       static_cast<uint32_t>(columns));
+    return hipGetLastError();
+}
+
+hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
+                  int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,
+                  hipStream_t stream) {
+    const uint64_t pairs = rows * steps * (head_dim / 2);
+    hipLaunchKernelGGL(rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0, stream, x, offsets,
+                       offsets_len, theta, sign, interleaved, out, static_cast<uint32_t>(rows / batch),
+                       static_cast<uint32_t>(steps), static_cast<uint32_t>(head_dim), pairs);
+    return hipGetLastError();
+}
+
+hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t count, hipStream_t stream) {
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const int vectorised = count % 4 == 0 && aligned(gate) && aligned(up) && aligned(out);
+    const uint64_t items = vectorised ? count / 4 : count;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream, gate, up,
+                       out, count, vectorised);
+    return hipGetLastError();
+}
+
+hipError_t argmax_rows(const float* logits, uint64_t rows, uint64_t columns, uint32_t* out, uint32_t* status,
+                       hipStream_t stream) {
+    hipLaunchKernelGGL(argmax_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, logits,
+                       static_cast<uint32_t>(columns), out, status);
+    return hipGetLastError();
+}
+
+hipError_t gather_rows(const void* table, uint64_t table_rows, uint64_t row_bytes, const void* indexes,
+                       int index_is_i64, uint64_t count, void* out, void* status, hipStream_t stream) {
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    auto* words = static_cast<unsigned long long*>(status);
+    if (row_bytes % 16 == 0 && aligned(table) && aligned(out))
+        hipLaunchKernelGGL(gather_rows_kernel<uint4>, dim3(static_cast<uint32_t>(count)), dim3(256), 0, stream,
+                           static_cast<const uint4*>(table), table_rows, row_bytes / 16, indexes, index_is_i64,
+                           static_cast<uint4*>(out), words);
+    else if (row_bytes % 2 == 0 && reinterpret_cast<uintptr_t>(table) % 2 == 0 && reinterpret_cast<uintptr_t>(out) % 2 == 0)
+        hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, dim3(static_cast<uint32_t>(count)), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(table), table_rows, row_bytes / 2, indexes, index_is_i64,
+                           static_cast<uint16_t*>(out), words);
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<uint8_t>, dim3(static_cast<uint32_t>(count)), dim3(256), 0, stream,
+                           static_cast<const uint8_t*>(table), table_rows, row_bytes, indexes, index_is_i64,
+                           static_cast<uint8_t*>(out), words);
+    return hipGetLastError();
+}
+
+}  // namespace et

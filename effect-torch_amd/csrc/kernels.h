@@ -117,6 +117,22 @@ KvLaunchShape kv_attention_shape(const KvAttention& p);
 // Attends, appends the new rows, merges; `workspace` holds kv_attention_shape(p).workspace_bytes.
 hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream);
 
+// ---- decode_ops.hip: the small operators next to the contraction in a decode step ----
+// Dense f32 rows; weight may be null. rows, columns < 2^32.
+hipError_t rms_norm(const float* x, const float* weight, double eps, float* out, uint64_t rows, uint64_t columns,
+                    hipStream_t stream);
+// x, out: [rows, steps, head_dim]; offsets: 1 or `batch` device words; rows % batch == 0.
+hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
+                  int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,
+                  hipStream_t stream);
+hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t count, hipStream_t stream);
+// out[row] = greedy token; status[row] = 0, or 1 + the first token whose logit is not finite.
+hipError_t argmax_rows(const float* logits, uint64_t rows, uint64_t columns, uint32_t* out, uint32_t* status,
+                       hipStream_t stream);
+// out[p, :] = table[indexes[p], :] as bytes; status[p] (8 bytes each) = 0, or bit 63 | the index.
+hipError_t gather_rows(const void* table, uint64_t table_rows, uint64_t row_bytes, const void* indexes,
+                       int index_is_i64, uint64_t count, void* out, void* status, hipStream_t stream);
+
 // ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
 // sink must hold 4 * `workgroups` words; bytes < 2^36.
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,

@@ -259,6 +259,53 @@ int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
 const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_heads,
                                        uint64_t tokens);
 
+/* ---- the small operators of a decode step ---------------------------------
+ *
+ * RMS norm, rotary embedding, SiLU(gate) * up, greedy token selection and the
+ * dense embedding lookup sit between the contractions of every decode step.
+ * All take contiguous tensors and enqueue one kernel on `stream`. */
+
+/* = rms_norm_forward_into (crates/runtime-cpu/src/composed.rs:1491-1533) for
+ * f32: out = x * (1 / sqrt(mean(x^2) + eps)) * weight over the last dimension,
+ * in f64, rounded once. weight: NULL or [columns]. */
+int et_hip_rms_norm_into(const et_tensor* x, const et_tensor* weight, double eps,
+                         const et_tensor* destination, void* stream);
+
+/* RotaryLayout (the pairs one angle rotates): (i, i + d/2) or (2i, 2i + 1). */
+typedef enum { ET_ROTARY_HALF_SPLIT = 0, ET_ROTARY_INTERLEAVED_PAIRS = 1 } et_rotary_layout;
+/* = rotary_forward_into (composed.rs:2735-2772) for f32 [.., steps, head_dim]:
+ * position = offset + step, angle = sign * position * theta^(-2i / head_dim),
+ * in f64, rounded once. `offsets` is a DEVICE array of 1 or batch (= shape[0], 1
+ * for rank 2) u32 entries - in a decode step, the kv cursors. */
+int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t offsets_len,
+                       double theta, double sign, int32_t layout, const et_tensor* destination,
+                       void* stream);
+
+/* out = silu(gate) * up with silu(x) = x * (tanh(x / 2) / 2 + 1 / 2), f32, every
+ * step rounded (Tensor.silu over Tensor.sigmoid, packages/core/src/Tensor.ts:1537-1540,
+ * :1240-1245; the reference builds it from four elementwise nodes). */
+int et_hip_silu_mul_into(const et_tensor* gate, const et_tensor* up, const et_tensor* destination,
+                         void* stream);
+
+/* = sample_logits with temperature 0 (crates/runtime/src/sampling.rs:86-103) for
+ * every row of f32 logits [.., vocabulary]: the largest logit, the lowest token
+ * among equals. tokens: device u32 [rows]. A logit that is not finite cannot
+ * fail the call; `status` (device, 4 bytes per row, written by the call) records
+ * it for et_hip_greedy_status_check ("sample: logit {token} is not finite"). */
+int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* status, void* stream);
+int et_hip_greedy_status_check(uint64_t rows, const void* status_host);
+
+/* = index_select_into along dimension 0 (crates/runtime-cpu/src/indexing.rs:396-430)
+ * of a [rows, width] table of any element type: destination[p, :] =
+ * table[indexes[p], :] (the dense embedding lookup; f16 tables stay f16).
+ * indexes: u32 or i64, any shape, contiguous; destination [count, width].
+ * `status`: device, 8 bytes per index, written by the call; an index outside
+ * the table leaves its row alone and et_hip_gather_rows_status_check returns
+ * "index_select: index {id} is out of bounds for extent {rows}". */
+int et_hip_gather_rows_into(const et_tensor* table, const et_tensor* indexes,
+                            const et_tensor* destination, void* status, void* stream);
+int et_hip_gather_rows_status_check(uint64_t table_rows, uint64_t count, const void* status_host);
+
 /* ---- int8 activation quantiser (stage 1 of ET_ACT_INT8) ------------------- */
 
 /* The activation quantiser on its own, exposed so that tests can check the

@@ -227,3 +227,31 @@ def test_kv_attention_launch_shapes_and_status_wording(et):
     assert message((1 << 32) | 0) == (2, "kv attention: advance 0 out of range for chunk length 7")
     assert message((2 << 32) | 70000) == (2, "kv attention: live context 70000 exceeds pool capacity 65536")
     assert message((3 << 32) | 41, slot=30) == (2, "kv attention: block table of slot 30 does not cover 41 tokens")
+
+
+def test_decode_operator_validation(et):
+    import torch
+    x = torch.zeros(2, 8)
+    with pytest.raises(et.QuantizedError, match="rms_norm: input must have rank at least 1"):
+        et.rms_norm_into(torch.zeros(()), None, 1e-5, torch.zeros(()), stream=0)
+    with pytest.raises(et.QuantizedError, match="rms_norm: weight must match the last dimension and dtype"):
+        et.rms_norm_into(x, torch.zeros(2, 4), 1e-5, torch.zeros(2, 8), stream=0)
+    with pytest.raises(et.QuantizedError, match="rms_norm: zero-sized dimensions are unsupported"):
+        et.rms_norm_into(torch.zeros(2, 0), None, 1e-5, torch.zeros(2, 0), stream=0)
+    offsets = torch.zeros(3, dtype=torch.int32)
+    with pytest.raises(et.QuantizedError, match="rotary: expected a float rank >= 2 tensor with even head dimension"):
+        et.rotary_into(torch.zeros(2, 7), offsets[:1], 1e4, 1.0, et.RotaryLayout.HALF_SPLIT, torch.zeros(2, 7), stream=0)
+    with pytest.raises(et.QuantizedError, match="rotary embedding: 3 offsets for batch 2"):
+        et.rotary_into(torch.zeros(2, 4, 1, 8), offsets, 1e4, 1.0, et.RotaryLayout.HALF_SPLIT,
+                       torch.zeros(2, 4, 1, 8), stream=0)
+    with pytest.raises(et.QuantizedError, match="silu_mul: gate, up and the destination must have one shape"):
+        et.silu_mul_into(x, torch.zeros(2, 4), torch.zeros(2, 8), stream=0)
+    with pytest.raises(et.QuantizedError, match="sample: logits must be non-empty"):
+        et.greedy_tokens(torch.zeros(2, 0), stream=0)
+    with pytest.raises(et.QuantizedError, match="sample: vocabulary 1048577 exceeds limit 1048576"):
+        et.greedy_tokens(torch.zeros(1, 1048577), stream=0)
+    table = torch.zeros(10, 4, dtype=torch.float16)
+    with pytest.raises(et.QuantizedError, match="index_select destination shape mismatch at dimension 0: expected 3, got 2"):
+        et.gather_rows_into(table, torch.zeros(3, dtype=torch.int64), torch.zeros(2, 4, dtype=torch.float16), stream=0)
+    with pytest.raises(et.QuantizedError, match="index_select: indexes must be u32 or i64"):
+        et.gather_rows_into(table, torch.zeros(3, dtype=torch.float32), torch.zeros(3, 4, dtype=torch.float16), stream=0)
