@@ -266,6 +266,128 @@ def kv_decode(args, et):
     print(json.dumps(result))
 
 
+DECODE_OPS = ("rms_norm_decode", "rotary_decode", "silu_mul_decode", "greedy_decode", "embedding_gather_decode")
+
+
+def decode_op(args, et):
+    """The small operators of one Llama-3-8B-shaped decode step for 32 slots, one launch per step:
+    RMS norm of [32, 4096], rotary of q [32, 32, 1, 128] at the slots' cursors, SiLU(gate) * up of
+    [32, 14336], greedy tokens of [32, 128256] logits, 32 rows of the f16 [128256, 4096] embedding
+    table. Inputs rotate over enough copies to stay out of the caches."""
+    import numpy as np
+    import torch
+    import oracle
+
+    device = torch.device("cuda:0")
+    rng = np.random.default_rng(11)
+    name = args.workload
+    slots = 32
+
+    def copies_for(nbytes):
+        return 1 if args.hot else max(2, -(-ROTATE_BYTES // max(nbytes, 1)))
+
+    if name == "rms_norm_decode":
+        x = rng.standard_normal((slots, 4096)).astype(np.float32)
+        w = rng.standard_normal(4096).astype(np.float32)
+        n = min(copies_for(x.nbytes), 64)
+        xs = [torch.from_numpy(np.roll(x, i, axis=1)).to(device) for i in range(n)]
+        wd, out = torch.from_numpy(w).to(device), torch.empty(slots, 4096, device=device)
+        step = lambda i: et.rms_norm_into(xs[i % n], wd, 1e-5, out)  # noqa: E731
+        check = lambda: np.abs(out.cpu().numpy() - oracle.rms_norm(np.roll(x, 0, axis=1), w, 1e-5)).max() <= 1e-6  # noqa: E731
+        algorithmic = 2 * x.nbytes + w.nbytes
+        cpu = lambda: oracle.rms_norm(x, w, 1e-5)  # noqa: E731
+        shape = "x [32, 4096] f32, weight [4096]"
+    elif name == "rotary_decode":
+        x = rng.standard_normal((slots, 32, 1, 128)).astype(np.float32)
+        cursors = rng.integers(0, 8192, slots).astype(np.int32)
+        n = min(copies_for(x.nbytes), 64)
+        xs = [torch.from_numpy(np.roll(x, i, axis=3)).to(device) for i in range(n)]
+        od, out = torch.from_numpy(cursors).to(device), torch.empty(x.shape, device=device)
+        step = lambda i: et.rotary_into(xs[i % n], od, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, out)  # noqa: E731
+        check = lambda: np.abs(out.cpu().numpy() - oracle.rotary(x, cursors, 500000.0)).max() <= 1e-6  # noqa: E731
+        algorithmic = 2 * x.nbytes + cursors.nbytes
+        cpu = lambda: oracle.rotary(x, cursors, 500000.0)  # noqa: E731
+        shape = "q [32, 32, 1, 128] f32, theta 5e5, half-split pairs, per-slot offsets"
+    elif name == "silu_mul_decode":
+        gate = (rng.standard_normal((slots, 14336)) * 3).astype(np.float32)
+        up = rng.standard_normal((slots, 14336)).astype(np.float32)
+        n = min(copies_for(2 * gate.nbytes), 64)
+        gs = [torch.from_numpy(np.roll(gate, i, axis=1)).to(device) for i in range(n)]
+        us = [torch.from_numpy(np.roll(up, i, axis=1)).to(device) for i in range(n)]
+        out = torch.empty(gate.shape, device=device)
+        step = lambda i: et.silu_mul_into(gs[i % n], us[i % n], out)  # noqa: E731
+        check = lambda: np.allclose(out.cpu().numpy(), oracle.silu_mul(gate, up), rtol=1e-6, atol=1e-6)  # noqa: E731
+        algorithmic = 3 * gate.nbytes
+        cpu = lambda: oracle.silu_mul(gate, up)  # noqa: E731
+        shape = "gate, up [32, 14336] f32"
+    elif name == "greedy_decode":
+        logits = rng.standard_normal((slots, 128256)).astype(np.float32)
+        n = min(copies_for(logits.nbytes), 48)
+        ls = [torch.from_numpy(np.roll(logits, 1000 * i, axis=1)).to(device) for i in range(n)]
+        tokens = torch.empty(slots, dtype=torch.int32, device=device)
+        status = torch.empty(4 * slots, dtype=torch.uint8, device=device)
+        from effect_torch_amd import _native
+        from effect_torch_amd.quantized import _Desc
+        descs = [_Desc(t) for t in ls]
+        scratch = torch.empty(et.greedy_workspace_bytes(slots, 128256), dtype=torch.uint8, device=device)
+
+        def step(i):
+            code = _native.lib().et_hip_greedy_tokens_into(descs[i % n].ref, tokens.data_ptr(), scratch.data_ptr(),
+                                                           scratch.numel(), status.data_ptr(),
+                                                           torch.cuda.current_stream().cuda_stream)
+            assert code == 0, _native.last_error()
+        check = lambda: np.array_equal(tokens.cpu().numpy(), oracle.argmax_rows(logits).astype(np.int32))  # noqa: E731
+        algorithmic = logits.nbytes + 8 * slots
+        cpu = lambda: oracle.argmax_rows(logits)  # noqa: E731
+        shape = "logits [32, 128256] f32"
+    else:
+        table = rng.standard_normal((128256, 4096)).astype(np.float16)
+        td = torch.from_numpy(table).to(device)
+        n = 64
+        ids_host = [rng.integers(0, 128256, slots) for _ in range(n)]
+        ids = [torch.from_numpy(a.astype(np.int32)).to(device).view(torch.uint32) for a in ids_host]
+        out = torch.empty((slots, 4096), dtype=torch.float16, device=device)
+        keep = []
+
+        def step(i):
+            keep.append(et.gather_rows_into(td, ids[i % n], out, synchronize=False))
+            if len(keep) > 4:
+                keep.pop(0)
+        check = lambda: np.array_equal(out.cpu().numpy().view(np.uint16),  # noqa: E731
+                                       oracle.gather_rows(table, ids_host[0]).view(np.uint16))
+        algorithmic = 2 * slots * 4096 * 2 + 4 * slots + 8 * slots
+        cpu = lambda: oracle.gather_rows(table, ids_host[0])  # noqa: E731
+        shape = "32 rows of the f16 [128256, 4096] table"
+
+    step(0)
+    torch.cuda.synchronize()
+    assert check(), f"parity gate failed for {name}"
+    ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    seconds = ms * 1e-3
+    gbs = algorithmic / seconds / 1e9
+    result = {
+        "metric": f"{name} GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16" if name == "embedding_gather_decode" else "f32", "data": "synthetic",
+        "config": {"workload": f"{name}: {shape}", "inputs": "hot" if args.hot else f"rotating over {n} copies",
+                   "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues",
+                   "host_wall_ms": round(wall * 1e3, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
+    }
+    if not args.no_cpu:
+        calls, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 3.0) or calls == 0:
+            cpu()
+            calls += 1
+        elapsed = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": round(algorithmic / (elapsed / calls) / 1e9, 4), "unit": "GB/s", "cores": 1,
+                                  "kind": "port", "sample": f"{calls} full call(s) of the same workload, "
+                                  f"{elapsed:.1f} s of CPU work ({elapsed / calls * 1e6:.0f} us per call)"}
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -282,12 +404,15 @@ def main():
 
     if args.workload in ("calibrate_read", "calibrate_copy"):
         return calibrate(args, et)
+    if args.workload in DECODE_OPS:
+        assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
+        return decode_op(args, et)
     if args.workload == "kv_attention_decode":
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return kv_decode(args, et)
     if args.workload not in synth.CONFIGS:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
-                 "or calibrate_read / calibrate_copy / kv_attention_decode")
+                 "or calibrate_read / calibrate_copy / kv_attention_decode / " + " / ".join(DECODE_OPS))
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")

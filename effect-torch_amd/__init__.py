@@ -39,6 +39,7 @@ from .decode_ops import (  # noqa: F401
     gather_rows_status_check,
     greedy_status_check,
     greedy_tokens,
+    greedy_workspace_bytes,
     rms_norm_into,
     rotary_into,
     silu_mul_into,

@@ -359,14 +359,19 @@ int et_hip_silu_mul_into(const et_tensor* gate, const et_tensor* up, const et_te
     });
 }
 
-int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* status, void* stream) {
+uint64_t et_hip_greedy_workspace_bytes(uint64_t rows, uint64_t vocabulary) {
+    return et::decode::greedy_workspace_bytes(rows, vocabulary);
+}
+
+int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* workspace, uint64_t workspace_bytes,
+                              void* status, void* stream) {
     return guarded([&](std::string* error) -> int {
         TensorView lv;
         if (!TensorView::from_c(logits, &lv, error)) {
             *error = "sample: " + *error;
             return ET_ERR_INVALID;
         }
-        return et::decode::greedy_tokens_into(lv, tokens, status, stream, error);
+        return et::decode::greedy_tokens_into(lv, tokens, workspace, workspace_bytes, status, stream, error);
     });
 }
 

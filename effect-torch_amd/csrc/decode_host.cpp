@@ -104,7 +104,10 @@ int silu_mul_into(const TensorView& gate, const TensorView& up, const TensorView
 }
 
 // validate (crates/runtime/src/sampling.rs:42-57) + the greedy branch (:86-103)
-int greedy_tokens_into(const TensorView& logits, uint32_t* tokens, void* status, void* stream, std::string* error) {
+uint64_t greedy_workspace_bytes(uint64_t rows, uint64_t vocabulary) { return argmax_workspace_bytes(rows, vocabulary); }
+
+int greedy_tokens_into(const TensorView& logits, uint32_t* tokens, void* workspace, uint64_t workspace_bytes,
+                       void* status, void* stream, std::string* error) {
     if (logits.dtype != ET_DTYPE_F32 || logits.shape.empty())
         return fail(error, ET_ERR_UNSUPPORTED, "sample: logits must be an f32 tensor of rank at least 1");
     const uint64_t columns = logits.shape.back();
@@ -115,9 +118,13 @@ int greedy_tokens_into(const TensorView& logits, uint32_t* tokens, void* status,
     const uint64_t rows = numel(logits) / columns;
     if (rows == 0) return ET_OK;
     if (rows > 0x7fffffffull) return fail(error, ET_ERR_UNSUPPORTED, "sample: too many rows");
-    if (logits.data == nullptr || tokens == nullptr || status == nullptr)
+    const uint64_t need = argmax_workspace_bytes(rows, columns);
+    if (workspace_bytes < need)
+        return fail(error, ET_ERR_EXECUTION, "sample: workspace of " + std::to_string(workspace_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(need) + " required");
+    if (logits.data == nullptr || tokens == nullptr || status == nullptr || workspace == nullptr)
         return fail(error, ET_ERR_INVALID, "sample: NULL device pointer");
-    return launched(argmax_rows(f32_data(logits), rows, columns, tokens, static_cast<uint32_t*>(status),
+    return launched(argmax_rows(f32_data(logits), rows, columns, tokens, static_cast<uint32_t*>(status), workspace,
                                 static_cast<hipStream_t>(stream)),
                     "sample", error);
 }

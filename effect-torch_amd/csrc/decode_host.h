@@ -20,7 +20,9 @@ int rotary_into(const TensorView& x, const uint32_t* offsets, uint64_t offsets_l
                 int32_t layout, const TensorView& destination, void* stream, std::string* error);
 int silu_mul_into(const TensorView& gate, const TensorView& up, const TensorView& destination, void* stream,
                   std::string* error);
-int greedy_tokens_into(const TensorView& logits, uint32_t* tokens, void* status, void* stream, std::string* error);
+uint64_t greedy_workspace_bytes(uint64_t rows, uint64_t vocabulary);
+int greedy_tokens_into(const TensorView& logits, uint32_t* tokens, void* workspace, uint64_t workspace_bytes,
+                       void* status, void* stream, std::string* error);
 int greedy_status_check(uint64_t rows, const void* status_host, std::string* error);
 int gather_rows_into(const TensorView& table, const TensorView& indexes, const TensorView& destination,
                      void* status, void* stream, std::string* error);

@@ -19,27 +19,72 @@
 namespace et {
 namespace {
 
+constexpr uint32_t kArgmaxChunk = 4096;  // logits per workgroup of the first stage
+
 __device__ __forceinline__ double wave_sum(double v) {
     for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset);
     return v;
 }
 
-// One workgroup of 256 per row.
+// One workgroup of 256 per row. VEC: the row is read as float4 (columns % 4 == 0, 16-byte aligned
+// rows); the first four vectors of a thread stay in registers for the second pass.
+template <bool VEC>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
                                                        double eps, float* __restrict__ out, uint32_t columns) {
     __shared__ double partial[4];
     const float* in = x + static_cast<uint64_t>(blockIdx.x) * columns;
     float* row = out + static_cast<uint64_t>(blockIdx.x) * columns;
+    constexpr int kHeld = 4;
+    float4 held[kHeld];
     double sum = 0.0;
-    for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
+    if constexpr (VEC) {
+        const uint32_t vectors = columns / 4;
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const uint32_t i = threadIdx.x + 256 * j;
+            held[j] = i < vectors ? reinterpret_cast<const float4*>(in)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const float4 v = held[j];
+            sum += (static_cast<double>(v.x) * v.x + static_cast<double>(v.y) * v.y) +
+                   (static_cast<double>(v.z) * v.z + static_cast<double>(v.w) * v.w);
+        }
+        for (uint32_t i = threadIdx.x + 256 * kHeld; i < vectors; i += 256) {
+            const float4 v = reinterpret_cast<const float4*>(in)[i];
+            sum += (static_cast<double>(v.x) * v.x + static_cast<double>(v.y) * v.y) +
+                   (static_cast<double>(v.z) * v.z + static_cast<double>(v.w) * v.w);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
+    }
     sum = wave_sum(sum);
     if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
     __syncthreads();
     const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
     const double scale = 1.0 / sqrt(mean_square + eps);
-    for (uint32_t i = threadIdx.x; i < columns; i += 256) {
-        const double w = weight != nullptr ? static_cast<double>(weight[i]) : 1.0;
-        row[i] = static_cast<float>(static_cast<double>(in[i]) * scale * w);
+    const auto one = [&](float value, float w) {
+        return static_cast<float>(static_cast<double>(value) * scale * static_cast<double>(w));
+    };
+    if constexpr (VEC) {
+        const uint32_t vectors = columns / 4;
+        const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
+#pragma unroll
+        for (int j = 0; j < kHeld; j++) {
+            const uint32_t i = threadIdx.x + 256 * j;
+            if (i < vectors) {
+                const float4 w = weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones;
+                const float4 v = held[j];
+                reinterpret_cast<float4*>(row)[i] = make_float4(one(v.x, w.x), one(v.y, w.y), one(v.z, w.z), one(v.w, w.w));
+            }
+        }
+        for (uint32_t i = threadIdx.x + 256 * kHeld; i < vectors; i += 256) {
+            const float4 w = weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones;
+            const float4 v = reinterpret_cast<const float4*>(in)[i];
+            reinterpret_cast<float4*>(row)[i] = make_float4(one(v.x, w.x), one(v.y, w.y), one(v.z, w.z), one(v.w, w.w));
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < columns; i += 256) row[i] = one(in[i], weight != nullptr ? weight[i] : 1.f);
     }
 }
 
@@ -87,32 +132,64 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     }
 }
 
-// One workgroup of 256 per row of logits: the largest value, the lowest token among equals, and
-// the first token that is not finite (status[row] = token + 1, 0 = none).
-__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, uint32_t columns,
-                                                     uint32_t* __restrict__ out, uint32_t* __restrict__ status) {
+// Greedy selection in two launches. Stage 1: one workgroup of 256 per (row, chunk of kArgmaxChunk
+// logits) writes the chunk's largest value, its lowest token and the first token that is not
+// finite. Stage 2: one wave per row combines the chunks (status[row] = that token + 1, 0 = none).
+struct ArgmaxPartial {
+    float value;
+    uint32_t token, bad;
+};
+
+__device__ __forceinline__ void argmax_merge(float& best, uint32_t& token, uint32_t& bad, float other,
+                                             uint32_t other_token, uint32_t other_bad) {
+    if (other > best || (other == best && other_token < token)) {
+        best = other;
+        token = other_token;
+    }
+    bad = min(bad, other_bad);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, uint32_t columns,
+                                                            uint32_t chunks, ArgmaxPartial* __restrict__ partials) {
     __shared__ float best_value[4];
     __shared__ uint32_t best_token[4], bad_token[4];
-    const float* row = logits + static_cast<uint64_t>(blockIdx.x) * columns;
+    const uint32_t chunk = blockIdx.x % chunks, row_index = blockIdx.x / chunks;
+    const float* row = logits + static_cast<uint64_t>(row_index) * columns;
+    const uint32_t begin = chunk * kArgmaxChunk, end = min(begin + kArgmaxChunk, columns);
     float best = -INFINITY;
     uint32_t token = 0xffffffffu, bad = 0xffffffffu;
-    for (uint32_t i = threadIdx.x; i < columns; i += 256) {
-        const float value = row[i];
+    const auto take = [&](float value, uint32_t i) {
         if (!isfinite(value)) bad = min(bad, i);
         if (value > best) {
             best = value;
             token = i;
         }
-    }
-    for (int offset = 32; offset > 0; offset >>= 1) {
-        const float other = __shfl_xor(best, offset);
-        const uint32_t other_token = __shfl_xor(token, offset);
-        if (other > best || (other == best && other_token < token)) {
-            best = other;
-            token = other_token;
+    };
+    if constexpr (VEC) {
+        // rows are 16-byte aligned and columns % 4 == 0: four loads of four logits in flight per thread
+        constexpr int kLoads = kArgmaxChunk / (4 * 256);
+        float4 v[kLoads];
+#pragma unroll
+        for (int j = 0; j < kLoads; j++) {
+            const uint32_t i = begin + 4 * (threadIdx.x + 256 * j);
+            v[j] = i < end ? *reinterpret_cast<const float4*>(row + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
         }
-        bad = min(bad, __shfl_xor(bad, offset));
+#pragma unroll
+        for (int j = 0; j < kLoads; j++) {
+            const uint32_t i = begin + 4 * (threadIdx.x + 256 * j);
+            if (i < end) {
+                take(v[j].x, i);
+                take(v[j].y, i + 1);
+                take(v[j].z, i + 2);
+                take(v[j].w, i + 3);
+            }
+        }
+    } else {
+        for (uint32_t i = begin + threadIdx.x; i < end; i += 256) take(row[i], i);
     }
+    for (int offset = 32; offset > 0; offset >>= 1)
+        argmax_merge(best, token, bad, __shfl_xor(best, offset), __shfl_xor(token, offset), __shfl_xor(bad, offset));
     if ((threadIdx.x & 63) == 0) {
         best_value[threadIdx.x >> 6] = best;
         best_token[threadIdx.x >> 6] = token;
@@ -120,14 +197,21 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; w++) {
-            if (best_value[w] > best || (best_value[w] == best && best_token[w] < token)) {
-                best = best_value[w];
-                token = best_token[w];
-            }
-            bad = min(bad, bad_token[w]);
-        }
-        // a row of -inf only (not finite) never selects a token: report token 0 as the CPU loop does
+        for (int w = 1; w < 4; w++) argmax_merge(best, token, bad, best_value[w], best_token[w], bad_token[w]);
+        partials[blockIdx.x] = ArgmaxPartial{best, token, bad};
+    }
+}
+
+__global__ __launch_bounds__(64) void argmax_rows_kernel(const ArgmaxPartial* __restrict__ partials, uint32_t chunks,
+                                                         uint32_t* __restrict__ out, uint32_t* __restrict__ status) {
+    const ArgmaxPartial* row = partials + static_cast<uint64_t>(blockIdx.x) * chunks;
+    float best = -INFINITY;
+    uint32_t token = 0xffffffffu, bad = 0xffffffffu;
+    for (uint32_t i = threadIdx.x; i < chunks; i += 64) argmax_merge(best, token, bad, row[i].value, row[i].token, row[i].bad);
+    for (int offset = 32; offset > 0; offset >>= 1)
+        argmax_merge(best, token, bad, __shfl_xor(best, offset), __shfl_xor(token, offset), __shfl_xor(bad, offset));
+    if (threadIdx.x == 0) {
+        // a row without any finite logit above -inf selects nothing; the status reports it
         out[blockIdx.x] = token == 0xffffffffu ? 0u : token;
         status[blockIdx.x] = bad == 0xffffffffu ? 0u : bad + 1;
     }
@@ -155,8 +239,13 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const Word* __restrict
 
 hipError_t rms_norm(const float* x, const float* weight, double eps, float* out, uint64_t rows, uint64_t columns,
                     hipStream_t stream) {
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps, out,
-                       static_cast<uint32_t>(columns));
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (columns % 4 == 0 && aligned(x) && aligned(out) && (weight == nullptr || aligned(weight)))
+        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps,
+                           out, static_cast<uint32_t>(columns));
+    else
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps,
+                           out, static_cast<uint32_t>(columns));
     return hipGetLastError();
 }
 
@@ -179,10 +268,24 @@ hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t cou
     return hipGetLastError();
 }
 
+uint64_t argmax_workspace_bytes(uint64_t rows, uint64_t columns) {
+    return rows * ((columns + kArgmaxChunk - 1) / kArgmaxChunk) * sizeof(ArgmaxPartial);
+}
+
 hipError_t argmax_rows(const float* logits, uint64_t rows, uint64_t columns, uint32_t* out, uint32_t* status,
-                       hipStream_t stream) {
-    hipLaunchKernelGGL(argmax_kernel, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, logits,
-                       static_cast<uint32_t>(columns), out, status);
+                       void* workspace, hipStream_t stream) {
+    const uint32_t chunks = static_cast<uint32_t>((columns + kArgmaxChunk - 1) / kArgmaxChunk);
+    auto* partials = static_cast<ArgmaxPartial*>(workspace);
+    if (columns % 4 == 0 && reinterpret_cast<uintptr_t>(logits) % 16 == 0)
+        hipLaunchKernelGGL(argmax_chunks_kernel<true>, dim3(static_cast<uint32_t>(rows * chunks)), dim3(256), 0, stream,
+                           logits, static_cast<uint32_t>(columns), chunks, partials);
+    else
+        hipLaunchKernelGGL(argmax_chunks_kernel<false>, dim3(static_cast<uint32_t>(rows * chunks)), dim3(256), 0, stream,
+                           logits, static_cast<uint32_t>(columns), chunks, partials);
+    hipError_t error = hipGetLastError();
+    if (error != hipSuccess) return error;
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(static_cast<uint32_t>(rows)), dim3(64), 0, stream, partials, chunks, out,
+                       status);
     return hipGetLastError();
 }
 

@@ -127,8 +127,10 @@ hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len,
                   hipStream_t stream);
 hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t count, hipStream_t stream);
 // out[row] = greedy token; status[row] = 0, or 1 + the first token whose logit is not finite.
+// `workspace` holds argmax_workspace_bytes(rows, columns), 4-byte aligned.
+uint64_t argmax_workspace_bytes(uint64_t rows, uint64_t columns);
 hipError_t argmax_rows(const float* logits, uint64_t rows, uint64_t columns, uint32_t* out, uint32_t* status,
-                       hipStream_t stream);
+                       void* workspace, hipStream_t stream);
 // out[p, :] = table[indexes[p], :] as bytes; status[p] (8 bytes each) = 0, or bit 63 | the index.
 hipError_t gather_rows(const void* table, uint64_t table_rows, uint64_t row_bytes, const void* indexes,
                        int index_is_i64, uint64_t count, void* out, void* status, hipStream_t stream);

@@ -49,15 +49,23 @@ def greedy_status_check(status: torch.Tensor) -> None:
     _check(N.lib().et_hip_greedy_status_check(len(host) // 4, ctypes.create_string_buffer(host, len(host))))
 
 
-def greedy_tokens(logits: torch.Tensor, *, stream=None, synchronize: bool = True):
+def greedy_workspace_bytes(rows: int, vocabulary: int) -> int:
+    return int(N.lib().et_hip_greedy_workspace_bytes(rows, vocabulary))
+
+
+def greedy_tokens(logits: torch.Tensor, *, workspace: Optional[torch.Tensor] = None, stream=None,
+                  synchronize: bool = True):
     """Greedy token per row of ``[.., vocabulary]`` logits as an int32 tensor. With ``synchronize`` a
     logit that is not finite raises the reference's error here; otherwise ``(tokens, status)``."""
     rows = logits.numel() // logits.shape[-1] if logits.dim() and logits.shape[-1] else 0
     tokens = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)
     status = torch.empty(4 * max(rows, 1), dtype=torch.uint8, device=logits.device)
+    if workspace is None:
+        need = greedy_workspace_bytes(rows, logits.shape[-1]) if rows else 0
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=logits.device)
     desc = _desc(logits)
-    _check(N.lib().et_hip_greedy_tokens_into(_ref(desc), tokens.data_ptr(), status.data_ptr(),
-                                             _stream_handle(stream)))
+    _check(N.lib().et_hip_greedy_tokens_into(_ref(desc), tokens.data_ptr(), workspace.data_ptr(), workspace.numel(),
+                                             status.data_ptr(), _stream_handle(stream)))
     if not synchronize:
         return tokens, status
     greedy_status_check(status[:4 * rows])

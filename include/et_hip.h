@@ -289,10 +289,14 @@ int et_hip_silu_mul_into(const et_tensor* gate, const et_tensor* up, const et_te
 
 /* = sample_logits with temperature 0 (crates/runtime/src/sampling.rs:86-103) for
  * every row of f32 logits [.., vocabulary]: the largest logit, the lowest token
- * among equals. tokens: device u32 [rows]. A logit that is not finite cannot
- * fail the call; `status` (device, 4 bytes per row, written by the call) records
- * it for et_hip_greedy_status_check ("sample: logit {token} is not finite"). */
-int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* status, void* stream);
+ * among equals. tokens: device u32 [rows]. workspace: device scratch of
+ * et_hip_greedy_workspace_bytes(rows, vocabulary), 4-byte aligned (the rows are
+ * scanned in chunks by many workgroups). A logit that is not finite cannot fail
+ * the call; `status` (device, 4 bytes per row, written by the call) records it
+ * for et_hip_greedy_status_check ("sample: logit {token} is not finite"). */
+uint64_t et_hip_greedy_workspace_bytes(uint64_t rows, uint64_t vocabulary);
+int et_hip_greedy_tokens_into(const et_tensor* logits, uint32_t* tokens, void* workspace,
+                              uint64_t workspace_bytes, void* status, void* stream);
 int et_hip_greedy_status_check(uint64_t rows, const void* status_host);
 
 /* = index_select_into along dimension 0 (crates/runtime-cpu/src/indexing.rs:396-430)
