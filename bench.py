@@ -50,7 +50,9 @@ def parse_args():
                    help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
-    p.add_argument("--context", type=int, default=2048, help="kv_attention_decode: positions per slot")
+    p.add_argument("--context", type=int, default=2048, help="kv_attention_decode / llama3_8b_batched_decode: "
+                   "positions per slot")
+    p.add_argument("--layers", type=int, default=32, help="llama3_8b_batched_decode: transformer layers")
     p.add_argument("--hot", action="store_true", help="reuse one weight buffer (cache-resident; not the headline)")
     p.add_argument("--no-graph", action="store_true", help="enqueue the steps one by one instead of replaying a HIP graph")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -388,6 +390,185 @@ def decode_op(args, et):
     print(json.dumps(result))
 
 
+def llama_decode(args, et):
+    """Workload ``llama3_8b_batched_decode`` (BASELINE config 4): one decode step of a Llama-3-8B-shaped
+    model for 32 slots at context 2048, every operator through the C ABI - per layer RMS norm, the
+    q / k / v / o and gate / up / down contractions on Q4_K weights (M = 32, f32 activations), rotary
+    on q and k at the slots' cursors, paged key/value-cache attention over f16 slabs, SiLU * up and the
+    two residual sums; then the final norm, the Q4_K output projection to 128256 logits, greedy
+    selection and the lookup of the chosen tokens' embeddings for the next step. Weights are
+    synthetic (one random matrix per shape, rolled by layer into 32 distinct buffers); the step is
+    captured once into a HIP graph and replayed."""
+    import numpy as np
+    import torch
+    import oracle
+    from effect_torch_amd import synth
+
+    device = torch.device("cuda:0")
+    hidden, heads, kv_heads, width, ffn, vocab = 4096, 32, 8, 128, 14336, 128256
+    layers, slots, context, block = args.layers, 32, args.context, 16
+    mode = et.ActivationMode.INT8 if args.mode == "int8" else et.ActivationMode.F32
+    Q4K = et.GgmlQuant.Q4_K
+    rng = np.random.default_rng(0x11A3A)
+
+    shapes = {"wq": (hidden, hidden), "wk": (kv_heads * width, hidden), "wv": (kv_heads * width, hidden),
+              "wo": (hidden, hidden), "gate": (ffn, hidden), "up": (ffn, hidden), "down": (hidden, ffn),
+              "head": (vocab, hidden)}
+    host = {name: synth.random_weight(synth.Q4_K, rows, columns, rng) for name, (rows, columns) in shapes.items()}
+    base = {name: torch.from_numpy(w).to(device) for name, w in host.items()}
+    weights = [{name: (base[name] if layer == 0 else torch.roll(base[name], layer, 0).contiguous())
+                for name in shapes if name != "head"} for layer in range(layers)]
+    norms_host = [rng.standard_normal((2, hidden)).astype(np.float32) for _ in range(layers)]
+    norms = [torch.from_numpy(n).to(device) for n in norms_host]
+    final_norm = torch.randn(hidden, device=device)
+    plans = {name: et.RawLinear(Q4K, rows, columns, slots, False, mode) for name, (rows, columns) in shapes.items()}
+    linear_ws = torch.empty(max(max(p.requirements.workspace_bytes for p in plans.values()), 16), dtype=torch.uint8,
+                            device=device)
+
+    blocks_per_slot = -(-context // block)
+    total_blocks = slots * blocks_per_slot
+    table_host = rng.permutation(total_blocks).reshape(slots, blocks_per_slot).astype(np.int32)
+    cursors_host = np.full(slots, context - 1, dtype=np.int32)
+    advances_host = np.ones(slots, dtype=np.int32)
+    table, cursors, advances = (torch.from_numpy(a).to(device) for a in (table_host, cursors_host, advances_host))
+    kv = [et.KvLayer(torch.randn(total_blocks * block, kv_heads, width, device=device, dtype=torch.float16),
+                     torch.randn(total_blocks * block, kv_heads, width, device=device, dtype=torch.float16),
+                     block, table, cursors, advances, context) for _ in range(layers)]
+    kv_ws = et.kv_attention_workspace(kv[0], heads, 1)
+    greedy_ws = torch.empty(et.greedy_workspace_bytes(slots, vocab), dtype=torch.uint8, device=device)
+    embedding = torch.randn(vocab, hidden, device=device)
+    tokens = torch.from_numpy(rng.integers(0, vocab, slots).astype(np.int32)).to(device)
+    scale = 1.0 / float(np.sqrt(width))
+
+    f32 = lambda *shape: torch.empty(shape, device=device)  # noqa: E731
+    x, h, q, k, v = f32(slots, hidden), f32(slots, hidden), f32(slots, hidden), f32(slots, kv_heads * width), \
+        f32(slots, kv_heads * width)
+    attended, projected, gate, up, down = f32(slots, hidden), f32(slots, hidden), f32(slots, ffn), f32(slots, ffn), \
+        f32(slots, hidden)
+    logits = f32(slots, vocab)
+    chosen = torch.empty(slots, dtype=torch.int32, device=device)
+    keep = []
+
+    def layer_step(index):
+        w, kvl = weights[index], kv[index]
+        et.rms_norm_into(x, norms[index][0], 1e-5, h)
+        plans["wq"].enqueue(h, w["wq"], None, q, linear_ws)
+        plans["wk"].enqueue(h, w["wk"], None, k, linear_ws)
+        plans["wv"].enqueue(h, w["wv"], None, v, linear_ws)
+        q4, k4, v4 = q.view(slots, heads, 1, width), k.view(slots, kv_heads, 1, width), v.view(slots, kv_heads, 1, width)
+        et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)
+        et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
+        keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
+                                         workspace=kv_ws, synchronize=False))
+        plans["wo"].enqueue(attended, w["wo"], None, projected, linear_ws)
+        et.add_into(x, projected, x)
+        et.rms_norm_into(x, norms[index][1], 1e-5, h)
+        plans["gate"].enqueue(h, w["gate"], None, gate, linear_ws)
+        plans["up"].enqueue(h, w["up"], None, up, linear_ws)
+        et.silu_mul_into(gate, up, gate)
+        plans["down"].enqueue(gate, w["down"], None, down, linear_ws)
+        et.add_into(x, down, x)
+
+    def step():
+        keep.clear()
+        keep.append(et.gather_rows_into(embedding, tokens.view(torch.uint32), x, synchronize=False))
+        for index in range(layers):
+            layer_step(index)
+        et.rms_norm_into(x, final_norm, 1e-5, h)
+        plans["head"].enqueue(h, base["head"], None, logits, linear_ws)
+        keep.append(et.greedy_tokens(logits, workspace=greedy_ws, synchronize=False)[1])
+
+    # Parity gate: layer 0 for two slots against the CPU oracle chained the same way.
+    et.gather_rows_into(embedding, tokens.view(torch.uint32), x)
+    x0 = x.cpu().numpy()[:2].copy()
+    layer_step(0)
+    torch.cuda.synchronize()
+    et.kv_attention_status_check(kv[0], 1, keep[-1])
+    got = x.cpu().numpy()[:2]
+    lin = lambda name, act: oracle.linear_rows(synth.Q4_K, shapes[name][0], shapes[name][1], act, host[name], None, 0,  # noqa: E731
+                                               shapes[name][0])
+    if args.mode == "int8":
+        def lin(name, act):  # noqa: F811
+            qa, sa, ta = oracle.quantize_q8(np.ascontiguousarray(act))
+            return oracle.linear_q8_rows(synth.Q4_K, shapes[name][0], shapes[name][1], qa, sa, ta, host[name], None, 0,
+                                         shapes[name][0])
+    hh = oracle.rms_norm(x0, norms_host[0][0], 1e-5)
+    q_ref = oracle.rotary(lin("wq", hh).reshape(2, heads, 1, width), cursors_host[:2], 500000.0)
+    k_ref = oracle.rotary(lin("wk", hh).reshape(2, kv_heads, 1, width), cursors_host[:2], 500000.0)
+    v_ref = lin("wv", hh).reshape(2, kv_heads, 1, width)
+    # the slabs already hold the rows this very step appended; the oracle writes the same values again
+    att = oracle.kv_attention(kv[0].k_slab.cpu().numpy(), kv[0].v_slab.cpu().numpy(), block,
+                              table_host[:2].view(np.uint32), cursors_host[:2].view(np.uint32),
+                              advances_host[:2].view(np.uint32), q_ref, k_ref, v_ref, scale)
+    x1 = oracle.add(x0, lin("wo", att.reshape(2, hidden)))
+    hh = oracle.rms_norm(x1, norms_host[0][1], 1e-5)
+    want = oracle.add(x1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
+    relative = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    assert relative <= (2e-2 if args.mode == "int8" else 1e-3), f"parity gate failed: relative L2 error {relative:.3g}"
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    start.record(stream)
+    for _ in range(args.steps):
+        graph.replay()
+    stop.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    ms = start.elapsed_time(stop) / args.steps
+    et.greedy_status_check(keep[-1])
+    seconds = ms * 1e-3
+    weight_bytes = layers * sum(host[n].size for n in shapes if n != "head") + host["head"].size
+    kv_bytes = layers * 2 * slots * context * kv_heads * width * 2
+    algorithmic = weight_bytes + kv_bytes + slots * vocab * 4 * 2
+    gbs = algorithmic / seconds / 1e9
+    result = {
+        "metric": "batched decode tok/s", "value": round(slots / seconds, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8" if args.mode == "int8" else "f32", "data": "synthetic",
+        "config": {"workload": f"llama3_8b_batched_decode: {layers} layers, hidden {hidden}, {heads}/{kv_heads} heads x {width}, "
+                               f"ffn {ffn}, vocab {vocab}; Q4_K weights, f16 kv slabs in blocks of {block}; {slots} slots at "
+                               f"context {context}; {'int8' if args.mode == 'int8' else 'f32'} activations",
+                   "launch": "one HIP graph of the whole step, replayed K times",
+                   "weight_bytes": weight_bytes, "kv_bytes_read": kv_bytes, "layer0_relative_l2_error": relative,
+                   "host_wall_ms": round(wall * 1e3, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 1)},
+    }
+    if not args.no_cpu:
+        # one layer for one slot and 2048 rows of the output projection on one core, scaled to the step
+        t0 = time.perf_counter()
+        one = x0[:1]
+        hh = oracle.rms_norm(one, norms_host[0][0], 1e-5)
+        q1 = oracle.rotary(lin("wq", hh).reshape(1, heads, 1, width), cursors_host[:1], 500000.0)
+        k1 = oracle.rotary(lin("wk", hh).reshape(1, kv_heads, 1, width), cursors_host[:1], 500000.0)
+        v1 = lin("wv", hh).reshape(1, kv_heads, 1, width)
+        a1 = oracle.kv_attention(kv[0].k_slab.cpu().numpy(), kv[0].v_slab.cpu().numpy(), block,
+                                 table_host[:1].view(np.uint32), cursors_host[:1].view(np.uint32),
+                                 advances_host[:1].view(np.uint32), q1, k1, v1, scale)
+        y1 = oracle.add(one, lin("wo", a1.reshape(1, hidden)))
+        hh = oracle.rms_norm(y1, norms_host[0][1], 1e-5)
+        oracle.add(y1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
+        t1 = time.perf_counter()
+        oracle.linear_rows(synth.Q4_K, vocab, hidden, hh, host["head"], None, 0, 2048)
+        t2 = time.perf_counter()
+        per_token = (t1 - t0) * layers + (t2 - t1) * vocab / 2048
+        result["cpu_baseline"] = {"value": round(1.0 / per_token, 4), "unit": "tok/s", "cores": 1, "kind": "port",
+                                  "sample": f"one layer for one slot ({t1 - t0:.2f} s incl. copying the slabs) x {layers} "
+                                            f"layers + 2048 of {vocab} output rows ({t2 - t1:.2f} s) scaled; scalar C "
+                                            f"restatement of the reference's loops ({per_token:.1f} s per token)"}
+    print(json.dumps(result))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -407,12 +588,15 @@ def main():
     if args.workload in DECODE_OPS:
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return decode_op(args, et)
+    if args.workload == "llama3_8b_batched_decode":
+        assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
+        return llama_decode(args, et)
     if args.workload == "kv_attention_decode":
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return kv_decode(args, et)
     if args.workload not in synth.CONFIGS:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
-                 "or calibrate_read / calibrate_copy / kv_attention_decode / " + " / ".join(DECODE_OPS))
+                 "or calibrate_read / calibrate_copy / kv_attention_decode / llama3_8b_batched_decode / " + " / ".join(DECODE_OPS))
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")

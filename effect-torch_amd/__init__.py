@@ -35,6 +35,7 @@ from .kv_cache import (  # noqa: F401
 )
 from .decode_ops import (  # noqa: F401
     RotaryLayout,
+    add_into,
     gather_rows_into,
     gather_rows_status_check,
     greedy_status_check,

@@ -347,6 +347,18 @@ int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t off
     });
 }
 
+int et_hip_add_into(const et_tensor* a, const et_tensor* b, const et_tensor* destination, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView av, bv, dst;
+        if (!TensorView::from_c(a, &av, error) || !TensorView::from_c(b, &bv, error) ||
+            !TensorView::from_c(destination, &dst, error)) {
+            *error = "add: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::add_into(av, bv, dst, stream, error);
+    });
+}
+
 int et_hip_silu_mul_into(const et_tensor* gate, const et_tensor* up, const et_tensor* destination, void* stream) {
     return guarded([&](std::string* error) -> int {
         TensorView gv, uv, dst;

@@ -86,6 +86,23 @@ int rotary_into(const TensorView& x, const uint32_t* offsets, uint64_t offsets_l
                     "rotary", error);
 }
 
+int add_into(const TensorView& a, const TensorView& b, const TensorView& destination, void* stream,
+             std::string* error) {
+    if (a.dtype != ET_DTYPE_F32 || b.dtype != ET_DTYPE_F32 || destination.dtype != ET_DTYPE_F32)
+        return fail(error, ET_ERR_UNSUPPORTED, "add: only f32 tensors are supported");
+    if (a.shape != b.shape || destination.shape != a.shape)
+        return fail(error, ET_ERR_UNSUPPORTED, "add: both operands and the destination must have one shape");
+    if (!a.is_contiguous() || !b.is_contiguous() || !destination.is_contiguous())
+        return fail(error, ET_ERR_UNSUPPORTED, "add: operands must be contiguous");
+    const uint64_t count = numel(a);
+    if (count == 0) return ET_OK;
+    if (count > (0x7fffffffull << 8)) return fail(error, ET_ERR_UNSUPPORTED, "add: geometry exceeds the launch limits");
+    if (a.data == nullptr || b.data == nullptr || destination.data == nullptr)
+        return fail(error, ET_ERR_INVALID, "add: NULL device pointer");
+    return launched(add(f32_data(a), f32_data(b), f32_out(destination), count, static_cast<hipStream_t>(stream)), "add",
+                    error);
+}
+
 int silu_mul_into(const TensorView& gate, const TensorView& up, const TensorView& destination, void* stream,
                   std::string* error) {
     if (gate.dtype != ET_DTYPE_F32 || up.dtype != ET_DTYPE_F32 || destination.dtype != ET_DTYPE_F32)

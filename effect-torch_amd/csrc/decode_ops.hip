@@ -5,6 +5,7 @@
 //   rms_norm_kernel     rms_norm_forward_into_impl (crates/runtime-cpu/src/composed.rs:1457-1487)
 //   rotary_kernel       rotary_forward_into_impl (composed.rs:2683-2729)
 //   silu_mul_kernel     Tensor.silu (packages/core/src/Tensor.ts:1537-1540) times the up projection
+//   add_kernel          the residual connections (binary add, crates/runtime-cpu/src/ops.rs)
 //   argmax_kernel       sample_logits with temperature 0 (crates/runtime/src/sampling.rs:86-103)
 //   gather_rows_kernel  index_select along dimension 0 (crates/runtime-cpu/src/indexing.rs:152-187)
 //
@@ -120,7 +121,7 @@ __device__ __forceinline__ float silu_mul_one(float gate, float up) {
 }
 
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
-                                                       float* __restrict__ out, uint64_t count, int vectorised) {
+                                                       float* out, uint64_t count, int vectorised) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (vectorised) {
         if (4 * i >= count) return;
@@ -129,6 +130,18 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
                                                         silu_mul_one(g.z, u.z), silu_mul_one(g.w, u.w));
     } else if (i < count) {
         out[i] = silu_mul_one(gate[i], up[i]);
+    }
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* a, const float* b,
+                                                  float* out, uint64_t count, int vectorised) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (vectorised) {
+        if (4 * i >= count) return;
+        const float4 x = reinterpret_cast<const float4*>(a)[i], y = reinterpret_cast<const float4*>(b)[i];
+        reinterpret_cast<float4*>(out)[i] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    } else if (i < count) {
+        out[i] = a[i] + b[i];
     }
 }
 
@@ -265,6 +278,15 @@ hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t cou
     const uint64_t items = vectorised ? count / 4 : count;
     hipLaunchKernelGGL(silu_mul_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream, gate, up,
                        out, count, vectorised);
+    return hipGetLastError();
+}
+
+hipError_t add(const float* a, const float* b, float* out, uint64_t count, hipStream_t stream) {
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const int vectorised = count % 4 == 0 && aligned(a) && aligned(b) && aligned(out);
+    const uint64_t items = vectorised ? count / 4 : count;
+    hipLaunchKernelGGL(add_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream, a, b, out,
+                       count, vectorised);
     return hipGetLastError();
 }
 

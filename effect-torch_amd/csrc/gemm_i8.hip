@@ -147,7 +147,8 @@ template <int CODEC, int MT, int LIMBS, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint8_t* __restrict__ weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
-    uint32_t vectors, uint32_t row_tiles, uint32_t vector_groups) {
+    uint32_t vectors, uint32_t row_tiles, uint32_t vector_groups, uint32_t k_splits,
+    float* __restrict__ partials) {
     using S = Shape<CODEC, MT, LIMBS, AX, AW>;
     using W = WeightLayout<CODEC>;
     constexpr int NB = kBlocksPerWave;
@@ -156,14 +157,21 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     // Workgroups are handed to the eight XCDs round-robin. All vector groups of one row tile
     // go to the same XCD, next to each other in time, so the later ones find the weights in L2.
     const uint32_t xcd = blockIdx.x & 7u, turn = blockIdx.x >> 3;
-    const uint32_t row_tile = (turn / vector_groups) * 8u + xcd;
-    const uint32_t vector_group = turn % vector_groups;
+    // With k_splits > 1 the stages of K are shared out over that many workgroups per tile, each
+    // leaving a partial result for reduce_partials_kernel.
+    const uint32_t units = vector_groups * k_splits;
+    const uint32_t row_tile = (turn / units) * 8u + xcd;
+    const uint32_t vector_group = (turn % units) % vector_groups;
+    const uint32_t k_share = (turn % units) / vector_groups;
     if (row_tile >= row_tiles) return;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: uniform branches
     const uint32_t tile0 = vector_group * MT;
-    const uint32_t stages = columns / 256u;  // whole: columns % 256 == 0
+    const uint32_t all_stages = columns / 256u;  // whole: columns % 256 == 0
+    const uint32_t share = (all_stages + k_splits - 1u) / k_splits;
+    const uint32_t first_stage = k_share * share;  // < all_stages: the launcher leaves no share empty
+    const uint32_t stages = min(share, all_stages - first_stage);
     const uint64_t row_bytes = static_cast<uint64_t>(columns / block_values(CODEC)) * block_bytes(CODEC);
     const uint32_t row0 = row_tile * kRows;
 
@@ -179,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 if (job >= static_cast<uint32_t>(S::kActivationJobs)) job -= S::kActivationJobs;
                 const uint32_t t = job / (S::kTile / 1024u), within = job % (S::kTile / 1024u);
                 const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
-                const uint8_t* src = tiles + (static_cast<uint64_t>(s) * vector_tiles + tile) * S::kBlob +
+                const uint8_t* src = tiles + (static_cast<uint64_t>(first_stage + s) * vector_tiles + tile) * S::kBlob +
                                      within * 1024u + lane * 16u;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
@@ -211,7 +219,8 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 if (job >= static_cast<uint32_t>(W::kJobs)) job -= W::kJobs;
                 const uint32_t at = job * 1024u + lane * 16u;  // byte of the slot this lane fills
                 const uint32_t row = min(row0 + at / W::kRowBytes, rows - 1u);
-                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(s) * W::kRowBytes + at % W::kRowBytes;
+                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * W::kRowBytes +
+                                     at % W::kRowBytes;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
             }
@@ -418,15 +427,50 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             for (int k = 1; k < kSplit; k++)
                 value += exchange[((((k - 1) * kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane];
             const uint32_t m = m0 + 32u * t + 8u * (r >> 2) + 4u * half + (r & 3u);
-            if (n_out < rows && m < vectors) y[static_cast<uint64_t>(m) * rows + n_out] = value + bias_value;
+            if (n_out < rows && m < vectors) {
+                if (k_splits == 1)
+                    y[static_cast<uint64_t>(m) * rows + n_out] = value + bias_value;
+                else
+                    partials[(static_cast<uint64_t>(k_share) * vectors + m) * rows + n_out] = value;
+            }
         }
         __builtin_amdgcn_sched_barrier(0);  // tile by tile: the sums of all tiles at once do not fit
     }
 }
 
+}  // namespace
+uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t columns, uint64_t vectors);
+namespace {
+
+// y[m, n] = bias[n] + sum over the K shares, in share order; four outputs per thread.
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partials,
+                                                              const float* __restrict__ bias, float* __restrict__ y,
+                                                              uint32_t rows, uint64_t outputs, uint32_t k_splits) {
+    const uint64_t i = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (i >= outputs) return;
+    if (rows % 4 == 0) {
+        const uint32_t n = static_cast<uint32_t>(i % rows);
+        float4 total = bias != nullptr ? *reinterpret_cast<const float4*>(bias + n) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (uint32_t k = 0; k < k_splits; k++) {
+            const float4 part = *reinterpret_cast<const float4*>(partials + k * outputs + i);
+            total.x += part.x;
+            total.y += part.y;
+            total.z += part.z;
+            total.w += part.w;
+        }
+        *reinterpret_cast<float4*>(y + i) = total;
+    } else {
+        for (uint64_t j = i; j < min(i + 4, outputs); j++) {
+            float total = bias != nullptr ? bias[j % rows] : 0.f;
+            for (uint32_t k = 0; k < k_splits; k++) total += partials[k * outputs + j];
+            y[j] = total;
+        }
+    }
+}
+
 template <int CODEC, int MT, int LIMBS, int AX, int AW>
 hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
-                  uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+                  uint32_t rows, uint32_t columns, uint32_t vectors, float* partials, hipStream_t stream) {
     using S = Shape<CODEC, MT, LIMBS, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, AX, AW>;
@@ -445,11 +489,18 @@ hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias
     const uint32_t vector_tiles = (vectors + 31u) / 32u;
     const uint32_t vector_groups = (vector_tiles + MT - 1) / MT;
     const uint32_t row_tiles = (rows + kRows - 1) / kRows;
-    const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_groups;
+    const uint32_t k_splits = partials != nullptr ? gemm_i8_k_splits(CODEC, LIMBS, rows, columns, vectors) : 1u;
+    const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_groups * k_splits;
     if (grid > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream,
                        weight, tiles, vector_tiles, bias, y, rows, columns, vectors, row_tiles,
-                       vector_groups);
+                       vector_groups, k_splits, partials);
+    if (hipError_t status = hipGetLastError()) return status;
+    if (k_splits > 1) {
+        const uint64_t outputs = static_cast<uint64_t>(vectors) * rows;
+        hipLaunchKernelGGL(reduce_partials_kernel, dim3(static_cast<uint32_t>((outputs + 1023) / 1024)), dim3(256), 0,
+                           stream, partials, bias, y, rows, outputs, k_splits);
+    }
     return hipGetLastError();
 }
 
@@ -469,27 +520,36 @@ constexpr int weight_lead() {
 }
 
 template <int CODEC, int MT, int LIMBS, int AX>
-hipError_t launch_shape(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
+hipError_t launch_shape(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y, float* partials,
                         uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
     constexpr int kWeightLead = weight_lead<CODEC, MT, LIMBS, AX>();
     static_assert(kWeightLead >= 1, "no room for a weight ring");
-    return launch<CODEC, MT, LIMBS, AX, kWeightLead>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    return launch<CODEC, MT, LIMBS, AX, kWeightLead>(weight, tiles, bias, y, rows, columns, vectors, partials, stream);
 }
 
 template <int CODEC>
 hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const float* bias,
-                        float* y, uint32_t rows, uint32_t columns, uint32_t vectors,
+                        float* y, float* partials, uint32_t rows, uint32_t columns, uint32_t vectors,
                         hipStream_t stream) {
     // Activations: 26 KiB per stage and 32-vector tile with three limbs, 10 KiB with one; two
     // stages of lead. The weight ring (9 to 20 KiB per stage) takes the rest of LDS.
     // One 32-vector tile per workgroup with three limbs: two tiles of three-limb results do not
     // fit in registers. Q4_K carries a second accumulator (the min term): at most two tiles.
-    if (limbs == 3) return launch_shape<CODEC, 1, 3, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    if (vectors <= 32) return launch_shape<CODEC, 1, 1, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
+    // (tiles_per_workgroup() below states the same choice for the launch geometry.)
+    if (limbs == 3)
+        return launch_shape<CODEC, 1, 3, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
+    if (vectors <= 32)
+        return launch_shape<CODEC, 1, 1, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
     if (vectors <= 64 || CODEC == kQ4_K)
-        return launch_shape<CODEC, 2, 1, 2>(weight, tiles, bias, y, rows, columns, vectors, stream);
-    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, bias, y, rows,
-                                                                                columns, vectors, stream);
+        return launch_shape<CODEC, 2, 1, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
+    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, bias, y, partials,
+                                                                                rows, columns, vectors, stream);
+}
+
+uint32_t tiles_per_workgroup(int32_t codec, int limbs, uint64_t vectors) {
+    if (limbs == 3 || vectors <= 32) return 1;
+    if (vectors <= 64 || codec == kQ4_K) return 2;
+    return 4;
 }
 
 }  // namespace
@@ -499,16 +559,30 @@ bool gemm_i8_supported(int32_t codec, uint64_t columns) {
     return (codec == kQ8_0 || codec == kQ4_0 || codec == kQ4_K) && columns % 256 == 0 && columns > 0;
 }
 
+uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t columns, uint64_t vectors) {
+    // One workgroup fits a compute unit. A launch with far fewer tiles than the 256 units shares
+    // the stages of K out over several workgroups per tile, no share empty.
+    const uint64_t vector_tiles = (vectors + 31) / 32, per_group = tiles_per_workgroup(codec, limbs, vectors);
+    const uint64_t tiles = ((rows + kRows - 1) / kRows) * ((vector_tiles + per_group - 1) / per_group);
+    const uint64_t stages = columns / 256;
+    if (tiles == 0 || stages < 2 || tiles >= 192) return 1;
+    uint64_t splits = 256 / tiles;
+    if (splits > stages) splits = stages;
+    if (splits < 2) return 1;
+    const uint64_t share = (stages + splits - 1) / splits;
+    return static_cast<uint32_t>((stages + share - 1) / share);
+}
+
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
-                   const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
-                   hipStream_t stream) {
+                   const float* bias, float* y, float* partials, uint64_t rows, uint64_t columns,
+                   uint64_t vectors, hipStream_t stream) {
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns),
                    m = static_cast<uint32_t>(vectors);
     switch (codec) {
-        case kQ8_0: return launch_codec<kQ8_0>(limbs, weight, tiles, bias, y, n, k, m, stream);
-        case kQ4_0: return launch_codec<kQ4_0>(limbs, weight, tiles, bias, y, n, k, m, stream);
-        case kQ4_K: return launch_codec<kQ4_K>(limbs, weight, tiles, bias, y, n, k, m, stream);
+        case kQ8_0: return launch_codec<kQ8_0>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
+        case kQ4_0: return launch_codec<kQ4_0>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
+        case kQ4_K: return launch_codec<kQ4_K>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -74,9 +74,12 @@ bool gemm_i8_supported(int32_t codec, uint64_t columns);
 // From this many vectors on, f32-mode requests use the matrix cores (3-limb activations):
 // measured on MI355X, two launches of the 3-vector GEMV are still faster below it.
 constexpr uint32_t kGemmMinVectors = 7;
+// Launches with few output tiles share K out over this many workgroups per tile (1 = no sharing);
+// `partials` then holds k_splits * vectors * rows floats. partials == nullptr: never share.
+uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t columns, uint64_t vectors);
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
-                   const float* bias, float* y, uint64_t rows, uint64_t columns, uint64_t vectors,
-                   hipStream_t stream);
+                   const float* bias, float* y, float* partials, uint64_t rows, uint64_t columns,
+                   uint64_t vectors, hipStream_t stream);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch
@@ -125,6 +128,7 @@ hipError_t rms_norm(const float* x, const float* weight, double eps, float* out,
 hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
                   int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,
                   hipStream_t stream);
+hipError_t add(const float* a, const float* b, float* out, uint64_t count, hipStream_t stream);
 hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t count, hipStream_t stream);
 // out[row] = greedy token; status[row] = 0, or 1 + the first token whose logit is not finite.
 // `workspace` holds argmax_workspace_bytes(rows, columns), 4-byte aligned.

@@ -97,7 +97,8 @@ int validate_weight(const char* operation, const TensorView& weight, int32_t cod
 // cf. linear_kernel_kind, crates/runtime-metal/src/quantized.rs:1204-1220.
 int select_kernel(et_linear_plan* plan, std::string* error) {
     plan->gather_offset = plan->gather_bytes = 0;
-    plan->q_offset = plan->bias_offset = 0;
+    plan->q_offset = plan->bias_offset = plan->partial_offset = 0;
+    plan->k_splits = 1;
     plan->workspace_bytes = 0;
     plan->vectors_per_launch = 0;
     if (plan->vectors == 0 || plan->rows == 0) {
@@ -118,6 +119,11 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         plan->kernel = kernel;
         plan->q_offset = cursor;  // activation tiles, see tile_blob_bytes()
         cursor = align_up(cursor + tile_workspace_bytes(limbs, plan->vectors, plan->columns), 256);
+        plan->k_splits = gemm_i8_k_splits(plan->codec, limbs, plan->rows, plan->columns, plan->vectors);
+        if (plan->k_splits > 1) {
+            plan->partial_offset = cursor;
+            cursor = align_up(cursor + plan->k_splits * plan->vectors * plan->rows * 4u, 256);
+        }
     };
     if (plan->activation_mode == ET_ACT_INT8) {
         if (!gemm_i8_supported(plan->codec, plan->columns))
@@ -236,8 +242,10 @@ const char* kernel_name(const et_linear_plan& plan) {
         case LinearKernel::kNone: return "none";
         case LinearKernel::kGemvLimb: return "gemv_limb";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
-        case LinearKernel::kGemmI8: return "quantize_act+gemm_i8";
-        case LinearKernel::kGemmLimb: return "quantize_limbs+gemm_i8";
+        case LinearKernel::kGemmI8:
+            return plan.k_splits > 1 ? "quantize_act+gemm_i8+reduce" : "quantize_act+gemm_i8";
+        case LinearKernel::kGemmLimb:
+            return plan.k_splits > 1 ? "quantize_limbs+gemm_i8+reduce" : "quantize_limbs+gemm_i8";
     }
     return "?";
 }
@@ -350,7 +358,8 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         if (hipError_t status =
                 quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs, tiles, s))
             return hip_failure(error, "quantized_linear", status);
-        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, bias, y, plan.rows,
+        float* partials = plan.k_splits > 1 ? reinterpret_cast<float*>(scratch + plan.partial_offset) : nullptr;
+        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, bias, y, partials, plan.rows,
                                         plan.columns, plan.vectors, s))
             return hip_failure(error, "quantized_linear", status);
         return ET_OK;

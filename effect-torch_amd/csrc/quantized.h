@@ -54,6 +54,8 @@ struct et_linear_plan {
     uint64_t gather_offset, gather_bytes;  // densified f32 input
     uint64_t bias_offset;                  // densified f32 bias
     uint64_t q_offset;                     // quantised activation tiles (matrix-core kernels)
+    uint64_t partial_offset;               // partial results of the K shares (0 splits: unused)
+    uint32_t k_splits;
     uint64_t workspace_bytes;
 };
 

@@ -39,6 +39,11 @@ def rotary_into(x: torch.Tensor, offsets: torch.Tensor, theta: float, sign: floa
                                       float(sign), int(layout), _ref(descs[1]), _stream_handle(stream)))
 
 
+def add_into(a: torch.Tensor, b: torch.Tensor, destination: torch.Tensor, *, stream=None) -> None:
+    descs = (_desc(a), _desc(b), _desc(destination))
+    _check(N.lib().et_hip_add_into(_ref(descs[0]), _ref(descs[1]), _ref(descs[2]), _stream_handle(stream)))
+
+
 def silu_mul_into(gate: torch.Tensor, up: torch.Tensor, destination: torch.Tensor, *, stream=None) -> None:
     descs = (_desc(gate), _desc(up), _desc(destination))
     _check(N.lib().et_hip_silu_mul_into(_ref(descs[0]), _ref(descs[1]), _ref(descs[2]), _stream_handle(stream)))

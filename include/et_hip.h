@@ -281,6 +281,11 @@ int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t off
                        double theta, double sign, int32_t layout, const et_tensor* destination,
                        void* stream);
 
+/* out = a + b, f32, same shapes (the residual connections; the reference's binary
+ * add without broadcasting, crates/runtime-cpu/src/ops.rs). `destination` may be `a`. */
+int et_hip_add_into(const et_tensor* a, const et_tensor* b, const et_tensor* destination,
+                    void* stream);
+
 /* out = silu(gate) * up with silu(x) = x * (tanh(x / 2) / 2 + 1 / 2), f32, every
  * step rounded (Tensor.silu over Tensor.sigmoid, packages/core/src/Tensor.ts:1537-1540,
  * :1240-1245; the reference builds it from four elementwise nodes). */

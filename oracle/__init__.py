@@ -85,6 +85,8 @@ def lib() -> ctypes.CDLL:
                                        ctypes.c_char_p, sz]
         L.et_oracle_silu_mul.restype = None
         L.et_oracle_silu_mul.argtypes = [vp, vp, vp, sz]
+        L.et_oracle_add.restype = None
+        L.et_oracle_add.argtypes = [vp, vp, vp, sz]
         L.et_oracle_argmax.restype = ci
         L.et_oracle_argmax.argtypes = [vp, sz, sz, vp, ctypes.c_char_p, sz]
         L.et_oracle_gather_rows.restype = ci
@@ -344,4 +346,13 @@ def gather_rows(table: np.ndarray, indexes) -> np.ndarray:
     if lib().et_oracle_gather_rows(_ptr(table), table.shape[0], row_bytes, _ptr(indexes), indexes.size,
                                    _ptr(out), err, 256) != 0:
         raise OracleError(err.value.decode())
+    return out
+
+
+def add(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    assert a.shape == b.shape
+    out = np.empty_like(a)
+    lib().et_oracle_add(_ptr(a), _ptr(b), _ptr(out), a.size)
     return out

@@ -67,6 +67,10 @@ void et_oracle_silu_mul(const float* gate, const float* up, float* out, size_t c
     }
 }
 
+void et_oracle_add(const float* a, const float* b, float* out, size_t count) {
+    for (size_t i = 0; i < count; i++) out[i] = a[i] + b[i];
+}
+
 /* sampling.rs:86-103 */
 int et_oracle_argmax(const float* logits, size_t rows, size_t columns, uint32_t* out, char* err,
                      size_t err_len) {

@@ -19,6 +19,8 @@
  *   et_oracle_argmax      sample_logits with temperature 0 (crates/runtime/src/sampling.rs:86-103):
  *                         the reference's tie test ([1, 4, 4, 2] -> 1, :223-238), numpy argmax on
  *                         random rows, the non-finite error message
+ *   et_oracle_add         elementwise f32 sum (the residual connections; ops.rs binary add): IEEE
+ *                         addition, identical to numpy's
  *   et_oracle_gather_rows index_select along dimension 0 (crates/runtime-cpu/src/indexing.rs:152-187):
  *                         numpy fancy indexing; the out-of-bounds message
  */
@@ -45,6 +47,9 @@ int et_oracle_rotary(const float* x, const uint32_t* offsets, size_t offsets_len
 
 /* out = (gate * (tanhf(gate / 2) / 2 + 0.5)) * up, every operation rounded to f32. */
 void et_oracle_silu_mul(const float* gate, const float* up, float* out, size_t count);
+
+/* out = a + b, f32. */
+void et_oracle_add(const float* a, const float* b, float* out, size_t count);
 
 /* Greedy token per row; 0, or -1 with "sample: logit {token} is not finite" for the first row
  * that holds one. */

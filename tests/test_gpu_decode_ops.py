@@ -127,3 +127,16 @@ def test_gather_rows(et, device, dtype, width, wide_index):
         idx = torch.from_numpy(bad.astype(np.int64)).to(device)
         with pytest.raises(et.QuantizedError, match="index_select: index -2 is out of bounds for extent 1000"):
             et.gather_rows_into(td, idx, out)
+
+
+def test_add(et, device):
+    rng = np.random.default_rng(8)
+    for count in (32 * 4096, 1001):
+        a = (rng.standard_normal(count) * 100).astype(np.float32)
+        b = rng.standard_normal(count).astype(np.float32)
+        ad, bd = torch.from_numpy(a).to(device), torch.from_numpy(b).to(device)
+        out = torch.empty_like(ad)
+        et.add_into(ad, bd, out)
+        assert np.array_equal(out.cpu().numpy(), oracle.add(a, b))
+        et.add_into(ad, bd, ad)  # in place, as the residual stream is updated
+        assert np.array_equal(ad.cpu().numpy(), oracle.add(a, b))

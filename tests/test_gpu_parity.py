@@ -221,7 +221,7 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
     bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   None, et.GgmlQuant(codec), (rows, columns))
-    assert plan.kernel == "quantize_limbs+gemm_i8"
+    assert plan.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
     got = run_linear(et, device, codec, rows, columns, x, weight, bias)
     if codec != oracle.Q4_K:
         # a width that is not a whole number of 256-column stages stays on the GEMV kernels
@@ -238,6 +238,34 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
     if bias is not None:
         exact = exact + bias.astype(np.float64)
     close(got, exact, oracle_noise=0)
+
+
+@pytest.mark.parametrize("mode", ["F32", "INT8"])
+@pytest.mark.parametrize("codec,vectors,rows,columns", [(oracle.Q4_K, 32, 1024, 4096), (oracle.Q4_K, 32, 4096, 4096),
+                                                        (oracle.Q4_K, 32, 4096, 14336), (oracle.Q8_0, 40, 700, 2304),
+                                                        (oracle.Q4_0, 9, 65, 1280)])
+def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vectors, rows, columns):
+    # decode-batch shapes: far fewer 64-row tiles than compute units, so the stages of K are shared
+    # out over several workgroups per tile and summed by a second kernel, in a fixed order
+    rng = np.random.default_rng(rows + columns + vectors)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    bias = rng.standard_normal(rows).astype(np.float32)
+    act = et.ActivationMode[mode]
+    plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
+                                  torch.zeros(rows), et.GgmlQuant(codec), (rows, columns), act)
+    assert plan.kernel.endswith("+gemm_i8+reduce")
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
+    again = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
+    assert np.array_equal(got, again)  # the same bits on every run
+    check_rows = min(rows, 192)
+    if mode == "F32":
+        want = oracle.linear_rows(codec, rows, columns, x, weight, bias, 0, check_rows)[:, :check_rows]
+        close(got[:, :check_rows], want)
+    else:
+        q, scale, total = oracle.quantize_q8(x)
+        want = oracle.linear_q8_rows(codec, rows, columns, q, scale, total, weight, bias, 0, check_rows)[:, :check_rows]
+        close(got[:, :check_rows], want)
 
 
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0, oracle.Q6_K])

@@ -49,7 +49,7 @@ def test_linear_plan_shapes(et):
     plan = et.linear_requirements(torch.zeros(2, 5, 512), _w(7, 288), torch.zeros(7), et.GgmlQuant.Q4_K, (7, 512))
     assert plan.output_shape == (2, 5, 7) and plan.vectors == 10
     # ten vectors: 3-limb activations on the matrix cores, with its workspace planned
-    assert plan.kernel == "quantize_limbs+gemm_i8" and plan.workspace_bytes > 3 * 10 * 512
+    assert plan.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce") and plan.workspace_bytes > 3 * 10 * 512
     for few in (3, 6):
         plan3 = et.linear_requirements(torch.zeros(few, 512), _w(7, 288), None, et.GgmlQuant.Q4_K, (7, 512))
         assert plan3.kernel == "gemv_limb"
@@ -59,6 +59,11 @@ def test_linear_plan_shapes(et):
     plan = et.linear_requirements(torch.zeros(64, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256),
                                   et.ActivationMode.INT8)
     assert plan.kernel == "quantize_act+gemm_i8" and plan.workspace_bytes > 64 * 256
+    # few 64-row tiles: K is shared over workgroups and a second kernel sums the shares
+    few = et.linear_requirements(torch.zeros(32, 4096), _w(1024, 2304), None, et.GgmlQuant.Q4_K, (1024, 4096))
+    many = et.linear_requirements(torch.zeros(32, 4096), _w(14336, 2304), None, et.GgmlQuant.Q4_K, (14336, 4096))
+    assert few.kernel == "quantize_limbs+gemm_i8+reduce" and many.kernel == "quantize_limbs+gemm_i8"
+    assert few.workspace_bytes >= 16 * 32 * 1024 * 4  # 16 tiles x 16 stages: one stage per share
     # empty output: nothing to dispatch
     plan = et.linear_requirements(torch.zeros(0, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256))
     assert plan.output_shape == (0, 2) and plan.kernel == "none"

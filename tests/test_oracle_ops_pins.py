@@ -100,3 +100,10 @@ def test_gather_rows():
     assert np.array_equal(oracle.gather_rows(table, indexes).view(np.uint16), table[indexes].view(np.uint16))
     with pytest.raises(oracle.OracleError, match="index_select: index 50 is out of bounds for extent 50"):
         oracle.gather_rows(table, [1, 50])
+
+
+def test_add_is_ieee_addition():
+    rng = np.random.default_rng(5)
+    a = (rng.standard_normal(10000) * 1e3).astype(np.float32)
+    b = (rng.standard_normal(10000) * 1e-3).astype(np.float32)
+    assert np.array_equal(oracle.add(a, b), a + b)
