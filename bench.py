@@ -179,6 +179,7 @@ def kv_decode(args, et):
     import torch
 
     device = torch.device("cuda:0")
+    torch.manual_seed(7)
     slots, query_heads, kv_heads, width, block, context = 32, 32, 8, 128, 16, args.context
     layers = 1 if args.hot else 2
     rng = np.random.default_rng(7)
@@ -405,6 +406,7 @@ def llama_decode(args, et):
     from effect_torch_amd import synth
 
     device = torch.device("cuda:0")
+    torch.manual_seed(0x11A3A)
     hidden, heads, kv_heads, width, ffn, vocab = 4096, 32, 8, 128, 14336, 128256
     layers, slots, context, block = args.layers, 32, args.context, 16
     mode = et.ActivationMode.INT8 if args.mode == "int8" else et.ActivationMode.F32
