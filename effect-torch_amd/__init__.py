@@ -45,3 +45,9 @@ from .decode_ops import (  # noqa: F401
     rotary_into,
     silu_mul_into,
 )
+from .gguf import (  # noqa: F401
+    GgufFile,
+    GgufMetadataValue,
+    GgufParseError,
+    GgufTensorDescriptor,
+)

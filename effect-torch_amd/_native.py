@@ -56,6 +56,22 @@ class EtKvLayer(ctypes.Structure):
     ]
 
 
+class EtGgufTensor(ctypes.Structure):
+    """``et_gguf_tensor`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("name", ctypes.c_void_p),
+        ("name_length", ctypes.c_uint64),
+        ("format", ctypes.c_int32),
+        ("logical_rank", ctypes.c_int32),
+        ("logical_shape", ctypes.c_uint64 * 4),
+        ("physical_rank", ctypes.c_int32),
+        ("physical_shape", ctypes.c_uint64 * 4),
+        ("data_offset", ctypes.c_uint64),
+        ("byte_len", ctypes.c_uint64),
+    ]
+
+
 # Every symbol include/et_hip.h declares: name -> (restype, argtypes).
 _vp, _u64, _i32 = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int32
 _T = ctypes.POINTER(EtTensor)
@@ -100,6 +116,25 @@ SIGNATURES = {
     "et_hip_greedy_status_check": (ctypes.c_int, [_u64, _vp]),
     "et_hip_gather_rows_into": (ctypes.c_int, [_T, _T, _T, _vp, _vp]),
     "et_hip_gather_rows_status_check": (ctypes.c_int, [_u64, _u64, _vp]),
+    "et_hip_gguf_open": (ctypes.c_int, [ctypes.c_char_p, _vp, _PP]),
+    "et_hip_gguf_close": (None, [_vp]),
+    "et_hip_gguf_architecture": (ctypes.c_char_p, [_vp]),
+    "et_hip_gguf_metadata_count": (_u64, [_vp]),
+    "et_hip_gguf_metadata_find": (ctypes.c_int64, [_vp, ctypes.c_char_p]),
+    "et_hip_gguf_metadata_key": (_vp, [_vp, _u64]),
+    "et_hip_gguf_metadata_key_length": (_u64, [_vp, _u64]),
+    "et_hip_gguf_metadata_type": (_i32, [_vp, _u64]),
+    "et_hip_gguf_metadata_element_type": (_i32, [_vp, _u64]),
+    "et_hip_gguf_metadata_length": (_u64, [_vp, _u64]),
+    "et_hip_gguf_metadata_unsigned": (ctypes.c_int, [_vp, _u64, _u64, ctypes.POINTER(_u64)]),
+    "et_hip_gguf_metadata_signed": (ctypes.c_int, [_vp, _u64, _u64, ctypes.POINTER(ctypes.c_int64)]),
+    "et_hip_gguf_metadata_real": (ctypes.c_int, [_vp, _u64, _u64, ctypes.POINTER(ctypes.c_double)]),
+    "et_hip_gguf_metadata_string": (_vp, [_vp, _u64, _u64, ctypes.POINTER(_u64)]),
+    "et_hip_gguf_tensor_count": (_u64, [_vp]),
+    "et_hip_gguf_tensor_find": (ctypes.c_int64, [_vp, ctypes.c_char_p]),
+    "et_hip_gguf_tensor_at": (ctypes.c_int, [_vp, _u64, ctypes.POINTER(EtGgufTensor)]),
+    "et_hip_gguf_read_tensor_into": (ctypes.c_int, [_vp, _u64, _vp, _u64, _vp]),
+    "et_hip_gguf_upload_tensor": (ctypes.c_int, [_vp, _u64, _vp, _u64, _vp, _vp]),
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),

@@ -37,6 +37,7 @@ SOURCES = {
     "quantized.cpp": [],
     "kv_cache.cpp": [],
     "decode_host.cpp": [],
+    "gguf.cpp": [],
     "c_api.cpp": [],
 }
 

@@ -12,6 +12,7 @@
 #include "et_hip.h"
 #include "kernels.h"
 #include "decode_host.h"
+#include "gguf.h"
 #include "kv_cache.h"
 #include "quantized.h"
 
@@ -41,6 +42,15 @@ int guarded(F&& body) {
 }
 
 using et::quantized::TensorView;
+
+int gguf_failure(const et::gguf::Error& error) {
+    g_last_error = error.message;
+    switch (error.kind) {
+        case et::gguf::Failure::kInvalid: return ET_ERR_UNSUPPORTED;
+        case et::gguf::Failure::kCancelled: return ET_ERR_CANCELLED;
+        default: return ET_ERR_EXECUTION;
+    }
+}
 
 }  // namespace
 
@@ -417,6 +427,151 @@ int et_hip_gather_rows_status_check(uint64_t table_rows, uint64_t count, const v
             return ET_ERR_INVALID;
         }
         return et::decode::gather_rows_status_check(table_rows, count, status_host, error);
+    });
+}
+
+int et_hip_gguf_open(const char* path, const volatile int32_t* cancel, et_gguf** out) {
+    return guarded([&](std::string* error) -> int {
+        if (path == nullptr || out == nullptr) {
+            *error = "gguf: path or output pointer is NULL";
+            return ET_ERR_INVALID;
+        }
+        *out = nullptr;
+        et::gguf::Error failure;
+        et::gguf::File* file = et::gguf::open(path, cancel, &failure);
+        if (file == nullptr) {
+            const int status = gguf_failure(failure);
+            *error = failure.message;
+            return status;
+        }
+        *out = reinterpret_cast<et_gguf*>(file);
+        return ET_OK;
+    });
+}
+
+}  // extern "C"
+namespace {
+const et::gguf::File* as_file(const et_gguf* file) { return reinterpret_cast<const et::gguf::File*>(file); }
+const et::gguf::Entry* entry_at(const et_gguf* file, uint64_t index) {
+    return file != nullptr && index < as_file(file)->metadata.size() ? &as_file(file)->metadata[index] : nullptr;
+}
+}  // namespace
+extern "C" {
+
+void et_hip_gguf_close(et_gguf* file) { delete reinterpret_cast<et::gguf::File*>(file); }
+const char* et_hip_gguf_architecture(const et_gguf* file) { return file ? as_file(file)->architecture.c_str() : ""; }
+uint64_t et_hip_gguf_metadata_count(const et_gguf* file) { return file ? as_file(file)->metadata.size() : 0; }
+int64_t et_hip_gguf_metadata_find(const et_gguf* file, const char* key) {
+    if (file == nullptr || key == nullptr) return -1;
+    const auto& metadata = as_file(file)->metadata;
+    for (size_t i = 0; i < metadata.size(); i++)
+        if (metadata[i].key == key) return static_cast<int64_t>(i);
+    return -1;
+}
+const char* et_hip_gguf_metadata_key(const et_gguf* file, uint64_t index) {
+    const auto* entry = entry_at(file, index);
+    return entry ? entry->key.c_str() : nullptr;
+}
+uint64_t et_hip_gguf_metadata_key_length(const et_gguf* file, uint64_t index) {
+    const auto* entry = entry_at(file, index);
+    return entry ? entry->key.size() : 0;
+}
+int32_t et_hip_gguf_metadata_type(const et_gguf* file, uint64_t index) {
+    const auto* entry = entry_at(file, index);
+    return entry ? static_cast<int32_t>(entry->value.type) : -1;
+}
+int32_t et_hip_gguf_metadata_element_type(const et_gguf* file, uint64_t index) {
+    const auto* entry = entry_at(file, index);
+    if (entry == nullptr) return -1;
+    return static_cast<int32_t>(entry->value.type == 9 ? entry->value.element_type : entry->value.type);
+}
+uint64_t et_hip_gguf_metadata_length(const et_gguf* file, uint64_t index) {
+    const auto* entry = entry_at(file, index);
+    return entry ? entry->value.length() : 0;
+}
+int et_hip_gguf_metadata_unsigned(const et_gguf* file, uint64_t index, uint64_t element, uint64_t* out) {
+    const auto* entry = entry_at(file, index);
+    if (entry == nullptr || out == nullptr || element >= entry->value.integers.size()) return ET_ERR_INVALID;
+    *out = entry->value.integers[element];
+    return ET_OK;
+}
+int et_hip_gguf_metadata_signed(const et_gguf* file, uint64_t index, uint64_t element, int64_t* out) {
+    const auto* entry = entry_at(file, index);
+    if (entry == nullptr || out == nullptr || element >= entry->value.signed_integers.size()) return ET_ERR_INVALID;
+    *out = entry->value.signed_integers[element];
+    return ET_OK;
+}
+int et_hip_gguf_metadata_real(const et_gguf* file, uint64_t index, uint64_t element, double* out) {
+    const auto* entry = entry_at(file, index);
+    if (entry == nullptr || out == nullptr || element >= entry->value.reals.size()) return ET_ERR_INVALID;
+    *out = entry->value.reals[element];
+    return ET_OK;
+}
+const char* et_hip_gguf_metadata_string(const et_gguf* file, uint64_t index, uint64_t element, uint64_t* length) {
+    const auto* entry = entry_at(file, index);
+    if (entry == nullptr || element >= entry->value.strings.size()) return nullptr;
+    if (length != nullptr) *length = entry->value.strings[element].size();
+    return entry->value.strings[element].c_str();
+}
+
+uint64_t et_hip_gguf_tensor_count(const et_gguf* file) { return file ? as_file(file)->tensors.size() : 0; }
+int64_t et_hip_gguf_tensor_find(const et_gguf* file, const char* name) {
+    if (file == nullptr || name == nullptr) return -1;
+    const auto& tensors = as_file(file)->tensors;
+    for (size_t i = 0; i < tensors.size(); i++)
+        if (tensors[i].name == name) return static_cast<int64_t>(i);
+    return -1;
+}
+int et_hip_gguf_tensor_at(const et_gguf* file, uint64_t index, et_gguf_tensor* out) {
+    if (file == nullptr || out == nullptr || index >= as_file(file)->tensors.size())
+        return set_error(ET_ERR_INVALID, "gguf: tensor index out of range");
+    const et::gguf::Tensor& tensor = as_file(file)->tensors[index];
+    std::memset(out, 0, sizeof *out);
+    out->name = tensor.name.c_str();
+    out->name_length = tensor.name.size();
+    out->format = static_cast<int32_t>(tensor.format);
+    out->logical_rank = static_cast<int32_t>(tensor.logical_shape.size());
+    for (size_t d = 0; d < tensor.logical_shape.size(); d++) out->logical_shape[d] = tensor.logical_shape[d];
+    out->physical_rank = static_cast<int32_t>(tensor.physical_shape.size());
+    for (size_t d = 0; d < tensor.physical_shape.size(); d++) out->physical_shape[d] = tensor.physical_shape[d];
+    out->data_offset = tensor.data_offset;
+    out->byte_len = tensor.byte_len;
+    return ET_OK;
+}
+
+int et_hip_gguf_read_tensor_into(const et_gguf* file, uint64_t index, void* destination,
+                                 uint64_t destination_bytes, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (file == nullptr || index >= as_file(file)->tensors.size() || (destination == nullptr && destination_bytes != 0)) {
+            *error = "gguf: file, tensor index or destination is invalid";
+            return ET_ERR_INVALID;
+        }
+        et::gguf::Error failure;
+        if (et::gguf::read_tensor(*as_file(file), as_file(file)->tensors[index], destination, destination_bytes, cancel,
+                                  &failure))
+            return ET_OK;
+        const int status = gguf_failure(failure);
+        *error = failure.message;
+        return status;
+    });
+}
+
+int et_hip_gguf_upload_tensor(et_gguf* file, uint64_t index, void* device_destination,
+                              uint64_t destination_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (file == nullptr || index >= as_file(file)->tensors.size() ||
+            (device_destination == nullptr && destination_bytes != 0)) {
+            *error = "gguf: file, tensor index or destination is invalid";
+            return ET_ERR_INVALID;
+        }
+        auto* owner = reinterpret_cast<et::gguf::File*>(file);
+        et::gguf::Error failure;
+        if (et::gguf::upload_tensor(*owner, owner->tensors[index], device_destination, destination_bytes, stream, cancel,
+                                    &failure))
+            return ET_OK;
+        const int status = gguf_failure(failure);
+        *error = failure.message;
+        return status;
     });
 }
 

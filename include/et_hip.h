@@ -315,6 +315,66 @@ int et_hip_gather_rows_into(const et_tensor* table, const et_tensor* indexes,
                             const et_tensor* destination, void* status, void* stream);
 int et_hip_gather_rows_status_check(uint64_t table_rows, uint64_t count, const void* status_host);
 
+/* ---- GGUF v3 files: the on-disk format that feeds the contraction ----------
+ *
+ * = parse_gguf / read_gguf_tensor_into (crates/runtime/src/gguf.rs:682-957,
+ * :959-994): the header is parsed with the reference's validation, resource
+ * limits and messages ("gguf: ..."); tensor payloads are validated for range and
+ * overlap, not read. Beyond the reference's F32 and K-quant tensors, GGML type
+ * codes 2 (Q4_0) and 8 (Q8_0) are accepted. Host calls; only the upload touches
+ * the device. */
+typedef struct et_gguf et_gguf; /* opaque; owns the open file */
+
+/* ET_ERR_UNSUPPORTED = the file violates the format or a limit
+ * (GgufParseError::Invalid), ET_ERR_EXECUTION = I/O failed, ET_ERR_CANCELLED. */
+int et_hip_gguf_open(const char* path, const volatile int32_t* cancel, et_gguf** out);
+void et_hip_gguf_close(et_gguf* file);
+const char* et_hip_gguf_architecture(const et_gguf* file); /* general.architecture */
+
+/* The metadata table in file order. Types are the GGUF value type codes: 0 u8, 1 i8,
+ * 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool, 8 string, 9 array, 10 u64, 11 i64, 12 f64. */
+uint64_t et_hip_gguf_metadata_count(const et_gguf* file);
+int64_t et_hip_gguf_metadata_find(const et_gguf* file, const char* key); /* index or -1 */
+const char* et_hip_gguf_metadata_key(const et_gguf* file, uint64_t index);
+uint64_t et_hip_gguf_metadata_key_length(const et_gguf* file, uint64_t index); /* bytes; a key may hold NULs */
+int32_t et_hip_gguf_metadata_type(const et_gguf* file, uint64_t index);
+int32_t et_hip_gguf_metadata_element_type(const et_gguf* file, uint64_t index); /* arrays, else = type */
+uint64_t et_hip_gguf_metadata_length(const et_gguf* file, uint64_t index);      /* elements; 1 for a scalar */
+/* Element `element` of entry `index`: unsigned / bool, signed, real (f32 widened exactly) or
+ * string (not NUL-terminated inside: `*length` bytes). Non-zero when the entry is of another kind. */
+int et_hip_gguf_metadata_unsigned(const et_gguf* file, uint64_t index, uint64_t element, uint64_t* out);
+int et_hip_gguf_metadata_signed(const et_gguf* file, uint64_t index, uint64_t element, int64_t* out);
+int et_hip_gguf_metadata_real(const et_gguf* file, uint64_t index, uint64_t element, double* out);
+const char* et_hip_gguf_metadata_string(const et_gguf* file, uint64_t index, uint64_t element,
+                                        uint64_t* length);
+
+/* GgufTensorDescriptor (gguf.rs:319-341). */
+typedef struct {
+    const char* name;
+    uint64_t name_length;      /* bytes */
+    int32_t format;            /* GGML type code: 0 F32, 2 Q4_0, 8 Q8_0, 10..14 Q2_K..Q6_K (= et_codec) */
+    int32_t logical_rank;
+    uint64_t logical_shape[4]; /* row-major */
+    int32_t physical_rank;     /* F32: the logical shape; quantized: [rows, encoded_row_bytes] */
+    uint64_t physical_shape[4];
+    uint64_t data_offset;      /* absolute file offset */
+    uint64_t byte_len;
+} et_gguf_tensor;
+uint64_t et_hip_gguf_tensor_count(const et_gguf* file);
+int64_t et_hip_gguf_tensor_find(const et_gguf* file, const char* name); /* index or -1 */
+int et_hip_gguf_tensor_at(const et_gguf* file, uint64_t index, et_gguf_tensor* out);
+
+/* = read_gguf_tensor_into (gguf.rs:959-994): exactly byte_len bytes into host memory. */
+int et_hip_gguf_read_tensor_into(const et_gguf* file, uint64_t index, void* destination,
+                                 uint64_t destination_bytes, const volatile int32_t* cancel);
+/* The same bytes into DEVICE memory: 8 MiB positioned reads into two pinned buffers (allocated
+ * at the first upload, owned by the file object) alternate with asynchronous copies on `stream`;
+ * returns when the tensor is in place. A quantized tensor arrives as the [rows,
+ * encoded_row_bytes] u8 matrix et_hip_linear_requirements takes as `weight`. */
+int et_hip_gguf_upload_tensor(et_gguf* file, uint64_t index, void* device_destination,
+                              uint64_t destination_bytes, void* stream,
+                              const volatile int32_t* cancel);
+
 /* ---- int8 activation quantiser (stage 1 of ET_ACT_INT8) ------------------- */
 
 /* The activation quantiser on its own, exposed so that tests can check the
