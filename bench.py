@@ -571,6 +571,115 @@ def llama_decode(args, et):
     print(json.dumps(result))
 
 
+def gguf_upload(args, et):
+    """Workload ``gguf_upload``: a synthetic GGUF v3 file with the tensor catalog of a Llama-3-8B Q4_K
+    model (291 tensors; ``--layers`` of them carry payloads, the default 4 make a 0.5 GB file) is
+    written to a temporary directory, parsed, and every tensor is uploaded into device memory. A step
+    = the upload of the whole file; the parse is timed separately. Bound by the host side (page cache
+    read + pinned staging + PCIe), not by HBM."""
+    import struct
+    import tempfile
+    import numpy as np
+    import torch
+    from effect_torch_amd import synth
+
+    device = torch.device("cuda:0")
+    layers = min(args.layers, 32)
+    rng = np.random.default_rng(5)
+    hidden, kv, ffn, vocab = 4096, 1024, 14336, 128256
+
+    def gstr(text):
+        raw = text.encode()
+        return struct.pack("<Q", len(raw)) + raw
+
+    catalog = [("token_embd.weight", (hidden, vocab), 12)]
+    for i in range(layers):
+        catalog += [(f"blk.{i}.attn_norm.weight", (hidden,), 0), (f"blk.{i}.attn_q.weight", (hidden, hidden), 12),
+                    (f"blk.{i}.attn_k.weight", (hidden, kv), 12), (f"blk.{i}.attn_v.weight", (hidden, kv), 12),
+                    (f"blk.{i}.attn_output.weight", (hidden, hidden), 12), (f"blk.{i}.ffn_norm.weight", (hidden,), 0),
+                    (f"blk.{i}.ffn_gate.weight", (hidden, ffn), 12), (f"blk.{i}.ffn_up.weight", (hidden, ffn), 12),
+                    (f"blk.{i}.ffn_down.weight", (ffn, hidden), 12)]
+    catalog += [("output_norm.weight", (hidden,), 0)]
+    sizes = [(int(np.prod(d)) * 4 if code == 0 else int(np.prod(d)) // 256 * 144) for _, d, code in catalog]
+    offsets, cursor = [], 0
+    for size in sizes:
+        offsets.append(cursor)
+        cursor = -(-(cursor + size) // 32) * 32
+    vocabulary = [f"token{i}" for i in range(vocab)]
+    meta = [gstr("general.architecture") + struct.pack("<I", 8) + gstr("llama"),
+            gstr("general.quantization_version") + struct.pack("<II", 4, 2),
+            gstr("llama.block_count") + struct.pack("<II", 4, layers),
+            gstr("tokenizer.ggml.tokens") + struct.pack("<IIQ", 9, 8, vocab) + b"".join(gstr(t) for t in vocabulary)]
+    head = b"GGUF" + struct.pack("<IQQ", 3, len(catalog), len(meta)) + b"".join(meta)
+    for (name, dims, code), offset in zip(catalog, offsets):
+        head += gstr(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+        head += struct.pack("<IQ", code, offset)
+    head += b"\0" * (-len(head) % 32)
+    block = rng.integers(0, 256, 64 << 20, dtype=np.uint8).tobytes()
+    with tempfile.TemporaryDirectory() as folder:
+        path = os.path.join(folder, "model.gguf")
+        with open(path, "wb") as out:
+            out.write(head)
+            written = 0
+            while written < cursor:
+                piece = block[: min(len(block), cursor - written)]
+                out.write(piece)
+                written += len(piece)
+        file_bytes = len(head) + cursor
+        import ctypes
+        from effect_torch_amd import _native
+        handle = ctypes.c_void_p()
+        t0 = time.perf_counter()
+        assert _native.lib().et_hip_gguf_open(path.encode(), None, ctypes.byref(handle)) == 0, _native.last_error()
+        parse_seconds = time.perf_counter() - t0
+        _native.lib().et_hip_gguf_close(handle)
+        model = et.GgufFile.open(path)
+        assert len(model.tensors) == len(catalog) and model.get("tokenizer.ggml.tokens").value[5] == "token5"
+        buffers = {t.name: torch.empty(t.physical_shape if t.format else t.logical_shape,
+                                       dtype=torch.uint8 if t.format else torch.float32, device=device)
+                   for t in model.tensors}
+
+        def step():
+            for t in model.tensors:
+                model.upload_tensor(t.name, device, buffers[t.name])
+
+        step()
+        probe = model.tensors[2]
+        assert np.array_equal(buffers[probe.name].cpu().numpy().reshape(-1),
+                              np.frombuffer(model.read_tensor(probe.name).tobytes(), dtype=np.uint8))
+        for _ in range(max(args.warmup, 0)):
+            step()
+        torch.cuda.synchronize()
+        steps = max(1, min(args.steps, 5))
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - t0) / steps
+        t0 = time.perf_counter()
+        host = np.empty(max(sizes), dtype=np.uint8)
+        for t in model.tensors:
+            model.read_tensor(t.name, host[: t.byte_len])
+        read_seconds = time.perf_counter() - t0
+        model.close()
+    gbs = cursor / seconds / 1e9
+    print(json.dumps({
+        "metric": "gguf_upload GB/s", "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"gguf_upload: {len(catalog)} tensors of a Llama-3-8B Q4_K catalog ({layers} layers), "
+                               f"{file_bytes} file bytes, vocabulary of {vocab} strings in the metadata",
+                   "parse_ms": round(parse_seconds * 1e3, 3), "host_read_GBps": round(cursor / read_seconds / 1e9, 2),
+                   "path": "page cache -> 2 x 8 MiB pinned staging -> hipMemcpyAsync -> HBM"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 5), "traffic": None,
+                     "note": "bound by the host link and the file read, not by HBM",
+                     "algorithmic_bytes_per_launch": cursor, "avg_launch_us": round(seconds * 1e6, 1)},
+        "cpu_baseline": {"value": round(cursor / read_seconds / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+                         "sample": "the same tensors read into host memory (read_gguf_tensor_into), one pass"},
+    }))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -590,6 +699,11 @@ def main():
     if args.workload in DECODE_OPS:
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return decode_op(args, et)
+    if args.workload == "gguf_upload":
+        assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
+        if args.layers == 32:
+            args.layers = 4
+        return gguf_upload(args, et)
     if args.workload == "llama3_8b_batched_decode":
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return llama_decode(args, et)
@@ -598,7 +712,7 @@ def main():
         return kv_decode(args, et)
     if args.workload not in synth.CONFIGS:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
-                 "or calibrate_read / calibrate_copy / kv_attention_decode / llama3_8b_batched_decode / " + " / ".join(DECODE_OPS))
+                 "or calibrate_read / calibrate_copy / kv_attention_decode / llama3_8b_batched_decode / gguf_upload / " + " / ".join(DECODE_OPS))
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")

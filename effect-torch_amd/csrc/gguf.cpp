@@ -110,6 +110,9 @@ struct Reader {
     uint64_t file_len;
     uint64_t position = 0;
     const volatile int32_t* cancel;
+    // read-ahead window: the header is a long run of small fields
+    std::vector<char> window;
+    uint64_t window_start = 0;
 
     void check_cancelled() const {
         if (cancel != nullptr && *cancel != 0) throw Stop{Failure::kCancelled, ""};
@@ -124,20 +127,34 @@ struct Reader {
         auto* out = static_cast<char*>(output);
         uint64_t done = 0;
         while (done < length) {
-            check_cancelled();
-            const uint64_t chunk = std::min(kHeaderReadChunkBytes, length - done);
-            uint64_t got = 0;
-            while (got < chunk) {
-                const ssize_t n = pread(fd, out + done + got, chunk - got, static_cast<off_t>(position + got));
-                if (n < 0) {
-                    if (errno == EINTR) continue;
-                    io_failed(std::strerror(errno));
-                }
-                if (n == 0) io_failed("failed to fill whole buffer");
-                got += static_cast<uint64_t>(n);
+            if (position < window_start || position >= window_start + window.size()) {
+                check_cancelled();  // once per chunk of header I/O
+                fill_window();
             }
+            const uint64_t at = position - window_start;
+            const uint64_t chunk = std::min<uint64_t>(window.size() - at, length - done);
+            std::memcpy(out + done, window.data() + at, chunk);
             done += chunk;
             position += chunk;
+        }
+    }
+    void fill_window() {
+        const uint64_t want = std::min(kHeaderReadChunkBytes, file_len - position);  // > 0: the caller checked
+        window.resize(want);
+        window_start = position;
+        uint64_t got = 0;
+        while (got < want) {
+            const ssize_t n = pread(fd, window.data() + got, want - got, static_cast<off_t>(position + got));
+            if (n < 0) {
+                if (errno == EINTR) continue;
+                window.clear();
+                io_failed(std::strerror(errno));
+            }
+            if (n == 0) {
+                window.clear();
+                io_failed("failed to fill whole buffer");
+            }
+            got += static_cast<uint64_t>(n);
         }
     }
     template <class T>
@@ -446,7 +463,7 @@ File* open(const char* path, const volatile int32_t* cancel, Error* error) {
         if (fstat(file->fd, &info) != 0) io_failed(std::strerror(errno));
         file->file_len = static_cast<uint64_t>(info.st_size);
         if (cancel != nullptr && *cancel != 0) throw Stop{Failure::kCancelled, ""};
-        Reader reader{file->fd, file->file_len, 0, cancel};
+        Reader reader{file->fd, file->file_len, 0, cancel, {}, 0};
         parse(reader, file);
         return file;
     } catch (const Stop& stop) {

@@ -400,3 +400,46 @@ def test_int8_full_size_prefill_row_ranges(et, device):
         want = oracle.linear_q8_rows(cfg["codec"], cfg["rows"], cfg["columns"], q, scale, total, weight,
                                      None, begin, begin + 16)
         close(got[:, begin:begin + 16], want[:, begin:begin + 16])
+
+
+def test_gguf_file_to_contraction(et, device, tmp_path):
+    # a GGUF file with Q4_K, Q8_0 and F32 tensors: parse, upload, contract - the file's bytes are the weights
+    import struct
+    from gguf_builder import build, entry
+    rng = np.random.default_rng(77)
+    rows, columns = 300, 1024
+    w4 = synth.random_weight(oracle.Q4_K, rows, columns, rng)
+    w8 = synth.random_weight(oracle.Q8_0, 70, 512, rng)
+    dense = rng.standard_normal((5, 33)).astype(np.float32)
+    big = rng.integers(0, 256, (20 << 20) + 144, dtype=np.uint8)  # more than two staging buffers
+    big = big[: big.size // 144 * 144]
+    tensors, payloads, cursor = [], {}, 0
+    for name, dims, code, data in (("blk.0.ffn_up.weight", (columns, rows), 12, w4.tobytes()),
+                                   ("blk.0.attn_q.weight", (512, 70), 8, w8.tobytes()),
+                                   ("norm.weight", (33, 5), 0, dense.tobytes()),
+                                   ("big.weight", (256, big.size // 144), 12, big.tobytes())):
+        cursor = -(-cursor // 32) * 32
+        tensors.append(dict(name=name, dimensions=list(dims), format=code, offset=cursor, bytes=len(data)))
+        payloads[name] = data
+        cursor += len(data)
+    data, _ = build([entry("general.quantization_version", "u32", 2), entry("llama.block_count", "u32", 1)],
+                    tensors, architecture="llama", payloads=payloads)
+    path = tmp_path / "model.gguf"
+    path.write_bytes(data)
+    with et.GgufFile.open(str(path)) as model:
+        assert model.architecture == "llama" and model.get("llama.block_count").value == 1
+        up = model.tensor("blk.0.ffn_up.weight")
+        assert up.format_name == "Q4_K" and up.logical_shape == (rows, columns) and up.physical_shape == (rows, 576)
+        weight = model.upload_tensor("blk.0.ffn_up.weight", device)
+        assert np.array_equal(weight.cpu().numpy(), w4)
+        x = synth.random_activations(9, columns, rng)
+        y = et.quantized_linear(to_dev(x, device), weight, None, et.GgmlQuant(up.format), up.logical_shape)
+        close(y.cpu().numpy(), oracle.linear_into(oracle.Q4_K, rows, columns, x, w4, None))
+        q = model.upload_tensor("blk.0.attn_q.weight", device)
+        x = synth.random_activations(2, 512, rng)
+        y = et.quantized_linear(to_dev(x, device), q, None, et.GgmlQuant.Q8_0, (70, 512))
+        close(y.cpu().numpy(), oracle.linear_into(oracle.Q8_0, 70, 512, x, w8, None))
+        assert np.array_equal(model.upload_tensor("norm.weight", device).cpu().numpy(), dense)
+        assert np.array_equal(model.upload_tensor("big.weight", device).cpu().numpy().reshape(-1), big)
+        with pytest.raises(et.GgufParseError, match="requires 38080 destination bytes, got 300"):
+            model.upload_tensor("blk.0.attn_q.weight", device, torch.empty(300, dtype=torch.uint8, device=device))
