@@ -1,4 +1,4 @@
-// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q4_0, Q8_0; 1-4 vectors):
+// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q6_K, Q4_0, Q8_0; 1-3 vectors):
 //     y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r])
 //
 // Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499)
@@ -44,6 +44,9 @@ struct XLimbs {
                       // limb 0 is the least significant (weight 1), limb 2 the most (65536)
     float s;          // value of one unit of limb 0
     float sum[2];     // exact f32 sums of elements 0..31 and 32..63
+    // Codecs whose lanes own four separate 16-column runs (Q6_K) use these instead of s / sum:
+    float s_pair[2];  // unit of runs 0, 1 and of runs 2, 3 (they lie in two 64-column chunks)
+    int bias[4][3];   // -32 * (sum of the limb bytes of run g): where the integer dots start
 };
 
 constexpr float kLimbRange = 8323072.0f;  // 127 * 2^16: |X| <= this
@@ -138,6 +141,10 @@ __device__ __forceinline__ float limb_value(const XLimbs& x, int d0, int d1, int
 // ---------------------------------------------------------------------------
 
 struct Q4KLimb {
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_limbs(stage, lane, active, out);
+    }
     struct Lane {
         uint32_t offset;  // byte offset of the lane's block within a row
         uint32_t p;       // pair within the block
@@ -220,6 +227,10 @@ struct __attribute__((packed, aligned(4))) Dwords17 {
 
 // Q4_0: two 18-byte blocks = 36 bytes = 9 dwords (dword aligned when columns % 64 == 0).
 struct Q40Limb {
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_limbs(stage, lane, active, out);
+    }
     struct Lane {
         uint32_t offset;
     };
@@ -274,6 +285,10 @@ struct Q40Limb {
 
 // Q8_0: two 34-byte blocks = 68 bytes = 17 dwords (dword aligned when columns % 64 == 0).
 struct Q80Limb {
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_limbs(stage, lane, active, out);
+    }
     struct Lane {
         uint32_t offset;
     };
@@ -314,6 +329,122 @@ struct Q80Limb {
         for (int m = 0; m < M; m++)
             value[m] = da * limb_value(x[m], da_[m][0], da_[m][1], da_[m][2]) +
                        db * limb_value(x[m], db_[m][0], db_[m][1], db_[m][2]);
+    }
+};
+
+// Sixteen bytes from an address that is only 2-byte aligned (odd Q6_K blocks start at 210 * b).
+#pragma clang diagnostic ignored "-Walign-mismatch"
+typedef uint4 __attribute__((aligned(2))) uint4_a2;
+typedef uint2 __attribute__((aligned(2))) uint2_a2;
+
+// Q6_K (decode_q6_k, crates/runtime-cpu/src/quantized.rs:238-261): 210 bytes per 256 values -
+// ql[128] low nibbles, qh[64] two high bits, scales[16] int8 per 16 values, d. Value e = half*128 +
+// quarter*32 + i of a block is d * scale[half*8 + quarter*2 + i/16] * (q - 32) with
+// q = nibble(ql[half*64 + (quarter & 1)*32 + i], quarter >> 1) | ((qh[half*32 + i] >> 2*quarter) & 3) << 4.
+// A lane takes (half, j = i / 16) of a block: the four 16-column runs quarter = 0..3, each with ONE
+// scale, out of exactly 48 bytes of quants - three 16-byte loads, nothing read twice. Its 64 columns
+// are not consecutive, so it gathers its activation limbs run by run (load_activations).
+struct Q6KLimb {
+    struct Lane {
+        uint32_t offset;  // byte offset of the lane's block within a row
+        uint32_t half, j;
+    };
+    struct Data {
+        uint4 qa, qb, qh;  // ql[half*64 + 16j ..], ql[half*64 + 32 + 16j ..], qh[half*32 + 16j ..]
+        uint2 scales;      // scales[half*8 .. half*8 + 8]
+        uint32_t d;        // f16 bits
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 8) * 210u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) {
+        return Lane{(chunk >> 2) * 210u, (chunk >> 1) & 1u, chunk & 1u};
+    }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        const uint8_t* base = row + lane.offset;
+        data.qa = *reinterpret_cast<const uint4_a2*>(base + 64u * lane.half + 16u * lane.j);
+        data.qb = *reinterpret_cast<const uint4_a2*>(base + 64u * lane.half + 32u + 16u * lane.j);
+        data.qh = *reinterpret_cast<const uint4_a2*>(base + 128u + 32u * lane.half + 16u * lane.j);
+        data.scales = *reinterpret_cast<const uint2_a2*>(base + 192u + 8u * lane.half);
+        data.d = *reinterpret_cast<const uint16_t*>(base + 208u);
+    }
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        // run g of lane (block b, half, j) is 16-column unit 16b + 8*half + 2g + j of the slice
+        const uint32_t first = 16u * (lane >> 2) + 8u * ((lane >> 1) & 1u) + (lane & 1u);
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint4 v = *reinterpret_cast<const uint4*>(&stage.limbs[k][limb_slot(first + 2u * g) * 4u]);
+                const int words[4] = {static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z),
+                                      static_cast<int>(v.w)};
+                int total = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    out.limb[k][4 * g + i] = active ? words[i] : 0;
+                    total = __builtin_amdgcn_sdot4(0x01010101, out.limb[k][4 * g + i], total, false);
+                }
+                out.bias[g][k] = -32 * total;
+            }
+        }
+        const uint32_t chunk = 4u * (lane >> 2) + 2u * ((lane >> 1) & 1u);
+        out.s_pair[0] = active ? stage.unit[chunk] : 0.f;
+        out.s_pair[1] = active ? stage.unit[chunk + 1u] : 0.f;
+        out.s = 0.f;
+        out.sum[0] = out.sum[1] = 0.f;
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
+                                                const XLimbs (&x)[M], float (&value)[M]) {
+        const uint32_t qa[4] = {data.qa.x, data.qa.y, data.qa.z, data.qa.w};
+        const uint32_t qb[4] = {data.qb.x, data.qb.y, data.qb.z, data.qb.w};
+        const uint32_t qh[4] = {data.qh.x, data.qh.y, data.qh.z, data.qh.w};
+        int dot[M][4][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) dot[m][g][k] = x[m].bias[g][k];  // sum (q - 32) x = sum q x - 32 sum x
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t low = (g & 1) ? qb[i] : qa[i];
+                const uint32_t nibbles = ((g & 2) ? (low >> 4) : low) & 0x0f0f0f0fu;
+                const uint32_t high = (qh[i] >> (2 * g)) & 0x03030303u;
+                const int q = static_cast<int>((high << 4) | nibbles);  // four values 0..63
+#pragma unroll
+                for (int m = 0; m < M; m++)
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        dot[m][g][k] = __builtin_amdgcn_sdot4(q, x[m].limb[k][4 * g + i], dot[m][g][k], false);
+            }
+        }
+        // scale of run g: signed byte j + 2g of the eight
+        const uint32_t shift = 8u * lane.j;
+        const auto signed_byte = [](uint32_t word, uint32_t at) {
+            return static_cast<float>(static_cast<int>(static_cast<int8_t>(word >> at)));
+        };
+        const float sc[4] = {signed_byte(data.scales.x, shift), signed_byte(data.scales.x, shift + 16u),
+                             signed_byte(data.scales.y, shift), signed_byte(data.scales.y, shift + 16u)};
+        const float d = half_bits_to_float(data.d);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float part[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                // the dots are below 2^21 in magnitude and convert exactly
+                float limb_sum[3];
+#pragma unroll
+                for (int k = 0; k < 3; k++)
+                    limb_sum[k] = fmaf(sc[2 * h + 1], static_cast<float>(dot[m][2 * h + 1][k]),
+                                       sc[2 * h] * static_cast<float>(dot[m][2 * h][k]));
+                part[h] = fmaf(65536.0f, limb_sum[2], fmaf(256.0f, limb_sum[1], limb_sum[0]));
+            }
+            value[m] = d * fmaf(x[m].s_pair[1], part[1], x[m].s_pair[0] * part[0]);
+        }
     }
 };
 
@@ -410,7 +541,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
         __syncthreads();
         if (s == slice) {
 #pragma unroll
-            for (int m = 0; m < M; m++) load_limbs(stage[m], lane_id, active, xr[m]);
+            for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -569,9 +700,15 @@ hipError_t launch_vectors(const uint8_t* weight, const float* x, uint64_t x_row_
 
 }  // namespace
 
+uint32_t gemv_limb_max_vectors(int32_t codec) {
+    // Q6_K keeps 62 registers of activation state per vector (48 limb words, 12 dot offsets, 2 units):
+    // three vectors do not fit next to the rows in flight.
+    return codec == kQ6_K ? 2u : kGemvLimbMaxVectors;
+}
+
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors) {
-    if (vectors == 0 || vectors > kGemvLimbMaxVectors || columns == 0 || columns > 65536u) return false;
-    if (codec == kQ4_K) return columns % 256 == 0;
+    if (vectors == 0 || vectors > gemv_limb_max_vectors(codec) || columns == 0 || columns > 65536u) return false;
+    if (codec == kQ4_K || codec == kQ6_K) return columns % 256 == 0;
     if (codec == kQ4_0 || codec == kQ8_0) return columns % 64 == 0;
     return false;
 }
@@ -582,6 +719,10 @@ hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint6
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
     switch (codec) {
         case kQ4_K: return launch_vectors<Q4KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ6_K:
+            if (vectors == 1) return launch_slices<Q6KLimb, 1>(weight, x, x_row_stride, bias, y, n, k, stream);
+            if (vectors == 2) return launch_slices<Q6KLimb, 2>(weight, x, x_row_stride, bias, y, n, k, stream);
+            return hipErrorInvalidValue;
         case kQ4_0: return launch_vectors<Q40Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         case kQ8_0: return launch_vectors<Q80Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         default: return hipErrorInvalidValue;

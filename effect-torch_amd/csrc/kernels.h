@@ -36,6 +36,7 @@ hipError_t gather_f32(const float* src, const IndexLayout& layout, uint64_t coun
 // y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r]) for v < vectors; f32-accurate.
 // x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
 constexpr uint32_t kGemvLimbMaxVectors = 3;
+uint32_t gemv_limb_max_vectors(int32_t codec);  // per launch: 3, or 2 for Q6_K
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors);
 hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,

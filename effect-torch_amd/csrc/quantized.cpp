@@ -132,8 +132,8 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
                             codec_name(plan->codec));
         plan_matrix_core(LinearKernel::kGemmI8, 1);
     } else if (plan->activation_mode == ET_ACT_F32) {
-        const uint32_t limb_launch = static_cast<uint32_t>(
-            plan->vectors < kGemvLimbMaxVectors ? plan->vectors : kGemvLimbMaxVectors);
+        const uint32_t limb_most = gemv_limb_max_vectors(plan->codec);
+        const uint32_t limb_launch = static_cast<uint32_t>(plan->vectors < limb_most ? plan->vectors : limb_most);
         if (plan->vectors >= kGemmMinVectors && gemm_i8_supported(plan->codec, plan->columns)) {
             plan_matrix_core(LinearKernel::kGemmLimb, 3);
         } else if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {

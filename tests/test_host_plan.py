@@ -55,6 +55,8 @@ def test_linear_plan_shapes(et):
         assert plan3.kernel == "gemv_limb"
     assert plan.algorithmic_bytes == 7 * 288 + 4 * 10 * 512 + 4 * 10 * 7 + 4 * 7
     plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 210), None, et.GgmlQuant.Q6_K, (2, 256))
+    assert plan.kernel == "gemv_limb"
+    plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 176), None, et.GgmlQuant.Q5_K, (2, 256))
     assert plan.kernel == "gemv_generic"
     plan = et.linear_requirements(torch.zeros(64, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256),
                                   et.ActivationMode.INT8)
