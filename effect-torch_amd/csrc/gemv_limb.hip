@@ -1,4 +1,4 @@
-// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q6_K, Q4_0, Q8_0; 1-3 vectors):
+// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q5_K, Q6_K, Q4_0, Q8_0; 1-3 vectors):
 //     y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r])
 //
 // Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499)
@@ -180,6 +180,94 @@ struct Q4KLimb {
             // low nibbles: elements 4j..4j+3 of sub-block 2p; high nibbles: of sub-block 2p+1
             const int ql = static_cast<int>(w[j] & 0x0f0f0f0fu);
             const int qh = static_cast<int>((w[j] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    lo[m][k] = __builtin_amdgcn_sdot4(ql, x[m].limb[k][j], lo[m][k], false);
+                    hi[m][k] = __builtin_amdgcn_sdot4(qh, x[m].limb[k][8 + j], hi[m][k], false);
+                }
+        }
+        // (scale, min) of sub-blocks 2p, 2p+1: crates/runtime-cpu/src/quantized.rs:77-86
+        const uint32_t shift = (lane.p & 1u) * 16u;
+        const uint32_t a = data.header.y >> shift, b = data.header.z >> shift, c = data.header.w >> shift;
+        uint32_t sc, mn;
+        if (lane.p < 2) {
+            sc = a & 0x3f3fu;
+            mn = b & 0x3f3fu;
+        } else {
+            sc = (c & 0x0f0fu) | ((a >> 2) & 0x3030u);
+            mn = ((c >> 4) & 0x0f0fu) | ((b >> 2) & 0x3030u);
+        }
+        const float sc_lo = static_cast<float>(sc & 0xffu), sc_hi = static_cast<float>((sc >> 8) & 0xffu);
+        const float m_lo = static_cast<float>(mn & 0xffu), m_hi = static_cast<float>((mn >> 8) & 0xffu);
+        const float d = half_bits_to_float(data.header.x & 0xffffu);
+        const float dmin = half_bits_to_float(data.header.x >> 16);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            // sub-block scales first, limb weights second, one f32 scale last
+            // (as floats: the dots are below 2^17 and convert exactly; a 32-bit
+            // integer multiply would run at quarter rate)
+            const float i1 = fmaf(sc_hi, static_cast<float>(hi[m][0]), sc_lo * static_cast<float>(lo[m][0]));
+            const float i2 = fmaf(sc_hi, static_cast<float>(hi[m][1]), sc_lo * static_cast<float>(lo[m][1]));
+            const float i3 = fmaf(sc_hi, static_cast<float>(hi[m][2]), sc_lo * static_cast<float>(lo[m][2]));
+            const float pos = x[m].s * fmaf(65536.0f, i3, fmaf(256.0f, i2, i1));
+            const float neg = fmaf(m_lo, x[m].sum[0], m_hi * x[m].sum[1]);
+            value[m] = d * pos - dmin * neg;
+        }
+    }
+};
+
+// Q5_K (decode_q5_k, crates/runtime-cpu/src/quantized.rs:203-234): Q4_K's layout with a fifth bit per
+// value in qh[32] between the scales and the nibbles - bit g of qh[i] belongs to element i of
+// sub-block g. 176 bytes per block, every field 16-byte aligned.
+struct Q5KLimb {
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_limbs(stage, lane, active, out);
+    }
+    struct Lane {
+        uint32_t offset;  // byte offset of the lane's block within a row
+        uint32_t p;       // pair within the block
+    };
+    struct Data {
+        uint4 header;  // d, dmin, scales[12]
+        uint4 h[2];    // qh[32]: the fifth bits of all eight sub-blocks
+        uint4 q[2];    // the pair's 32 bytes of nibbles
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 8) * 176u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) {
+        return Lane{(chunk >> 2) * 176u, chunk & 3u};
+    }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        const uint8_t* base = row + lane.offset;
+        data.header = *reinterpret_cast<const uint4*>(base);
+        data.h[0] = *reinterpret_cast<const uint4*>(base + 16);
+        data.h[1] = *reinterpret_cast<const uint4*>(base + 32);
+        data.q[0] = *reinterpret_cast<const uint4*>(base + 48 + 32 * lane.p);
+        data.q[1] = *reinterpret_cast<const uint4*>(base + 64 + 32 * lane.p);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
+                                                const XLimbs (&x)[M], float (&value)[M]) {
+        const uint32_t w[8] = {data.q[0].x, data.q[0].y, data.q[0].z, data.q[0].w,
+                               data.q[1].x, data.q[1].y, data.q[1].z, data.q[1].w};
+        const uint32_t h[8] = {data.h[0].x, data.h[0].y, data.h[0].z, data.h[0].w,
+                               data.h[1].x, data.h[1].y, data.h[1].z, data.h[1].w};
+        const uint32_t bit = 2u * lane.p;  // sub-blocks 2p and 2p + 1
+        int lo[M][3], hi[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int k = 0; k < 3; k++) lo[m][k] = hi[m][k] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            // low nibbles: elements 4j..4j+3 of sub-block 2p; high nibbles: of sub-block 2p+1
+            const uint32_t fifth = h[j] >> bit;
+            const int ql = static_cast<int>((w[j] & 0x0f0f0f0fu) | ((fifth & 0x01010101u) << 4));
+            const int qh = static_cast<int>(((w[j] >> 4) & 0x0f0f0f0fu) | ((fifth & 0x02020202u) << 3));
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
@@ -708,7 +796,7 @@ uint32_t gemv_limb_max_vectors(int32_t codec) {
 
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors) {
     if (vectors == 0 || vectors > gemv_limb_max_vectors(codec) || columns == 0 || columns > 65536u) return false;
-    if (codec == kQ4_K || codec == kQ6_K) return columns % 256 == 0;
+    if (codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) return columns % 256 == 0;
     if (codec == kQ4_0 || codec == kQ8_0) return columns % 64 == 0;
     return false;
 }
@@ -719,6 +807,7 @@ hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint6
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
     switch (codec) {
         case kQ4_K: return launch_vectors<Q4KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ5_K: return launch_vectors<Q5KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         case kQ6_K:
             if (vectors == 1) return launch_slices<Q6KLimb, 1>(weight, x, x_row_stride, bias, y, n, k, stream);
             if (vectors == 2) return launch_slices<Q6KLimb, 2>(weight, x, x_row_stride, bias, y, n, k, stream);

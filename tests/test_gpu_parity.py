@@ -443,3 +443,23 @@ def test_gguf_file_to_contraction(et, device, tmp_path):
         assert np.array_equal(model.upload_tensor("big.weight", device).cpu().numpy().reshape(-1), big)
         with pytest.raises(et.GgufParseError, match="requires 38080 destination bytes, got 300"):
             model.upload_tensor("blk.0.attn_q.weight", device, torch.empty(300, dtype=torch.uint8, device=device))
+
+
+@pytest.mark.parametrize("codec", [oracle.Q5_K, oracle.Q6_K])
+@pytest.mark.parametrize("vectors", [1, 2, 5])
+def test_k_quant_gemv_at_full_size(et, device, codec, vectors):
+    # the integer-dot GEMV for the other K-quants at 14336 x 4096: a row range against the oracle,
+    # and linearity in x over all rows
+    rng = np.random.default_rng(900 + codec + vectors)
+    rows, columns = 14336, 4096
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
+                                  None, et.GgmlQuant(codec), (rows, columns))
+    assert plan.kernel == "gemv_limb"
+    got = run_linear(et, device, codec, rows, columns, x, weight)
+    for start in (0, rows - 128):
+        want = oracle.linear_rows(codec, rows, columns, x, weight, None, start, start + 128)[:, start:start + 128]
+        close(got[:, start:start + 128], want)
+    doubled = run_linear(et, device, codec, rows, columns, 2.0 * x, weight)
+    assert np.array_equal(doubled, 2.0 * got)  # scaling by two is exact in every step
