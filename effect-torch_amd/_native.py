@@ -95,6 +95,9 @@ SIGNATURES = {
     "et_hip_linear_into": (ctypes.c_int, [_vp, _T, _T, _T, _T, _vp, _u64, _vp, _vp]),
     "et_hip_linear_plan_create": (ctypes.c_int, [_i32, _u64, _u64, _u64, _i32, _i32, _PP]),
     "et_hip_linear_enqueue": (ctypes.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
+    "et_hip_linear_plan_prepared_input_bytes": (_u64, [_vp]),
+    "et_hip_linear_prepare_input": (ctypes.c_int, [_vp, _vp, _u64, _vp, _u64, _vp]),
+    "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
     "et_hip_embedding_plan_destroy": (None, [_vp]),
     "et_hip_embedding_plan_output_rank": (_i32, [_vp]),

@@ -188,6 +188,34 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
     });
 }
 
+uint64_t et_hip_linear_plan_prepared_input_bytes(const et_linear_plan* plan) {
+    return plan ? et::quantized::prepared_input_bytes(*plan) : 0;
+}
+
+int et_hip_linear_prepare_input(const et_linear_plan* plan, const float* x, uint64_t x_row_stride, void* prepared,
+                                uint64_t prepared_bytes, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_prepare_input(*plan, x, x_row_stride, prepared, prepared_bytes, stream, error);
+    });
+}
+
+int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepared, const uint8_t* weight,
+                                   const float* bias, const float* residual, float* y, void* workspace,
+                                   uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_enqueue_prepared(*plan, prepared, weight, bias, residual, y, workspace,
+                                                      workspace_bytes, stream, cancel, error);
+    });
+}
+
 int et_hip_embedding_requirements(const et_tensor* indexes, const et_tensor* weight, int32_t codec,
                                   uint64_t rows, uint64_t columns, et_embedding_plan** out) {
     return guarded([&](std::string* error) -> int {

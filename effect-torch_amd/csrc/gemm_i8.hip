@@ -146,7 +146,7 @@ struct Shape {
 template <int CODEC, int MT, int LIMBS, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint8_t* __restrict__ weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
-    const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
+    const float* __restrict__ bias, const float* residual, float* y, uint32_t rows, uint32_t columns,
     uint32_t vectors, uint32_t row_tiles, uint32_t vector_groups, uint32_t k_splits,
     float* __restrict__ partials) {
     using S = Shape<CODEC, MT, LIMBS, AX, AW>;
@@ -428,9 +428,11 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 value += exchange[((((k - 1) * kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane];
             const uint32_t m = m0 + 32u * t + 8u * (r >> 2) + 4u * half + (r & 3u);
             if (n_out < rows && m < vectors) {
-                if (k_splits == 1)
-                    y[static_cast<uint64_t>(m) * rows + n_out] = value + bias_value;
-                else
+                if (k_splits == 1) {
+                    // residual may be y itself: every output is read, then written, by this lane only
+                    const uint64_t at = static_cast<uint64_t>(m) * rows + n_out;
+                    y[at] = residual != nullptr ? (value + bias_value) + residual[at] : value + bias_value;
+                } else
                     partials[(static_cast<uint64_t>(k_share) * vectors + m) * rows + n_out] = value;
             }
         }
@@ -442,10 +444,12 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t columns, uint64_t vectors);
 namespace {
 
-// y[m, n] = bias[n] + sum over the K shares, in share order; four outputs per thread.
+// y[m, n] = bias[n] + sum over the K shares, in share order (+ residual[m, n], which may be y
+// itself); four outputs per thread.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ partials,
-                                                              const float* __restrict__ bias, float* __restrict__ y,
-                                                              uint32_t rows, uint64_t outputs, uint32_t k_splits) {
+                                                              const float* __restrict__ bias, const float* residual,
+                                                              float* y, uint32_t rows, uint64_t outputs,
+                                                              uint32_t k_splits) {
     const uint64_t i = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
     if (i >= outputs) return;
     if (rows % 4 == 0) {
@@ -458,19 +462,29 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
             total.z += part.z;
             total.w += part.w;
         }
+        if (residual != nullptr) {
+            const float4 r = *reinterpret_cast<const float4*>(residual + i);
+            total.x += r.x;
+            total.y += r.y;
+            total.z += r.z;
+            total.w += r.w;
+        }
         *reinterpret_cast<float4*>(y + i) = total;
     } else {
         for (uint64_t j = i; j < min(i + 4, outputs); j++) {
             float total = bias != nullptr ? bias[j % rows] : 0.f;
             for (uint32_t k = 0; k < k_splits; k++) total += partials[k * outputs + j];
-            y[j] = total;
+            y[j] = residual != nullptr ? total + residual[j] : total;
         }
     }
 }
 
 template <int CODEC, int MT, int LIMBS, int AX, int AW>
-hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y,
-                  uint32_t rows, uint32_t columns, uint32_t vectors, float* partials, hipStream_t stream) {
+hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out, uint32_t rows,
+                  uint32_t columns, uint32_t vectors, hipStream_t stream) {
+    const float* bias = out.bias;
+    float* y = out.y;
+    float* partials = out.partials;
     using S = Shape<CODEC, MT, LIMBS, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, AX, AW>;
@@ -493,13 +507,13 @@ hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const float* bias
     const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_groups * k_splits;
     if (grid > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream,
-                       weight, tiles, vector_tiles, bias, y, rows, columns, vectors, row_tiles,
+                       weight, tiles, vector_tiles, bias, out.residual, y, rows, columns, vectors, row_tiles,
                        vector_groups, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
     if (k_splits > 1) {
         const uint64_t outputs = static_cast<uint64_t>(vectors) * rows;
         hipLaunchKernelGGL(reduce_partials_kernel, dim3(static_cast<uint32_t>((outputs + 1023) / 1024)), dim3(256), 0,
-                           stream, partials, bias, y, rows, outputs, k_splits);
+                           stream, partials, bias, out.residual, y, rows, outputs, k_splits);
     }
     return hipGetLastError();
 }
@@ -520,30 +534,29 @@ constexpr int weight_lead() {
 }
 
 template <int CODEC, int MT, int LIMBS, int AX>
-hipError_t launch_shape(const uint8_t* weight, const uint8_t* tiles, const float* bias, float* y, float* partials,
-                        uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+hipError_t launch_shape(const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out, uint32_t rows,
+                        uint32_t columns, uint32_t vectors, hipStream_t stream) {
     constexpr int kWeightLead = weight_lead<CODEC, MT, LIMBS, AX>();
     static_assert(kWeightLead >= 1, "no room for a weight ring");
-    return launch<CODEC, MT, LIMBS, AX, kWeightLead>(weight, tiles, bias, y, rows, columns, vectors, partials, stream);
+    return launch<CODEC, MT, LIMBS, AX, kWeightLead>(weight, tiles, out, rows, columns, vectors, stream);
 }
 
 template <int CODEC>
-hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const float* bias,
-                        float* y, float* partials, uint32_t rows, uint32_t columns, uint32_t vectors,
-                        hipStream_t stream) {
+hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
+                        uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
     // Activations: 26 KiB per stage and 32-vector tile with three limbs, 10 KiB with one; two
     // stages of lead. The weight ring (9 to 20 KiB per stage) takes the rest of LDS.
     // One 32-vector tile per workgroup with three limbs: two tiles of three-limb results do not
     // fit in registers. Q4_K carries a second accumulator (the min term): at most two tiles.
     // (tiles_per_workgroup() below states the same choice for the launch geometry.)
     if (limbs == 3)
-        return launch_shape<CODEC, 1, 3, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
+        return launch_shape<CODEC, 1, 3, 2>(weight, tiles, out, rows, columns, vectors, stream);
     if (vectors <= 32)
-        return launch_shape<CODEC, 1, 1, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
+        return launch_shape<CODEC, 1, 1, 2>(weight, tiles, out, rows, columns, vectors, stream);
     if (vectors <= 64 || CODEC == kQ4_K)
-        return launch_shape<CODEC, 2, 1, 2>(weight, tiles, bias, y, partials, rows, columns, vectors, stream);
-    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, bias, y, partials,
-                                                                                rows, columns, vectors, stream);
+        return launch_shape<CODEC, 2, 1, 2>(weight, tiles, out, rows, columns, vectors, stream);
+    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, out, rows, columns,
+                                                                                vectors, stream);
 }
 
 uint32_t tiles_per_workgroup(int32_t codec, int limbs, uint64_t vectors) {
@@ -574,15 +587,15 @@ uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t colu
 }
 
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
-                   const float* bias, float* y, float* partials, uint64_t rows, uint64_t columns,
-                   uint64_t vectors, hipStream_t stream) {
+                   const GemmOutput& out, uint64_t rows, uint64_t columns, uint64_t vectors,
+                   hipStream_t stream) {
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns),
                    m = static_cast<uint32_t>(vectors);
     switch (codec) {
-        case kQ8_0: return launch_codec<kQ8_0>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
-        case kQ4_0: return launch_codec<kQ4_0>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
-        case kQ4_K: return launch_codec<kQ4_K>(limbs, weight, tiles, bias, y, partials, n, k, m, stream);
+        case kQ8_0: return launch_codec<kQ8_0>(limbs, weight, tiles, out, n, k, m, stream);
+        case kQ4_0: return launch_codec<kQ4_0>(limbs, weight, tiles, out, n, k, m, stream);
+        case kQ4_K: return launch_codec<kQ4_K>(limbs, weight, tiles, out, n, k, m, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -78,9 +78,15 @@ constexpr uint32_t kGemmMinVectors = 7;
 // Launches with few output tiles share K out over this many workgroups per tile (1 = no sharing);
 // `partials` then holds k_splits * vectors * rows floats. partials == nullptr: never share.
 uint32_t gemm_i8_k_splits(int32_t codec, int limbs, uint64_t rows, uint64_t columns, uint64_t vectors);
+struct GemmOutput {
+    const float* bias;      // [rows] or null
+    const float* residual;  // [vectors, rows] added to the result, or null; may be y itself
+    float* y;               // [vectors, rows]
+    float* partials;        // see gemm_i8_k_splits, or null
+};
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
-                   const float* bias, float* y, float* partials, uint64_t rows, uint64_t columns,
-                   uint64_t vectors, hipStream_t stream);
+                   const GemmOutput& out, uint64_t rows, uint64_t columns, uint64_t vectors,
+                   hipStream_t stream);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch

@@ -312,6 +312,59 @@ int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint6
                                activation_mode, plan, error);
 }
 
+namespace {
+bool on_matrix_cores(const et_linear_plan& plan) {
+    return plan.kernel == LinearKernel::kGemmI8 || plan.kernel == LinearKernel::kGemmLimb;
+}
+int limbs_of(const et_linear_plan& plan) { return plan.kernel == LinearKernel::kGemmI8 ? 1 : 3; }
+}  // namespace
+
+uint64_t prepared_input_bytes(const et_linear_plan& plan) {
+    return on_matrix_cores(plan) ? tile_workspace_bytes(limbs_of(plan), plan.vectors, plan.columns) : 0;
+}
+
+int linear_prepare_input(const et_linear_plan& plan, const float* x, uint64_t x_row_stride, void* prepared,
+                         uint64_t prepared_bytes, void* stream, std::string* error) {
+    if (!on_matrix_cores(plan))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: this plan's kernel takes the activations as they are");
+    if (prepared == nullptr || prepared_bytes < prepared_input_bytes(plan))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: prepared-input buffer of " + std::to_string(prepared_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(prepared_input_bytes(plan)) +
+                                                 " required");
+    if (x == nullptr || reinterpret_cast<uintptr_t>(x) % 16 != 0 || x_row_stride % 4 != 0 || x_row_stride < plan.columns ||
+        reinterpret_cast<uintptr_t>(prepared) % 16 != 0)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
+    if (hipError_t status = quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs_of(plan),
+                                           static_cast<uint8_t*>(prepared), as_stream(stream)))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
+int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
+                            const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
+                            const volatile int32_t* cancel, std::string* error) {
+    if (!on_matrix_cores(plan))
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: this plan's kernel takes the activations as they are");
+    if ((bias != nullptr) != plan.has_bias)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias does not match the immutable plan");
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (prepared == nullptr || weight == nullptr || y == nullptr)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: NULL operand");
+    float* partials = nullptr;
+    if (plan.k_splits > 1) {
+        if (workspace == nullptr || workspace_bytes < plan.workspace_bytes)
+            return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                                                     " bytes is smaller than the planned " +
+                                                     std::to_string(plan.workspace_bytes));
+        partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + plan.partial_offset);
+    }
+    if (hipError_t status = gemm_i8(plan.codec, limbs_of(plan), weight, static_cast<const uint8_t*>(prepared),
+                                    GemmOutput{bias, residual, y, partials}, plan.rows, plan.columns, plan.vectors,
+                                    as_stream(stream)))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
 int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
                    const uint8_t* weight, const float* bias, float* y, void* workspace,
                    uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
@@ -359,8 +412,8 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
                 quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs, tiles, s))
             return hip_failure(error, "quantized_linear", status);
         float* partials = plan.k_splits > 1 ? reinterpret_cast<float*>(scratch + plan.partial_offset) : nullptr;
-        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, bias, y, partials, plan.rows,
-                                        plan.columns, plan.vectors, s))
+        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, GemmOutput{bias, nullptr, y, partials},
+                                        plan.rows, plan.columns, plan.vectors, s))
             return hip_failure(error, "quantized_linear", status);
         return ET_OK;
     }

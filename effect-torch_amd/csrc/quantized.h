@@ -88,6 +88,16 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
                    uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
                    std::string* error);
 
+// The quantised form of the activations a matrix-core plan consumes, made once and shared by every
+// plan of the same columns, vectors and activation mode; 0 bytes when the plan's kernel reads x itself.
+uint64_t prepared_input_bytes(const et_linear_plan& plan);
+int linear_prepare_input(const et_linear_plan& plan, const float* x, uint64_t x_row_stride, void* prepared,
+                         uint64_t prepared_bytes, void* stream, std::string* error);
+// y = W x (+ bias) (+ residual, which may be y itself) from a prepared input.
+int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
+                            const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
+                            const volatile int32_t* cancel, std::string* error);
+
 int embedding_requirements(const TensorView& indexes, const TensorView& weight, int32_t codec,
                            uint64_t rows, uint64_t columns, et_embedding_plan* plan,
                            std::string* error);

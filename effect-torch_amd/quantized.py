@@ -327,6 +327,30 @@ class RawLinear:
                                              cancelled.ptr if cancelled is not None else None))
 
 
+    @property
+    def prepared_input_bytes(self) -> int:
+        """Bytes of the shared quantised activations this plan consumes; 0 = it reads x itself."""
+        return int(N.lib().et_hip_linear_plan_prepared_input_bytes(self.requirements._handle))
+
+    def prepare_input(self, x: torch.Tensor, prepared: torch.Tensor, stream=None) -> None:
+        _check(N.lib().et_hip_linear_prepare_input(self.requirements._handle, x.data_ptr(), x.stride(0),
+                                                   prepared.data_ptr(), prepared.numel() * prepared.element_size(),
+                                                   _stream_handle(stream)))
+
+    def enqueue_prepared(self, prepared: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                         y: torch.Tensor, workspace: Optional[torch.Tensor] = None,
+                         residual: Optional[torch.Tensor] = None, stream=None,
+                         cancelled: Optional[CancellationFlag] = None) -> None:
+        """``y = W x (+ bias) (+ residual)`` from activations prepared once by any plan of the same
+        columns, vectors and activation mode; ``residual`` may be ``y``."""
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+        _check(N.lib().et_hip_linear_enqueue_prepared(
+            self.requirements._handle, prepared.data_ptr(), weight.data_ptr(),
+            bias.data_ptr() if bias is not None else None, residual.data_ptr() if residual is not None else None,
+            y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
+
+
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""
     assert sink.numel() >= 4 * workgroups and sink.element_size() == 4

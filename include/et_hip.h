@@ -162,6 +162,22 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
                           const uint8_t* weight, const float* bias, float* y, void* workspace,
                           uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel);
 
+/* Contractions that share their activations (q / k / v, gate / up of a decode step) can share the
+ * quantised form the matrix-core kernels consume: prepare it once, then enqueue every plan of the
+ * same columns, vectors and activation mode from it. `residual` (dense [vectors, rows], may be y
+ * itself) is added to the result in the kernel's epilogue, which saves the separate sum of a
+ * residual connection. Only plans whose kernel runs on the matrix cores have a prepared form
+ * (et_hip_linear_plan_prepared_input_bytes > 0); the others return ET_ERR_UNSUPPORTED here and
+ * use et_hip_linear_enqueue. No counterpart in the reference, whose executor runs one operator
+ * at a time. */
+uint64_t et_hip_linear_plan_prepared_input_bytes(const et_linear_plan* plan);
+int et_hip_linear_prepare_input(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
+                                void* prepared, uint64_t prepared_bytes, void* stream);
+int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepared,
+                                   const uint8_t* weight, const float* bias, const float* residual,
+                                   float* y, void* workspace, uint64_t workspace_bytes, void* stream,
+                                   const volatile int32_t* cancel);
+
 /* ---- quantized_embedding (= bit-exact dequantisation of selected rows) ---- */
 
 /* Plan step = embedding_requirements (crates/runtime-cpu/src/quantized.rs:340-365).

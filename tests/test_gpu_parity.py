@@ -463,3 +463,40 @@ def test_k_quant_gemv_at_full_size(et, device, codec, vectors):
         close(got[:, start:start + 128], want)
     doubled = run_linear(et, device, codec, rows, columns, 2.0 * x, weight)
     assert np.array_equal(doubled, 2.0 * got)  # scaling by two is exact in every step
+
+
+@pytest.mark.parametrize("mode", ["F32", "INT8"])
+def test_shared_prepared_input_and_residual_epilogue(et, device, mode):
+    # q / k / v style: one quantisation of the activations feeds plans of different row counts; the
+    # residual rides in the epilogue. Every result has the bits of the unfused sequence.
+    rng = np.random.default_rng(61)
+    columns, vectors = 4096, 32
+    act = et.ActivationMode[mode]
+    x = to_dev(synth.random_activations(vectors, columns, rng), device)
+    plans, prepared = {}, None
+    for rows in (4096, 1024, 14336):  # K shares of 4, 16 and none
+        plans[rows] = et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors, rows == 1024, act)
+    sizes = {p.prepared_input_bytes for p in plans.values()}
+    assert len(sizes) == 1 and sizes.pop() > 0
+    prepared = torch.empty(plans[4096].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[1024].prepare_input(x, prepared)  # any of the plans may prepare it
+    for rows, plan in plans.items():
+        weight = to_dev(synth.random_weight(oracle.Q4_K, rows, columns, rng), device)
+        bias = to_dev(rng.standard_normal(rows).astype(np.float32), device) if rows == 1024 else None
+        workspace = torch.empty(max(plan.requirements.workspace_bytes, 16), dtype=torch.uint8, device=device)
+        plain = torch.empty(vectors, rows, device=device)
+        plan.enqueue(x, weight, bias, plain, workspace)
+        shared = torch.empty_like(plain)
+        plan.enqueue_prepared(prepared, weight, bias, shared, workspace)
+        assert torch.equal(plain, shared)
+        residual = torch.randn(vectors, rows, device=device)
+        fused = torch.empty_like(plain)
+        plan.enqueue_prepared(prepared, weight, bias, fused, workspace, residual=residual)
+        assert torch.equal(fused, plain + residual)
+        stream = residual.clone()  # in place, as a residual stream is updated
+        plan.enqueue_prepared(prepared, weight, bias, stream, workspace, residual=stream)
+        assert torch.equal(stream, plain + residual)
+    small = et.RawLinear(et.GgmlQuant.Q4_K, 64, columns, 2, False, et.ActivationMode.F32)
+    assert small.prepared_input_bytes == 0
+    with pytest.raises(et.QuantizedError, match="takes the activations as they are"):
+        small.prepare_input(x[:2], prepared)
