@@ -38,7 +38,7 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # script; the runs and their figures are in profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md.
 MEASURED_TRAFFIC = {("q4_k_gemv_14336x4096", 1, "f32"): 33338900,
                     # attend kernel; profiles/kv_attend_decode_32slots_ctx2048_f16.md
-                    ("kv_attention_decode", 2048): 271028400}
+                    ("kv_attention_decode", 2048): 270009600}
 
 
 def parse_args():

@@ -119,6 +119,7 @@ struct KvAttention {
 };
 struct KvLaunchShape {
     bool streaming;
+    int waves;  // per workgroup of the streaming kernel: 4 or 8
     uint32_t splits;
     uint64_t workgroups;
     uint64_t workspace_bytes;

@@ -30,8 +30,6 @@
 namespace et {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
 constexpr uint32_t kNoBlock = 0xffffffffu;
 constexpr float kLowest = -1.0e30f;  // "no score yet": finite, so that exp2(kLowest - m) = 0 without NaN
 
@@ -356,10 +354,14 @@ __device__ __forceinline__ void merge_splits(const KvArgs& a, uint64_t query, ui
 
 // Streaming kernel. LPT lanes share one position (each holds Piece<T>::kDims of the width,
 // width == LPT * kDims), so a wave covers 64 / LPT positions per load and the workgroup
-// 4 * 64 / LPT; U such loads are in flight per step. G query heads of one kv head are
-// served from the same K / V registers.
-template <typename T, int LPT, int G, int U>
-__global__ __launch_bounds__(kThreads) void kv_attend_kernel(const KvArgs a) {
+// WAVES * 64 / LPT; U such loads are in flight per step. G query heads of one kv head are
+// served from the same K / V registers. WAVES = 8 when the launch has enough rows of queries to give
+// every compute unit a workgroup without splitting the context (no partial records, no merge
+// launch), else 4.
+template <typename T, int LPT, int G, int U, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
+    constexpr int kWaves = WAVES;
+    constexpr int kThreads = 64 * WAVES;
     constexpr int DPL = Piece<T>::kDims;
     constexpr int PPW = 64 / LPT;        // positions per wave per load
     constexpr int PPG = kWaves * PPW;    // per workgroup per load
@@ -640,28 +642,31 @@ __global__ void kv_merge_kernel(const KvArgs a) {
 }
 
 template <typename T, int LPT, int G>
-hipError_t launch_streaming(const KvArgs& a, uint32_t workgroups, hipStream_t stream) {
+hipError_t launch_streaming(const KvArgs& a, uint32_t workgroups, int waves, hipStream_t stream) {
     constexpr int U = G >= 8 ? 2 : 4;
-    hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U>), dim3(workgroups), dim3(kThreads), 0, stream, a);
+    if (waves == 8)
+        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
+    else
+        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4>), dim3(workgroups), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
 template <typename T, int LPT>
-hipError_t launch_streaming_group(const KvArgs& a, int g, uint32_t workgroups, hipStream_t stream) {
+hipError_t launch_streaming_group(const KvArgs& a, int g, uint32_t workgroups, int waves, hipStream_t stream) {
     switch (g) {
-        case 8: return launch_streaming<T, LPT, 8>(a, workgroups, stream);
-        case 4: return launch_streaming<T, LPT, 4>(a, workgroups, stream);
-        case 2: return launch_streaming<T, LPT, 2>(a, workgroups, stream);
-        default: return launch_streaming<T, LPT, 1>(a, workgroups, stream);
+        case 8: return launch_streaming<T, LPT, 8>(a, workgroups, waves, stream);
+        case 4: return launch_streaming<T, LPT, 4>(a, workgroups, waves, stream);
+        case 2: return launch_streaming<T, LPT, 2>(a, workgroups, waves, stream);
+        default: return launch_streaming<T, LPT, 1>(a, workgroups, waves, stream);
     }
 }
 
 template <typename T>
-hipError_t launch_streaming_width(const KvArgs& a, int g, uint32_t workgroups, hipStream_t stream) {
+hipError_t launch_streaming_width(const KvArgs& a, int g, uint32_t workgroups, int waves, hipStream_t stream) {
     switch (a.width / Piece<T>::kDims) {
-        case 32: return launch_streaming_group<T, 32>(a, g, workgroups, stream);
-        case 16: return launch_streaming_group<T, 16>(a, g, workgroups, stream);
-        default: return launch_streaming_group<T, 8>(a, g, workgroups, stream);
+        case 32: return launch_streaming_group<T, 32>(a, g, workgroups, waves, stream);
+        case 16: return launch_streaming_group<T, 16>(a, g, workgroups, waves, stream);
+        default: return launch_streaming_group<T, 8>(a, g, workgroups, waves, stream);
     }
 }
 
@@ -677,9 +682,9 @@ int streaming_group(const KvAttention& p) {
     return 1;
 }
 
-uint32_t positions_per_step(const KvAttention& p, int g) {
+uint32_t positions_per_step(const KvAttention& p, int g, int waves) {
     const uint32_t lanes = p.width / (p.slab_is_f16 ? 8 : 4);
-    return kWaves * (64 / lanes) * (g >= 8 ? 2 : 4);
+    return waves * (64 / lanes) * (g >= 8 ? 2 : 4);
 }
 
 }  // namespace
@@ -693,11 +698,15 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     // Enough workgroups for every compute unit several times over, and no split shorter than
     // a few steps; the block list of a split must fit the kernel's table.
     const uint64_t context = p.max_context == 0 ? 1 : p.max_context;
-    const uint64_t step = shape.streaming ? positions_per_step(p, g) : 64;
+    // A compute unit keeps eight waves of the streaming kernel resident: two workgroups of four, or
+    // one of eight. With all workgroups resident at once none waits for a second round (measured for 32
+    // slots x 8 kv heads at context 2048: 512 x 4 waves 58.9 us, 1024 x 4 waves 63.7, 256 x 8 waves
+    // without any split - no partial records, no merge launch - 55.6). Eight waves need enough rows
+    // of queries to go round without splitting.
+    shape.waves = shape.streaming && rows >= 128 ? 8 : 4;
+    const uint64_t step = shape.streaming ? positions_per_step(p, g, shape.waves) : 64;
     uint64_t splits = 1;
-    // The streaming kernel keeps two workgroups per compute unit resident; with all of them
-    // resident at once no workgroup waits for a second round (measured: 512 beat 1024 and 2048).
-    const uint64_t wanted = shape.streaming ? 512 : 4096;
+    const uint64_t wanted = shape.streaming ? (shape.waves == 8 ? 256 : 512) : 4096;
     if (rows < wanted) splits = shape.streaming ? wanted / (rows == 0 ? 1 : rows)
                                                 : (wanted + rows - 1) / (rows == 0 ? 1 : rows);
     const uint64_t most = (context + 2 * step - 1) / (2 * step);
@@ -762,8 +771,8 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     if (shape.streaming) {
         const int g = streaming_group(p);
         error = p.slab_is_f16
-                    ? launch_streaming_width<__half>(a, g, static_cast<uint32_t>(shape.workgroups), stream)
-                    : launch_streaming_width<float>(a, g, static_cast<uint32_t>(shape.workgroups), stream);
+                    ? launch_streaming_width<__half>(a, g, static_cast<uint32_t>(shape.workgroups), shape.waves, stream)
+                    : launch_streaming_width<float>(a, g, static_cast<uint32_t>(shape.workgroups), shape.waves, stream);
     } else {
         if (p.slab_is_f16)
             hipLaunchKernelGGL(kv_attend_any_kernel<__half>, dim3(static_cast<uint32_t>(shape.workgroups)),

@@ -93,6 +93,25 @@ def test_streaming_kernel_shapes(et, device, dtype, lanes, group, kv_heads):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("lanes", [8, 16, 32])
+@pytest.mark.parametrize("group", [1, 4, 8])
+def test_eight_wave_workgroups_without_context_splits(et, device, dtype, lanes, group):
+    # 256 rows of queries: one eight-wave workgroup per (slot, kv head), no partial records
+    width = lanes * (4 if dtype == np.float32 else 8)
+    rng = np.random.default_rng(7000 + 100 * lanes + group)
+    slots, kv_heads = 32, 8
+    contexts = rng.integers(0, 150, slots)
+    contexts[:2] = [0, 600]
+    case = make_case(rng, slots=slots, query_heads=group * kv_heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=contexts, tokens=1, advances=[1] * slots, dtype=dtype)
+    scale = 1.0 / np.sqrt(width)
+    got = run_gpu(et, device, case, scale)
+    assert et.kv_attention_kernel(got[3], group * kv_heads, 1) == "kv_attend"
+    assert et.kv_attention_workspace_bytes(got[3], group * kv_heads, 1) == 0
+    compare(got, run_oracle(case, scale))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("block_size", [1, 5, 16, 64])
 @pytest.mark.parametrize("tokens,advances", [(1, [1, 1, 1, 1]), (4, [4, 1, 3, 2])])
 def test_paging_chunks_and_ragged_advances(et, device, dtype, block_size, tokens, advances):

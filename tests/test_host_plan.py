@@ -210,8 +210,13 @@ def test_kv_attention_launch_shapes_and_status_wording(et):
     from effect_torch_amd import _native
     decode = _kv_layer(et, torch, slots=32, kv_heads=8, width=128, max_tokens=32 * 2048, block_size=16,
                        dtype=torch.float16, max_context=2048)
-    assert et.kv_attention_kernel(decode, 32, 1) == "kv_attend+kv_merge"
-    assert et.kv_attention_workspace_bytes(decode, 32, 1) % (32 * 32 * 130 * 4) == 0
+    # 256 rows of queries: one eight-wave workgroup per compute unit, the context is not split
+    assert et.kv_attention_kernel(decode, 32, 1) == "kv_attend"
+    assert et.kv_attention_workspace_bytes(decode, 32, 1) == 0
+    few = _kv_layer(et, torch, slots=4, kv_heads=8, width=128, max_tokens=4 * 2048, block_size=16,
+                    dtype=torch.float16, max_context=2048)
+    assert et.kv_attention_kernel(few, 32, 1) == "kv_attend+kv_merge"
+    assert et.kv_attention_workspace_bytes(few, 32, 1) % (4 * 32 * 130 * 4) == 0
     short = _kv_layer(et, torch, slots=512, kv_heads=8, width=128, max_tokens=4096, block_size=16,
                       dtype=torch.float16, max_context=8)
     assert et.kv_attention_kernel(short, 32, 1) == "kv_attend"
