@@ -1,4 +1,4 @@
-// Dequant-GEMV on integer dot products for gfx950 (Q4_K, Q5_K, Q6_K, Q4_0, Q8_0; 1-3 vectors):
+// Dequant-GEMV on integer dot products for gfx950 (the five K-quants, Q4_0, Q8_0; 1-3 vectors):
 //     y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r])
 //
 // Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499)
@@ -46,7 +46,8 @@ struct XLimbs {
     float sum[2];     // exact f32 sums of elements 0..31 and 32..63
     // Codecs whose lanes own four separate 16-column runs (Q6_K) use these instead of s / sum:
     float s_pair[2];  // unit of runs 0, 1 and of runs 2, 3 (they lie in two 64-column chunks)
-    int bias[4][3];   // -32 * (sum of the limb bytes of run g): where the integer dots start
+    int bias[4][3];   // -offset * (sum of the limb bytes of run g): where the integer dots start
+    float run_sum[4]; // sum of the (quantised) activations of run g, for codecs with block minima
 };
 
 constexpr float kLimbRange = 8323072.0f;  // 127 * 2^16: |X| <= this
@@ -425,6 +426,44 @@ struct Q80Limb {
 typedef uint4 __attribute__((aligned(2))) uint4_a2;
 typedef uint2 __attribute__((aligned(2))) uint2_a2;
 
+// Activations of a lane that owns four 16-column runs of a 256-column block (Q2_K, Q3_K, Q6_K):
+// lane (block b, half, j) takes runs g = 0..3 = 16-column units 16b + 8*half + 2g + j of the slice.
+// OFFSET is what the codec subtracts from every quant: the integer dots start at -OFFSET * (sum of
+// the run's limb bytes), so that sum (q - OFFSET) x needs no per-row work.
+template <int OFFSET>
+__device__ __forceinline__ void load_run_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                     XLimbs& out) {
+    const uint32_t first = 16u * (lane >> 2) + 8u * ((lane >> 1) & 1u) + (lane & 1u);
+    int totals[4][3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint4 v = *reinterpret_cast<const uint4*>(&stage.limbs[k][limb_slot(first + 2u * g) * 4u]);
+            const int words[4] = {static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z),
+                                  static_cast<int>(v.w)};
+            int total = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out.limb[k][4 * g + i] = active ? words[i] : 0;
+                total = __builtin_amdgcn_sdot4(0x01010101, out.limb[k][4 * g + i], total, false);
+            }
+            totals[g][k] = total;
+            out.bias[g][k] = -OFFSET * total;
+        }
+    }
+    const uint32_t chunk = 4u * (lane >> 2) + 2u * ((lane >> 1) & 1u);
+    out.s_pair[0] = active ? stage.unit[chunk] : 0.f;
+    out.s_pair[1] = active ? stage.unit[chunk + 1u] : 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+        out.run_sum[g] = out.s_pair[g >> 1] * fmaf(65536.0f, static_cast<float>(totals[g][2]),
+                                                   fmaf(256.0f, static_cast<float>(totals[g][1]),
+                                                        static_cast<float>(totals[g][0])));
+    out.s = 0.f;
+    out.sum[0] = out.sum[1] = 0.f;
+}
+
 // Q6_K (decode_q6_k, crates/runtime-cpu/src/quantized.rs:238-261): 210 bytes per 256 values -
 // ql[128] low nibbles, qh[64] two high bits, scales[16] int8 per 16 values, d. Value e = half*128 +
 // quarter*32 + i of a block is d * scale[half*8 + quarter*2 + i/16] * (q - 32) with
@@ -458,29 +497,7 @@ struct Q6KLimb {
     }
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
-        // run g of lane (block b, half, j) is 16-column unit 16b + 8*half + 2g + j of the slice
-        const uint32_t first = 16u * (lane >> 2) + 8u * ((lane >> 1) & 1u) + (lane & 1u);
-#pragma unroll
-        for (int k = 0; k < 3; k++) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&stage.limbs[k][limb_slot(first + 2u * g) * 4u]);
-                const int words[4] = {static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z),
-                                      static_cast<int>(v.w)};
-                int total = 0;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    out.limb[k][4 * g + i] = active ? words[i] : 0;
-                    total = __builtin_amdgcn_sdot4(0x01010101, out.limb[k][4 * g + i], total, false);
-                }
-                out.bias[g][k] = -32 * total;
-            }
-        }
-        const uint32_t chunk = 4u * (lane >> 2) + 2u * ((lane >> 1) & 1u);
-        out.s_pair[0] = active ? stage.unit[chunk] : 0.f;
-        out.s_pair[1] = active ? stage.unit[chunk + 1u] : 0.f;
-        out.s = 0.f;
-        out.sum[0] = out.sum[1] = 0.f;
+        load_run_activations<32>(stage, lane, active, out);
     }
     template <int M>
     static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
@@ -533,6 +550,178 @@ struct Q6KLimb {
             }
             value[m] = d * fmaf(x[m].s_pair[1], part[1], x[m].s_pair[0] * part[0]);
         }
+    }
+};
+
+// s_pair[0] * (limb-combined, scale-weighted dots of runs 0, 1) + s_pair[1] * (those of runs 2, 3)
+template <int M>
+__device__ __forceinline__ void combine_runs(const int (&dot)[M][4][3], const float (&sc)[4], const XLimbs (&x)[M],
+                                             float (&out)[M]) {
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+        float part[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float limb_sum[3];
+#pragma unroll
+            for (int k = 0; k < 3; k++)
+                limb_sum[k] = fmaf(sc[2 * h + 1], static_cast<float>(dot[m][2 * h + 1][k]),
+                                   sc[2 * h] * static_cast<float>(dot[m][2 * h][k]));
+            part[h] = fmaf(65536.0f, limb_sum[2], fmaf(256.0f, limb_sum[1], limb_sum[0]));
+        }
+        out[m] = fmaf(x[m].s_pair[1], part[1], x[m].s_pair[0] * part[0]);
+    }
+}
+
+typedef uint4 __attribute__((aligned(4))) uint4_a4;
+typedef struct __attribute__((packed, aligned(2))) { uint32_t v[3]; } Dwords3_a2;
+
+// Q2_K (decode_q2_k, crates/runtime-cpu/src/quantized.rs:117-138): 84 bytes per 256 values - scales[16]
+// (4-bit scale, 4-bit minimum per 16 values), qs[64] (2-bit quants), d, dmin. Value e = half*128 + 32g +
+// 16j + i is d * (scales[8*half + 2g + j] & 15) * ((qs[32*half + 16j + i] >> 2g) & 3) - dmin *
+// (scales[..] >> 4). A lane takes (half, j): runs g = 0..3, sixteen bytes of quants.
+struct Q2KLimb {
+    struct Lane {
+        uint32_t offset, half, j;
+    };
+    struct Data {
+        uint4 qs;
+        uint2 scales;  // scales[8*half .. 8*half + 8]
+        uint32_t dd;   // d | dmin << 16 (f16 bits)
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 8) * 84u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) {
+        return Lane{(chunk >> 2) * 84u, (chunk >> 1) & 1u, chunk & 1u};
+    }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        const uint8_t* base = row + lane.offset;  // 84 b: dword aligned
+        data.qs = *reinterpret_cast<const uint4_a4*>(base + 16u + 32u * lane.half + 16u * lane.j);
+        data.scales = *reinterpret_cast<const uint2_a2*>(base + 8u * lane.half);
+        data.dd = *reinterpret_cast<const uint32_t*>(base + 80u);
+    }
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_run_activations<0>(stage, lane, active, out);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
+                                                const XLimbs (&x)[M], float (&value)[M]) {
+        const uint32_t qs[4] = {data.qs.x, data.qs.y, data.qs.z, data.qs.w};
+        int dot[M][4][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) dot[m][g][k] = 0;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int q = static_cast<int>((qs[i] >> (2 * g)) & 0x03030303u);
+#pragma unroll
+                for (int m = 0; m < M; m++)
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        dot[m][g][k] = __builtin_amdgcn_sdot4(q, x[m].limb[k][4 * g + i], dot[m][g][k], false);
+            }
+        // (scale, minimum) of run g: byte j + 2g of the eight
+        const uint32_t shift = 8u * lane.j;
+        const uint32_t bytes[4] = {(data.scales.x >> shift) & 0xffu, (data.scales.x >> (shift + 16u)) & 0xffu,
+                                   (data.scales.y >> shift) & 0xffu, (data.scales.y >> (shift + 16u)) & 0xffu};
+        float sc[4], mn[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            sc[g] = static_cast<float>(bytes[g] & 15u);
+            mn[g] = static_cast<float>(bytes[g] >> 4);
+        }
+        float pos[M];
+        combine_runs<M>(dot, sc, x, pos);
+        const float d = half_bits_to_float(data.dd & 0xffffu), dmin = half_bits_to_float(data.dd >> 16);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float neg = fmaf(mn[3], x[m].run_sum[3],
+                                   fmaf(mn[2], x[m].run_sum[2], fmaf(mn[1], x[m].run_sum[1], mn[0] * x[m].run_sum[0])));
+            value[m] = d * pos[m] - dmin * neg;
+        }
+    }
+};
+
+// Q3_K (decode_q3_k, crates/runtime-cpu/src/quantized.rs:142-176): 110 bytes per 256 values - hmask[32]
+// (third bits), qs[64] (2-bit quants), scales[12] (sixteen 6-bit scales, packed), d. Value e = half*128 +
+// 32g + 16j + i is d * (scale[8*half + 2g + j] - 32) * (((qs[32*half + 16j + i] >> 2g) & 3) -
+// (hmask[16j + i] bit (4*half + g) ? 0 : 4)). A lane takes (half, j): runs g = 0..3.
+struct Q3KLimb {
+    struct Lane {
+        uint32_t offset, half, j;
+    };
+    struct Data {
+        uint4 qs, hm;
+        uint32_t packed[3];  // scales[12]
+        uint32_t d;
+    };
+    static __device__ __forceinline__ uint64_t row_bytes(uint32_t columns) {
+        return static_cast<uint64_t>(columns >> 8) * 110u;
+    }
+    static __device__ __forceinline__ Lane lane_setup(uint32_t chunk) {
+        return Lane{(chunk >> 2) * 110u, (chunk >> 1) & 1u, chunk & 1u};
+    }
+    static __device__ __forceinline__ void load(const uint8_t* row, const Lane& lane, Data& data) {
+        const uint8_t* base = row + lane.offset;  // 110 b: odd blocks start 2 bytes off a dword
+        data.hm = *reinterpret_cast<const uint4_a2*>(base + 16u * lane.j);
+        data.qs = *reinterpret_cast<const uint4_a2*>(base + 32u + 32u * lane.half + 16u * lane.j);
+        const Dwords3_a2 packed = *reinterpret_cast<const Dwords3_a2*>(base + 96u);
+        data.packed[0] = packed.v[0];
+        data.packed[1] = packed.v[1];
+        data.packed[2] = packed.v[2];
+        data.d = *reinterpret_cast<const uint16_t*>(base + 108u);
+    }
+    static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
+                                                            XLimbs& out) {
+        load_run_activations<4>(stage, lane, active, out);
+    }
+    template <int M>
+    static __device__ __forceinline__ void fold(const Data& data, const Lane& lane,
+                                                const XLimbs (&x)[M], float (&value)[M]) {
+        const uint32_t qs[4] = {data.qs.x, data.qs.y, data.qs.z, data.qs.w};
+        const uint32_t hm[4] = {data.hm.x, data.hm.y, data.hm.z, data.hm.w};
+        int dot[M][4][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) dot[m][g][k] = x[m].bias[g][k];  // sum (v - 4) x = sum v x - 4 sum x
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t low = (qs[i] >> (2 * g)) & 0x03030303u;
+                const uint32_t third = (hm[i] >> (4u * lane.half + g)) & 0x01010101u;
+                const int v = static_cast<int>(low | (third << 2));  // four values 0..7
+#pragma unroll
+                for (int m = 0; m < M; m++)
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        dot[m][g][k] = __builtin_amdgcn_sdot4(v, x[m].limb[k][4 * g + i], dot[m][g][k], false);
+            }
+        // scale of group G = 8*half + 2g + j: low four bits = nibble `half` of byte 2g + j of scales[0..8],
+        // top two bits = bits 2*(2*half + g/2) of byte 8 + 2*(g & 1) + j; minus 32
+        float sc[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t word = g < 2 ? data.packed[0] : data.packed[1];
+            const uint32_t low = (word >> (8u * (2u * (g & 1) + lane.j) + 4u * lane.half)) & 15u;
+            const uint32_t high = (data.packed[2] >> (8u * (2u * (g & 1) + lane.j) + 2u * (2u * lane.half + (g >> 1)))) & 3u;
+            sc[g] = static_cast<float>(static_cast<int>(low | (high << 4)) - 32);
+        }
+        float pos[M];
+        combine_runs<M>(dot, sc, x, pos);
+        const float d = half_bits_to_float(data.d);
+#pragma unroll
+        for (int m = 0; m < M; m++) value[m] = d * pos[m];
     }
 };
 
@@ -786,17 +975,26 @@ hipError_t launch_vectors(const uint8_t* weight, const float* x, uint64_t x_row_
     }
 }
 
+// One or two vectors per launch (the codecs whose lanes own four runs).
+template <class T>
+hipError_t launch_pair(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias, float* y,
+                       uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+    if (vectors == 1) return launch_slices<T, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    if (vectors == 2) return launch_slices<T, 2>(weight, x, x_row_stride, bias, y, rows, columns, stream);
+    return hipErrorInvalidValue;
+}
+
 }  // namespace
 
 uint32_t gemv_limb_max_vectors(int32_t codec) {
-    // Q6_K keeps 62 registers of activation state per vector (48 limb words, 12 dot offsets, 2 units):
-    // three vectors do not fit next to the rows in flight.
-    return codec == kQ6_K ? 2u : kGemvLimbMaxVectors;
+    // Q2_K, Q3_K and Q6_K keep 62 and more registers of activation state per vector (48 limb words,
+    // 12 dot offsets, 2 units, run sums): three vectors do not fit next to the rows in flight.
+    return codec == kQ6_K || codec == kQ3_K || codec == kQ2_K ? 2u : kGemvLimbMaxVectors;
 }
 
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors) {
     if (vectors == 0 || vectors > gemv_limb_max_vectors(codec) || columns == 0 || columns > 65536u) return false;
-    if (codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) return columns % 256 == 0;
+    if (codec == kQ2_K || codec == kQ3_K || codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) return columns % 256 == 0;
     if (codec == kQ4_0 || codec == kQ8_0) return columns % 64 == 0;
     return false;
 }
@@ -808,10 +1006,9 @@ hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint6
     switch (codec) {
         case kQ4_K: return launch_vectors<Q4KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         case kQ5_K: return launch_vectors<Q5KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
-        case kQ6_K:
-            if (vectors == 1) return launch_slices<Q6KLimb, 1>(weight, x, x_row_stride, bias, y, n, k, stream);
-            if (vectors == 2) return launch_slices<Q6KLimb, 2>(weight, x, x_row_stride, bias, y, n, k, stream);
-            return hipErrorInvalidValue;
+        case kQ6_K: return launch_pair<Q6KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ3_K: return launch_pair<Q3KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ2_K: return launch_pair<Q2KLimb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         case kQ4_0: return launch_vectors<Q40Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         case kQ8_0: return launch_vectors<Q80Limb>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
         default: return hipErrorInvalidValue;

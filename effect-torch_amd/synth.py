@@ -53,6 +53,8 @@ CONFIGS = {
     "q8_0_gemv_4096x4096": dict(codec=Q8_0, rows=4096, columns=4096, vectors=(1,), x_scale=1.0, seed=0xE77C0DE0),
     "q4_0_gemv_11008x4096": dict(codec=Q4_0, rows=11008, columns=4096, vectors=(1, 4, 8), x_scale=1.0, seed=0xE77C0DE1),
     "q4_k_gemv_14336x4096": dict(codec=Q4_K, rows=14336, columns=4096, vectors=(1, 16, 64), x_scale=1.0, seed=0xE77C0DE2),
+    "q2_k_gemv_14336x4096": dict(codec=Q2_K, rows=14336, columns=4096, vectors=(1, 2), x_scale=1.0, seed=0xE77C0DE2),
+    "q3_k_gemv_14336x4096": dict(codec=Q3_K, rows=14336, columns=4096, vectors=(1, 2), x_scale=1.0, seed=0xE77C0DE3),
     "q5_k_gemv_14336x4096": dict(codec=Q5_K, rows=14336, columns=4096, vectors=(1, 2), x_scale=1.0, seed=0xE77C0DE5),
     "q6_k_gemv_14336x4096": dict(codec=Q6_K, rows=14336, columns=4096, vectors=(1, 2), x_scale=1.0, seed=0xE77C0DE6),
     "q8_0_gemm_i8_512x14336x4096": dict(codec=Q8_0, rows=4096, columns=14336, vectors=(512,), x_scale=0.5, seed=0xE77C0DE3),

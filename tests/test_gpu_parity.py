@@ -445,7 +445,7 @@ def test_gguf_file_to_contraction(et, device, tmp_path):
             model.upload_tensor("blk.0.attn_q.weight", device, torch.empty(300, dtype=torch.uint8, device=device))
 
 
-@pytest.mark.parametrize("codec", [oracle.Q5_K, oracle.Q6_K])
+@pytest.mark.parametrize("codec", [oracle.Q2_K, oracle.Q3_K, oracle.Q5_K, oracle.Q6_K])
 @pytest.mark.parametrize("vectors", [1, 2, 5])
 def test_k_quant_gemv_at_full_size(et, device, codec, vectors):
     # the integer-dot GEMV for the other K-quants at 14336 x 4096: a row range against the oracle,

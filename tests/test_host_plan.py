@@ -59,7 +59,9 @@ def test_linear_plan_shapes(et):
     plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 176), None, et.GgmlQuant.Q5_K, (2, 256))
     assert plan.kernel == "gemv_limb"
     plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 110), None, et.GgmlQuant.Q3_K, (2, 256))
-    assert plan.kernel == "gemv_generic"
+    assert plan.kernel == "gemv_limb"
+    plan = et.linear_requirements(torch.zeros(2, 512), _w(2, 168), None, et.GgmlQuant.Q2_K, (2, 512))
+    assert plan.kernel == "gemv_limb"
     plan = et.linear_requirements(torch.zeros(64, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256),
                                   et.ActivationMode.INT8)
     assert plan.kernel == "quantize_act+gemm_i8" and plan.workspace_bytes > 64 * 256
