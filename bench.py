@@ -50,6 +50,7 @@ def parse_args():
                    help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
+    p.add_argument("--codec", default="q4_k", help="quantized_embedding_vocab: the table's codec (q2_k ... q6_k, q4_0, q8_0)")
     p.add_argument("--context", type=int, default=2048, help="kv_attention_decode / llama3_8b_batched_decode: "
                    "positions per slot")
     p.add_argument("--unfused", action="store_true", help="llama3_8b_batched_decode: one launch sequence per "
@@ -390,6 +391,78 @@ def decode_op(args, et):
         result["cpu_baseline"] = {"value": round(algorithmic / (elapsed / calls) / 1e9, 4), "unit": "GB/s", "cores": 1,
                                   "kind": "port", "sample": f"{calls} full call(s) of the same workload, "
                                   f"{elapsed:.1f} s of CPU work ({elapsed / calls * 1e6:.0f} us per call)"}
+    print(json.dumps(result))
+
+
+def quantized_embedding(args, et):
+    """Workload ``quantized_embedding_vocab``: ``embedding_into`` on a vocabulary-sized packed table
+    ([128256, 4096] in Q4_K, Q6_K with ``--codec q6_k`` ...): ``--vectors`` token ids (default 8192, a
+    prefill chunk of 4 sequences x 2048) are gathered and decoded bit-exactly to f32 rows. The bytes
+    that must move: the ids, every selected packed row once, every f32 output row once (the stores
+    dominate: 16 384 B written per 2 304 B read for Q4_K)."""
+    import numpy as np
+    import torch
+    import oracle
+    from effect_torch_amd import synth
+
+    device = torch.device("cuda:0")
+    codec = et.GgmlQuant.from_name(args.codec.upper())
+    assert codec is not None, f"unknown codec {args.codec}"
+    rows, columns = 128256, 4096
+    tokens = args.vectors if args.vectors is not None else 8192
+    rng = np.random.default_rng(0xE77C0DE9)
+    base_rows = 8192  # distinct random rows; the table repeats them rolled by one row per repeat
+    block = synth.random_weight(int(codec), base_rows, columns, rng)
+    table_host = np.concatenate([np.roll(block, r, axis=0) for r in range(-(-rows // base_rows))])[:rows]
+    table = torch.from_numpy(table_host).to(device)
+    n = 1 if args.hot else 8
+    ids_host = [rng.integers(0, rows, tokens).astype(np.int64) for _ in range(n)]
+    ids = [torch.from_numpy(a).to(device) for a in ids_host]
+    outs = [torch.empty((tokens, columns), dtype=torch.float32, device=device) for _ in range(2)]
+    plan = et.embedding_requirements(ids[0], table, codec, (rows, columns))
+    keep = []
+
+    def step(i):
+        keep.append(et.embedding_into(ids[i % n], table, codec, outs[i % 2], plan, synchronize=False))
+        if len(keep) > 4:
+            keep.pop(0)
+
+    step(0)
+    torch.cuda.synchronize()
+    et.embedding_status_check(plan, keep[-1])
+    sample = min(tokens, 256)
+    want = oracle.embedding_into(int(codec), rows, columns, ids_host[0][:sample], table_host)
+    got = outs[0][:sample].cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "parity gate failed: decoded rows differ"
+    ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    row_bytes = codec.encoded_row_bytes(columns)
+    algorithmic = tokens * (8 + row_bytes + 4 * columns)
+    gbs = algorithmic / (ms * 1e-3) / 1e9
+    result = {
+        "metric": "quantized embedding GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"quantized_embedding_vocab: {tokens} i64 ids into the {codec.ggml_name} "
+                               f"[{rows}, {columns}] table -> f32 [{tokens}, {columns}]",
+                   "inputs": "hot" if args.hot else f"rotating over {n} id sets and 2 outputs",
+                   "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues",
+                   "host_wall_ms": round(wall * 1e3, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
+    }
+    if not args.no_cpu:
+        cpu_tokens = min(tokens, 512)
+        calls, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 5.0) or calls == 0:
+            oracle.embedding_into(int(codec), rows, columns, ids_host[0][:cpu_tokens], table_host)
+            calls += 1
+        elapsed = time.perf_counter() - t0
+        per_token = elapsed / calls / cpu_tokens
+        result["cpu_baseline"] = {"value": round((8 + row_bytes + 4 * columns) / per_token / 1e9, 4), "unit": "GB/s",
+                                  "cores": 1, "kind": "port",
+                                  "sample": f"{calls} call(s) on the first {cpu_tokens} ids, {elapsed:.1f} s of CPU "
+                                            f"work ({per_token * 1e6:.1f} us per row); scalar C restatement"}
     print(json.dumps(result))
 
 
@@ -739,9 +812,13 @@ def main():
     if args.workload == "kv_attention_decode":
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return kv_decode(args, et)
+    if args.workload == "quantized_embedding_vocab":
+        assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
+        return quantized_embedding(args, et)
     if args.workload not in synth.CONFIGS:
         sys.exit(f"unknown workload {args.workload}; choose from {sorted(synth.CONFIGS)} "
-                 "or calibrate_read / calibrate_copy / kv_attention_decode / llama3_8b_batched_decode / gguf_upload / " + " / ".join(DECODE_OPS))
+                 "or calibrate_read / calibrate_copy / kv_attention_decode / llama3_8b_batched_decode / gguf_upload / "
+                 "quantized_embedding_vocab / " + " / ".join(DECODE_OPS))
     cfg = synth.CONFIGS[args.workload]
     vectors = args.vectors if args.vectors is not None else cfg["vectors"][0]
     mode_name = args.mode or ("int8" if "i8" in args.workload else "f32")

@@ -31,6 +31,7 @@ SOURCES = {
     "gemv_generic.hip": [],
     "quantize_act.hip": ["-ffp-contract=off"],
     "gemm_i8.hip": [],
+    "gemm_h16.hip": [],
     "kv_attention.hip": [],
     "decode_ops.hip": ["-ffp-contract=off"],
     "calibrate.hip": [],

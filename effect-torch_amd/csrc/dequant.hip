@@ -41,6 +41,7 @@ __device__ __forceinline__ uint64_t source_index(const IndexLayout& layout, uint
 }
 
 constexpr uint64_t kNoBadIndex = ~0ull;
+constexpr uint32_t kChunksPerPass = 4;  // 1024-column chunks a workgroup decodes per pass
 
 __global__ void status_init_kernel(unsigned long long* status) {
     if (threadIdx.x == 0) {
@@ -63,6 +64,9 @@ __global__ void status_finalize_kernel(const void* indexes, int index_is_i64, In
     status[1] = static_cast<unsigned long long>(value);
 }
 
+// One workgroup per (output row, four 1024-column chunks): the row's index is read once per workgroup
+// and everything per lane is 32-bit arithmetic (a 64-bit division per item, as a flat grid-stride
+// loop over all outputs needs, costs more than the decode itself).
 template <int CODEC>
 __global__ __launch_bounds__(256) void dequant_rows_kernel(
     const uint8_t* __restrict__ weight, const void* __restrict__ indexes, int index_is_i64,
@@ -70,13 +74,8 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
     uint64_t row_bytes, float* __restrict__ out, unsigned long long* status) {
     constexpr uint32_t kValues = block_values(CODEC);
     constexpr uint32_t kBytes = block_bytes(CODEC);
-    const uint32_t quads_per_row = columns >> 2;
-    const uint64_t total = out_rows * quads_per_row;
-    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
-    for (uint64_t item = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; item < total;
-         item += stride) {
-        const uint64_t p = item / quads_per_row;
-        const uint32_t column = static_cast<uint32_t>(item - p * quads_per_row) << 2;
+    const uint32_t chunks = (columns + 1023u) >> 10;
+    for (uint64_t p = blockIdx.x; p < out_rows; p += gridDim.x) {
         uint64_t row = p;
         if (indexes != nullptr) {
             const uint64_t source = source_index(layout, p);
@@ -90,17 +89,31 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(
                 bad = row >= table_rows;
             }
             if (bad) {
-                if (column == 0) atomicMin(status, static_cast<unsigned long long>(p));
+                if (blockIdx.y == 0 && threadIdx.x == 0) atomicMin(status, static_cast<unsigned long long>(p));
                 continue;  // skipped, like the reference's Metal kernel
             }
         }
-        const uint32_t block_index = column / kValues;
-        const uint32_t e = column - block_index * kValues;
-        const uint8_t* block = weight + row * row_bytes + static_cast<uint64_t>(block_index) * kBytes;
-        float values[4];
-        decode4<CODEC>(block, e, values);
-        float4 packed = make_float4(values[0], values[1], values[2], values[3]);
-        *reinterpret_cast<float4*>(out + p * columns + column) = packed;
+        const uint8_t* packed_row = weight + row * row_bytes;
+        float* out_row = out + p * columns;
+        // Four chunks per pass, all decoded before the first store: their loads are in flight together.
+        for (uint32_t first = blockIdx.y * kChunksPerPass; first < chunks; first += gridDim.y * kChunksPerPass) {
+            float values[kChunksPerPass][4];
+#pragma unroll
+            for (uint32_t u = 0; u < kChunksPerPass; u++) {
+                const uint32_t column = ((first + u) << 10) + (threadIdx.x << 2);
+                if (column >= columns) continue;  // columns is a multiple of the block width, so of four
+                const uint32_t block_index = column / kValues;
+                decode4<CODEC>(packed_row + static_cast<uint64_t>(block_index) * kBytes, column - block_index * kValues,
+                               values[u]);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kChunksPerPass; u++) {
+                const uint32_t column = ((first + u) << 10) + (threadIdx.x << 2);
+                if (column >= columns) continue;
+                *reinterpret_cast<float4*>(out_row + column) =
+                    make_float4(values[u][0], values[u][1], values[u][2], values[u][3]);
+            }
+        }
     }
 }
 
@@ -109,16 +122,16 @@ hipError_t launch_dequant(const uint8_t* weight, const void* indexes, int index_
                           const IndexLayout& layout, uint64_t out_rows, uint64_t table_rows,
                           uint64_t columns, float* out, void* status, hipStream_t stream) {
     const uint64_t row_bytes = columns / block_values(CODEC) * block_bytes(CODEC);
-    const uint64_t total = out_rows * (columns >> 2);
-    if (total == 0) return hipSuccess;
-    uint64_t blocks = (total + 255) / 256;
-    // Enough workgroups to fill 256 CUs many times over; the grid-stride loop takes the rest.
-    if (blocks > (1u << 20)) blocks = 1u << 20;
+    if (out_rows == 0 || columns == 0) return hipSuccess;
+    // The loops in the kernel take what the grid limits leave over.
+    const uint64_t chunks = (((columns + 1023) >> 10) + kChunksPerPass - 1) / kChunksPerPass;
+    const uint32_t grid_x = static_cast<uint32_t>(out_rows < (1u << 24) ? out_rows : (1u << 24));
+    const uint32_t grid_y = static_cast<uint32_t>(chunks < 1024 ? chunks : 1024);
     auto* status_words = static_cast<unsigned long long*>(status);
     if (indexes != nullptr) {
         hipLaunchKernelGGL(status_init_kernel, dim3(1), dim3(64), 0, stream, status_words);
     }
-    hipLaunchKernelGGL(dequant_rows_kernel<CODEC>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+    hipLaunchKernelGGL(dequant_rows_kernel<CODEC>, dim3(grid_x, grid_y), dim3(256), 0,
                        stream, weight, indexes, index_is_i64, layout, out_rows, table_rows,
                        static_cast<uint32_t>(columns), row_bytes, out, status_words);
     if (indexes != nullptr) {

@@ -1,0 +1,348 @@
+// f32-accurate contraction of Q4_K weights with a batch of activation vectors on the gfx950
+// matrix cores, with every operand an exact small integer held in a half float.
+//
+//   y[m, n] = sum_s  unit[m, s] * d[n, s] * sum_g sum_i (sc_g[n] * nib[n, g, i]) * X[m, g, i]
+//           - sum_s  dmin[n, s] * sum_g m_g[n] * xsum[m, g]
+// s = 256-column stage (one Q4_K super-block), g = its eight 32-column sub-blocks.
+//
+// Activations are 24-bit fixed point per vector and stage, X = rint(x * (2^23 - 1) / max|x|), split
+// into two balanced 12-bit halves X = 4096 * hi + lo with |lo|, |hi| <= 2048: integers a half float
+// holds exactly. On the weight side the 6-bit sub-block scale is folded into the operand:
+// sc_g * nib <= 63 * 15 = 945, exact in a half float as well. Every product (< 2^21) is exact in
+// the f32 the matrix core accumulates in, so v_mfma_f32_32x32x16_f16 sums whole super-blocks with
+// f32 accumulation error only, and the f32 scales unit[m] * d[n] are applied once per stage instead
+// of once per 32-column block: the per-element VALU work, which bounds the int8 kernel with
+// three-byte activations (gemm_i8.hip: a convert and multiply-adds per element and block), shrinks
+// by the eight blocks of a stage. The contraction computed is linear_into's
+// (crates/runtime-cpu/src/quantized.rs:419-499); the reference's own batch kernel decodes weights
+// to f32 and uses f32 simdgroup MMA (crates/runtime-metal/src/quantized.rs:1016-1097).
+//
+// Tiling, operand streams and barriers are those of gemm_i8.hip: a workgroup owns 64 weight rows x
+// 32 vectors and walks K in stages; eight consumer waves (four share a 32-row group and split the
+// eight sub-blocks of a stage), two loader waves per operand stream that only issue
+// global_load_lds copies into LDS rings, one s_barrier per stage.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "et_codecs.h"
+#include "gemv_common.h"
+#include "kernels.h"
+
+namespace et {
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kStageBlocks = 8;
+constexpr int kConsumers = 8;
+constexpr int kWeightLoaders = 2;
+constexpr int kActivationLoaders = 2;
+constexpr int kLoaders = kWeightLoaders + kActivationLoaders;
+constexpr int kThreads = 64 * (kConsumers + kLoaders);
+constexpr int kSplit = 4;
+constexpr int kRowGroups = kConsumers / kSplit;
+constexpr int kBlocksPerWave = kStageBlocks / kSplit;
+constexpr uint32_t kRows = 32 * kRowGroups;
+
+constexpr uint32_t kBlob = tile_blob_bytes(2);  // in memory and in LDS
+constexpr uint32_t kUnitAt = 32768u;            // unit[m]
+constexpr uint32_t kSumsAt = 32768u + 128u;     // xsum[g][m]
+constexpr uint32_t kRowBytes = 144u;            // a row's share of a stage
+constexpr uint32_t kWeightBytes = kRows * kRowBytes;
+constexpr int kWeightJobs = kWeightBytes / 1024;
+constexpr int kActivationJobs = kBlob / 1024;
+static_assert(kWeightBytes % 1024 == 0 && kBlob % 1024 == 0, "whole copy instructions");
+
+// (scale, min) of Q4_K sub-block g (crates/runtime-cpu/src/quantized.rs:77-86).
+__device__ __forceinline__ void q4k_scale_min(const uint4& header, uint32_t g, uint32_t& sc, uint32_t& mn) {
+    const uint32_t shift = 8u * (g & 3u);
+    const uint32_t s0 = (header.y >> shift) & 0xffu;
+    const uint32_t s1 = (header.z >> shift) & 0xffu;
+    const uint32_t s2 = (header.w >> shift) & 0xffu;
+    sc = g < 4 ? (s0 & 63u) : ((s2 & 0x0fu) | ((s0 >> 6) << 4));
+    mn = g < 4 ? (s1 & 63u) : ((s2 >> 4) | ((s1 >> 6) << 4));
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) {
+    return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
+}
+
+template <int AX, int AW>
+struct Shape {
+    static constexpr int kActivationDepth = AX + 1, kWeightDepth = AW + 1;
+    static constexpr uint32_t kWeightRingAt = kActivationDepth * kBlob;
+    static constexpr uint32_t kRingBytes = kWeightRingAt + kWeightDepth * kWeightBytes;
+    static constexpr int kActivationRounds = (kActivationJobs + kActivationLoaders - 1) / kActivationLoaders;
+    static constexpr int kWeightRounds = (kWeightJobs + kWeightLoaders - 1) / kWeightLoaders;
+    static constexpr int kActivationWait = (AX - 1) * kActivationRounds < 63 ? (AX - 1) * kActivationRounds : 63;
+    static constexpr int kWeightWait = (AW - 1) * kWeightRounds < 63 ? (AW - 1) * kWeightRounds : 63;
+    static constexpr uint32_t kExchangeBytes = (kSplit - 1) * kRowGroups * 16 * 64 * 4;
+    static constexpr uint32_t kLdsBytes = kRingBytes > kExchangeBytes ? kRingBytes : kExchangeBytes;
+};
+
+// Eight nibbles (two dwords of four, one per byte) as eight half floats times `scale`:
+// 0x6400 | n is the half float 1024 + n, and (1024 + n) * scale - 1024 * scale, one fused
+// multiply-add per pair, is n * scale exactly (1024 * scale <= 64512 is a half float).
+__device__ __forceinline__ v8h nibbles_times(uint32_t first, uint32_t second, v2h scale) {
+    const v2h offset = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    union {
+        uint32_t word[4];
+        v2h pair[4];
+        v8h all;
+    } u;
+    u.word[0] = __builtin_amdgcn_perm(0x64646464u, first, 0x04010400u);   // bytes 0, 1
+    u.word[1] = __builtin_amdgcn_perm(0x64646464u, first, 0x04030402u);   // bytes 2, 3
+    u.word[2] = __builtin_amdgcn_perm(0x64646464u, second, 0x04010400u);
+    u.word[3] = __builtin_amdgcn_perm(0x64646464u, second, 0x04030402u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) u.pair[i] = __builtin_elementwise_fma(u.pair[i], scale, -(offset * scale));
+    return u.all;
+}
+
+template <int AX, int AW>
+__global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
+    const uint8_t* __restrict__ weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
+    const float* __restrict__ bias, const float* residual, float* y, uint32_t rows, uint32_t columns,
+    uint32_t vectors, uint32_t row_tiles, uint32_t k_splits, float* __restrict__ partials) {
+    using S = Shape<AX, AW>;
+    constexpr int NB = kBlocksPerWave;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    // Workgroups go to the eight XCDs round-robin; all vector tiles and K shares of one row tile
+    // run on the same XCD, next to each other in time, so the later ones find the weights in L2.
+    const uint32_t xcd = blockIdx.x & 7u, turn = blockIdx.x >> 3;
+    const uint32_t units = vector_tiles * k_splits;
+    const uint32_t row_tile = (turn / units) * 8u + xcd;
+    const uint32_t tile = (turn % units) % vector_tiles;
+    const uint32_t k_share = (turn % units) / vector_tiles;
+    if (row_tile >= row_tiles) return;
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t all_stages = columns / 256u;
+    const uint32_t share = (all_stages + k_splits - 1u) / k_splits;
+    const uint32_t first_stage = k_share * share;  // < all_stages: the launcher leaves no share empty
+    const uint32_t stages = min(share, all_stages - first_stage);
+    const uint64_t row_bytes = static_cast<uint64_t>(all_stages) * kRowBytes;
+    const uint32_t row0 = row_tile * kRows;
+
+    if (wave >= static_cast<uint32_t>(kConsumers + kWeightLoaders)) {
+        // ---- activation loaders: linear copies of the stage's blob ----
+        const uint32_t loader = wave - (kConsumers + kWeightLoaders);
+        const auto request = [&](uint32_t stage) {
+            const uint32_t s = min(stage, stages - 1u);  // past the end: a copy nobody reads
+            uint8_t* slot = lds + (stage % S::kActivationDepth) * kBlob;
+            const uint8_t* blob = tiles + (static_cast<uint64_t>(first_stage + s) * vector_tiles + tile) * kBlob;
+#pragma unroll
+            for (int i = 0; i < S::kActivationRounds; i++) {
+                uint32_t job = i * kActivationLoaders + loader;
+                if (job >= static_cast<uint32_t>(kActivationJobs)) job -= kActivationJobs;
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(blob + job * 1024u + lane * 16u),
+                                                 reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
+            }
+        };
+        for (uint32_t a = 0; a < static_cast<uint32_t>(AX); a++) request(a);
+        for (uint32_t stage = 0; stage < stages; stage++) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kActivationWait));  // all but the newest AX - 1 requests
+            __builtin_amdgcn_s_barrier();  // "stage is in LDS" / "the slots of stage - 1 are free"
+            request(stage + AX);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));  // nothing may still write the ring
+        __builtin_amdgcn_s_barrier();               // the consumers' two exchange barriers
+        __builtin_amdgcn_s_barrier();
+        return;
+    }
+    if (wave >= static_cast<uint32_t>(kConsumers)) {
+        // ---- weight loaders: the stage's bytes of the 64 rows, row after row as in memory ----
+        const uint32_t loader = wave - kConsumers;
+        const auto request = [&](uint32_t stage) {
+            const uint32_t s = min(stage, stages - 1u);
+            uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * kWeightBytes;
+#pragma unroll
+            for (int i = 0; i < S::kWeightRounds; i++) {
+                uint32_t job = i * kWeightLoaders + loader;
+                if (job >= static_cast<uint32_t>(kWeightJobs)) job -= kWeightJobs;
+                const uint32_t at = job * 1024u + lane * 16u;
+                const uint32_t row = min(row0 + at / kRowBytes, rows - 1u);
+                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * kRowBytes +
+                                     at % kRowBytes;
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
+                                                 reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
+            }
+        };
+        for (uint32_t a = 0; a < static_cast<uint32_t>(AW); a++) request(a);
+        for (uint32_t stage = 0; stage < stages; stage++) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(S::kWeightWait));
+            __builtin_amdgcn_s_barrier();
+            request(stage + AW);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_s_barrier();
+        return;
+    }
+
+    // ---- consumer waves ----
+    const uint32_t half = lane >> 5, in_half = lane & 31u;
+    const uint32_t wave_n = wave % kRowGroups;  // row group
+    const uint32_t wave_k = wave / kRowGroups;  // share of the stage's sub-blocks
+    const uint32_t n0 = row0 + wave_n * 32u;
+    const uint32_t m0 = tile * 32u;
+    float acc[16];
+    v16f acc_min, zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        acc[r] = 0.f;
+        acc_min[r] = 0.f;
+        zero[r] = 0.f;
+    }
+
+    for (uint32_t stage = 0; stage < stages; stage++) {
+        __builtin_amdgcn_s_barrier();
+        const uint8_t* slot = lds + (stage % S::kActivationDepth) * kBlob;
+        const uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * kWeightBytes;
+        const uint32_t b_base = wave_k * NB;
+        const uint8_t* row_in_slot = region + (wave_n * 32u + in_half) * kRowBytes;  // this lane's weight row
+
+        const uint4 header = *reinterpret_cast<const uint4*>(row_in_slot);
+        const float d_block = half_bits_to_float(header.x & 0xffffu);
+        const float dmin_block = half_bits_to_float(header.x >> 16);
+        const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
+
+        // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA, lane half h
+        // supplies sub-block 2j + h.
+#pragma unroll
+        for (int jj = 0; jj < NB / 2; jj++) {
+            const uint32_t g = b_base + 2u * jj + half;
+            uint32_t sc, mn;
+            q4k_scale_min(header, g, sc, mn);
+            const float a_operand = *reinterpret_cast<const float*>(slot + kSumsAt + g * 128u + in_half * 4u);
+            acc_min = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, dmin_block * static_cast<float>(mn), acc_min,
+                                                           0, 0, 0);
+        }
+
+        // The stage's products: both halves of X against sc_g * nib, summed over this wave's sub-blocks.
+        // The weight operands of sub-block bb + 1 are prepared (VALU) between the MFMAs of sub-block bb.
+        const auto prepare = [&](int bb, v8h& b0, v8h& b1) {
+            const uint32_t b = b_base + bb;
+            // sub-block 2p + side: low (side 0) or high (side 1) nibbles of the 32 bytes of pair p; this
+            // lane half takes bytes 16 * half .. + 16 = columns 16 * half .. + 16 of the sub-block
+            const uint4 raw = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 32u * (b >> 1) + 16u * half);
+            const uint32_t shift = (b & 1u) * 4u;
+            const uint32_t w0 = (raw.x >> shift) & 0x0f0f0f0fu, w1 = (raw.y >> shift) & 0x0f0f0f0fu,
+                           w2 = (raw.z >> shift) & 0x0f0f0f0fu, w3 = (raw.w >> shift) & 0x0f0f0f0fu;
+            uint32_t sc, mn;
+            q4k_scale_min(header, b, sc, mn);
+            const _Float16 sc_h = static_cast<_Float16>(static_cast<float>(sc));
+            const v2h sc2 = {sc_h, sc_h};
+            b0 = nibbles_times(w0, w1, sc2);
+            b1 = nibbles_times(w2, w3, sc2);
+        };
+        v16f p_lo = zero, p_hi = zero;
+        v8h b0, b1;
+        prepare(0, b0, b1);
+#pragma unroll
+        for (int bb = 0; bb < NB; bb++) {
+            const uint8_t* chunk = slot + ((2u * (b_base + bb) + half) * 2u) * 512u + in_half * 16u;
+            const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
+            const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
+                      hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
+            p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
+            p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
+            p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
+            p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
+            if (bb + 1 < NB) {
+                v8h n0, n1;
+                prepare(bb + 1, n0, n1);
+                b0 = n0;
+                b1 = n1;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 12, 0);  // twelve VALU
+                }
+            }
+        }
+        // unit[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1 product in the
+        // result layout (only the k = 0 half of the lanes carries a value).
+        const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+                                                             zero, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
+    }
+
+    // ---- combine the sub-block shares, add bias, store ----
+    __syncthreads();  // the loaders arrive here with nothing in flight: the ring is free
+    float* exchange = reinterpret_cast<float*>(lds);  // [wave_k - 1][wave_n][16][64 lanes]
+    if (wave_k > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            exchange[(((wave_k - 1u) * kRowGroups + wave_n) * 16 + r) * 64 + lane] = acc[r] - acc_min[r];
+    }
+    __syncthreads();
+    if (wave_k > 0) return;
+    const uint32_t n_out = n0 + in_half;
+    const float bias_value = bias != nullptr && n_out < rows ? bias[n_out] : 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        float value = acc[r] - acc_min[r];
+#pragma unroll
+        for (int k = 1; k < kSplit; k++) value += exchange[(((k - 1) * kRowGroups + wave_n) * 16 + r) * 64 + lane];
+        const uint32_t m = m0 + 8u * (r >> 2) + 4u * half + (r & 3u);
+        if (n_out < rows && m < vectors) {
+            if (k_splits == 1) {
+                // residual may be y itself: every output is read, then written, by this lane only
+                const uint64_t at = static_cast<uint64_t>(m) * rows + n_out;
+                y[at] = residual != nullptr ? (value + bias_value) + residual[at] : value + bias_value;
+            } else {
+                partials[(static_cast<uint64_t>(k_share) * vectors + m) * rows + n_out] = value;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool gemm_h16_supported(int32_t codec, uint64_t columns) {
+    return codec == kQ4_K && columns % 256 == 0 && columns > 0;
+}
+
+hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
+                    uint64_t rows64, uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+    if (!gemm_h16_supported(codec, columns64)) return hipErrorInvalidValue;
+    constexpr int AX = 2, AW = 3;
+    using S = Shape<AX, AW>;
+    static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
+    const auto kernel = gemm_h16_kernel<AX, AW>;
+    const uint32_t rows = static_cast<uint32_t>(rows64), columns = static_cast<uint32_t>(columns64),
+                   vectors = static_cast<uint32_t>(vectors64);
+    // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
+    static bool allowed[64] = {};
+    int device = 0;
+    if (hipError_t status = hipGetDevice(&device)) return status;
+    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+    if (!allowed[device]) {
+        if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes))
+            return status;
+        allowed[device] = true;
+    }
+    const uint32_t vector_tiles = (vectors + 31u) / 32u;
+    const uint32_t row_tiles = (rows + kRows - 1) / kRows;
+    const uint32_t k_splits = out.partials != nullptr ? gemm_i8_k_splits(codec, 2, rows, columns, vectors) : 1u;
+    const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_tiles * k_splits;
+    if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, weight, tiles,
+                       vector_tiles, out.bias, out.residual, out.y, rows, columns, vectors, row_tiles, k_splits,
+                       out.partials);
+    if (hipError_t status = hipGetLastError()) return status;
+    if (k_splits > 1)
+        return reduce_partials(out.partials, out.bias, out.residual, out.y, rows, vectors, k_splits, stream);
+    return hipSuccess;
+}
+
+}  // namespace et

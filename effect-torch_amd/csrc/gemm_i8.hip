@@ -510,12 +510,8 @@ hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const GemmOutput&
                        weight, tiles, vector_tiles, bias, out.residual, y, rows, columns, vectors, row_tiles,
                        vector_groups, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
-    if (k_splits > 1) {
-        const uint64_t outputs = static_cast<uint64_t>(vectors) * rows;
-        hipLaunchKernelGGL(reduce_partials_kernel, dim3(static_cast<uint32_t>((outputs + 1023) / 1024)), dim3(256), 0,
-                           stream, partials, bias, out.residual, y, rows, outputs, k_splits);
-    }
-    return hipGetLastError();
+    if (k_splits > 1) return reduce_partials(partials, bias, out.residual, y, rows, vectors, k_splits, stream);
+    return hipSuccess;
 }
 
 // Weight lead (stages) that fills what the activation ring leaves of LDS.
@@ -560,12 +556,20 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
 }
 
 uint32_t tiles_per_workgroup(int32_t codec, int limbs, uint64_t vectors) {
-    if (limbs == 3 || vectors <= 32) return 1;
+    if (limbs != 1 || vectors <= 32) return 1;
     if (vectors <= 64 || codec == kQ4_K) return 2;
     return 4;
 }
 
 }  // namespace
+
+hipError_t reduce_partials(const float* partials, const float* bias, const float* residual, float* y,
+                           uint32_t rows, uint32_t vectors, uint32_t k_splits, hipStream_t stream) {
+    const uint64_t outputs = static_cast<uint64_t>(vectors) * rows;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3(static_cast<uint32_t>((outputs + 1023) / 1024)), dim3(256), 0,
+                       stream, partials, bias, residual, y, rows, outputs, k_splits);
+    return hipGetLastError();
+}
 
 bool gemm_i8_supported(int32_t codec, uint64_t columns) {
     // Whole stages of 256 columns, also for the 32-wide codecs.

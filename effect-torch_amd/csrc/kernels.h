@@ -63,7 +63,13 @@ hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 // and padding up to a multiple of 4096 bytes.
 // limbs = 1: int8 activations, scale = max|x| / 127.
 // limbs = 3: 24-bit fixed point in three balanced signed bytes, scale = max|x| / (127 * 65536).
-constexpr uint32_t tile_blob_bytes(int limbs) { return limbs == 1 ? 12288u : 28672u; }
+// limbs = 2 is the layout of gemm_h16: 24-bit fixed point per vector and 256-column stage in two
+// balanced 12-bit halves, each a half float:
+//   half l (0 low, 1 high), 8-column part c (0..31), vector m: 8 half floats at  l*16384 + c*512 + m*16
+//   unit[m] f32 (max|x| / (2^23 - 1)) at  32768 + m*4
+//   xsum[sub-block g (0..7)][m] f32 at  32768 + 128 + g*128 + m*4
+// and padding up to 34 KiB.
+constexpr uint32_t tile_blob_bytes(int limbs) { return limbs == 1 ? 12288u : limbs == 2 ? 34816u : 28672u; }
 constexpr uint64_t tile_workspace_bytes(int limbs, uint64_t vectors, uint64_t columns) {
     return ((columns + 255) / 256) * ((vectors + 31) / 32) * tile_blob_bytes(limbs);
 }
@@ -87,6 +93,15 @@ struct GemmOutput {
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
                    const GemmOutput& out, uint64_t rows, uint64_t columns, uint64_t vectors,
                    hipStream_t stream);
+// y = bias + the k_splits partial results in share order (+ residual); the second kernel of a launch
+// that shared K out.
+hipError_t reduce_partials(const float* partials, const float* bias, const float* residual, float* y,
+                           uint32_t rows, uint32_t vectors, uint32_t k_splits, hipStream_t stream);
+
+// ---- gemm_h16.hip: Q4_K on the half-float matrix cores, exact integer operands (limbs = 2 tiles) ----
+bool gemm_h16_supported(int32_t codec, uint64_t columns);
+hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
+                    uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch

@@ -124,6 +124,61 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
     }
 }
 
+
+// Activations for gemm_h16: per vector and 256-column stage, X = clamp(rint(x * (2^23 - 1) / amax))
+// as two balanced 12-bit halves, X = 4096 * hi + lo with lo in [-2048, 2047], both written as half
+// floats (exact); unit = amax / (2^23 - 1); xsum[g] = unit * (integer sum of X over sub-block g).
+// One wave per (vector, stage): lane q holds columns 4q .. 4q + 3 of the stage. Blob layout: see
+// tile_blob_bytes() in kernels.h.
+__global__ __launch_bounds__(64) void quantize_halves_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+                                                             uint32_t vectors, uint32_t stages,
+                                                             uint8_t* __restrict__ tiles) {
+    constexpr float kRange = 8388607.f;  // 2^23 - 1
+    const uint32_t vector_tiles = (vectors + 31u) >> 5;
+    const uint32_t quad = threadIdx.x;
+    for (uint64_t item = blockIdx.x; item < static_cast<uint64_t>(vectors) * stages; item += gridDim.x) {
+        const uint32_t v = static_cast<uint32_t>(item / stages), stage = static_cast<uint32_t>(item % stages);
+        const float4 in = *reinterpret_cast<const float4*>(x + v * x_row_stride + 256u * stage + 4u * quad);
+        float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
+#pragma unroll
+        for (int step = 1; step < 64; step <<= 1) amax = fmaxf(amax, __shfl_xor(amax, step));
+        const float inv = amax > 0.f ? kRange / amax : 0.f;
+        const float values[4] = {in.x, in.y, in.z, in.w};
+        int total = 0;
+        _Float16 low[4], high[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float r = fminf(fmaxf(rintf(values[i] * inv), -kRange), kRange);
+            const int q = static_cast<int>(r);
+            const int lo = ((q + 2048) & 4095) - 2048;
+            total += q;
+            low[i] = static_cast<_Float16>(lo);
+            high[i] = static_cast<_Float16>((q - lo) >> 12);  // exact: q - lo is a multiple of 4096
+        }
+        total += dpp_i32<0xB1>(total);   // the eight lanes of a 32-column sub-block
+        total += dpp_i32<0x4E>(total);
+        total += dpp_i32<0x141>(total);
+        const float unit = amax / kRange;
+        uint8_t* blob = tiles + (static_cast<uint64_t>(stage) * vector_tiles + (v >> 5)) * tile_blob_bytes(2);
+        // columns 4 quad .. + 3 = sub-block quad / 8, 16-column half, 8-column part, first or second four
+        const uint32_t at = (quad >> 1) * 512u + (v & 31u) * 16u + (quad & 1u) * 8u;
+        union {
+            _Float16 h[4];
+            uint2 words;
+        } lo_words, hi_words;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lo_words.h[i] = low[i];
+            hi_words.h[i] = high[i];
+        }
+        *reinterpret_cast<uint2*>(blob + at) = lo_words.words;
+        *reinterpret_cast<uint2*>(blob + 16384u + at) = hi_words.words;
+        float* tables = reinterpret_cast<float*>(blob + 32768u);
+        if (quad == 0) tables[v & 31u] = unit;
+        if ((quad & 7u) == 0) tables[32u + (quad >> 3) * 32u + (v & 31u)] = unit * static_cast<float>(total);
+    }
+}
+
 // Small batches are latency-bound: one wave per workgroup spreads them over all CUs.
 struct Geometry {
     uint32_t blocks, threads;
@@ -152,6 +207,14 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
                           int limbs, uint8_t* tiles, hipStream_t stream) {
     const uint64_t total = vectors * (((columns + 255) & ~255ull) >> 2);
     if (total == 0) return hipSuccess;
+    if (limbs == 2) {
+        if (columns % 256 != 0) return hipErrorInvalidValue;
+        const uint64_t items = vectors * (columns / 256);
+        hipLaunchKernelGGL(quantize_halves_kernel, dim3(static_cast<uint32_t>(items < 65536 ? items : 65536)), dim3(64),
+                           0, stream, x, x_row_stride, static_cast<uint32_t>(vectors),
+                           static_cast<uint32_t>(columns / 256), tiles);
+        return hipGetLastError();
+    }
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
     const Geometry g = geometry_for(total);
     const dim3 grid(g.blocks), block(g.threads);

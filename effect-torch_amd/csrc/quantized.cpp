@@ -134,7 +134,9 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     } else if (plan->activation_mode == ET_ACT_F32) {
         const uint32_t limb_most = gemv_limb_max_vectors(plan->codec);
         const uint32_t limb_launch = static_cast<uint32_t>(plan->vectors < limb_most ? plan->vectors : limb_most);
-        if (plan->vectors >= kGemmMinVectors && gemm_i8_supported(plan->codec, plan->columns)) {
+        if (plan->vectors >= kGemmMinVectors && gemm_h16_supported(plan->codec, plan->columns)) {
+            plan_matrix_core(LinearKernel::kGemmHalf, 2);
+        } else if (plan->vectors >= kGemmMinVectors && gemm_i8_supported(plan->codec, plan->columns)) {
             plan_matrix_core(LinearKernel::kGemmLimb, 3);
         } else if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
             plan->kernel = LinearKernel::kGemvLimb;
@@ -246,6 +248,8 @@ const char* kernel_name(const et_linear_plan& plan) {
             return plan.k_splits > 1 ? "quantize_act+gemm_i8+reduce" : "quantize_act+gemm_i8";
         case LinearKernel::kGemmLimb:
             return plan.k_splits > 1 ? "quantize_limbs+gemm_i8+reduce" : "quantize_limbs+gemm_i8";
+        case LinearKernel::kGemmHalf:
+            return plan.k_splits > 1 ? "quantize_halves+gemm_h16+reduce" : "quantize_halves+gemm_h16";
     }
     return "?";
 }
@@ -314,9 +318,19 @@ int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint6
 
 namespace {
 bool on_matrix_cores(const et_linear_plan& plan) {
-    return plan.kernel == LinearKernel::kGemmI8 || plan.kernel == LinearKernel::kGemmLimb;
+    return plan.kernel == LinearKernel::kGemmI8 || plan.kernel == LinearKernel::kGemmLimb ||
+           plan.kernel == LinearKernel::kGemmHalf;
 }
-int limbs_of(const et_linear_plan& plan) { return plan.kernel == LinearKernel::kGemmI8 ? 1 : 3; }
+int limbs_of(const et_linear_plan& plan) {
+    return plan.kernel == LinearKernel::kGemmI8 ? 1 : plan.kernel == LinearKernel::kGemmHalf ? 2 : 3;
+}
+// The contraction over prepared activation tiles, on whichever matrix-core kernel the plan chose.
+hipError_t contract_tiles(const et_linear_plan& plan, const uint8_t* weight, const uint8_t* tiles,
+                          const GemmOutput& out, hipStream_t stream) {
+    if (plan.kernel == LinearKernel::kGemmHalf)
+        return gemm_h16(plan.codec, weight, tiles, out, plan.rows, plan.columns, plan.vectors, stream);
+    return gemm_i8(plan.codec, limbs_of(plan), weight, tiles, out, plan.rows, plan.columns, plan.vectors, stream);
+}
 }  // namespace
 
 uint64_t prepared_input_bytes(const et_linear_plan& plan) {
@@ -358,9 +372,8 @@ int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, co
                                                      std::to_string(plan.workspace_bytes));
         partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + plan.partial_offset);
     }
-    if (hipError_t status = gemm_i8(plan.codec, limbs_of(plan), weight, static_cast<const uint8_t*>(prepared),
-                                    GemmOutput{bias, residual, y, partials}, plan.rows, plan.columns, plan.vectors,
-                                    as_stream(stream)))
+    if (hipError_t status = contract_tiles(plan, weight, static_cast<const uint8_t*>(prepared),
+                                           GemmOutput{bias, residual, y, partials}, as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);
     return ET_OK;
 }
@@ -400,20 +413,18 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         x_row_stride = plan.columns;
     }
 
-    if (plan.kernel == LinearKernel::kGemmI8 || plan.kernel == LinearKernel::kGemmLimb) {
+    if (on_matrix_cores(plan)) {
         if (scratch == nullptr || workspace_bytes < plan.workspace_bytes)
             return fail(error, ET_ERR_EXECUTION,
                         "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
                             " bytes is smaller than the planned " +
                             std::to_string(plan.workspace_bytes));
-        const int limbs = plan.kernel == LinearKernel::kGemmI8 ? 1 : 3;
         auto* tiles = scratch + plan.q_offset;
         if (hipError_t status =
-                quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs, tiles, s))
+                quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs_of(plan), tiles, s))
             return hip_failure(error, "quantized_linear", status);
         float* partials = plan.k_splits > 1 ? reinterpret_cast<float*>(scratch + plan.partial_offset) : nullptr;
-        if (hipError_t status = gemm_i8(plan.codec, limbs, weight, tiles, GemmOutput{bias, nullptr, y, partials},
-                                        plan.rows, plan.columns, plan.vectors, s))
+        if (hipError_t status = contract_tiles(plan, weight, tiles, GemmOutput{bias, nullptr, y, partials}, s))
             return hip_failure(error, "quantized_linear", status);
         return ET_OK;
     }

@@ -33,6 +33,7 @@ enum class LinearKernel {
     kGemvGeneric,  // portable dequant-GEMV (gemv_generic.hip)
     kGemmI8,       // int8 activations: quantize_act.hip + gemm_i8.hip
     kGemmLimb,     // f32-accurate 3-limb activations on the same matrix-core kernel
+    kGemmHalf,     // f32-accurate two-half activations on the half-float matrix cores (gemm_h16)
 };
 
 }  // namespace quantized

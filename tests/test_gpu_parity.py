@@ -212,8 +212,9 @@ def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
 @pytest.mark.parametrize("vectors,rows,columns", [(7, 129, 256), (12, 64, 2304), (33, 1, 512), (65, 300, 1024),
                                                   (100, 130, 4096), (130, 257, 768), (200, 63, 256)])
 def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, rows, columns):
-    # seven or more vectors: 3-limb activations on the matrix cores; ragged tiles on both sides,
-    # one and several stages of 256 columns, ring turns with padding stages
+    # seven or more vectors: fixed-point activations on the matrix cores (two 12-bit halves as half
+    # floats for Q4_K, three byte limbs for the 32-wide codecs); ragged tiles on both sides, one and
+    # several stages of 256 columns, ring turns with padding stages
     rng = np.random.default_rng(codec * 11 + vectors + rows + columns)
     weight = synth.random_weight(codec, rows, columns, rng)
     x = synth.random_activations(vectors, columns, rng)
@@ -221,7 +222,8 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
     bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   None, et.GgmlQuant(codec), (rows, columns))
-    assert plan.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
+    family = "quantize_halves+gemm_h16" if codec == oracle.Q4_K else "quantize_limbs+gemm_i8"
+    assert plan.kernel in (family, family + "+reduce")
     got = run_linear(et, device, codec, rows, columns, x, weight, bias)
     if codec != oracle.Q4_K:
         # a width that is not a whole number of 256-column stages stays on the GEMV kernels
@@ -254,7 +256,7 @@ def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vecto
     act = et.ActivationMode[mode]
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   torch.zeros(rows), et.GgmlQuant(codec), (rows, columns), act)
-    assert plan.kernel.endswith("+gemm_i8+reduce")
+    assert plan.kernel.endswith("+gemm_h16+reduce" if (mode, codec) == ("F32", oracle.Q4_K) else "+gemm_i8+reduce")
     got = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
     again = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
     assert np.array_equal(got, again)  # the same bits on every run
@@ -443,6 +445,38 @@ def test_gguf_file_to_contraction(et, device, tmp_path):
         assert np.array_equal(model.upload_tensor("big.weight", device).cpu().numpy().reshape(-1), big)
         with pytest.raises(et.GgufParseError, match="requires 38080 destination bytes, got 300"):
             model.upload_tensor("blk.0.attn_q.weight", device, torch.empty(300, dtype=torch.uint8, device=device))
+
+
+@pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q6_K])
+def test_embedding_at_vocabulary_scale(et, device, codec):
+    # a [128256, 4096] table, 8192 ids (repeats, the first and the last row): sampled rows against the
+    # oracle bit for bit; every output row equals the first output row of the same id; a table row
+    # gathered is that row of the whole-table decode
+    rng = np.random.default_rng(1200 + codec)
+    rows, columns, base = 128256, 4096, 2048
+    block = synth.random_weight(codec, base, columns, rng)
+    table = np.concatenate([np.roll(block, r, axis=0) for r in range(-(-rows // base))])[:rows]
+    ids = rng.integers(0, rows, 8192).astype(np.int64)
+    ids[:4] = [0, rows - 1, 0, rows - 1]
+    w, index = to_dev(table, device), torch.from_numpy(ids).to(device)
+    plan = et.embedding_requirements(index, w, et.GgmlQuant(codec), (rows, columns))
+    out = torch.full(plan.output_shape, float("nan"), dtype=torch.float32, device=device)
+    et.embedding_into(index, w, et.GgmlQuant(codec), out, plan)
+    got = out.cpu().numpy()
+    picks = np.concatenate([np.arange(4), rng.integers(0, ids.size, 60)])
+    want = oracle.embedding_into(codec, rows, columns, ids[picks], table)
+    assert np.array_equal(bits(got[picks]), bits(want))
+    order = np.argsort(ids, kind="stable")
+    first_of = order[np.searchsorted(ids[order], ids)]  # first position holding the same id
+    assert np.array_equal(bits(got), bits(got[first_of]))
+    # ids of rows that repeat `block` decode to the same values as the block's rows
+    whole = et.dequantize_rows(to_dev(block, device), et.GgmlQuant(codec), (base, columns)).cpu().numpy()
+    source = (ids % base - ids // base) % base  # table row r holds block row (r % base - r // base) mod base
+    assert np.array_equal(bits(got), bits(whole[source]))
+    bad = index.clone()
+    bad[4097] = rows
+    with pytest.raises(et.QuantizedError, match=f"outside 0..{rows}"):
+        et.embedding_into(bad, w, et.GgmlQuant(codec), out, plan)
 
 
 @pytest.mark.parametrize("codec", [oracle.Q2_K, oracle.Q3_K, oracle.Q5_K, oracle.Q6_K])

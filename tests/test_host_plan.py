@@ -48,8 +48,10 @@ def test_linear_plan_shapes(et):
     assert plan.output_bytes == 24  # crates/runtime-metal/src/quantized.rs:1393-1449
     plan = et.linear_requirements(torch.zeros(2, 5, 512), _w(7, 288), torch.zeros(7), et.GgmlQuant.Q4_K, (7, 512))
     assert plan.output_shape == (2, 5, 7) and plan.vectors == 10
-    # ten vectors: 3-limb activations on the matrix cores, with its workspace planned
-    assert plan.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce") and plan.workspace_bytes > 3 * 10 * 512
+    # ten vectors: fixed-point activations on the matrix cores, with its workspace planned
+    assert plan.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce") and plan.workspace_bytes > 4 * 10 * 512
+    plan8 = et.linear_requirements(torch.zeros(10, 512), _w(7, 544), None, et.GgmlQuant.Q8_0, (7, 512))
+    assert plan8.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
     for few in (3, 6):
         plan3 = et.linear_requirements(torch.zeros(few, 512), _w(7, 288), None, et.GgmlQuant.Q4_K, (7, 512))
         assert plan3.kernel == "gemv_limb"
@@ -68,7 +70,7 @@ def test_linear_plan_shapes(et):
     # few 64-row tiles: K is shared over workgroups and a second kernel sums the shares
     few = et.linear_requirements(torch.zeros(32, 4096), _w(1024, 2304), None, et.GgmlQuant.Q4_K, (1024, 4096))
     many = et.linear_requirements(torch.zeros(32, 4096), _w(14336, 2304), None, et.GgmlQuant.Q4_K, (14336, 4096))
-    assert few.kernel == "quantize_limbs+gemm_i8+reduce" and many.kernel == "quantize_limbs+gemm_i8"
+    assert few.kernel == "quantize_halves+gemm_h16+reduce" and many.kernel == "quantize_halves+gemm_h16"
     assert few.workspace_bytes >= 16 * 32 * 1024 * 4  # 16 tiles x 16 stages: one stage per share
     # empty output: nothing to dispatch
     plan = et.linear_requirements(torch.zeros(0, 256), _w(2, 144), None, et.GgmlQuant.Q4_K, (2, 256))
