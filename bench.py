@@ -532,14 +532,29 @@ def llama_decode(args, et):
     chosen = torch.empty(slots, dtype=torch.int32, device=device)
     keep = []
 
+    # the norms and SiLU * up are applied while their results are quantised, where the plans can;
+    # q / k / v, and gate / up, then run as one launch each
+    on_the_fly = fused and all(plans[name].fused_prepare for name in ("wq", "gate", "down", "head"))
+    if on_the_fly:
+        qkv_group = et.LinearGroup([plans["wq"], plans["wk"], plans["wv"]])
+        ffn_group = et.LinearGroup([plans["gate"], plans["up"]])
+        group_ws = torch.empty(max(qkv_group.workspace_bytes, ffn_group.workspace_bytes, 16), dtype=torch.uint8,
+                               device=device)
+
     def layer_step(index):
         w, kvl = weights[index], kv[index]
-        et.rms_norm_into(x, norms[index][0], 1e-5, h)
+        if on_the_fly:
+            plans["wq"].prepare_input_rms_norm(x, norms[index][0], 1e-5, shared_hidden)
+        else:
+            et.rms_norm_into(x, norms[index][0], 1e-5, h)
         if fused:
-            plans["wq"].prepare_input(h, shared_hidden)
-            plans["wq"].enqueue_prepared(shared_hidden, w["wq"], None, q, linear_ws)
-            plans["wk"].enqueue_prepared(shared_hidden, w["wk"], None, k, linear_ws)
-            plans["wv"].enqueue_prepared(shared_hidden, w["wv"], None, v, linear_ws)
+            if on_the_fly:
+                qkv_group.enqueue_prepared(shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v], group_ws)
+            else:
+                plans["wq"].prepare_input(h, shared_hidden)
+                plans["wq"].enqueue_prepared(shared_hidden, w["wq"], None, q, linear_ws)
+                plans["wk"].enqueue_prepared(shared_hidden, w["wk"], None, k, linear_ws)
+                plans["wv"].enqueue_prepared(shared_hidden, w["wv"], None, v, linear_ws)
         else:
             plans["wq"].enqueue(h, w["wq"], None, q, linear_ws)
             plans["wk"].enqueue(h, w["wk"], None, k, linear_ws)
@@ -555,17 +570,27 @@ def llama_decode(args, et):
         else:
             plans["wo"].enqueue(attended, w["wo"], None, projected, linear_ws)
             et.add_into(x, projected, x)
-        et.rms_norm_into(x, norms[index][1], 1e-5, h)
+        if on_the_fly:
+            plans["gate"].prepare_input_rms_norm(x, norms[index][1], 1e-5, shared_hidden)
+        else:
+            et.rms_norm_into(x, norms[index][1], 1e-5, h)
         if fused:
-            plans["gate"].prepare_input(h, shared_hidden)
-            plans["gate"].enqueue_prepared(shared_hidden, w["gate"], None, gate, linear_ws)
-            plans["up"].enqueue_prepared(shared_hidden, w["up"], None, up, linear_ws)
+            if on_the_fly:
+                ffn_group.enqueue_prepared(shared_hidden, [w["gate"], w["up"]], [gate, up], group_ws)
+            else:
+                plans["gate"].prepare_input(h, shared_hidden)
+                plans["gate"].enqueue_prepared(shared_hidden, w["gate"], None, gate, linear_ws)
+                plans["up"].enqueue_prepared(shared_hidden, w["up"], None, up, linear_ws)
         else:
             plans["gate"].enqueue(h, w["gate"], None, gate, linear_ws)
             plans["up"].enqueue(h, w["up"], None, up, linear_ws)
-        et.silu_mul_into(gate, up, gate)
+        if on_the_fly:
+            plans["down"].prepare_input_silu_mul(gate, up, shared_ffn)
+        else:
+            et.silu_mul_into(gate, up, gate)
         if fused:
-            plans["down"].prepare_input(gate, shared_ffn)
+            if not on_the_fly:
+                plans["down"].prepare_input(gate, shared_ffn)
             plans["down"].enqueue_prepared(shared_ffn, w["down"], None, x, linear_ws, residual=x)
         else:
             plans["down"].enqueue(gate, w["down"], None, down, linear_ws)
@@ -576,8 +601,12 @@ def llama_decode(args, et):
         keep.append(et.gather_rows_into(embedding, tokens.view(torch.uint32), x, synchronize=False))
         for index in range(layers):
             layer_step(index)
-        et.rms_norm_into(x, final_norm, 1e-5, h)
-        plans["head"].enqueue(h, base["head"], None, logits, linear_ws)
+        if on_the_fly:
+            plans["head"].prepare_input_rms_norm(x, final_norm, 1e-5, shared_hidden)
+            plans["head"].enqueue_prepared(shared_hidden, base["head"], None, logits, linear_ws)
+        else:
+            et.rms_norm_into(x, final_norm, 1e-5, h)
+            plans["head"].enqueue(h, base["head"], None, logits, linear_ws)
         keep.append(et.greedy_tokens(logits, workspace=greedy_ws, synchronize=False)[1])
 
     # Parity gate: layer 0 for two slots against the CPU oracle chained the same way.

@@ -12,6 +12,7 @@ from .quantized import (  # noqa: F401
     GgmlQuant,
     QuantizedError,
     QuantizedRequirements,
+    LinearGroup,
     RawLinear,
     calibration_copy,
     calibration_read,

@@ -34,6 +34,21 @@ class EtTensor(ctypes.Structure):
     ]
 
 
+class EtPrepareSource(ctypes.Structure):
+    """``et_prepare_source`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("kind", ctypes.c_int32),
+        ("x", ctypes.c_void_p),
+        ("x_row_stride", ctypes.c_uint64),
+        ("second", ctypes.c_void_p),
+        ("eps", ctypes.c_double),
+    ]
+
+
+PREPARE_PLAIN, PREPARE_RMS_NORM, PREPARE_SILU_MUL = 0, 1, 2
+
+
 class EtKvLayer(ctypes.Structure):
     """``et_kv_layer`` of include/et_hip.h."""
 
@@ -97,6 +112,11 @@ SIGNATURES = {
     "et_hip_linear_enqueue": (ctypes.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_linear_plan_prepared_input_bytes": (_u64, [_vp]),
     "et_hip_linear_prepare_input": (ctypes.c_int, [_vp, _vp, _u64, _vp, _u64, _vp]),
+    "et_hip_linear_plan_fused_prepare": (ctypes.c_int, [_vp]),
+    "et_hip_linear_group_workspace_bytes": (ctypes.c_int, [_vp, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint64)]),
+    "et_hip_linear_enqueue_prepared_group": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _u64,
+                                                            _vp, _vp]),
+    "et_hip_linear_prepare_input_from": (ctypes.c_int, [_vp, ctypes.POINTER(EtPrepareSource), _vp, _u64, _vp]),
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
     "et_hip_embedding_plan_destroy": (None, [_vp]),

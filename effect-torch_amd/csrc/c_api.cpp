@@ -203,6 +203,41 @@ int et_hip_linear_prepare_input(const et_linear_plan* plan, const float* x, uint
     });
 }
 
+int et_hip_linear_plan_fused_prepare(const et_linear_plan* plan) {
+    return plan != nullptr && et::quantized::fused_prepare(*plan) ? 1 : 0;
+}
+
+int et_hip_linear_prepare_input_from(const et_linear_plan* plan, const et_prepare_source* source, void* prepared,
+                                     uint64_t prepared_bytes, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr || source == nullptr) {
+            *error = "quantized_linear: plan or source is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_prepare_input_from(*plan, *source, prepared, prepared_bytes, stream, error);
+    });
+}
+
+int et_hip_linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes) {
+    return guarded([&](std::string* error) -> int {
+        if (bytes == nullptr) {
+            *error = "quantized_linear: bytes is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_group_workspace_bytes(plans, count, bytes, error);
+    });
+}
+
+int et_hip_linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                         const uint8_t* const* weights, const float* const* biases,
+                                         const float* const* residuals, float* const* ys, void* workspace,
+                                         uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        return et::quantized::linear_enqueue_prepared_group(plans, count, prepared, weights, biases, residuals, ys,
+                                                            workspace, workspace_bytes, stream, cancel, error);
+    });
+}
+
 int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepared, const uint8_t* weight,
                                    const float* bias, const float* residual, float* y, void* workspace,
                                    uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel) {

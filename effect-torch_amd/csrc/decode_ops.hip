@@ -15,17 +15,13 @@
 
 #include <cmath>
 
+#include "decode_math.h"
 #include "kernels.h"
 
 namespace et {
 namespace {
 
 constexpr uint32_t kArgmaxChunk = 4096;  // logits per workgroup of the first stage
-
-__device__ __forceinline__ double wave_sum(double v) {
-    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset);
-    return v;
-}
 
 // One workgroup of 256 per row. VEC: the row is read as float4 (columns % 4 == 0, 16-byte aligned
 // rows); the first four vectors of a thread stay in registers for the second pass.
@@ -35,57 +31,31 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     __shared__ double partial[4];
     const float* in = x + static_cast<uint64_t>(blockIdx.x) * columns;
     float* row = out + static_cast<uint64_t>(blockIdx.x) * columns;
-    constexpr int kHeld = 4;
-    float4 held[kHeld];
-    double sum = 0.0;
     if constexpr (VEC) {
-        const uint32_t vectors = columns / 4;
-#pragma unroll
-        for (int j = 0; j < kHeld; j++) {
-            const uint32_t i = threadIdx.x + 256 * j;
-            held[j] = i < vectors ? reinterpret_cast<const float4*>(in)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-#pragma unroll
-        for (int j = 0; j < kHeld; j++) {
-            const float4 v = held[j];
-            sum += (static_cast<double>(v.x) * v.x + static_cast<double>(v.y) * v.y) +
-                   (static_cast<double>(v.z) * v.z + static_cast<double>(v.w) * v.w);
-        }
-        for (uint32_t i = threadIdx.x + 256 * kHeld; i < vectors; i += 256) {
-            const float4 v = reinterpret_cast<const float4*>(in)[i];
-            sum += (static_cast<double>(v.x) * v.x + static_cast<double>(v.y) * v.y) +
-                   (static_cast<double>(v.z) * v.z + static_cast<double>(v.w) * v.w);
-        }
-    } else {
-        for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
-    }
-    sum = wave_sum(sum);
-    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
-    __syncthreads();
-    const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
-    const double scale = 1.0 / sqrt(mean_square + eps);
-    const auto one = [&](float value, float w) {
-        return static_cast<float>(static_cast<double>(value) * scale * static_cast<double>(w));
-    };
-    if constexpr (VEC) {
+        float4 held[kRmsHeld];
+        const double scale = rms_row_scale(in, columns, eps, held, partial);
         const uint32_t vectors = columns / 4;
         const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
 #pragma unroll
-        for (int j = 0; j < kHeld; j++) {
+        for (int j = 0; j < kRmsHeld; j++) {
             const uint32_t i = threadIdx.x + 256 * j;
-            if (i < vectors) {
-                const float4 w = weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones;
-                const float4 v = held[j];
-                reinterpret_cast<float4*>(row)[i] = make_float4(one(v.x, w.x), one(v.y, w.y), one(v.z, w.z), one(v.w, w.w));
-            }
+            if (i < vectors)
+                reinterpret_cast<float4*>(row)[i] =
+                    rms_four(held[j], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones);
         }
-        for (uint32_t i = threadIdx.x + 256 * kHeld; i < vectors; i += 256) {
-            const float4 w = weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones;
-            const float4 v = reinterpret_cast<const float4*>(in)[i];
-            reinterpret_cast<float4*>(row)[i] = make_float4(one(v.x, w.x), one(v.y, w.y), one(v.z, w.z), one(v.w, w.w));
-        }
+        for (uint32_t i = threadIdx.x + 256 * kRmsHeld; i < vectors; i += 256)
+            reinterpret_cast<float4*>(row)[i] =
+                rms_four(reinterpret_cast<const float4*>(in)[i], scale,
+                         weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones);
     } else {
-        for (uint32_t i = threadIdx.x; i < columns; i += 256) row[i] = one(in[i], weight != nullptr ? weight[i] : 1.f);
+        double sum = 0.0;
+        for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
+        sum = wave_sum(sum);
+        if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
+        __syncthreads();
+        const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
+        const double scale = 1.0 / sqrt(mean_square + eps);
+        for (uint32_t i = threadIdx.x; i < columns; i += 256) row[i] = rms_one(in[i], scale, weight != nullptr ? weight[i] : 1.f);
     }
 }
 
@@ -112,12 +82,6 @@ __global__ __launch_bounds__(256) void rotary_kernel(const float* __restrict__ x
     const double a = x[first], b = x[second];
     out[first] = static_cast<float>(a * c - b * s);
     out[second] = static_cast<float>(b * c + a * s);
-}
-
-__device__ __forceinline__ float silu_mul_one(float gate, float up) {
-    // Tensor.sigmoid: tanh(x / 2) / 2 + 1 / 2, every step rounded to f32 (Tensor.ts:1240-1245)
-    const float sigmoid = tanhf(gate * 0.5f) * 0.5f + 0.5f;
-    return (gate * sigmoid) * up;
 }
 
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,

@@ -103,11 +103,26 @@ __device__ __forceinline__ v8h nibbles_times(uint32_t first, uint32_t second, v2
     return u.all;
 }
 
+// The matrices of one launch: contractions that share their activations (the q / k / v projections
+// of a decode step) run as one grid over the row tiles of all of them.
+struct Member {
+    const uint8_t* weight;
+    const float* bias;
+    const float* residual;
+    float* y;
+    uint32_t rows;
+    uint32_t first_tile;  // of the launch's row tiles
+};
+struct Group {
+    Member member[kGemmGroupMost];
+    uint32_t count;
+    uint32_t row_tiles;  // of all members together
+};
+
 template <int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
-    const uint8_t* __restrict__ weight, const uint8_t* __restrict__ tiles, uint32_t vector_tiles,
-    const float* __restrict__ bias, const float* residual, float* y, uint32_t rows, uint32_t columns,
-    uint32_t vectors, uint32_t row_tiles, uint32_t k_splits, float* __restrict__ partials) {
+    const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
+    uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
     using S = Shape<AX, AW>;
     constexpr int NB = kBlocksPerWave;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -119,7 +134,13 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const uint32_t row_tile = (turn / units) * 8u + xcd;
     const uint32_t tile = (turn % units) % vector_tiles;
     const uint32_t k_share = (turn % units) / vector_tiles;
-    if (row_tile >= row_tiles) return;
+    if (row_tile >= group.row_tiles) return;
+    uint32_t which = 0;
+    for (uint32_t i = 1; i < group.count; i++)
+        if (row_tile >= group.member[i].first_tile) which = i;
+    const Member& member = group.member[which];
+    const uint8_t* __restrict__ weight = member.weight;
+    const uint32_t rows = member.rows;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -128,7 +149,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const uint32_t first_stage = k_share * share;  // < all_stages: the launcher leaves no share empty
     const uint32_t stages = min(share, all_stages - first_stage);
     const uint64_t row_bytes = static_cast<uint64_t>(all_stages) * kRowBytes;
-    const uint32_t row0 = row_tile * kRows;
+    const uint32_t row0 = (row_tile - member.first_tile) * kRows;  // in the member's own rows
 
     if (wave >= static_cast<uint32_t>(kConsumers + kWeightLoaders)) {
         // ---- activation loaders: linear copies of the stage's blob ----
@@ -286,7 +307,12 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     __syncthreads();
     if (wave_k > 0) return;
     const uint32_t n_out = n0 + in_half;
+    const float* bias = member.bias;
+    const float* residual = member.residual;
+    float* y = member.y;
     const float bias_value = bias != nullptr && n_out < rows ? bias[n_out] : 0.f;
+    const uint32_t launch_row = row_tile * kRows + wave_n * 32u + in_half;  // among the rows of all members
+    const uint64_t launch_rows = static_cast<uint64_t>(group.row_tiles) * kRows;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         float value = acc[r] - acc_min[r];
@@ -299,9 +325,49 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const uint64_t at = static_cast<uint64_t>(m) * rows + n_out;
                 y[at] = residual != nullptr ? (value + bias_value) + residual[at] : value + bias_value;
             } else {
-                partials[(static_cast<uint64_t>(k_share) * vectors + m) * rows + n_out] = value;
+                partials[(static_cast<uint64_t>(k_share) * vectors + m) * launch_rows + launch_row] = value;
             }
         }
+    }
+}
+
+// y[m, n] = bias[n] + the K shares in share order (+ residual[m, n], which may be y itself), for every
+// member of the launch; partials are [share][vector][launch row], four launch rows per thread (a tile
+// of 64 rows belongs to one member).
+__global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, const float* __restrict__ partials,
+                                                           uint32_t vectors, uint32_t k_splits) {
+    const uint64_t launch_rows = static_cast<uint64_t>(group.row_tiles) * kRows;
+    const uint64_t item = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+    if (item >= launch_rows * vectors) return;
+    const uint32_t m = static_cast<uint32_t>(item / launch_rows);
+    const uint32_t launch_row = static_cast<uint32_t>(item - m * launch_rows);
+    const uint32_t row_tile = launch_row / kRows;
+    uint32_t which = 0;
+    for (uint32_t i = 1; i < group.count; i++)
+        if (row_tile >= group.member[i].first_tile) which = i;
+    const Member& member = group.member[which];
+    const uint32_t n = launch_row - member.first_tile * kRows;
+    if (n >= member.rows) return;
+    float4 total = make_float4(0.f, 0.f, 0.f, 0.f);
+    const uint64_t share_stride = launch_rows * vectors;
+    for (uint32_t k = 0; k < k_splits; k++) {
+        const float4 part = *reinterpret_cast<const float4*>(partials + k * share_stride + item);
+        if (k == 0) {
+            total = part;
+        } else {
+            total.x += part.x;
+            total.y += part.y;
+            total.z += part.z;
+            total.w += part.w;
+        }
+    }
+    const float sums[4] = {total.x, total.y, total.z, total.w};
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        if (n + i >= member.rows) break;
+        const uint64_t at = static_cast<uint64_t>(m) * member.rows + n + i;
+        const float with_bias = member.bias != nullptr ? sums[i] + member.bias[n + i] : sums[i];
+        member.y[at] = member.residual != nullptr ? with_bias + member.residual[at] : with_bias;
     }
 }
 
@@ -311,15 +377,41 @@ bool gemm_h16_supported(int32_t codec, uint64_t columns) {
     return codec == kQ4_K && columns % 256 == 0 && columns > 0;
 }
 
-hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
-                    uint64_t rows64, uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
-    if (!gemm_h16_supported(codec, columns64)) return hipErrorInvalidValue;
+uint64_t gemm_h16_group_row_tiles(const GemmMember* members, uint32_t count) {
+    uint64_t tiles = 0;
+    for (uint32_t i = 0; i < count; i++) tiles += (members[i].rows + kRows - 1) / kRows;
+    return tiles;
+}
+
+uint32_t gemm_h16_group_k_splits(uint64_t row_tiles, uint64_t columns, uint64_t vectors) {
+    // the rule of gemm_i8_k_splits for row_tiles tiles of 64 rows
+    return gemm_i8_k_splits(kQ4_K, 2, row_tiles * kRows, columns, vectors);
+}
+
+uint64_t gemm_h16_group_partial_bytes(uint64_t row_tiles, uint64_t columns, uint64_t vectors) {
+    const uint32_t splits = gemm_h16_group_k_splits(row_tiles, columns, vectors);
+    return splits > 1 ? splits * vectors * row_tiles * kRows * 4u : 0;
+}
+
+hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+                          uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+    if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
     constexpr int AX = 2, AW = 3;
     using S = Shape<AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_h16_kernel<AX, AW>;
-    const uint32_t rows = static_cast<uint32_t>(rows64), columns = static_cast<uint32_t>(columns64),
-                   vectors = static_cast<uint32_t>(vectors64);
+    const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
+    Group group = {};
+    group.count = count;
+    uint64_t row_tiles = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        group.member[i] = Member{members[i].weight, members[i].bias, members[i].residual, members[i].y,
+                                 static_cast<uint32_t>(members[i].rows), static_cast<uint32_t>(row_tiles)};
+        if (members[i].rows == 0 || members[i].rows > 0xffffffffull) return hipErrorInvalidValue;
+        row_tiles += (members[i].rows + kRows - 1) / kRows;
+    }
+    if (row_tiles > 0x00ffffffull) return hipErrorInvalidValue;
+    group.row_tiles = static_cast<uint32_t>(row_tiles);
     // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
     static bool allowed[64] = {};
     int device = 0;
@@ -332,17 +424,25 @@ hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, 
         allowed[device] = true;
     }
     const uint32_t vector_tiles = (vectors + 31u) / 32u;
-    const uint32_t row_tiles = (rows + kRows - 1) / kRows;
-    const uint32_t k_splits = out.partials != nullptr ? gemm_i8_k_splits(codec, 2, rows, columns, vectors) : 1u;
-    const uint64_t grid = static_cast<uint64_t>((row_tiles + 7u) / 8u) * 8u * vector_tiles * k_splits;
+    const uint32_t k_splits = partials != nullptr ? gemm_h16_group_k_splits(row_tiles, columns, vectors) : 1u;
+    const uint64_t grid = ((row_tiles + 7u) / 8u) * 8u * vector_tiles * k_splits;
     if (grid > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, weight, tiles,
-                       vector_tiles, out.bias, out.residual, out.y, rows, columns, vectors, row_tiles, k_splits,
-                       out.partials);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, group, tiles,
+                       vector_tiles, columns, vectors, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
-    if (k_splits > 1)
-        return reduce_partials(out.partials, out.bias, out.residual, out.y, rows, vectors, k_splits, stream);
-    return hipSuccess;
+    if (k_splits > 1) {
+        const uint64_t items = row_tiles * kRows * vectors / 4;
+        hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
+                           group, partials, vectors, k_splits);
+    }
+    return hipGetLastError();
+}
+
+hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
+                    uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream) {
+    if (!gemm_h16_supported(codec, columns)) return hipErrorInvalidValue;
+    const GemmMember one = {weight, out.bias, out.residual, out.y, rows};
+    return gemm_h16_group(&one, 1, tiles, out.partials, columns, vectors, stream);
 }
 
 }  // namespace et

@@ -75,6 +75,13 @@ constexpr uint64_t tile_workspace_bytes(int limbs, uint64_t vectors, uint64_t co
 }
 hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vectors, uint64_t columns,
                           int limbs, uint8_t* tiles, hipStream_t stream);
+// The limbs = 2 tiles of silu(gate) * up / of rms_norm(x) * weight (weight may be null), computed
+// on the fly with the arithmetic of silu_mul() / rms_norm() below: the same bits as the operator
+// followed by quantize_tiles, one launch less. columns % 256 == 0, 16-byte aligned rows.
+hipError_t quantize_tiles_silu_mul(const float* gate, const float* up, uint64_t row_stride, uint64_t vectors,
+                                   uint64_t columns, uint8_t* tiles, hipStream_t stream);
+hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const float* weight, double eps,
+                                   uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream);
 
 // ---- gemm_i8.hip: matrix-core contraction over quantised activation tiles ---------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
@@ -102,6 +109,23 @@ hipError_t reduce_partials(const float* partials, const float* bias, const float
 bool gemm_h16_supported(int32_t codec, uint64_t columns);
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream);
+// Several Q4_K matrices of the same width against the same activation tiles in one launch (the q / k /
+// v projections of a decode step): the grid runs over the 64-row tiles of all of them, and K is shared
+// out by the rule of gemm_i8_k_splits for that many tiles. `partials` holds
+// gemm_h16_group_partial_bytes(...) bytes when that is not zero.
+constexpr uint32_t kGemmGroupMost = 4;
+struct GemmMember {
+    const uint8_t* weight;
+    const float* bias;      // [rows] or null
+    const float* residual;  // [vectors, rows] or null; may be y
+    float* y;               // [vectors, rows]
+    uint64_t rows;
+};
+uint64_t gemm_h16_group_row_tiles(const GemmMember* members, uint32_t count);
+uint32_t gemm_h16_group_k_splits(uint64_t row_tiles, uint64_t columns, uint64_t vectors);
+uint64_t gemm_h16_group_partial_bytes(uint64_t row_tiles, uint64_t columns, uint64_t vectors);
+hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+                          uint64_t columns, uint64_t vectors, hipStream_t stream);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch

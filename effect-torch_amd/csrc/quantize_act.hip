@@ -25,6 +25,7 @@
 
 #include <cstdint>
 
+#include "decode_math.h"
 #include "kernels.h"
 
 namespace et {
@@ -128,54 +129,95 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 // Activations for gemm_h16: per vector and 256-column stage, X = clamp(rint(x * (2^23 - 1) / amax))
 // as two balanced 12-bit halves, X = 4096 * hi + lo with lo in [-2048, 2047], both written as half
 // floats (exact); unit = amax / (2^23 - 1); xsum[g] = unit * (integer sum of X over sub-block g).
-// One wave per (vector, stage): lane q holds columns 4q .. 4q + 3 of the stage. Blob layout: see
-// tile_blob_bytes() in kernels.h.
-__global__ __launch_bounds__(64) void quantize_halves_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+// One wave per (vector, stage): lane `quad` holds columns 4 quad .. 4 quad + 3 of the stage. Blob
+// layout: see tile_blob_bytes() in kernels.h.
+__device__ __forceinline__ void quantize_halves_store(const float4& in, uint32_t v, uint32_t stage, uint32_t quad,
+                                                      uint32_t vector_tiles, uint8_t* __restrict__ tiles) {
+    constexpr float kRange = 8388607.f;  // 2^23 - 1
+    float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) amax = fmaxf(amax, __shfl_xor(amax, step));
+    const float inv = amax > 0.f ? kRange / amax : 0.f;
+    const float values[4] = {in.x, in.y, in.z, in.w};
+    int total = 0;
+    union {
+        _Float16 h[4];
+        uint2 words;
+    } low, high;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float r = fminf(fmaxf(rintf(values[i] * inv), -kRange), kRange);
+        const int q = static_cast<int>(r);
+        const int lo = ((q + 2048) & 4095) - 2048;
+        total += q;
+        low.h[i] = static_cast<_Float16>(lo);
+        high.h[i] = static_cast<_Float16>((q - lo) >> 12);  // exact: q - lo is a multiple of 4096
+    }
+    total += dpp_i32<0xB1>(total);   // the eight lanes of a 32-column sub-block
+    total += dpp_i32<0x4E>(total);
+    total += dpp_i32<0x141>(total);
+    const float unit = amax / kRange;
+    uint8_t* blob = tiles + (static_cast<uint64_t>(stage) * vector_tiles + (v >> 5)) * tile_blob_bytes(2);
+    // columns 4 quad .. + 3 = sub-block quad / 8, 16-column half, 8-column part, first or second four
+    const uint32_t at = (quad >> 1) * 512u + (v & 31u) * 16u + (quad & 1u) * 8u;
+    *reinterpret_cast<uint2*>(blob + at) = low.words;
+    *reinterpret_cast<uint2*>(blob + 16384u + at) = high.words;
+    float* tables = reinterpret_cast<float*>(blob + 32768u);
+    if (quad == 0) tables[v & 31u] = unit;
+    if ((quad & 7u) == 0) tables[32u + (quad >> 3) * 32u + (v & 31u)] = unit * static_cast<float>(total);
+}
+
+// SILU_MUL: the activations are silu(x) * second, element by element (the input of a gated
+// feed-forward's down projection), computed on the fly with silu_mul_kernel's arithmetic.
+template <bool SILU_MUL>
+__global__ __launch_bounds__(64) void quantize_halves_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ second, uint64_t x_row_stride,
                                                              uint32_t vectors, uint32_t stages,
                                                              uint8_t* __restrict__ tiles) {
-    constexpr float kRange = 8388607.f;  // 2^23 - 1
     const uint32_t vector_tiles = (vectors + 31u) >> 5;
     const uint32_t quad = threadIdx.x;
     for (uint64_t item = blockIdx.x; item < static_cast<uint64_t>(vectors) * stages; item += gridDim.x) {
         const uint32_t v = static_cast<uint32_t>(item / stages), stage = static_cast<uint32_t>(item % stages);
-        const float4 in = *reinterpret_cast<const float4*>(x + v * x_row_stride + 256u * stage + 4u * quad);
-        float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
-#pragma unroll
-        for (int step = 1; step < 64; step <<= 1) amax = fmaxf(amax, __shfl_xor(amax, step));
-        const float inv = amax > 0.f ? kRange / amax : 0.f;
-        const float values[4] = {in.x, in.y, in.z, in.w};
-        int total = 0;
-        _Float16 low[4], high[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float r = fminf(fmaxf(rintf(values[i] * inv), -kRange), kRange);
-            const int q = static_cast<int>(r);
-            const int lo = ((q + 2048) & 4095) - 2048;
-            total += q;
-            low[i] = static_cast<_Float16>(lo);
-            high[i] = static_cast<_Float16>((q - lo) >> 12);  // exact: q - lo is a multiple of 4096
+        const uint64_t at = v * x_row_stride + 256u * stage + 4u * quad;
+        float4 in = *reinterpret_cast<const float4*>(x + at);
+        if constexpr (SILU_MUL) {
+            const float4 up = *reinterpret_cast<const float4*>(second + at);
+            in = make_float4(silu_mul_one(in.x, up.x), silu_mul_one(in.y, up.y), silu_mul_one(in.z, up.z),
+                             silu_mul_one(in.w, up.w));
         }
-        total += dpp_i32<0xB1>(total);   // the eight lanes of a 32-column sub-block
-        total += dpp_i32<0x4E>(total);
-        total += dpp_i32<0x141>(total);
-        const float unit = amax / kRange;
-        uint8_t* blob = tiles + (static_cast<uint64_t>(stage) * vector_tiles + (v >> 5)) * tile_blob_bytes(2);
-        // columns 4 quad .. + 3 = sub-block quad / 8, 16-column half, 8-column part, first or second four
-        const uint32_t at = (quad >> 1) * 512u + (v & 31u) * 16u + (quad & 1u) * 8u;
-        union {
-            _Float16 h[4];
-            uint2 words;
-        } lo_words, hi_words;
+        quantize_halves_store(in, v, stage, quad, vector_tiles, tiles);
+    }
+}
+
+// The activations are rms_norm(x) * weight, with rms_norm_kernel's arithmetic: one workgroup of 256
+// per vector finds the row's scale, then wave w quantises stages w, w + 4, ... - float4 number
+// threadIdx.x + 256 j of the row is lane threadIdx.x % 64 of stage threadIdx.x / 64 + 4 j.
+__global__ __launch_bounds__(256) void quantize_halves_rms_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+                                                                  const float* __restrict__ weight, double eps,
+                                                                  uint32_t vectors, uint32_t columns,
+                                                                  uint8_t* __restrict__ tiles) {
+    __shared__ double partial[4];
+    const uint32_t v = blockIdx.x;
+    const float* in = x + v * x_row_stride;
+    float4 held[kRmsHeld];
+    const double scale = rms_row_scale(in, columns, eps, held, partial);
+    const uint32_t vector_tiles = (vectors + 31u) >> 5, stages = columns >> 8;
+    const uint32_t wave = threadIdx.x >> 6, quad = threadIdx.x & 63u;
+    const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            lo_words.h[i] = low[i];
-            hi_words.h[i] = high[i];
+    for (int j = 0; j < kRmsHeld; j++) {
+        const uint32_t stage = wave + 4u * j;  // uniform in the wave
+        if (stage < stages) {
+            const uint32_t i = threadIdx.x + 256u * j;
+            quantize_halves_store(rms_four(held[j], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
+                                  v, stage, quad, vector_tiles, tiles);
         }
-        *reinterpret_cast<uint2*>(blob + at) = lo_words.words;
-        *reinterpret_cast<uint2*>(blob + 16384u + at) = hi_words.words;
-        float* tables = reinterpret_cast<float*>(blob + 32768u);
-        if (quad == 0) tables[v & 31u] = unit;
-        if ((quad & 7u) == 0) tables[32u + (quad >> 3) * 32u + (v & 31u)] = unit * static_cast<float>(total);
+    }
+    for (uint32_t stage = wave + 4u * kRmsHeld; stage < stages; stage += 4u) {
+        const uint32_t i = 64u * stage + quad;
+        quantize_halves_store(rms_four(reinterpret_cast<const float4*>(in)[i], scale,
+                                       weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
+                              v, stage, quad, vector_tiles, tiles);
     }
 }
 
@@ -210,8 +252,8 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
     if (limbs == 2) {
         if (columns % 256 != 0) return hipErrorInvalidValue;
         const uint64_t items = vectors * (columns / 256);
-        hipLaunchKernelGGL(quantize_halves_kernel, dim3(static_cast<uint32_t>(items < 65536 ? items : 65536)), dim3(64),
-                           0, stream, x, x_row_stride, static_cast<uint32_t>(vectors),
+        hipLaunchKernelGGL(quantize_halves_kernel<false>, dim3(static_cast<uint32_t>(items < 65536 ? items : 65536)),
+                           dim3(64), 0, stream, x, nullptr, x_row_stride, static_cast<uint32_t>(vectors),
                            static_cast<uint32_t>(columns / 256), tiles);
         return hipGetLastError();
     }
@@ -226,6 +268,26 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
         hipLaunchKernelGGL((quantize_kernel<3, true>), grid, block, 0, stream, x, x_row_stride,
                            static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns),
                            reinterpret_cast<int8_t*>(tiles), nullptr, nullptr);
+    return hipGetLastError();
+}
+
+hipError_t quantize_tiles_silu_mul(const float* gate, const float* up, uint64_t row_stride, uint64_t vectors,
+                                   uint64_t columns, uint8_t* tiles, hipStream_t stream) {
+    if (columns % 256 != 0) return hipErrorInvalidValue;
+    const uint64_t items = vectors * (columns / 256);
+    if (items == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_halves_kernel<true>, dim3(static_cast<uint32_t>(items < 65536 ? items : 65536)),
+                       dim3(64), 0, stream, gate, up, row_stride, static_cast<uint32_t>(vectors),
+                       static_cast<uint32_t>(columns / 256), tiles);
+    return hipGetLastError();
+}
+
+hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const float* weight, double eps,
+                                   uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream) {
+    if (columns % 256 != 0 || vectors > 0x7fffffffull) return hipErrorInvalidValue;
+    if (vectors == 0 || columns == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_halves_rms_kernel, dim3(static_cast<uint32_t>(vectors)), dim3(256), 0, stream, x,
+                       x_row_stride, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
 }
 

@@ -122,7 +122,9 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         plan->k_splits = gemm_i8_k_splits(plan->codec, limbs, plan->rows, plan->columns, plan->vectors);
         if (plan->k_splits > 1) {
             plan->partial_offset = cursor;
-            cursor = align_up(cursor + plan->k_splits * plan->vectors * plan->rows * 4u, 256);
+            // gemm_h16 keeps its partial results by whole 64-row tiles
+            const uint64_t partial_rows = limbs == 2 ? (plan->rows + 63) / 64 * 64 : plan->rows;
+            cursor = align_up(cursor + plan->k_splits * plan->vectors * partial_rows * 4u, 256);
         }
     };
     if (plan->activation_mode == ET_ACT_INT8) {
@@ -350,6 +352,96 @@ int linear_prepare_input(const et_linear_plan& plan, const float* x, uint64_t x_
         return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
     if (hipError_t status = quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs_of(plan),
                                            static_cast<uint8_t*>(prepared), as_stream(stream)))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
+bool fused_prepare(const et_linear_plan& plan) { return plan.kernel == LinearKernel::kGemmHalf; }
+
+int linear_prepare_input_from(const et_linear_plan& plan, const et_prepare_source& source, void* prepared,
+                              uint64_t prepared_bytes, void* stream, std::string* error) {
+    if (source.kind == ET_PREPARE_PLAIN)
+        return linear_prepare_input(plan, source.x, source.x_row_stride, prepared, prepared_bytes, stream, error);
+    if (source.kind != ET_PREPARE_RMS_NORM && source.kind != ET_PREPARE_SILU_MUL)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: unknown prepared-input kind " + std::to_string(source.kind));
+    if (!fused_prepare(plan))
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "quantized_linear: this plan's prepared input cannot be computed from an operator on the fly");
+    if (prepared == nullptr || prepared_bytes < prepared_input_bytes(plan))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: prepared-input buffer of " + std::to_string(prepared_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(prepared_input_bytes(plan)) +
+                                                 " required");
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (source.x == nullptr || !aligned(source.x) || source.x_row_stride % 4 != 0 || source.x_row_stride < plan.columns ||
+        !aligned(prepared) || !aligned(source.second) || (source.kind == ET_PREPARE_SILU_MUL && source.second == nullptr))
+        return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
+    hipError_t status;
+    if (source.kind == ET_PREPARE_RMS_NORM) {
+        if (!(source.eps == source.eps))
+            return fail(error, ET_ERR_INVALID, "quantized_linear: rms norm epsilon is not a number");
+        status = quantize_tiles_rms_norm(source.x, source.x_row_stride, source.second, source.eps, plan.vectors,
+                                         plan.columns, static_cast<uint8_t*>(prepared), as_stream(stream));
+    } else {
+        status = quantize_tiles_silu_mul(source.x, source.second, source.x_row_stride, plan.vectors, plan.columns,
+                                         static_cast<uint8_t*>(prepared), as_stream(stream));
+    }
+    if (status != hipSuccess) return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
+namespace {
+// What a group launch needs of its members: the same prepared input, all on gemm_h16.
+int check_group(const et_linear_plan* const* plans, uint32_t count, std::string* error) {
+    if (plans == nullptr || count == 0 || count > kGemmGroupMost)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: a group holds 1 to " + std::to_string(kGemmGroupMost) + " plans");
+    for (uint32_t i = 0; i < count; i++) {
+        if (plans[i] == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: plan is NULL");
+        if (plans[i]->kernel != LinearKernel::kGemmHalf)
+            return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: this plan's kernel has no group launch");
+        if (plans[i]->columns != plans[0]->columns || plans[i]->vectors != plans[0]->vectors)
+            return fail(error, ET_ERR_INVALID, "quantized_linear: the plans of a group must share columns and vectors");
+    }
+    return ET_OK;
+}
+uint64_t group_row_tiles(const et_linear_plan* const* plans, uint32_t count) {
+    uint64_t tiles = 0;
+    for (uint32_t i = 0; i < count; i++) tiles += (plans[i]->rows + 63) / 64;
+    return tiles;
+}
+}  // namespace
+
+int linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes, std::string* error) {
+    if (int rc = check_group(plans, count, error)) return rc;
+    *bytes = gemm_h16_group_partial_bytes(group_row_tiles(plans, count), plans[0]->columns, plans[0]->vectors);
+    return ET_OK;
+}
+
+int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                  const uint8_t* const* weights, const float* const* biases,
+                                  const float* const* residuals, float* const* ys, void* workspace,
+                                  uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                                  std::string* error) {
+    if (int rc = check_group(plans, count, error)) return rc;
+    if (weights == nullptr || ys == nullptr || prepared == nullptr)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+    GemmMember members[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) {
+        const float* bias = biases != nullptr ? biases[i] : nullptr;
+        if ((bias != nullptr) != plans[i]->has_bias)
+            return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias presence does not match the immutable plan");
+        if (weights[i] == nullptr || ys[i] == nullptr)
+            return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+        members[i] = GemmMember{weights[i], bias, residuals != nullptr ? residuals[i] : nullptr, ys[i], plans[i]->rows};
+    }
+    if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (plans[0]->vectors == 0) return ET_OK;
+    const uint64_t need = gemm_h16_group_partial_bytes(group_row_tiles(plans, count), plans[0]->columns, plans[0]->vectors);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(need) + " the group needs");
+    if (hipError_t status = gemm_h16_group(members, count, static_cast<const uint8_t*>(prepared),
+                                           need > 0 ? static_cast<float*>(workspace) : nullptr, plans[0]->columns,
+                                           plans[0]->vectors, as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);
     return ET_OK;
 }

@@ -94,6 +94,19 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
 uint64_t prepared_input_bytes(const et_linear_plan& plan);
 int linear_prepare_input(const et_linear_plan& plan, const float* x, uint64_t x_row_stride, void* prepared,
                          uint64_t prepared_bytes, void* stream, std::string* error);
+// The prepared input of rms_norm(x) * second or silu(x) * second (et_prepare_source in et_hip.h):
+// only for plans whose prepared form has a quantiser that applies the operator on the fly.
+bool fused_prepare(const et_linear_plan& plan);
+int linear_prepare_input_from(const et_linear_plan& plan, const et_prepare_source& source, void* prepared,
+                              uint64_t prepared_bytes, void* stream, std::string* error);
+// Several plans of the same columns and vectors against one prepared input in one launch (see
+// et_hip_linear_enqueue_prepared_group in et_hip.h).
+int linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes, std::string* error);
+int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                  const uint8_t* const* weights, const float* const* biases,
+                                  const float* const* residuals, float* const* ys, void* workspace,
+                                  uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
+                                  std::string* error);
 // y = W x (+ bias) (+ residual, which may be y itself) from a prepared input.
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,

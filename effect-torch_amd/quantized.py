@@ -337,6 +337,31 @@ class RawLinear:
                                                    prepared.data_ptr(), prepared.numel() * prepared.element_size(),
                                                    _stream_handle(stream)))
 
+    @property
+    def fused_prepare(self) -> bool:
+        """Whether :meth:`prepare_input_rms_norm` and :meth:`prepare_input_silu_mul` exist for this plan."""
+        return bool(N.lib().et_hip_linear_plan_fused_prepare(self.requirements._handle))
+
+    def _prepare_from(self, kind: int, x: torch.Tensor, second: Optional[torch.Tensor], eps: float,
+                      prepared: torch.Tensor, stream) -> None:
+        source = N.EtPrepareSource(kind, x.data_ptr(), x.stride(0), second.data_ptr() if second is not None else None,
+                                   float(eps))
+        _check(N.lib().et_hip_linear_prepare_input_from(self.requirements._handle, ctypes.byref(source),
+                                                        prepared.data_ptr(), prepared.numel() * prepared.element_size(),
+                                                        _stream_handle(stream)))
+
+    def prepare_input_rms_norm(self, x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
+                               prepared: torch.Tensor, stream=None) -> None:
+        """The prepared input of ``rms_norm(x) * weight`` without the operator's own launch: the same
+        bytes as :func:`rms_norm_into` followed by :meth:`prepare_input`."""
+        self._prepare_from(N.PREPARE_RMS_NORM, x, weight, eps, prepared, stream)
+
+    def prepare_input_silu_mul(self, gate: torch.Tensor, up: torch.Tensor, prepared: torch.Tensor, stream=None) -> None:
+        """The prepared input of ``silu(gate) * up`` (rows of ``up`` laid out like those of ``gate``)."""
+        if up.stride(0) != gate.stride(0):
+            raise QuantizedError(N.ERR_INVALID, "quantized_linear: gate and up must share their row stride")
+        self._prepare_from(N.PREPARE_SILU_MUL, gate, up, 0.0, prepared, stream)
+
     def enqueue_prepared(self, prepared: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                          y: torch.Tensor, workspace: Optional[torch.Tensor] = None,
                          residual: Optional[torch.Tensor] = None, stream=None,
@@ -349,6 +374,34 @@ class RawLinear:
             self.requirements._handle, prepared.data_ptr(), weight.data_ptr(),
             bias.data_ptr() if bias is not None else None, residual.data_ptr() if residual is not None else None,
             y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
+
+
+class LinearGroup:
+    """Up to four :class:`RawLinear` plans of the same columns and vectors that run from one prepared
+    input in one launch (``et_hip_linear_enqueue_prepared_group``)."""
+
+    def __init__(self, plans: Sequence["RawLinear"]):
+        self.plans = list(plans)
+        self._handles = (ctypes.c_void_p * len(self.plans))(*[p.requirements._handle for p in self.plans])
+        size = ctypes.c_uint64()
+        _check(N.lib().et_hip_linear_group_workspace_bytes(self._handles, len(self.plans), ctypes.byref(size)))
+        self.workspace_bytes = int(size.value)
+
+    def enqueue_prepared(self, prepared: torch.Tensor, weights: Sequence[torch.Tensor],
+                         ys: Sequence[torch.Tensor], workspace: Optional[torch.Tensor] = None,
+                         biases: Optional[Sequence[Optional[torch.Tensor]]] = None,
+                         residuals: Optional[Sequence[Optional[torch.Tensor]]] = None, stream=None,
+                         cancelled: Optional[CancellationFlag] = None) -> None:
+        count = len(self.plans)
+        pointers = lambda tensors: (ctypes.c_void_p * count)(  # noqa: E731
+            *[t.data_ptr() if t is not None else None for t in tensors])
+        _check(N.lib().et_hip_linear_enqueue_prepared_group(
+            self._handles, count, prepared.data_ptr(), pointers(weights),
+            pointers(biases) if biases is not None else None,
+            pointers(residuals) if residuals is not None else None, pointers(ys),
+            workspace.data_ptr() if workspace is not None else None,
+            workspace.numel() * workspace.element_size() if workspace is not None else 0,
+            _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
 
 
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:

@@ -173,6 +173,41 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
 uint64_t et_hip_linear_plan_prepared_input_bytes(const et_linear_plan* plan);
 int et_hip_linear_prepare_input(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
                                 void* prepared, uint64_t prepared_bytes, void* stream);
+/* The prepared input of an operator's RESULT, without the operator's own launch or its f32 output:
+ * the activations are computed element by element while they are quantised, with the arithmetic of
+ * the stand-alone operator, so the prepared bytes are those of the operator followed by
+ * et_hip_linear_prepare_input. Kinds: ET_PREPARE_RMS_NORM, rms_norm(x) * second (second = the
+ * weight [columns], or NULL; et_hip_rms_norm_into, crates/runtime-cpu/src/composed.rs:1491-1533),
+ * and ET_PREPARE_SILU_MUL, silu(x) * second (second = the up projection, laid out like x;
+ * et_hip_silu_mul_into). ET_PREPARE_PLAIN is et_hip_linear_prepare_input. Only plans with
+ * et_hip_linear_plan_fused_prepare(plan) != 0 take the first two; the others return
+ * ET_ERR_UNSUPPORTED and the caller runs the operator itself. No counterpart in the reference,
+ * whose executor runs one operator at a time. */
+typedef enum { ET_PREPARE_PLAIN = 0, ET_PREPARE_RMS_NORM = 1, ET_PREPARE_SILU_MUL = 2 } et_prepare_kind;
+typedef struct et_prepare_source {
+    int32_t kind;           /* et_prepare_kind */
+    const float* x;         /* [vectors, columns] f32, rows x_row_stride elements apart, 16-byte aligned */
+    uint64_t x_row_stride;
+    const float* second;    /* see the kinds above */
+    double eps;             /* ET_PREPARE_RMS_NORM */
+} et_prepare_source;
+int et_hip_linear_plan_fused_prepare(const et_linear_plan* plan);
+int et_hip_linear_prepare_input_from(const et_linear_plan* plan, const et_prepare_source* source,
+                                     void* prepared, uint64_t prepared_bytes, void* stream);
+/* Up to four contractions from the same prepared input in ONE launch: the q / k / v projections of
+ * a decode step are three small matrices, each of which alone leaves most of the device idle.
+ * The grid runs over the 64-row tiles of all members; results are those of
+ * et_hip_linear_enqueue_prepared per member up to the order of the K shares (the same order on
+ * every run). Every plan must have et_hip_linear_plan_fused_prepare(plan) != 0 and share columns
+ * and vectors; weights / biases / residuals / ys hold one device pointer per plan (biases and
+ * residuals may be NULL, or hold NULL entries). The workspace is the group's own:
+ * et_hip_linear_group_workspace_bytes. No counterpart in the reference. */
+int et_hip_linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes);
+int et_hip_linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                         const uint8_t* const* weights, const float* const* biases,
+                                         const float* const* residuals, float* const* ys, void* workspace,
+                                         uint64_t workspace_bytes, void* stream,
+                                         const volatile int32_t* cancel);
 int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepared,
                                    const uint8_t* weight, const float* bias, const float* residual,
                                    float* y, void* workspace, uint64_t workspace_bytes, void* stream,

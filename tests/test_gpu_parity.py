@@ -534,3 +534,92 @@ def test_shared_prepared_input_and_residual_epilogue(et, device, mode):
     assert small.prepared_input_bytes == 0
     with pytest.raises(et.QuantizedError, match="takes the activations as they are"):
         small.prepare_input(x[:2], prepared)
+
+
+def test_prepared_input_of_an_operator_on_the_fly(et, device):
+    # rms_norm(x) * w and silu(gate) * up applied while the activations are quantised: the prepared
+    # bytes, and so every contraction from them, are those of the operator followed by prepare_input
+    rng = np.random.default_rng(77)
+    vectors = 33
+    for columns in (4096, 5632):  # 16 stages: all in registers; 22: the tail loop of the norm
+        plan = et.RawLinear(et.GgmlQuant.Q4_K, 64, columns, vectors)
+        assert plan.fused_prepare and plan.prepared_input_bytes > 0
+        x = to_dev(synth.random_activations(vectors, columns, rng, 3.0), device)
+        x[5, 256:512] = 0.0
+        weight = to_dev(rng.standard_normal(columns).astype(np.float32), device)
+        plain, fused = (torch.zeros(plan.prepared_input_bytes, dtype=torch.uint8, device=device) for _ in range(2))
+        for w in (weight, None):
+            normed = torch.empty_like(x)
+            et.rms_norm_into(x, w, 1e-5, normed)
+            plan.prepare_input(normed, plain)
+            plan.prepare_input_rms_norm(x, w, 1e-5, fused)
+            assert torch.equal(plain, fused)
+        gate, up = x * 2.0, to_dev(synth.random_activations(vectors, columns, rng), device)
+        product = torch.empty_like(gate)
+        et.silu_mul_into(gate, up, product)
+        plan.prepare_input(product, plain)
+        plan.prepare_input_silu_mul(gate, up, fused)
+        assert torch.equal(plain, fused)
+    # plans without such a quantiser say so
+    small = et.RawLinear(et.GgmlQuant.Q4_K, 64, 4096, 2)
+    int8 = et.RawLinear(et.GgmlQuant.Q4_K, 64, 4096, vectors, False, et.ActivationMode.INT8)
+    assert not small.fused_prepare and not int8.fused_prepare
+    buffer = torch.zeros(max(int8.prepared_input_bytes, 16), dtype=torch.uint8, device=device)
+    with pytest.raises(et.QuantizedError, match="on the fly"):
+        int8.prepare_input_rms_norm(x[:, :4096].contiguous(), None, 1e-5, buffer)
+
+
+def test_group_launch_of_contractions_sharing_their_input(et, device):
+    # q / k / v style: three matrices, one prepared input, one launch over the row tiles of all
+    rng = np.random.default_rng(88)
+    columns, vectors = 4096, 32
+    x_host = synth.random_activations(vectors, columns, rng)
+    x = to_dev(x_host, device)
+    sizes = (4096, 1024, 1000)  # the last one ends in a ragged tile
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors, rows == 1024) for rows in sizes]
+    group = et.LinearGroup(plans)
+    assert group.workspace_bytes >= 2 * vectors * sum(-(-rows // 64) * 64 for rows in sizes) * 4  # two K shares
+    prepared = torch.empty(plans[0].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[0].prepare_input(x, prepared)
+    host_weights = [synth.random_weight(oracle.Q4_K, rows, columns, rng) for rows in sizes]
+    weights = [to_dev(w, device) for w in host_weights]
+    bias_host = rng.standard_normal(1024).astype(np.float32)
+    biases = [None, to_dev(bias_host, device), None]
+    residual = to_dev(rng.standard_normal((vectors, 4096)).astype(np.float32), device)
+    workspace = torch.empty(group.workspace_bytes, dtype=torch.uint8, device=device)
+    runs = []
+    for _ in range(2):
+        ys = [torch.full((vectors, rows), float("nan"), device=device) for rows in sizes]
+        group.enqueue_prepared(prepared, weights, ys, workspace, biases=biases, residuals=[residual, None, None])
+        runs.append([y.cpu().numpy() for y in ys])
+    for first, second in zip(*runs):
+        assert np.array_equal(first, second)  # the same bits on every run
+    for index, rows in enumerate(sizes):
+        want = oracle.linear_rows(oracle.Q4_K, rows, columns, x_host, host_weights[index],
+                                  bias_host if index == 1 else None, 0, min(rows, 192))[:, :min(rows, 192)]
+        got = runs[0][index][:, :min(rows, 192)]
+        if index == 0:
+            got = got - residual.cpu().numpy()[:, :192]
+        close(got, want)
+        # all rows against the member's own launch (another order of the K shares: not the same bits)
+        alone = torch.empty((vectors, rows), device=device)
+        single_ws = torch.empty(max(plans[index].requirements.workspace_bytes, 16), dtype=torch.uint8, device=device)
+        plans[index].enqueue_prepared(prepared, weights[index], biases[index], alone, single_ws,
+                                      residual=residual if index == 0 else None)
+        close(runs[0][index], alone.cpu().numpy())
+    # two large members: no K shares either way, so the group writes the bits of the single launches
+    big = [et.RawLinear(et.GgmlQuant.Q4_K, 14336, columns, vectors) for _ in range(2)]
+    pair = et.LinearGroup(big)
+    assert pair.workspace_bytes == 0
+    big_weights = [to_dev(synth.random_weight(oracle.Q4_K, 14336, columns, rng), device) for _ in range(2)]
+    together = [torch.empty((vectors, 14336), device=device) for _ in range(2)]
+    pair.enqueue_prepared(prepared, big_weights, together)
+    for index in range(2):
+        alone = torch.empty((vectors, 14336), device=device)
+        big[index].enqueue_prepared(prepared, big_weights[index], None, alone, None)
+        assert torch.equal(alone, together[index])
+    # members must share the prepared input, and run on the kernel that has the group launch
+    with pytest.raises(et.QuantizedError, match="share columns and vectors"):
+        et.LinearGroup([plans[0], et.RawLinear(et.GgmlQuant.Q4_K, 64, 512, vectors)])
+    with pytest.raises(et.QuantizedError, match="no group launch"):
+        et.LinearGroup([et.RawLinear(et.GgmlQuant.Q4_K, 64, columns, 2)])
