@@ -42,19 +42,17 @@ constexpr int kWeightLoaders = 2;
 constexpr int kActivationLoaders = 2;
 constexpr int kLoaders = kWeightLoaders + kActivationLoaders;
 constexpr int kThreads = 64 * (kConsumers + kLoaders);
-constexpr int kSplit = 4;
-constexpr int kRowGroups = kConsumers / kSplit;
-constexpr int kBlocksPerWave = kStageBlocks / kSplit;
-constexpr uint32_t kRows = 32 * kRowGroups;
+// RG = 32-row groups per workgroup (2 or 4): the eight consumers are RG groups of 8 / RG waves that
+// split the eight sub-blocks of a stage, RG each. Four groups (128 rows) halve the activation bytes a
+// workgroup copies per weight row; two groups (64 rows) make twice as many workgroups.
+constexpr uint32_t kSmallRows = 64;  // rows of a workgroup with RG = 2: the unit of the K-share rule
 
 constexpr uint32_t kBlob = tile_blob_bytes(2);  // in memory and in LDS
 constexpr uint32_t kUnitAt = 32768u;            // unit[m]
 constexpr uint32_t kSumsAt = 32768u + 128u;     // xsum[g][m]
 constexpr uint32_t kRowBytes = 144u;            // a row's share of a stage
-constexpr uint32_t kWeightBytes = kRows * kRowBytes;
-constexpr int kWeightJobs = kWeightBytes / 1024;
 constexpr int kActivationJobs = kBlob / 1024;
-static_assert(kWeightBytes % 1024 == 0 && kBlob % 1024 == 0, "whole copy instructions");
+static_assert(kBlob % 1024 == 0, "whole copy instructions");
 
 // (scale, min) of Q4_K sub-block g (crates/runtime-cpu/src/quantized.rs:77-86).
 __device__ __forceinline__ void q4k_scale_min(const uint4& header, uint32_t g, uint32_t& sc, uint32_t& mn) {
@@ -71,8 +69,13 @@ constexpr int vmcnt_only(int n) {
     return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
 }
 
-template <int AX, int AW>
+template <int RG, int AX, int AW>
 struct Shape {
+    static constexpr int kRowGroups = RG, kSplit = kConsumers / RG, kBlocksPerWave = kStageBlocks / kSplit;
+    static constexpr uint32_t kRows = 32 * RG;
+    static constexpr uint32_t kWeightBytes = kRows * kRowBytes;
+    static constexpr int kWeightJobs = kWeightBytes / 1024;
+    static_assert(kWeightBytes % 1024 == 0, "whole copy instructions");
     static constexpr int kActivationDepth = AX + 1, kWeightDepth = AW + 1;
     static constexpr uint32_t kWeightRingAt = kActivationDepth * kBlob;
     static constexpr uint32_t kRingBytes = kWeightRingAt + kWeightDepth * kWeightBytes;
@@ -119,12 +122,14 @@ struct Group {
     uint32_t row_tiles;  // of all members together
 };
 
-template <int AX, int AW>
+template <int RG, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
     uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
-    using S = Shape<AX, AW>;
-    constexpr int NB = kBlocksPerWave;
+    using S = Shape<RG, AX, AW>;
+    constexpr int NB = S::kBlocksPerWave;
+    constexpr int kSplit = S::kSplit, kRowGroups = S::kRowGroups, kWeightJobs = S::kWeightJobs;
+    constexpr uint32_t kRows = S::kRows, kWeightBytes = S::kWeightBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     // Workgroups go to the eight XCDs round-robin; all vector tiles and K shares of one row tile
@@ -333,9 +338,9 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
 
 // y[m, n] = bias[n] + the K shares in share order (+ residual[m, n], which may be y itself), for every
 // member of the launch; partials are [share][vector][launch row], four launch rows per thread (a tile
-// of 64 rows belongs to one member).
+// of kRows rows belongs to one member).
 __global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, const float* __restrict__ partials,
-                                                           uint32_t vectors, uint32_t k_splits) {
+                                                           uint32_t vectors, uint32_t k_splits, uint32_t kRows) {
     const uint64_t launch_rows = static_cast<uint64_t>(group.row_tiles) * kRows;
     const uint64_t item = (static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
     if (item >= launch_rows * vectors) return;
@@ -377,38 +382,49 @@ bool gemm_h16_supported(int32_t codec, uint64_t columns) {
     return codec == kQ4_K && columns % 256 == 0 && columns > 0;
 }
 
-uint64_t gemm_h16_group_row_tiles(const GemmMember* members, uint32_t count) {
-    uint64_t tiles = 0;
-    for (uint32_t i = 0; i < count; i++) tiles += (members[i].rows + kRows - 1) / kRows;
-    return tiles;
+GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors) {
+    const uint64_t stages = columns / 256, vector_tiles = (vectors + 31) / 32;
+    // The rule of gemm_i8_k_splits: a launch with far fewer workgroups than compute units shares the
+    // stages of K out over several workgroups per tile, no share empty.
+    const auto shares = [&](uint64_t tiles) -> uint32_t {
+        if (tiles == 0 || stages < 2 || tiles >= 192) return 1;
+        uint64_t splits = 256 / tiles;
+        if (splits > stages) splits = stages;
+        if (splits < 2) return 1;
+        const uint64_t share = (stages + splits - 1) / splits;
+        return static_cast<uint32_t>((stages + share - 1) / share);
+    };
+    uint64_t small = 0, large = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        small += (rows[i] + 63) / 64;
+        large += (rows[i] + 127) / 128;
+    }
+    // 128-row workgroups (half the activation copies per weight row) once they fill the device without
+    // sharing K. (With K shares they measured slower than 64-row workgroups: 14336 x 4096 with 32 vectors
+    // 25.1 against 23.7 us, 4096 x 4096 16.3 against 13.8 us.)
+    if (large * vector_tiles >= 192) return GemmGroupGeometry{128, large, 1};
+    return GemmGroupGeometry{64, small, shares(small * vector_tiles)};
 }
 
-uint32_t gemm_h16_group_k_splits(uint64_t row_tiles, uint64_t columns, uint64_t vectors) {
-    // the rule of gemm_i8_k_splits for row_tiles tiles of 64 rows
-    return gemm_i8_k_splits(kQ4_K, 2, row_tiles * kRows, columns, vectors);
+uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors) {
+    const GemmGroupGeometry g = gemm_h16_group_geometry(rows, count, columns, vectors);
+    return g.k_splits > 1 ? g.k_splits * vectors * g.row_tiles * g.tile_rows * 4u : 0;
 }
 
-uint64_t gemm_h16_group_partial_bytes(uint64_t row_tiles, uint64_t columns, uint64_t vectors) {
-    const uint32_t splits = gemm_h16_group_k_splits(row_tiles, columns, vectors);
-    return splits > 1 ? splits * vectors * row_tiles * kRows * 4u : 0;
-}
-
-hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
-                          uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
-    if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
-    constexpr int AX = 2, AW = 3;
-    using S = Shape<AX, AW>;
+namespace {
+template <int RG, int AX, int AW>
+hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream) {
+    using S = Shape<RG, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
-    const auto kernel = gemm_h16_kernel<AX, AW>;
-    const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
+    const auto kernel = gemm_h16_kernel<RG, AX, AW>;
     Group group = {};
     group.count = count;
     uint64_t row_tiles = 0;
     for (uint32_t i = 0; i < count; i++) {
         group.member[i] = Member{members[i].weight, members[i].bias, members[i].residual, members[i].y,
                                  static_cast<uint32_t>(members[i].rows), static_cast<uint32_t>(row_tiles)};
-        if (members[i].rows == 0 || members[i].rows > 0xffffffffull) return hipErrorInvalidValue;
-        row_tiles += (members[i].rows + kRows - 1) / kRows;
+        row_tiles += (members[i].rows + S::kRows - 1) / S::kRows;
     }
     if (row_tiles > 0x00ffffffull) return hipErrorInvalidValue;
     group.row_tiles = static_cast<uint32_t>(row_tiles);
@@ -424,18 +440,36 @@ hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8
         allowed[device] = true;
     }
     const uint32_t vector_tiles = (vectors + 31u) / 32u;
-    const uint32_t k_splits = partials != nullptr ? gemm_h16_group_k_splits(row_tiles, columns, vectors) : 1u;
     const uint64_t grid = ((row_tiles + 7u) / 8u) * 8u * vector_tiles * k_splits;
     if (grid > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, group, tiles,
                        vector_tiles, columns, vectors, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
     if (k_splits > 1) {
-        const uint64_t items = row_tiles * kRows * vectors / 4;
+        const uint64_t items = row_tiles * S::kRows * vectors / 4;
         hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
-                           group, partials, vectors, k_splits);
+                           group, partials, vectors, k_splits, S::kRows);
     }
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+                          uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+    if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
+    const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
+    uint64_t rows[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) {
+        if (members[i].rows == 0 || members[i].rows > 0xffffffffull) return hipErrorInvalidValue;
+        rows[i] = members[i].rows;
+    }
+    GemmGroupGeometry g = gemm_h16_group_geometry(rows, count, columns, vectors);
+    if (partials == nullptr && g.k_splits > 1) {  // nowhere to keep shares: 64-row workgroups, whole K each
+        g = GemmGroupGeometry{64, 0, 1};
+    }
+    if (g.tile_rows == 128)
+        return launch_group<4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+    return launch_group<2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,

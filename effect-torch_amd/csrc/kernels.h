@@ -110,7 +110,7 @@ bool gemm_h16_supported(int32_t codec, uint64_t columns);
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream);
 // Several Q4_K matrices of the same width against the same activation tiles in one launch (the q / k /
-// v projections of a decode step): the grid runs over the 64-row tiles of all of them, and K is shared
+// v projections of a decode step): the grid runs over the row tiles of all of them, and K is shared
 // out by the rule of gemm_i8_k_splits for that many tiles. `partials` holds
 // gemm_h16_group_partial_bytes(...) bytes when that is not zero.
 constexpr uint32_t kGemmGroupMost = 4;
@@ -121,9 +121,14 @@ struct GemmMember {
     float* y;               // [vectors, rows]
     uint64_t rows;
 };
-uint64_t gemm_h16_group_row_tiles(const GemmMember* members, uint32_t count);
-uint32_t gemm_h16_group_k_splits(uint64_t row_tiles, uint64_t columns, uint64_t vectors);
-uint64_t gemm_h16_group_partial_bytes(uint64_t row_tiles, uint64_t columns, uint64_t vectors);
+// Rows per workgroup (64 or 128), row tiles of that height over all members, K shares.
+struct GemmGroupGeometry {
+    uint32_t tile_rows;
+    uint64_t row_tiles;
+    uint32_t k_splits;
+};
+GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
+uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
 hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
                           uint64_t columns, uint64_t vectors, hipStream_t stream);
 

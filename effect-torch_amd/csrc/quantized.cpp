@@ -119,12 +119,18 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         plan->kernel = kernel;
         plan->q_offset = cursor;  // activation tiles, see tile_blob_bytes()
         cursor = align_up(cursor + tile_workspace_bytes(limbs, plan->vectors, plan->columns), 256);
+        if (limbs == 2) {  // gemm_h16 chooses its own tile height and keeps partial results by whole tiles
+            plan->k_splits = gemm_h16_group_geometry(&plan->rows, 1, plan->columns, plan->vectors).k_splits;
+            if (plan->k_splits > 1) {
+                plan->partial_offset = cursor;
+                cursor = align_up(cursor + gemm_h16_group_partial_bytes(&plan->rows, 1, plan->columns, plan->vectors), 256);
+            }
+            return;
+        }
         plan->k_splits = gemm_i8_k_splits(plan->codec, limbs, plan->rows, plan->columns, plan->vectors);
         if (plan->k_splits > 1) {
             plan->partial_offset = cursor;
-            // gemm_h16 keeps its partial results by whole 64-row tiles
-            const uint64_t partial_rows = limbs == 2 ? (plan->rows + 63) / 64 * 64 : plan->rows;
-            cursor = align_up(cursor + plan->k_splits * plan->vectors * partial_rows * 4u, 256);
+            cursor = align_up(cursor + plan->k_splits * plan->vectors * plan->rows * 4u, 256);
         }
     };
     if (plan->activation_mode == ET_ACT_INT8) {
@@ -403,16 +409,16 @@ int check_group(const et_linear_plan* const* plans, uint32_t count, std::string*
     }
     return ET_OK;
 }
-uint64_t group_row_tiles(const et_linear_plan* const* plans, uint32_t count) {
-    uint64_t tiles = 0;
-    for (uint32_t i = 0; i < count; i++) tiles += (plans[i]->rows + 63) / 64;
-    return tiles;
+uint64_t group_partial_bytes(const et_linear_plan* const* plans, uint32_t count) {
+    uint64_t rows[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) rows[i] = plans[i]->rows;
+    return gemm_h16_group_partial_bytes(rows, count, plans[0]->columns, plans[0]->vectors);
 }
 }  // namespace
 
 int linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes, std::string* error) {
     if (int rc = check_group(plans, count, error)) return rc;
-    *bytes = gemm_h16_group_partial_bytes(group_row_tiles(plans, count), plans[0]->columns, plans[0]->vectors);
+    *bytes = group_partial_bytes(plans, count);
     return ET_OK;
 }
 
@@ -435,7 +441,7 @@ int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t c
     }
     if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
     if (plans[0]->vectors == 0) return ET_OK;
-    const uint64_t need = gemm_h16_group_partial_bytes(group_row_tiles(plans, count), plans[0]->columns, plans[0]->vectors);
+    const uint64_t need = group_partial_bytes(plans, count);
     if (need > 0 && (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0))
         return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
                                                  " bytes is smaller than the " + std::to_string(need) + " the group needs");

@@ -607,17 +607,25 @@ def test_group_launch_of_contractions_sharing_their_input(et, device):
         plans[index].enqueue_prepared(prepared, weights[index], biases[index], alone, single_ws,
                                       residual=residual if index == 0 else None)
         close(runs[0][index], alone.cpu().numpy())
-    # two large members: no K shares either way, so the group writes the bits of the single launches
+    # two large members (gate / up): enough 128-row tiles for every compute unit, no K shares
     big = [et.RawLinear(et.GgmlQuant.Q4_K, 14336, columns, vectors) for _ in range(2)]
     pair = et.LinearGroup(big)
     assert pair.workspace_bytes == 0
-    big_weights = [to_dev(synth.random_weight(oracle.Q4_K, 14336, columns, rng), device) for _ in range(2)]
+    big_host = [synth.random_weight(oracle.Q4_K, 14336, columns, rng) for _ in range(2)]
+    big_weights = [to_dev(w, device) for w in big_host]
     together = [torch.empty((vectors, 14336), device=device) for _ in range(2)]
     pair.enqueue_prepared(prepared, big_weights, together)
+    again = [torch.empty((vectors, 14336), device=device) for _ in range(2)]
+    pair.enqueue_prepared(prepared, big_weights, again)
     for index in range(2):
+        assert torch.equal(together[index], again[index])
         alone = torch.empty((vectors, 14336), device=device)
-        big[index].enqueue_prepared(prepared, big_weights[index], None, alone, None)
-        assert torch.equal(alone, together[index])
+        big_ws = torch.empty(max(big[index].requirements.workspace_bytes, 16), dtype=torch.uint8, device=device)
+        big[index].enqueue_prepared(prepared, big_weights[index], None, alone, big_ws)
+        close(together[index].cpu().numpy(), alone.cpu().numpy())
+        for start in (0, 14336 - 128):
+            want = oracle.linear_rows(oracle.Q4_K, 14336, columns, x_host, big_host[index], None, start, start + 128)
+            close(together[index].cpu().numpy()[:, start:start + 128], want[:, start:start + 128])
     # members must share the prepared input, and run on the kernel that has the group launch
     with pytest.raises(et.QuantizedError, match="share columns and vectors"):
         et.LinearGroup([plans[0], et.RawLinear(et.GgmlQuant.Q4_K, 64, 512, vectors)])
