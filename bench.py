@@ -560,8 +560,11 @@ def llama_decode(args, et):
             plans["wk"].enqueue(h, w["wk"], None, k, linear_ws)
             plans["wv"].enqueue(h, w["wv"], None, v, linear_ws)
         q4, k4, v4 = q.view(slots, heads, 1, width), k.view(slots, kv_heads, 1, width), v.view(slots, kv_heads, 1, width)
-        et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)
-        et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
+        if fused:
+            et.rotary_pair_into(q4, k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4, k4)
+        else:
+            et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)
+            et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
         keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
                                          workspace=kv_ws, synchronize=False))
         if fused:

@@ -44,6 +44,7 @@ from .decode_ops import (  # noqa: F401
     greedy_workspace_bytes,
     rms_norm_into,
     rotary_into,
+    rotary_pair_into,
     silu_mul_into,
 )
 from .gguf import (  # noqa: F401

@@ -132,6 +132,7 @@ SIGNATURES = {
     "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
     "et_hip_rms_norm_into": (ctypes.c_int, [_T, _T, ctypes.c_double, _T, _vp]),
     "et_hip_rotary_into": (ctypes.c_int, [_T, _vp, _u64, ctypes.c_double, ctypes.c_double, _i32, _T, _vp]),
+    "et_hip_rotary_pair_into": (ctypes.c_int, [_T, _T, _vp, _u64, ctypes.c_double, ctypes.c_double, _i32, _T, _T, _vp]),
     "et_hip_add_into": (ctypes.c_int, [_T, _T, _T, _vp]),
     "et_hip_silu_mul_into": (ctypes.c_int, [_T, _T, _T, _vp]),
     "et_hip_greedy_workspace_bytes": (_u64, [_u64, _u64]),

@@ -420,6 +420,20 @@ int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t off
     });
 }
 
+int et_hip_rotary_pair_into(const et_tensor* x, const et_tensor* second, const uint32_t* offsets, uint64_t offsets_len,
+                            double theta, double sign, int32_t layout, const et_tensor* destination,
+                            const et_tensor* second_destination, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        TensorView xv, sv, dst, sdst;
+        if (!TensorView::from_c(x, &xv, error) || !TensorView::from_c(second, &sv, error) ||
+            !TensorView::from_c(destination, &dst, error) || !TensorView::from_c(second_destination, &sdst, error)) {
+            *error = "rotary: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::decode::rotary_pair_into(xv, sv, offsets, offsets_len, theta, sign, layout, dst, sdst, stream, error);
+    });
+}
+
 int et_hip_add_into(const et_tensor* a, const et_tensor* b, const et_tensor* destination, void* stream) {
     return guarded([&](std::string* error) -> int {
         TensorView av, bv, dst;

@@ -56,33 +56,71 @@ int rms_norm_into(const TensorView& x, const TensorView* weight, double eps, con
                     "rms_norm", error);
 }
 
-// rotary_forward_into (composed.rs:2735-2772)
-int rotary_into(const TensorView& x, const uint32_t* offsets, uint64_t offsets_len, double theta, double sign,
-                int32_t layout, const TensorView& destination, void* stream, std::string* error) {
+namespace {
+struct RotaryShape {
+    uint64_t batch, rows, steps, head_dim, elements;
+};
+// The checks of rotary_forward_into (composed.rs:2735-2772) for one tensor.
+int rotary_shape(const TensorView& x, uint64_t offsets_len, const TensorView& destination, RotaryShape* shape,
+                 std::string* error) {
     const size_t rank = x.shape.size();
     if (rank < 2 || x.shape[rank - 1] % 2 != 0 || x.dtype != ET_DTYPE_F32)
         return fail(error, ET_ERR_UNSUPPORTED, "rotary: expected a float rank >= 2 tensor with even head dimension");
-    const uint64_t batch = rank == 2 ? 1 : x.shape[0];
-    if (offsets_len != 1 && offsets_len != batch)
+    shape->batch = rank == 2 ? 1 : x.shape[0];
+    if (offsets_len != 1 && offsets_len != shape->batch)
         return fail(error, ET_ERR_UNSUPPORTED, "rotary embedding: " + std::to_string(offsets_len) +
-                                                   " offsets for batch " + std::to_string(batch));
-    if (layout != ET_ROTARY_HALF_SPLIT && layout != ET_ROTARY_INTERLEAVED_PAIRS)
-        return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(layout));
+                                                   " offsets for batch " + std::to_string(shape->batch));
     if (destination.dtype != x.dtype || destination.shape != x.shape)
         return fail(error, ET_ERR_EXECUTION, "rotary output: destination does not match the input shape");
     if (!x.is_contiguous() || !destination.is_contiguous())
         return fail(error, ET_ERR_UNSUPPORTED, "rotary: operands must be contiguous");
-    const uint64_t steps = x.shape[rank - 2], head_dim = x.shape[rank - 1];
-    const uint64_t elements = numel(x);
-    if (elements == 0) return ET_OK;
-    const uint64_t rows = elements / (steps * head_dim);
-    if (steps > kLimit || head_dim > kLimit || rows / batch > kLimit || elements / 2 > (0x7fffffffull << 8))
+    shape->steps = x.shape[rank - 2];
+    shape->head_dim = x.shape[rank - 1];
+    shape->elements = numel(x);
+    shape->rows = shape->elements == 0 ? 0 : shape->elements / (shape->steps * shape->head_dim);
+    if (shape->elements != 0 && (shape->steps > kLimit || shape->head_dim > kLimit || shape->rows / shape->batch > kLimit ||
+                                 shape->elements / 2 > (0x7fffffffull << 8)))
         return fail(error, ET_ERR_UNSUPPORTED, "rotary: geometry exceeds the launch limits");
-    if (x.data == nullptr || destination.data == nullptr || offsets == nullptr)
+    if (shape->elements != 0 && (x.data == nullptr || destination.data == nullptr))
         return fail(error, ET_ERR_INVALID, "rotary: NULL device pointer");
+    return ET_OK;
+}
+}  // namespace
+
+// rotary_forward_into (composed.rs:2735-2772)
+int rotary_into(const TensorView& x, const uint32_t* offsets, uint64_t offsets_len, double theta, double sign,
+                int32_t layout, const TensorView& destination, void* stream, std::string* error) {
+    if (layout != ET_ROTARY_HALF_SPLIT && layout != ET_ROTARY_INTERLEAVED_PAIRS)
+        return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(layout));
+    RotaryShape shape;
+    if (int rc = rotary_shape(x, offsets_len, destination, &shape, error)) return rc;
+    if (shape.elements == 0) return ET_OK;
+    if (offsets == nullptr) return fail(error, ET_ERR_INVALID, "rotary: NULL device pointer");
     return launched(rotary(f32_data(x), offsets, static_cast<uint32_t>(offsets_len), theta, sign,
-                           layout == ET_ROTARY_INTERLEAVED_PAIRS, f32_out(destination), batch, rows, steps, head_dim,
-                           static_cast<hipStream_t>(stream)),
+                           layout == ET_ROTARY_INTERLEAVED_PAIRS, f32_out(destination), shape.batch, shape.rows,
+                           shape.steps, shape.head_dim, static_cast<hipStream_t>(stream)),
+                    "rotary", error);
+}
+
+// Two tensors at the same positions (the queries and the keys of a step) in one launch.
+int rotary_pair_into(const TensorView& x, const TensorView& second, const uint32_t* offsets, uint64_t offsets_len,
+                     double theta, double sign, int32_t layout, const TensorView& destination,
+                     const TensorView& second_destination, void* stream, std::string* error) {
+    if (layout != ET_ROTARY_HALF_SPLIT && layout != ET_ROTARY_INTERLEAVED_PAIRS)
+        return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(layout));
+    RotaryShape a, b;
+    if (int rc = rotary_shape(x, offsets_len, destination, &a, error)) return rc;
+    if (int rc = rotary_shape(second, offsets_len, second_destination, &b, error)) return rc;
+    if (a.batch != b.batch || a.steps != b.steps || a.head_dim != b.head_dim)
+        return fail(error, ET_ERR_UNSUPPORTED, "rotary: both tensors must share batch, steps and head dimension");
+    if (a.elements == 0 && b.elements == 0) return ET_OK;
+    if (offsets == nullptr) return fail(error, ET_ERR_INVALID, "rotary: NULL device pointer");
+    if ((a.elements + b.elements) / 2 > (0x7fffffffull << 8))
+        return fail(error, ET_ERR_UNSUPPORTED, "rotary: geometry exceeds the launch limits");
+    return launched(rotary_pair(f32_data(x), f32_out(destination), a.rows, f32_data(second), f32_out(second_destination),
+                                b.rows, offsets, static_cast<uint32_t>(offsets_len), theta, sign,
+                                layout == ET_ROTARY_INTERLEAVED_PAIRS, a.batch, a.steps, a.head_dim,
+                                static_cast<hipStream_t>(stream)),
                     "rotary", error);
 }
 

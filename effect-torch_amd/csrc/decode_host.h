@@ -18,6 +18,9 @@ int rms_norm_into(const TensorView& x, const TensorView* weight, double eps, con
                   void* stream, std::string* error);
 int rotary_into(const TensorView& x, const uint32_t* offsets, uint64_t offsets_len, double theta, double sign,
                 int32_t layout, const TensorView& destination, void* stream, std::string* error);
+int rotary_pair_into(const TensorView& x, const TensorView& second, const uint32_t* offsets, uint64_t offsets_len,
+                     double theta, double sign, int32_t layout, const TensorView& destination,
+                     const TensorView& second_destination, void* stream, std::string* error);
 int add_into(const TensorView& a, const TensorView& b, const TensorView& destination, void* stream,
              std::string* error);
 int silu_mul_into(const TensorView& gate, const TensorView& up, const TensorView& destination, void* stream,

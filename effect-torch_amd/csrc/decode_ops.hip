@@ -59,13 +59,25 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
     }
 }
 
-// One thread per (row, step, pair).
-__global__ __launch_bounds__(256) void rotary_kernel(const float* __restrict__ x, const uint32_t* __restrict__ offsets,
-                                                     uint32_t offsets_len, double theta, double sign, int interleaved,
-                                                     float* __restrict__ out, uint32_t rows_per_batch, uint32_t steps,
-                                                     uint32_t head_dim, uint64_t pairs) {
-    const uint64_t item = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (item >= pairs) return;
+// One thread per (row, step, pair), over one tensor or two of the same steps and head width (the
+// queries and the keys of a decode step).
+struct RotaryTensor {
+    const float* x;
+    float* out;
+    uint32_t rows_per_batch;
+    uint64_t pairs;
+};
+__global__ __launch_bounds__(256) void rotary_kernel(RotaryTensor first, RotaryTensor second,
+                                                     const uint32_t* __restrict__ offsets, uint32_t offsets_len,
+                                                     double theta, double sign, int interleaved, uint32_t steps,
+                                                     uint32_t head_dim) {
+    uint64_t item = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= first.pairs + second.pairs) return;
+    const bool in_second = item >= first.pairs;
+    if (in_second) item -= first.pairs;
+    const float* x = in_second ? second.x : first.x;
+    float* out = in_second ? second.out : first.out;
+    const uint32_t rows_per_batch = in_second ? second.rows_per_batch : first.rows_per_batch;
     const uint32_t half = head_dim / 2;
     const uint32_t index = static_cast<uint32_t>(item % half);
     const uint64_t row_step = item / half;
@@ -77,11 +89,11 @@ __global__ __launch_bounds__(256) void rotary_kernel(const float* __restrict__ x
     double s, c;
     sincos(angle, &s, &c);
     const uint64_t base = row_step * head_dim;
-    const uint64_t first = interleaved ? base + 2 * index : base + index;
-    const uint64_t second = interleaved ? base + 2 * index + 1 : base + half + index;
-    const double a = x[first], b = x[second];
-    out[first] = static_cast<float>(a * c - b * s);
-    out[second] = static_cast<float>(b * c + a * s);
+    const uint64_t lo = interleaved ? base + 2 * index : base + index;
+    const uint64_t hi = interleaved ? base + 2 * index + 1 : base + half + index;
+    const double a = x[lo], b = x[hi];
+    out[lo] = static_cast<float>(a * c - b * s);
+    out[hi] = static_cast<float>(b * c + a * s);
 }
 
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
@@ -229,10 +241,21 @@ hipError_t rms_norm(const float* x, const float* weight, double eps, float* out,
 hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
                   int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,
                   hipStream_t stream) {
-    const uint64_t pairs = rows * steps * (head_dim / 2);
-    hipLaunchKernelGGL(rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0, stream, x, offsets,
-                       offsets_len, theta, sign, interleaved, out, static_cast<uint32_t>(rows / batch),
-                       static_cast<uint32_t>(steps), static_cast<uint32_t>(head_dim), pairs);
+    return rotary_pair(x, out, rows, nullptr, nullptr, 0, offsets, offsets_len, theta, sign, interleaved, batch, steps,
+                       head_dim, stream);
+}
+
+hipError_t rotary_pair(const float* x, float* out, uint64_t rows, const float* second, float* second_out,
+                       uint64_t second_rows, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
+                       int interleaved, uint64_t batch, uint64_t steps, uint64_t head_dim, hipStream_t stream) {
+    const RotaryTensor a = {x, out, static_cast<uint32_t>(rows / batch), rows * steps * (head_dim / 2)};
+    const RotaryTensor b = {second, second_out, static_cast<uint32_t>(second_rows / batch),
+                            second_rows * steps * (head_dim / 2)};
+    const uint64_t pairs = a.pairs + b.pairs;
+    if (pairs == 0) return hipSuccess;
+    hipLaunchKernelGGL(rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0, stream, a, b,
+                       offsets, offsets_len, theta, sign, interleaved, static_cast<uint32_t>(steps),
+                       static_cast<uint32_t>(head_dim));
     return hipGetLastError();
 }
 

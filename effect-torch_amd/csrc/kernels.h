@@ -180,6 +180,11 @@ hipError_t rms_norm(const float* x, const float* weight, double eps, float* out,
 hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
                   int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,
                   hipStream_t stream);
+// The same for two tensors of the same batch, steps and head width in one launch (rows = elements /
+// (steps * head_dim) of each).
+hipError_t rotary_pair(const float* x, float* out, uint64_t rows, const float* second, float* second_out,
+                       uint64_t second_rows, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
+                       int interleaved, uint64_t batch, uint64_t steps, uint64_t head_dim, hipStream_t stream);
 hipError_t add(const float* a, const float* b, float* out, uint64_t count, hipStream_t stream);
 hipError_t silu_mul(const float* gate, const float* up, float* out, uint64_t count, hipStream_t stream);
 // out[row] = greedy token; status[row] = 0, or 1 + the first token whose logit is not finite.

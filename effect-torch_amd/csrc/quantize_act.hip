@@ -135,8 +135,18 @@ __device__ __forceinline__ void quantize_halves_store(const float4& in, uint32_t
                                                       uint32_t vector_tiles, uint8_t* __restrict__ tiles) {
     constexpr float kRange = 8388607.f;  // 2^23 - 1
     float amax = fmaxf(fmaxf(fabsf(in.x), fabsf(in.y)), fmaxf(fabsf(in.z), fabsf(in.w)));
-#pragma unroll
-    for (int step = 1; step < 64; step <<= 1) amax = fmaxf(amax, __shfl_xor(amax, step));
+    // over the wave: inside rows of 16 lanes with DPP, then the four rows through scalar registers
+    amax = fmaxf(amax, dpp_f32<0xB1>(amax));   // quad_perm [1,0,3,2]
+    amax = fmaxf(amax, dpp_f32<0x4E>(amax));   // quad_perm [2,3,0,1]
+    amax = fmaxf(amax, dpp_f32<0x141>(amax));  // row_half_mirror
+    amax = fmaxf(amax, dpp_f32<0x140>(amax));  // row_mirror
+    {
+        const int bits = __float_as_int(amax);
+        amax = fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(bits, 0)),
+                           __int_as_float(__builtin_amdgcn_readlane(bits, 16))),
+                     fmaxf(__int_as_float(__builtin_amdgcn_readlane(bits, 32)),
+                           __int_as_float(__builtin_amdgcn_readlane(bits, 48))));
+    }
     const float inv = amax > 0.f ? kRange / amax : 0.f;
     const float values[4] = {in.x, in.y, in.z, in.w};
     int total = 0;

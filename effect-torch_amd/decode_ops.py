@@ -39,6 +39,18 @@ def rotary_into(x: torch.Tensor, offsets: torch.Tensor, theta: float, sign: floa
                                       float(sign), int(layout), _ref(descs[1]), _stream_handle(stream)))
 
 
+def rotary_pair_into(x: torch.Tensor, second: torch.Tensor, offsets: torch.Tensor, theta: float, sign: float,
+                     layout: RotaryLayout, destination: torch.Tensor, second_destination: torch.Tensor, *,
+                     stream=None) -> None:
+    """:func:`rotary_into` for two tensors of one batch, steps and head width (queries and keys) in one launch."""
+    if offsets.dtype not in (torch.int32, torch.uint32) or not offsets.is_contiguous():
+        raise QuantizedError(N.ERR_UNSUPPORTED, "rotary: offsets must be contiguous 32-bit integers")
+    descs = (_desc(x), _desc(second), _desc(destination), _desc(second_destination))
+    _check(N.lib().et_hip_rotary_pair_into(_ref(descs[0]), _ref(descs[1]), offsets.data_ptr(), offsets.numel(),
+                                           float(theta), float(sign), int(layout), _ref(descs[2]), _ref(descs[3]),
+                                           _stream_handle(stream)))
+
+
 def add_into(a: torch.Tensor, b: torch.Tensor, destination: torch.Tensor, *, stream=None) -> None:
     descs = (_desc(a), _desc(b), _desc(destination))
     _check(N.lib().et_hip_add_into(_ref(descs[0]), _ref(descs[1]), _ref(descs[2]), _stream_handle(stream)))

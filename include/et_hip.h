@@ -331,6 +331,12 @@ typedef enum { ET_ROTARY_HALF_SPLIT = 0, ET_ROTARY_INTERLEAVED_PAIRS = 1 } et_ro
 int et_hip_rotary_into(const et_tensor* x, const uint32_t* offsets, uint64_t offsets_len,
                        double theta, double sign, int32_t layout, const et_tensor* destination,
                        void* stream);
+/* The same for two tensors of one batch, steps and head_dim at the same offsets - the queries and
+ * the keys of a decode step - in one launch; each result is et_hip_rotary_into's. */
+int et_hip_rotary_pair_into(const et_tensor* x, const et_tensor* second, const uint32_t* offsets,
+                            uint64_t offsets_len, double theta, double sign, int32_t layout,
+                            const et_tensor* destination, const et_tensor* second_destination,
+                            void* stream);
 
 /* out = a + b, f32, same shapes (the residual connections; the reference's binary
  * add without broadcasting, crates/runtime-cpu/src/ops.rs). `destination` may be `a`. */

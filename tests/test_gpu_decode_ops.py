@@ -66,6 +66,25 @@ def test_rotary(et, device, layout, shape, offsets):
     assert np.abs(back.cpu().numpy() - x).max() <= 2e-6  # the reference's own round-trip bar
 
 
+@pytest.mark.parametrize("layout", ["HALF_SPLIT", "INTERLEAVED_PAIRS"])
+def test_rotary_pair_is_two_rotaries(et, device, layout):
+    # queries and keys of a step in one launch: the bits of the two separate launches, in place too
+    rng = np.random.default_rng(17)
+    for q_shape, k_shape in (((32, 32, 1, 128), (32, 8, 1, 128)), ((3, 5, 4, 16), (3, 1, 4, 16))):
+        q = torch.from_numpy(rng.standard_normal(q_shape).astype(np.float32)).to(device)
+        k = torch.from_numpy(rng.standard_normal(k_shape).astype(np.float32)).to(device)
+        offsets = torch.tensor(rng.integers(0, 9000, q_shape[0]), dtype=torch.int32, device=device)
+        q_alone, k_alone = torch.empty_like(q), torch.empty_like(k)
+        et.rotary_into(q, offsets, 500000.0, 1.0, et.RotaryLayout[layout], q_alone)
+        et.rotary_into(k, offsets, 500000.0, 1.0, et.RotaryLayout[layout], k_alone)
+        q_pair, k_pair = q.clone(), k.clone()
+        et.rotary_pair_into(q_pair, k_pair, offsets, 500000.0, 1.0, et.RotaryLayout[layout], q_pair, k_pair)
+        assert torch.equal(q_pair, q_alone) and torch.equal(k_pair, k_alone)
+    with pytest.raises(et.QuantizedError, match="share batch, steps and head dimension"):
+        shorter = k[:, :, :2].contiguous()  # other steps
+        et.rotary_pair_into(q, shorter, offsets, 500000.0, 1.0, et.RotaryLayout[layout], q, shorter)
+
+
 def test_silu_mul(et, device):
     rng = np.random.default_rng(5)
     for count in (32 * 14336, 1001, 3):
