@@ -1,4 +1,4 @@
-// f32-accurate contraction of Q4_K weights with a batch of activation vectors on the gfx950
+// f32-accurate contraction of Q4_K or Q5_K weights with a batch of activation vectors on the gfx950
 // matrix cores, with every operand an exact small integer held in a half float.
 //
 //   y[m, n] = sum_s  unit[m, s] * d[n, s] * sum_g sum_i (sc_g[n] * nib[n, g, i]) * X[m, g, i]
@@ -8,7 +8,7 @@
 // Activations are 24-bit fixed point per vector and stage, X = rint(x * (2^23 - 1) / max|x|), split
 // into two balanced 12-bit halves X = 4096 * hi + lo with |lo|, |hi| <= 2048: integers a half float
 // holds exactly. On the weight side the 6-bit sub-block scale is folded into the operand:
-// sc_g * nib <= 63 * 15 = 945, exact in a half float as well. Every product (< 2^21) is exact in
+// sc_g * nib <= 63 * 15 = 945 (Q5_K: 63 * 31 = 1953), exact in a half float as well. Every product (< 2^21) is exact in
 // the f32 the matrix core accumulates in, so v_mfma_f32_32x32x16_f16 sums whole super-blocks with
 // f32 accumulation error only, and the f32 scales unit[m] * d[n] are applied once per stage instead
 // of once per 32-column block: the per-element VALU work, which bounds the int8 kernel with
@@ -50,7 +50,6 @@ constexpr uint32_t kSmallRows = 64;  // rows of a workgroup with RG = 2: the uni
 constexpr uint32_t kBlob = tile_blob_bytes(2);  // in memory and in LDS
 constexpr uint32_t kUnitAt = 32768u;            // unit[m]
 constexpr uint32_t kSumsAt = 32768u + 128u;     // xsum[g][m]
-constexpr uint32_t kRowBytes = 144u;            // a row's share of a stage
 constexpr int kActivationJobs = kBlob / 1024;
 static_assert(kBlob % 1024 == 0, "whole copy instructions");
 
@@ -69,8 +68,19 @@ constexpr int vmcnt_only(int n) {
     return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
 }
 
-template <int RG, int AX, int AW>
+// A row's share of a stage, as it lies in memory: a Q4_K super-block is d, dmin, scales[12], qs[128];
+// a Q5_K one d, dmin, scales[12], qh[32] (the fifth bits: bit g of qh[c] belongs to column c of
+// sub-block g), qs[128] (crates/runtime-cpu/src/quantized.rs:180-234).
+template <int CODEC>
+struct Codec {
+    static_assert(CODEC == kQ4_K || CODEC == kQ5_K, "the codecs whose scaled quants a half float holds exactly");
+    static constexpr uint32_t kRowBytes = CODEC == kQ5_K ? 176u : 144u;
+    static constexpr uint32_t kQuantsAt = CODEC == kQ5_K ? 48u : 16u;
+};
+
+template <int CODEC, int RG, int AX, int AW>
 struct Shape {
+    static constexpr uint32_t kRowBytes = Codec<CODEC>::kRowBytes;
     static constexpr int kRowGroups = RG, kSplit = kConsumers / RG, kBlocksPerWave = kStageBlocks / kSplit;
     static constexpr uint32_t kRows = 32 * RG;
     static constexpr uint32_t kWeightBytes = kRows * kRowBytes;
@@ -122,11 +132,12 @@ struct Group {
     uint32_t row_tiles;  // of all members together
 };
 
-template <int RG, int AX, int AW>
+template <int CODEC, int RG, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
     uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
-    using S = Shape<RG, AX, AW>;
+    using S = Shape<CODEC, RG, AX, AW>;
+    constexpr uint32_t kRowBytes = S::kRowBytes, kQuantsAt = Codec<CODEC>::kQuantsAt;
     constexpr int NB = S::kBlocksPerWave;
     constexpr int kSplit = S::kSplit, kRowGroups = S::kRowGroups, kWeightJobs = S::kWeightJobs;
     constexpr uint32_t kRows = S::kRows, kWeightBytes = S::kWeightBytes;
@@ -238,6 +249,8 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const float d_block = half_bits_to_float(header.x & 0xffffu);
         const float dmin_block = half_bits_to_float(header.x >> 16);
         const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
+        uint4 fifth = make_uint4(0u, 0u, 0u, 0u);  // Q5_K: qh of this lane half's sixteen columns
+        if constexpr (CODEC == kQ5_K) fifth = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 16u * half);
 
         // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA, lane half h
         // supplies sub-block 2j + h.
@@ -257,10 +270,16 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             const uint32_t b = b_base + bb;
             // sub-block 2p + side: low (side 0) or high (side 1) nibbles of the 32 bytes of pair p; this
             // lane half takes bytes 16 * half .. + 16 = columns 16 * half .. + 16 of the sub-block
-            const uint4 raw = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 32u * (b >> 1) + 16u * half);
+            const uint4 raw = *reinterpret_cast<const uint4*>(row_in_slot + kQuantsAt + 32u * (b >> 1) + 16u * half);
             const uint32_t shift = (b & 1u) * 4u;
-            const uint32_t w0 = (raw.x >> shift) & 0x0f0f0f0fu, w1 = (raw.y >> shift) & 0x0f0f0f0fu,
-                           w2 = (raw.z >> shift) & 0x0f0f0f0fu, w3 = (raw.w >> shift) & 0x0f0f0f0fu;
+            uint32_t w0 = (raw.x >> shift) & 0x0f0f0f0fu, w1 = (raw.y >> shift) & 0x0f0f0f0fu,
+                     w2 = (raw.z >> shift) & 0x0f0f0f0fu, w3 = (raw.w >> shift) & 0x0f0f0f0fu;
+            if constexpr (CODEC == kQ5_K) {  // the fifth bit of column c of sub-block b: bit b of qh[c]
+                w0 |= ((fifth.x >> b) & 0x01010101u) << 4;
+                w1 |= ((fifth.y >> b) & 0x01010101u) << 4;
+                w2 |= ((fifth.z >> b) & 0x01010101u) << 4;
+                w3 |= ((fifth.w >> b) & 0x01010101u) << 4;
+            }
             uint32_t sc, mn;
             q4k_scale_min(header, b, sc, mn);
             const _Float16 sc_h = static_cast<_Float16>(static_cast<float>(sc));
@@ -379,7 +398,7 @@ __global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, co
 }  // namespace
 
 bool gemm_h16_supported(int32_t codec, uint64_t columns) {
-    return codec == kQ4_K && columns % 256 == 0 && columns > 0;
+    return (codec == kQ4_K || codec == kQ5_K) && columns % 256 == 0 && columns > 0;
 }
 
 GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors) {
@@ -412,12 +431,12 @@ uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint
 }
 
 namespace {
-template <int RG, int AX, int AW>
+template <int CODEC, int RG, int AX, int AW>
 hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
                         uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream) {
-    using S = Shape<RG, AX, AW>;
+    using S = Shape<CODEC, RG, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
-    const auto kernel = gemm_h16_kernel<RG, AX, AW>;
+    const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW>;
     Group group = {};
     group.count = count;
     uint64_t row_tiles = 0;
@@ -454,8 +473,9 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
 }
 }  // namespace
 
-hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
-                          uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
+                          float* partials, uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+    if (!gemm_h16_supported(codec, columns64)) return hipErrorInvalidValue;
     if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
     const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
     uint64_t rows[kGemmGroupMost];
@@ -467,16 +487,21 @@ hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8
     if (partials == nullptr && g.k_splits > 1) {  // nowhere to keep shares: 64-row workgroups, whole K each
         g = GemmGroupGeometry{64, 0, 1};
     }
+    // weight lead: what the activation ring (three slots of 34 KiB) leaves of LDS
+    if (codec == kQ5_K) {
+        if (g.tile_rows == 128)
+            return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+    }
     if (g.tile_rows == 128)
-        return launch_group<4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
-    return launch_group<2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream) {
-    if (!gemm_h16_supported(codec, columns)) return hipErrorInvalidValue;
     const GemmMember one = {weight, out.bias, out.residual, out.y, rows};
-    return gemm_h16_group(&one, 1, tiles, out.partials, columns, vectors, stream);
+    return gemm_h16_group(codec, &one, 1, tiles, out.partials, columns, vectors, stream);
 }
 
 }  // namespace et

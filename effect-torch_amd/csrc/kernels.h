@@ -105,11 +105,11 @@ hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_
 hipError_t reduce_partials(const float* partials, const float* bias, const float* residual, float* y,
                            uint32_t rows, uint32_t vectors, uint32_t k_splits, hipStream_t stream);
 
-// ---- gemm_h16.hip: Q4_K on the half-float matrix cores, exact integer operands (limbs = 2 tiles) ----
+// ---- gemm_h16.hip: Q4_K and Q5_K on the half-float matrix cores, exact integer operands (limbs = 2 tiles) ----
 bool gemm_h16_supported(int32_t codec, uint64_t columns);
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream);
-// Several Q4_K matrices of the same width against the same activation tiles in one launch (the q / k /
+// Several matrices of one codec and the same width against the same activation tiles in one launch (the q / k /
 // v projections of a decode step): the grid runs over the row tiles of all of them, and K is shared
 // out by the rule of gemm_i8_k_splits for that many tiles. `partials` holds
 // gemm_h16_group_partial_bytes(...) bytes when that is not zero.
@@ -129,8 +129,8 @@ struct GemmGroupGeometry {
 };
 GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
 uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
-hipError_t gemm_h16_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
-                          uint64_t columns, uint64_t vectors, hipStream_t stream);
+hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
+                          float* partials, uint64_t columns, uint64_t vectors, hipStream_t stream);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch

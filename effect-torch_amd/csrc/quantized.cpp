@@ -404,8 +404,9 @@ int check_group(const et_linear_plan* const* plans, uint32_t count, std::string*
         if (plans[i] == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: plan is NULL");
         if (plans[i]->kernel != LinearKernel::kGemmHalf)
             return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: this plan's kernel has no group launch");
-        if (plans[i]->columns != plans[0]->columns || plans[i]->vectors != plans[0]->vectors)
-            return fail(error, ET_ERR_INVALID, "quantized_linear: the plans of a group must share columns and vectors");
+        if (plans[i]->columns != plans[0]->columns || plans[i]->vectors != plans[0]->vectors ||
+            plans[i]->codec != plans[0]->codec)
+            return fail(error, ET_ERR_INVALID, "quantized_linear: the plans of a group must share columns and vectors and codec");
     }
     return ET_OK;
 }
@@ -445,7 +446,7 @@ int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t c
     if (need > 0 && (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0))
         return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
                                                  " bytes is smaller than the " + std::to_string(need) + " the group needs");
-    if (hipError_t status = gemm_h16_group(members, count, static_cast<const uint8_t*>(prepared),
+    if (hipError_t status = gemm_h16_group(plans[0]->codec, members, count, static_cast<const uint8_t*>(prepared),
                                            need > 0 ? static_cast<float*>(workspace) : nullptr, plans[0]->columns,
                                            plans[0]->vectors, as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);

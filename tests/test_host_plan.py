@@ -50,6 +50,10 @@ def test_linear_plan_shapes(et):
     assert plan.output_shape == (2, 5, 7) and plan.vectors == 10
     # ten vectors: fixed-point activations on the matrix cores, with its workspace planned
     assert plan.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce") and plan.workspace_bytes > 4 * 10 * 512
+    plan5 = et.linear_requirements(torch.zeros(10, 512), _w(7, 352), None, et.GgmlQuant.Q5_K, (7, 512))
+    assert plan5.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce")
+    plan6 = et.linear_requirements(torch.zeros(10, 512), _w(7, 420), None, et.GgmlQuant.Q6_K, (7, 512))
+    assert plan6.kernel == "gemv_limb"  # no batch kernel yet: repeated two-vector launches
     plan8 = et.linear_requirements(torch.zeros(10, 512), _w(7, 544), None, et.GgmlQuant.Q8_0, (7, 512))
     assert plan8.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
     for few in (3, 6):
