@@ -71,11 +71,20 @@ constexpr int vmcnt_only(int n) {
 // A row's share of a stage, as it lies in memory: a Q4_K super-block is d, dmin, scales[12], qs[128];
 // a Q5_K one d, dmin, scales[12], qh[32] (the fifth bits: bit g of qh[c] belongs to column c of
 // sub-block g), qs[128] (crates/runtime-cpu/src/quantized.rs:180-234).
+// A Q6_K super-block is ql[128], qh[64], sixteen int8 scales (one per 16 columns), d: 210 bytes, so
+// the stages of a row start on 2-byte boundaries. Its LDS row is 224 bytes: chunks 0..12 are bytes
+// 0..207 of the stage, chunk 13 is bytes 194..209 (d at offset 222) so that no copy reads past the
+// stage (crates/runtime-cpu/src/quantized.rs:238-261).
 template <int CODEC>
 struct Codec {
-    static_assert(CODEC == kQ4_K || CODEC == kQ5_K, "the codecs whose scaled quants a half float holds exactly");
-    static constexpr uint32_t kRowBytes = CODEC == kQ5_K ? 176u : 144u;
+    static_assert(CODEC == kQ4_K || CODEC == kQ5_K || CODEC == kQ6_K, "the K-quants with a half-float form");
+    static constexpr uint32_t kStageBytes = CODEC == kQ6_K ? 210u : CODEC == kQ5_K ? 176u : 144u;  // in memory
+    static constexpr uint32_t kRowBytes = CODEC == kQ6_K ? 224u : kStageBytes;                     // in LDS
     static constexpr uint32_t kQuantsAt = CODEC == kQ5_K ? 48u : 16u;
+    // byte of the stage that LDS byte `within` (a multiple of 16) of the row holds
+    static __device__ __forceinline__ uint32_t source_of(uint32_t within) {
+        return CODEC == kQ6_K && within == 208u ? 194u : within;
+    }
 };
 
 template <int CODEC, int RG, int AX, int AW>
@@ -100,8 +109,10 @@ struct Shape {
 // Eight nibbles (two dwords of four, one per byte) as eight half floats times `scale`:
 // 0x6400 | n is the half float 1024 + n, and (1024 + n) * scale - 1024 * scale, one fused
 // multiply-add per pair, is n * scale exactly (1024 * scale <= 64512 is a half float).
+template <int OFFSET = 0>
 __device__ __forceinline__ v8h nibbles_times(uint32_t first, uint32_t second, v2h scale) {
-    const v2h offset = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+    // OFFSET is subtracted from every byte first: (1024 + n) * scale - (1024 + OFFSET) * scale
+    const v2h offset = {static_cast<_Float16>(1024.0f + OFFSET), static_cast<_Float16>(1024.0f + OFFSET)};
     union {
         uint32_t word[4];
         v2h pair[4];
@@ -137,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
     uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
     using S = Shape<CODEC, RG, AX, AW>;
-    constexpr uint32_t kRowBytes = S::kRowBytes, kQuantsAt = Codec<CODEC>::kQuantsAt;
+    constexpr uint32_t kRowBytes = S::kRowBytes, kQuantsAt = Codec<CODEC>::kQuantsAt, kStageBytes = Codec<CODEC>::kStageBytes;
     constexpr int NB = S::kBlocksPerWave;
     constexpr int kSplit = S::kSplit, kRowGroups = S::kRowGroups, kWeightJobs = S::kWeightJobs;
     constexpr uint32_t kRows = S::kRows, kWeightBytes = S::kWeightBytes;
@@ -164,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const uint32_t share = (all_stages + k_splits - 1u) / k_splits;
     const uint32_t first_stage = k_share * share;  // < all_stages: the launcher leaves no share empty
     const uint32_t stages = min(share, all_stages - first_stage);
-    const uint64_t row_bytes = static_cast<uint64_t>(all_stages) * kRowBytes;
+    const uint64_t row_bytes = static_cast<uint64_t>(all_stages) * kStageBytes;
     const uint32_t row0 = (row_tile - member.first_tile) * kRows;  // in the member's own rows
 
     if (wave >= static_cast<uint32_t>(kConsumers + kWeightLoaders)) {
@@ -205,8 +216,8 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 if (job >= static_cast<uint32_t>(kWeightJobs)) job -= kWeightJobs;
                 const uint32_t at = job * 1024u + lane * 16u;
                 const uint32_t row = min(row0 + at / kRowBytes, rows - 1u);
-                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * kRowBytes +
-                                     at % kRowBytes;
+                const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * kStageBytes +
+                                     Codec<CODEC>::source_of(at % kRowBytes);
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
             }
@@ -244,6 +255,55 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * kWeightBytes;
         const uint32_t b_base = wave_k * NB;
         const uint8_t* row_in_slot = region + (wave_n * 32u + in_half) * kRowBytes;  // this lane's weight row
+
+        if constexpr (CODEC == kQ6_K) {
+            // value = d * sc * (q - 32) with an int8 scale per 16 columns: a lane half's sixteen columns
+            // of a 32-column block are one such run. sc * (q - 32) reaches 4096, too wide for a half
+            // float, so sc = 16 * s_hi + s_lo (s_lo 0..15, s_hi -8..7) and both parts are contracted:
+            // four accumulators, (X_lo, X_hi) x (s_lo, s_hi), joined once per stage.
+            const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + 222u));
+            const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
+            v16f p_ll = zero, p_lh = zero, p_hl = zero, p_hh = zero;  // activation half, scale part
+#pragma unroll
+            for (int bb = 0; bb < NB; bb++) {
+                const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
+                // columns 32 t + 16 half .. + 16 of 128-column half n: low four bits in ql[64 n + 32 (t & 1) + l]
+                // (high nibbles for t >= 2), bits 4-5 in qh[32 n + l] >> 2 t, l = 16 half .. + 16
+                const uint4 ql = *reinterpret_cast<const uint4*>(row_in_slot + 64u * n + 32u * (t & 1u) + 16u * half);
+                const uint4 qh = *reinterpret_cast<const uint4*>(row_in_slot + 128u + 32u * n + 16u * half);
+                const int sc = *reinterpret_cast<const int8_t*>(row_in_slot + 192u + 8u * n + 2u * t + half);
+                const uint32_t low_shift = (t >> 1) * 4u, high_shift = 2u * t;
+                const uint32_t w0 = ((ql.x >> low_shift) & 0x0f0f0f0fu) | (((qh.x >> high_shift) & 0x03030303u) << 4),
+                               w1 = ((ql.y >> low_shift) & 0x0f0f0f0fu) | (((qh.y >> high_shift) & 0x03030303u) << 4),
+                               w2 = ((ql.z >> low_shift) & 0x0f0f0f0fu) | (((qh.z >> high_shift) & 0x03030303u) << 4),
+                               w3 = ((ql.w >> low_shift) & 0x0f0f0f0fu) | (((qh.w >> high_shift) & 0x03030303u) << 4);
+                const _Float16 s_lo = static_cast<_Float16>(static_cast<float>(sc & 15));
+                const _Float16 s_hi = static_cast<_Float16>(static_cast<float>(sc >> 4));
+                const v2h lo2 = {s_lo, s_lo}, hi2 = {s_hi, s_hi};
+                const v8h bl0 = nibbles_times<32>(w0, w1, lo2), bl1 = nibbles_times<32>(w2, w3, lo2);
+                const v8h bh0 = nibbles_times<32>(w0, w1, hi2), bh1 = nibbles_times<32>(w2, w3, hi2);
+                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
+                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
+                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
+                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
+                p_ll = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bl0, p_ll, 0, 0, 0);
+                p_lh = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bh0, p_lh, 0, 0, 0);
+                p_hl = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bl0, p_hl, 0, 0, 0);
+                p_hh = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bh0, p_hh, 0, 0, 0);
+                p_ll = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bl1, p_ll, 0, 0, 0);
+                p_lh = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bh1, p_lh, 0, 0, 0);
+                p_hl = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bl1, p_hl, 0, 0, 0);
+                p_hh = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bh1, p_hh, 0, 0, 0);
+            }
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+                                                                 zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float high = fmaf(16.0f, p_hh[r], p_hl[r]), low = fmaf(16.0f, p_lh[r], p_ll[r]);
+                acc[r] = fmaf(fmaf(4096.0f, high, low), sd[r], acc[r]);
+            }
+            continue;
+        }
 
         const uint4 header = *reinterpret_cast<const uint4*>(row_in_slot);
         const float d_block = half_bits_to_float(header.x & 0xffffu);
@@ -398,10 +458,11 @@ __global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, co
 }  // namespace
 
 bool gemm_h16_supported(int32_t codec, uint64_t columns) {
-    return (codec == kQ4_K || codec == kQ5_K) && columns % 256 == 0 && columns > 0;
+    return (codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) && columns % 256 == 0 && columns > 0;
 }
 
-GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors) {
+GemmGroupGeometry gemm_h16_group_geometry(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
+                                          uint64_t vectors) {
     const uint64_t stages = columns / 256, vector_tiles = (vectors + 31) / 32;
     // The rule of gemm_i8_k_splits: a launch with far fewer workgroups than compute units shares the
     // stages of K out over several workgroups per tile, no share empty.
@@ -421,12 +482,14 @@ GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, 
     // 128-row workgroups (half the activation copies per weight row) once they fill the device without
     // sharing K. (With K shares they measured slower than 64-row workgroups: 14336 x 4096 with 32 vectors
     // 25.1 against 23.7 us, 4096 x 4096 16.3 against 13.8 us.)
-    if (large * vector_tiles >= 192) return GemmGroupGeometry{128, large, 1};
+    // (Q6_K: 128 rows of 224 bytes per stage leave no room for a weight ring.)
+    if (codec != kQ6_K && large * vector_tiles >= 192) return GemmGroupGeometry{128, large, 1};
     return GemmGroupGeometry{64, small, shares(small * vector_tiles)};
 }
 
-uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors) {
-    const GemmGroupGeometry g = gemm_h16_group_geometry(rows, count, columns, vectors);
+uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
+                                      uint64_t vectors) {
+    const GemmGroupGeometry g = gemm_h16_group_geometry(codec, rows, count, columns, vectors);
     return g.k_splits > 1 ? g.k_splits * vectors * g.row_tiles * g.tile_rows * 4u : 0;
 }
 
@@ -483,11 +546,13 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
         if (members[i].rows == 0 || members[i].rows > 0xffffffffull) return hipErrorInvalidValue;
         rows[i] = members[i].rows;
     }
-    GemmGroupGeometry g = gemm_h16_group_geometry(rows, count, columns, vectors);
+    GemmGroupGeometry g = gemm_h16_group_geometry(codec, rows, count, columns, vectors);
     if (partials == nullptr && g.k_splits > 1) {  // nowhere to keep shares: 64-row workgroups, whole K each
         g = GemmGroupGeometry{64, 0, 1};
     }
     // weight lead: what the activation ring (three slots of 34 KiB) leaves of LDS
+    if (codec == kQ6_K)  // 64-row tiles only (gemm_h16_group_geometry): 128 rows of 224 bytes leave no room for a ring
+        return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
             return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);

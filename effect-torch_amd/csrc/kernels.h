@@ -105,7 +105,7 @@ hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_
 hipError_t reduce_partials(const float* partials, const float* bias, const float* residual, float* y,
                            uint32_t rows, uint32_t vectors, uint32_t k_splits, hipStream_t stream);
 
-// ---- gemm_h16.hip: Q4_K and Q5_K on the half-float matrix cores, exact integer operands (limbs = 2 tiles) ----
+// ---- gemm_h16.hip: Q4_K, Q5_K and Q6_K on the half-float matrix cores, exact integer operands (limbs = 2 tiles) ----
 bool gemm_h16_supported(int32_t codec, uint64_t columns);
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream);
@@ -127,8 +127,10 @@ struct GemmGroupGeometry {
     uint64_t row_tiles;
     uint32_t k_splits;
 };
-GemmGroupGeometry gemm_h16_group_geometry(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
-uint64_t gemm_h16_group_partial_bytes(const uint64_t* rows, uint32_t count, uint64_t columns, uint64_t vectors);
+GemmGroupGeometry gemm_h16_group_geometry(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
+                                          uint64_t vectors);
+uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
+                                      uint64_t vectors);
 hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
                           float* partials, uint64_t columns, uint64_t vectors, hipStream_t stream);
 

@@ -120,10 +120,11 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         plan->q_offset = cursor;  // activation tiles, see tile_blob_bytes()
         cursor = align_up(cursor + tile_workspace_bytes(limbs, plan->vectors, plan->columns), 256);
         if (limbs == 2) {  // gemm_h16 chooses its own tile height and keeps partial results by whole tiles
-            plan->k_splits = gemm_h16_group_geometry(&plan->rows, 1, plan->columns, plan->vectors).k_splits;
+            plan->k_splits = gemm_h16_group_geometry(plan->codec, &plan->rows, 1, plan->columns, plan->vectors).k_splits;
             if (plan->k_splits > 1) {
                 plan->partial_offset = cursor;
-                cursor = align_up(cursor + gemm_h16_group_partial_bytes(&plan->rows, 1, plan->columns, plan->vectors), 256);
+                cursor = align_up(cursor + gemm_h16_group_partial_bytes(plan->codec, &plan->rows, 1, plan->columns,
+                                                                        plan->vectors), 256);
             }
             return;
         }
@@ -413,7 +414,7 @@ int check_group(const et_linear_plan* const* plans, uint32_t count, std::string*
 uint64_t group_partial_bytes(const et_linear_plan* const* plans, uint32_t count) {
     uint64_t rows[kGemmGroupMost];
     for (uint32_t i = 0; i < count; i++) rows[i] = plans[i]->rows;
-    return gemm_h16_group_partial_bytes(rows, count, plans[0]->columns, plans[0]->vectors);
+    return gemm_h16_group_partial_bytes(plans[0]->codec, rows, count, plans[0]->columns, plans[0]->vectors);
 }
 }  // namespace
 
