@@ -68,6 +68,8 @@ class EtKvLayer(ctypes.Structure):
         ("active_batch", ctypes.c_uint64),
         ("context_window", ctypes.c_uint64),
         ("max_context", ctypes.c_uint64),
+        ("k_scales", ctypes.c_void_p),
+        ("v_scales", ctypes.c_void_p),
     ]
 
 

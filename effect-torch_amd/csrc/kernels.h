@@ -148,7 +148,9 @@ enum : uint32_t {
 struct KvAttention {
     void* k_slab;
     void* v_slab;
-    bool slab_is_f16;
+    int32_t slab_dtype;  // ET_DTYPE_F32, _F16, _BF16 or _U8 (the int8-quantized tier)
+    float* k_scales;     // [max_tokens, kv_heads], ET_DTYPE_U8 only
+    float* v_scales;
     uint32_t max_tokens, kv_heads, width, block_size;
     const uint32_t* block_table;  // [batch, table_stride]
     uint32_t table_stride;

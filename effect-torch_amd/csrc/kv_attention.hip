@@ -24,7 +24,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
+#include "et_hip.h"
 #include "kernels.h"
 
 namespace et {
@@ -33,9 +35,19 @@ namespace {
 constexpr uint32_t kNoBlock = 0xffffffffu;
 constexpr float kLowest = -1.0e30f;  // "no score yet": finite, so that exp2(kLowest - m) = 0 without NaN
 
+// Element types of a slab besides float and __half.
+struct Bf16 {
+    uint16_t bits;
+};
+struct U8 {  // the int8-quantized tier: byte = round(x / scale) + 128, one f32 scale per row and head
+    uint8_t byte;
+};
+
 struct KvArgs {
     void* k_slab;
     void* v_slab;
+    float* k_scales;  // [max_tokens, kv_heads], the U8 tier only
+    float* v_scales;
     const uint32_t* table;
     const uint32_t* cursors;
     const uint32_t* advances;
@@ -102,6 +114,28 @@ __device__ __forceinline__ float slab_round(const __half*, float value) {
 }
 __device__ __forceinline__ float slab_load(const float* slab, uint64_t at) { return slab[at]; }
 __device__ __forceinline__ float slab_load(const __half* slab, uint64_t at) { return __half2float(slab[at]); }
+// bf16::from_f32 (half 2.7.1): NaN keeps its top bits and gets a quiet bit, else round to nearest even.
+__device__ __forceinline__ uint32_t bf16_bits(float value) {
+    const uint32_t x = __float_as_uint(value);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (x >> 16) | 0x0040u;
+    return (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ void slab_store(Bf16* slab, uint64_t at, float value) {
+    slab[at].bits = static_cast<uint16_t>(bf16_bits(value));
+}
+__device__ __forceinline__ float slab_round(const Bf16*, float value) { return __uint_as_float(bf16_bits(value) << 16); }
+__device__ __forceinline__ float slab_load(const Bf16* slab, uint64_t at) {
+    return __uint_as_float(static_cast<uint32_t>(slab[at].bits) << 16);
+}
+// The U8 tier (napi/mod.rs:3397-3437, :3467-3478): scale = max|x| / 127 + 1e-12 over the row of a
+// head, byte = clamp(round(x / scale), +-127) + 128 (halves away from zero), value = (byte - 128) * scale.
+__device__ __forceinline__ float u8_scale(float row_maximum) { return row_maximum / 127.0f + 1e-12f; }
+__device__ __forceinline__ uint32_t u8_byte(float value, float scale) {
+    return static_cast<uint32_t>(fminf(fmaxf(roundf(value / scale), -127.0f), 127.0f) + 128.0f);
+}
+__device__ __forceinline__ float u8_value(uint32_t byte, float scale) {
+    return (static_cast<float>(byte) - 128.0f) * scale;
+}
 
 __global__ void kv_zero_kernel(float* out, uint64_t count, unsigned long long* status, uint32_t slots) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -157,18 +191,32 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+template <int LANES>
+__device__ __forceinline__ float group_max(float v) {
+    if constexpr (LANES >= 2) v = fmaxf(v, dpp_f32<0xB1>(v));
+    if constexpr (LANES >= 4) v = fmaxf(v, dpp_f32<0x4E>(v));
+    if constexpr (LANES >= 8) v = fmaxf(v, dpp_f32<0x141>(v));
+    if constexpr (LANES >= 16) v = fmaxf(v, dpp_f32<0x140>(v));
+    if constexpr (LANES >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+    if constexpr (LANES >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
 // Sixteen bytes of a slab row as floats.
 template <typename T>
 struct Piece;
 template <>
 struct Piece<float> {
     static constexpr int kDims = 4;
+    static constexpr int kElementBytes = 4;
+    static constexpr bool kScaled = false;
     uint4 raw;
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = i == 0 ? raw.x : i == 1 ? raw.y : i == 2 ? raw.z : raw.w;
         return __uint_as_float(w);
     }
-    // what the slab would hold for these input values
+    // what the slab would hold for these input values (LANES lanes share the row of a head)
+    template <int LANES>
     __device__ __forceinline__ void from_input(const float* source) {
         raw = *reinterpret_cast<const uint4*>(source);
     }
@@ -176,11 +224,14 @@ struct Piece<float> {
 template <>
 struct Piece<__half> {
     static constexpr int kDims = 8;
+    static constexpr int kElementBytes = 2;
+    static constexpr bool kScaled = false;
     uint4 raw;
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = (i >> 1) == 0 ? raw.x : (i >> 1) == 1 ? raw.y : (i >> 1) == 2 ? raw.z : raw.w;
         return __half2float(__ushort_as_half(static_cast<unsigned short>((i & 1) ? (w >> 16) : (w & 0xffffu))));
     }
+    template <int LANES>
     __device__ __forceinline__ void from_input(const float* source) {
         const float4 low = *reinterpret_cast<const float4*>(source);
         const float4 high = *reinterpret_cast<const float4*>(source + 4);
@@ -189,6 +240,59 @@ struct Piece<__half> {
                    (static_cast<uint32_t>(__half_as_ushort(__float2half_rn(y))) << 16);
         };
         raw = make_uint4(pack(low.x, low.y), pack(low.z, low.w), pack(high.x, high.y), pack(high.z, high.w));
+    }
+};
+template <>
+struct Piece<Bf16> {
+    static constexpr int kDims = 8;
+    static constexpr int kElementBytes = 2;
+    static constexpr bool kScaled = false;
+    uint4 raw;
+    __device__ __forceinline__ float get(int i) const {
+        const uint32_t w = (i >> 1) == 0 ? raw.x : (i >> 1) == 1 ? raw.y : (i >> 1) == 2 ? raw.z : raw.w;
+        return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    }
+    template <int LANES>
+    __device__ __forceinline__ void from_input(const float* source) {
+        const float4 low = *reinterpret_cast<const float4*>(source);
+        const float4 high = *reinterpret_cast<const float4*>(source + 4);
+        const auto pack = [](float x, float y) { return bf16_bits(x) | (bf16_bits(y) << 16); };
+        raw = make_uint4(pack(low.x, low.y), pack(low.z, low.w), pack(high.x, high.y), pack(high.z, high.w));
+    }
+};
+template <>
+struct Piece<U8> {
+    static constexpr int kDims = 16;
+    static constexpr int kElementBytes = 1;
+    static constexpr bool kScaled = true;
+    uint4 raw;
+    float scale;  // of the row and head these bytes belong to
+    __device__ __forceinline__ float get(int i) const {
+        const uint32_t w = (i >> 2) == 0 ? raw.x : (i >> 2) == 1 ? raw.y : (i >> 2) == 2 ? raw.z : raw.w;
+        // (byte - 128) * scale, one rounding: -128 * scale is exact
+        return fmaf(static_cast<float>((w >> (8 * (i & 3))) & 0xffu), scale, -128.0f * scale);
+    }
+    template <int LANES>
+    __device__ __forceinline__ void from_input(const float* source) {
+        float values[16];
+        float maximum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float4 v = *reinterpret_cast<const float4*>(source + 4 * j);
+            values[4 * j] = v.x;
+            values[4 * j + 1] = v.y;
+            values[4 * j + 2] = v.z;
+            values[4 * j + 3] = v.w;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i++) maximum = fmaxf(maximum, fabsf(values[i]));
+        scale = u8_scale(group_max<LANES>(maximum));
+        uint32_t words[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            words[j] = u8_byte(values[4 * j], scale) | (u8_byte(values[4 * j + 1], scale) << 8) |
+                       (u8_byte(values[4 * j + 2], scale) << 16) | (u8_byte(values[4 * j + 3], scale) << 24);
+        raw = make_uint4(words[0], words[1], words[2], words[3]);
     }
 };
 
@@ -432,8 +536,8 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
         for (int d = 0; d < DPL; d++) acc[g][d] = 0.f;
     }
 
-    const uint64_t row_bytes = static_cast<uint64_t>(a.kv_heads) * a.width * sizeof(T);
-    const uint64_t lane_offset = (static_cast<uint64_t>(kv_head) * a.width + sub * DPL) * sizeof(T);
+    const uint64_t row_bytes = static_cast<uint64_t>(a.kv_heads) * a.width * Piece<T>::kElementBytes;
+    const uint64_t lane_offset = (static_cast<uint64_t>(kv_head) * a.width + sub * DPL) * Piece<T>::kElementBytes;
     char* k_base = static_cast<char*>(a.k_slab) + lane_offset;
     char* v_base = static_cast<char*>(a.v_slab) + lane_offset;
     const auto row_of = [&](uint32_t position) {
@@ -449,6 +553,10 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
                 const uint32_t row = row_of(min(step_begin + u * PPG + group, cached_end - 1));
                 kp[u].raw = *reinterpret_cast<const uint4*>(k_base + row * row_bytes);
                 vp[u].raw = *reinterpret_cast<const uint4*>(v_base + row * row_bytes);
+                if constexpr (Piece<T>::kScaled) {
+                    kp[u].scale = a.k_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head];
+                    vp[u].scale = a.v_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head];
+                }
             }
         };
         const auto consume = [&](uint32_t step, const Piece<T> (&kp)[U], const Piece<T> (&vp)[U]) {
@@ -482,14 +590,20 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
         const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + kv_head) * a.tokens + arrival) *
                                     a.width + sub * DPL;
         Piece<T> kp[1], vp[1];
-        kp[0].from_input(a.k + source);
-        vp[0].from_input(a.v + source);
+        kp[0].template from_input<LPT>(a.k + source);
+        vp[0].template from_input<LPT>(a.v + source);
         if (live[0] && arrival == token && chunk == 0) {
             const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
             const uint32_t row = base + within_block(a, position);
             if (base != kNoBlock && row < a.max_tokens) {
                 *reinterpret_cast<uint4*>(k_base + row * row_bytes) = kp[0].raw;
                 *reinterpret_cast<uint4*>(v_base + row * row_bytes) = vp[0].raw;
+                if constexpr (Piece<T>::kScaled) {
+                    if (sub == 0) {
+                        a.k_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head] = kp[0].scale;
+                        a.v_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head] = vp[0].scale;
+                    }
+                }
             }
         }
         if constexpr (kScatter)
@@ -589,23 +703,70 @@ __global__ __launch_bounds__(64) void kv_attend_any_kernel(const KvArgs a) {
         const bool appends = arriving && arrival == token && head % group_size == 0 && inside;
         float key[kKvAnyWidthPerLane], value[kKvAnyWidthPerLane];
         float part = 0.f;
+        if constexpr (std::is_same<T, U8>::value) {
+            // the row's scales: of the cached row, or what the write computes for the arriving one
+            float k_scale, v_scale;
+            if (arriving) {
+                float k_top = 0.f, v_top = 0.f;
 #pragma unroll
-        for (int i = 0; i < kKvAnyWidthPerLane; i++) {
-            const uint32_t column = lane + 64 * i;
-            key[i] = value[i] = 0.f;
-            if (column < a.width) {
-                if (arriving) {
-                    key[i] = slab_round(keys, a.k[source + column]);
-                    value[i] = slab_round(values, a.v[source + column]);
-                    if (appends) {
-                        slab_store(keys, at + column, a.k[source + column]);
-                        slab_store(values, at + column, a.v[source + column]);
+                for (int i = 0; i < kKvAnyWidthPerLane; i++) {
+                    const uint32_t column = lane + 64 * i;
+                    if (column < a.width) {
+                        k_top = fmaxf(k_top, fabsf(a.k[source + column]));
+                        v_top = fmaxf(v_top, fabsf(a.v[source + column]));
                     }
-                } else {
-                    key[i] = slab_load(keys, at + column);
-                    value[i] = slab_load(values, at + column);
                 }
-                part = fmaf(q[i], key[i], part);
+                k_scale = u8_scale(group_max<64>(k_top));
+                v_scale = u8_scale(group_max<64>(v_top));
+                if (appends && lane == 0) {
+                    a.k_scales[row * a.kv_heads + kv_head] = k_scale;
+                    a.v_scales[row * a.kv_heads + kv_head] = v_scale;
+                }
+            } else {
+                k_scale = a.k_scales[row * a.kv_heads + kv_head];
+                v_scale = a.v_scales[row * a.kv_heads + kv_head];
+            }
+#pragma unroll
+            for (int i = 0; i < kKvAnyWidthPerLane; i++) {
+                const uint32_t column = lane + 64 * i;
+                key[i] = value[i] = 0.f;
+                if (column < a.width) {
+                    uint32_t k_byte, v_byte;
+                    if (arriving) {
+                        k_byte = u8_byte(a.k[source + column], k_scale);
+                        v_byte = u8_byte(a.v[source + column], v_scale);
+                        if (appends) {
+                            keys[at + column].byte = static_cast<uint8_t>(k_byte);
+                            values[at + column].byte = static_cast<uint8_t>(v_byte);
+                        }
+                    } else {
+                        k_byte = keys[at + column].byte;
+                        v_byte = values[at + column].byte;
+                    }
+                    key[i] = u8_value(k_byte, k_scale);
+                    value[i] = u8_value(v_byte, v_scale);
+                    part = fmaf(q[i], key[i], part);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kKvAnyWidthPerLane; i++) {
+                const uint32_t column = lane + 64 * i;
+                key[i] = value[i] = 0.f;
+                if (column < a.width) {
+                    if (arriving) {
+                        key[i] = slab_round(keys, a.k[source + column]);
+                        value[i] = slab_round(values, a.v[source + column]);
+                        if (appends) {
+                            slab_store(keys, at + column, a.k[source + column]);
+                            slab_store(values, at + column, a.v[source + column]);
+                        }
+                    } else {
+                        key[i] = slab_load(keys, at + column);
+                        value[i] = slab_load(values, at + column);
+                    }
+                    part = fmaf(q[i], key[i], part);
+                }
             }
         }
         const float score = group_sum<64>(part);
@@ -644,8 +805,15 @@ __global__ void kv_merge_kernel(const KvArgs a) {
 template <typename T, int LPT, int G>
 hipError_t launch_streaming(const KvArgs& a, uint32_t workgroups, int waves, hipStream_t stream) {
     constexpr int U = G >= 8 ? 2 : 4;
-    if (waves == 8)
-        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
+    // (kv_attention_shape never asks for eight waves of the u8 tier with groups of eight heads: the
+    // merge area of 16-value pieces would not fit LDS)
+    if constexpr (!(std::is_same<T, U8>::value && G >= 8)) {
+        if (waves == 8) {
+            hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
+            return hipGetLastError();
+        }
+    }
+    if (waves == 8) return hipErrorInvalidValue;
     else
         hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4>), dim3(workgroups), dim3(256), 0, stream, a);
     return hipGetLastError();
@@ -671,8 +839,13 @@ hipError_t launch_streaming_width(const KvArgs& a, int g, uint32_t workgroups, i
 }
 
 // Query heads of one kv head served together by the streaming kernel; 0 = not covered.
+// Elements of a slab row in sixteen bytes.
+uint32_t piece_dims(const KvAttention& p) {
+    return p.slab_dtype == ET_DTYPE_F32 ? 4 : p.slab_dtype == ET_DTYPE_U8 ? 16 : 8;
+}
+
 int streaming_group(const KvAttention& p) {
-    const uint32_t dims = p.slab_is_f16 ? 8 : 4;
+    const uint32_t dims = piece_dims(p);
     if (p.width % dims != 0) return 0;
     const uint32_t lanes = p.width / dims;
     if (lanes != 8 && lanes != 16 && lanes != 32) return 0;
@@ -683,7 +856,7 @@ int streaming_group(const KvAttention& p) {
 }
 
 uint32_t positions_per_step(const KvAttention& p, int g, int waves) {
-    const uint32_t lanes = p.width / (p.slab_is_f16 ? 8 : 4);
+    const uint32_t lanes = p.width / piece_dims(p);
     return waves * (64 / lanes) * (g >= 8 ? 2 : 4);
 }
 
@@ -703,7 +876,7 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     // slots x 8 kv heads at context 2048: 512 x 4 waves 58.9 us, 1024 x 4 waves 63.7, 256 x 8 waves
     // without any split - no partial records, no merge launch - 55.6). Eight waves need enough rows
     // of queries to go round without splitting.
-    shape.waves = shape.streaming && rows >= 128 ? 8 : 4;
+    shape.waves = shape.streaming && rows >= 128 && !(p.slab_dtype == ET_DTYPE_U8 && g >= 8) ? 8 : 4;
     const uint64_t step = shape.streaming ? positions_per_step(p, g, shape.waves) : 64;
     uint64_t splits = 1;
     const uint64_t wanted = shape.streaming ? (shape.waves == 8 ? 256 : 512) : 4096;
@@ -730,6 +903,8 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     KvArgs a{};
     a.k_slab = p.k_slab;
     a.v_slab = p.v_slab;
+    a.k_scales = p.k_scales;
+    a.v_scales = p.v_scales;
     a.table = p.block_table;
     a.cursors = p.cursors;
     a.advances = p.advances;
@@ -770,16 +945,21 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     hipError_t error;
     if (shape.streaming) {
         const int g = streaming_group(p);
-        error = p.slab_is_f16
-                    ? launch_streaming_width<__half>(a, g, static_cast<uint32_t>(shape.workgroups), shape.waves, stream)
-                    : launch_streaming_width<float>(a, g, static_cast<uint32_t>(shape.workgroups), shape.waves, stream);
+        const uint32_t workgroups = static_cast<uint32_t>(shape.workgroups);
+        switch (p.slab_dtype) {
+            case ET_DTYPE_F16: error = launch_streaming_width<__half>(a, g, workgroups, shape.waves, stream); break;
+            case ET_DTYPE_BF16: error = launch_streaming_width<Bf16>(a, g, workgroups, shape.waves, stream); break;
+            case ET_DTYPE_U8: error = launch_streaming_width<U8>(a, g, workgroups, shape.waves, stream); break;
+            default: error = launch_streaming_width<float>(a, g, workgroups, shape.waves, stream); break;
+        }
     } else {
-        if (p.slab_is_f16)
-            hipLaunchKernelGGL(kv_attend_any_kernel<__half>, dim3(static_cast<uint32_t>(shape.workgroups)),
-                               dim3(64), 0, stream, a);
-        else
-            hipLaunchKernelGGL(kv_attend_any_kernel<float>, dim3(static_cast<uint32_t>(shape.workgroups)),
-                               dim3(64), 0, stream, a);
+        const dim3 grid(static_cast<uint32_t>(shape.workgroups));
+        switch (p.slab_dtype) {
+            case ET_DTYPE_F16: hipLaunchKernelGGL(kv_attend_any_kernel<__half>, grid, dim3(64), 0, stream, a); break;
+            case ET_DTYPE_BF16: hipLaunchKernelGGL(kv_attend_any_kernel<Bf16>, grid, dim3(64), 0, stream, a); break;
+            case ET_DTYPE_U8: hipLaunchKernelGGL(kv_attend_any_kernel<U8>, grid, dim3(64), 0, stream, a); break;
+            default: hipLaunchKernelGGL(kv_attend_any_kernel<float>, grid, dim3(64), 0, stream, a); break;
+        }
         error = hipGetLastError();
     }
     if (error != hipSuccess) return error;

@@ -19,8 +19,10 @@ constexpr uint64_t kLimit = 0xffffffffull;
 
 // Geometry of the layer alone; `p` receives what the kernels need of it.
 int layer_geometry(const et_kv_layer& layer, KvAttention* p, std::string* error) {
-    if (layer.slab_dtype != ET_DTYPE_F32 && layer.slab_dtype != ET_DTYPE_F16)
-        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: slabs must be f32 or f16");
+    // NativeKvPool::new (napi/mod.rs:3652-3658)
+    if (layer.slab_dtype != ET_DTYPE_F32 && layer.slab_dtype != ET_DTYPE_F16 && layer.slab_dtype != ET_DTYPE_BF16 &&
+        layer.slab_dtype != ET_DTYPE_U8)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv pool: dtype must be f32, f16, bf16 or u8 (int8-quantized)");
     if (layer.kv_heads == 0 || layer.head_dim == 0 || layer.block_size == 0 || layer.max_tokens == 0)
         return fail(error, ET_ERR_UNSUPPORTED, "kv attention: empty pool geometry");
     if (layer.max_tokens > kLimit || layer.kv_heads > kLimit || layer.head_dim > kLimit ||
@@ -32,7 +34,7 @@ int layer_geometry(const et_kv_layer& layer, KvAttention* p, std::string* error)
     if (layer.active_batch > layer.slots)
         return fail(error, ET_ERR_UNSUPPORTED, "kv attention: active batch " + std::to_string(layer.active_batch) +
                                                    " exceeds " + std::to_string(layer.slots) + " kv slots");
-    p->slab_is_f16 = layer.slab_dtype == ET_DTYPE_F16;
+    p->slab_dtype = layer.slab_dtype;
     p->max_tokens = static_cast<uint32_t>(layer.max_tokens);
     p->kv_heads = static_cast<uint32_t>(layer.kv_heads);
     p->width = static_cast<uint32_t>(layer.head_dim);
@@ -130,8 +132,14 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
         layer.cursors == nullptr || layer.advances == nullptr || q.data == nullptr || k.data == nullptr ||
         v.data == nullptr || destination.data == nullptr)
         return fail(error, ET_ERR_INVALID, "kv attention: NULL device pointer");
+    if (layer.slab_dtype == ET_DTYPE_U8 &&
+        (layer.k_scales == nullptr || layer.v_scales == nullptr || reinterpret_cast<uintptr_t>(layer.k_scales) % 4 != 0 ||
+         reinterpret_cast<uintptr_t>(layer.v_scales) % 4 != 0))
+        return fail(error, ET_ERR_INVALID, "kv attention: the u8 tier needs its f32 scale slabs");
     p.k_slab = layer.k_slab;
     p.v_slab = layer.v_slab;
+    p.k_scales = layer.slab_dtype == ET_DTYPE_U8 ? layer.k_scales : nullptr;
+    p.v_scales = layer.slab_dtype == ET_DTYPE_U8 ? layer.v_scales : nullptr;
     p.block_table = layer.block_table;
     p.cursors = layer.cursors;
     p.advances = layer.advances;

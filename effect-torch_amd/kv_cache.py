@@ -16,19 +16,31 @@ import torch
 from . import _native as N
 from .quantized import CancellationFlag, QuantizedError, _check, _desc, _ref, _stream_handle
 
-_SLAB_DTYPES = {torch.float32: N.DTYPE_F32, torch.float16: N.DTYPE_F16}
+_SLAB_DTYPES = {torch.float32: N.DTYPE_F32, torch.float16: N.DTYPE_F16, torch.bfloat16: N.DTYPE_BF16,
+                torch.uint8: N.DTYPE_U8}
 
 
 class KvLayer:
-    """Device state of one layer. ``k_slab`` / ``v_slab``: ``[max_tokens, kv_heads, head_dim]`` f32 or
-    f16; ``block_table``: uint32/int32 ``[slots, table_stride]``; ``cursors`` / ``advances``:
+    """Device state of one layer. ``k_slab`` / ``v_slab``: ``[max_tokens, kv_heads, head_dim]`` f32,
+    f16, bf16 or uint8 (the int8-quantized tier, with f32 ``k_scales`` / ``v_scales``
+    ``[max_tokens, kv_heads]``); ``block_table``: uint32/int32 ``[slots, table_stride]``; ``cursors`` / ``advances``:
     uint32/int32 ``[slots]``. ``max_context`` bounds ``cursor + advance`` (it sizes the launch)."""
 
     def __init__(self, k_slab: torch.Tensor, v_slab: torch.Tensor, block_size: int, block_table: torch.Tensor,
                  cursors: torch.Tensor, advances: torch.Tensor, max_context: int,
-                 active_batch: Optional[int] = None, context_window: int = 0):
+                 active_batch: Optional[int] = None, context_window: int = 0,
+                 k_scales: Optional[torch.Tensor] = None, v_scales: Optional[torch.Tensor] = None):
         if k_slab.dtype not in _SLAB_DTYPES or v_slab.dtype != k_slab.dtype:
-            raise QuantizedError(N.ERR_UNSUPPORTED, "kv attention: slabs must be f32 or f16")
+            raise QuantizedError(N.ERR_UNSUPPORTED, "kv pool: dtype must be f32, f16, bf16 or u8 (int8-quantized)")
+        if k_slab.dtype == torch.uint8:
+            for scales in (k_scales, v_scales):
+                if scales is None or scales.dtype != torch.float32 or not scales.is_contiguous() or \
+                        tuple(scales.shape) != tuple(k_slab.shape[:2]):
+                    raise QuantizedError(N.ERR_UNSUPPORTED,
+                                         "kv attention: the u8 tier needs contiguous f32 scales [tokens, heads]")
+        elif k_scales is not None or v_scales is not None:
+            raise QuantizedError(N.ERR_UNSUPPORTED, "kv attention: only the u8 tier has scale slabs")
+        self.k_scales, self.v_scales = k_scales, v_scales
         if k_slab.dim() != 3 or k_slab.shape != v_slab.shape or not k_slab.is_contiguous() or \
                 not v_slab.is_contiguous():
             raise QuantizedError(N.ERR_UNSUPPORTED, "kv attention: slabs must be contiguous [tokens, heads, width]")
@@ -50,7 +62,9 @@ class KvLayer:
         return N.EtKvLayer(self.k_slab.data_ptr(), self.v_slab.data_ptr(), _SLAB_DTYPES[self.k_slab.dtype],
                            max_tokens, kv_heads, width, self.block_size, self.block_table.data_ptr(),
                            self.block_table.shape[1], self.cursors.data_ptr(), self.advances.data_ptr(),
-                           self.cursors.numel(), self.active_batch, self.context_window, self.max_context)
+                           self.cursors.numel(), self.active_batch, self.context_window, self.max_context,
+                           self.k_scales.data_ptr() if self.k_scales is not None else None,
+                           self.v_scales.data_ptr() if self.v_scales is not None else None)
 
 
 def kv_attention_workspace_bytes(layer: KvLayer, query_heads: int, tokens: int) -> int:

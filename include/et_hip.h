@@ -258,9 +258,11 @@ int et_hip_dequantize_rows(int32_t codec, uint64_t rows, uint64_t columns, const
  * :2501-2513; slabs crates/runtime-cpu/src/pool.rs). All pointers are device
  * pointers. */
 typedef struct {
-    void* k_slab;                /* [max_tokens, kv_heads, head_dim], f32 or f16; written and read */
+    void* k_slab;                /* [max_tokens, kv_heads, head_dim] of slab_dtype; written and read */
     void* v_slab;
-    int32_t slab_dtype;          /* ET_DTYPE_F32 or ET_DTYPE_F16 (the reference's int8 tier is not covered) */
+    int32_t slab_dtype;          /* ET_DTYPE_F32, ET_DTYPE_F16, ET_DTYPE_BF16, or ET_DTYPE_U8: the
+                                    int8-quantized tier (napi/mod.rs:3397-3437), byte = round(x / scale) +
+                                    128 with one f32 scale per row and head in k_scales / v_scales */
     uint64_t max_tokens;         /* pool.max_tokens */
     uint64_t kv_heads;           /* pool.kv_heads */
     uint64_t head_dim;           /* pool.head_dim */
@@ -275,6 +277,9 @@ typedef struct {
     uint64_t context_window;     /* context.window, 0 = none */
     uint64_t max_context;        /* host-side upper bound of cursor + advance over the active slots;
                                     it sizes the launch and the workspace */
+    float* k_scales;             /* [max_tokens, kv_heads] f32, ET_DTYPE_U8 only (pool.scales[2 * layer],
+                                    napi/mod.rs:3727-3734); written with the rows; NULL otherwise */
+    float* v_scales;
 } et_kv_layer;
 
 /* Device scratch et_hip_kv_attention_into needs for these sizes (partial results

@@ -93,9 +93,11 @@ def lib() -> ctypes.CDLL:
         L.et_oracle_gather_rows.argtypes = [vp, sz, sz, vp, sz, vp, ctypes.c_char_p, sz]
         L.et_oracle_f32_to_fp16.restype = ctypes.c_uint16
         L.et_oracle_f32_to_fp16.argtypes = [ctypes.c_float]
-        L.et_oracle_kv_attention.restype = ci
-        L.et_oracle_kv_attention.argtypes = [ci, vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, sz, sz, sz,
-                                             vp, vp, vp, ctypes.c_double, sz, sz, vp, ctypes.c_char_p, sz]
+        L.et_oracle_f32_to_bf16.restype = ctypes.c_uint16
+        L.et_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.et_oracle_kv_attention_scaled.restype = ci
+        L.et_oracle_kv_attention_scaled.argtypes = [ci, vp, vp, vp, vp, sz, sz, sz, sz, vp, sz, vp, vp, sz, sz, sz, sz,
+                                                    vp, vp, vp, ctypes.c_double, sz, sz, vp, ctypes.c_char_p, sz]
         _lib = L
     return _lib
 
@@ -263,13 +265,27 @@ def f32_to_fp16_bits(value) -> int:
     return int(lib().et_oracle_f32_to_fp16(ctypes.c_float(float(np.float32(value)))))
 
 
+def f32_to_bf16_bits(value) -> int:
+    """binary32 -> bfloat16 bits, round to nearest even (et_oracle_f32_to_bf16)."""
+    return int(lib().et_oracle_f32_to_bf16(ctypes.c_float(float(np.float32(value)))))
+
+
 def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_table: np.ndarray,
                  cursors, advances, q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float,
-                 window: int = 0, active_batch=None, context_window: int = 0) -> np.ndarray:
-    """Paged KV attention (et_oracle_kv_attention): writes the new rows of ``k`` / ``v`` into the
-    slabs IN PLACE (float32 or float16 ``[max_tokens, kv_heads, width]``), then attends.
-    ``q`` is ``[batch, query_heads, tokens, width]``; returns the output of the same shape."""
-    assert k_slab.dtype == v_slab.dtype and k_slab.dtype in (np.float32, np.float16)
+                 window: int = 0, active_batch=None, context_window: int = 0, k_scales=None,
+                 v_scales=None) -> np.ndarray:
+    """Paged KV attention (et_oracle_kv_attention_scaled): writes the new rows of ``k`` / ``v`` into
+    the slabs IN PLACE, then attends. Slabs are ``[max_tokens, kv_heads, width]`` in float32, float16,
+    uint16 (bfloat16 bits) or uint8 (the int8-quantized tier, with float32 ``k_scales`` / ``v_scales``
+    ``[max_tokens, kv_heads]``, written in place too). ``q`` is ``[batch, query_heads, tokens, width]``;
+    returns the output of the same shape."""
+    codes = {np.dtype(np.float32): 0, np.dtype(np.float16): 2, np.dtype(np.uint16): 3, np.dtype(np.uint8): 4}
+    assert k_slab.dtype == v_slab.dtype and k_slab.dtype in codes
+    code = codes[k_slab.dtype]
+    if code == 4:
+        for scales in (k_scales, v_scales):
+            assert scales is not None and scales.dtype == np.float32 and scales.flags.c_contiguous
+            assert scales.shape == k_slab.shape[:2]
     assert k_slab.flags.c_contiguous and v_slab.flags.c_contiguous and k_slab.shape == v_slab.shape
     max_tokens, kv_heads, width = k_slab.shape
     q = np.ascontiguousarray(q, dtype=np.float32)
@@ -282,11 +298,14 @@ def kv_attention(k_slab: np.ndarray, v_slab: np.ndarray, block_size: int, block_
     advances = np.ascontiguousarray(advances, dtype=np.uint32)
     out = np.zeros_like(q)
     err = ctypes.create_string_buffer(256)
-    rc = lib().et_oracle_kv_attention(0 if k_slab.dtype == np.float32 else 2, _ptr(k_slab), _ptr(v_slab),
-                                      max_tokens, kv_heads, width, block_size, _ptr(table), table.shape[1],
-                                      _ptr(cursors), _ptr(advances), batch,
-                                      batch if active_batch is None else active_batch, query_heads, tokens,
-                                      _ptr(q), _ptr(k), _ptr(v), float(scale), context_window, window, _ptr(out), err, 256)
+    rc = lib().et_oracle_kv_attention_scaled(code, _ptr(k_slab), _ptr(v_slab),
+                                             _ptr(k_scales) if code == 4 else None,
+                                             _ptr(v_scales) if code == 4 else None,
+                                             max_tokens, kv_heads, width, block_size, _ptr(table), table.shape[1],
+                                             _ptr(cursors), _ptr(advances), batch,
+                                             batch if active_batch is None else active_batch, query_heads, tokens,
+                                             _ptr(q), _ptr(k), _ptr(v), float(scale), context_window, window,
+                                             _ptr(out), err, 256)
     if rc != 0:
         raise OracleError(err.value.decode())
     return out

@@ -39,21 +39,63 @@ uint16_t et_oracle_f32_to_fp16(float value) {
     return (uint16_t)(sign | half);
 }
 
+/* bf16::from_f32 (half 2.7.1): NaN keeps its top bits and gets a quiet bit; otherwise round to
+ * nearest even on the sixteen dropped bits. */
+uint16_t et_oracle_f32_to_bf16(float value) {
+    uint32_t x;
+    memcpy(&x, &value, sizeof x);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    const uint32_t round_bit = 0x00008000u;
+    if ((x & round_bit) != 0 && (x & (3u * round_bit - 1u)) != 0) return (uint16_t)((x >> 16) + 1u);
+    return (uint16_t)(x >> 16);
+}
+
+static float bf16_to_f32(uint16_t bits) {
+    const uint32_t x = (uint32_t)bits << 16;
+    float value;
+    memcpy(&value, &x, sizeof value);
+    return value;
+}
+
 static int fail(char* err, size_t err_len, const char* message) {
     if (err != NULL && err_len > 0) snprintf(err, err_len, "%s", message);
     return -1;
 }
 
-static float slab_get(int dtype, const void* slab, size_t index) {
+/* SlabReader::get_f32 (pool.rs) and, for the u8 tier, `cached` (napi/mod.rs:3467-3478):
+ * (raw - 128) * scale of the row and head. */
+static float slab_get(int dtype, const void* slab, const float* scales, size_t index, size_t width) {
     if (dtype == 0) return ((const float*)slab)[index];
-    return et_oracle_fp16_to_f32(((const uint16_t*)slab)[index]);
+    if (dtype == 2) return et_oracle_fp16_to_f32(((const uint16_t*)slab)[index]);
+    if (dtype == 3) return bf16_to_f32(((const uint16_t*)slab)[index]);
+    return ((float)((const uint8_t*)slab)[index] - 128.0f) * scales[index / width];
 }
 
 static void slab_set(int dtype, void* slab, size_t index, float value) {
     if (dtype == 0)
         ((float*)slab)[index] = value;
-    else
+    else if (dtype == 2)
         ((uint16_t*)slab)[index] = et_oracle_f32_to_fp16(value);
+    else
+        ((uint16_t*)slab)[index] = et_oracle_f32_to_bf16(value);
+}
+
+/* The u8 tier's write (napi/mod.rs:3397-3437): one scale per row and head, max|x| / 127 + 1e-12,
+ * bytes round(x / scale) clamped to +-127, plus 128. f32::round rounds halves away from zero. */
+static void slab_set_row_u8(uint8_t* slab, float* scales, size_t row_head, const float* values, size_t width) {
+    float maximum = 0.0f;
+    for (size_t column = 0; column < width; column++) {
+        const float magnitude = fabsf(values[column]);
+        if (magnitude > maximum) maximum = magnitude; /* f32::max ignores a NaN operand the same way */
+    }
+    const float scale = maximum / 127.0f + 1e-12f;
+    scales[row_head] = scale;
+    for (size_t column = 0; column < width; column++) {
+        float value = roundf(values[column] / scale);
+        if (value < -127.0f) value = -127.0f;
+        if (value > 127.0f) value = 127.0f;
+        slab[row_head * width + column] = (uint8_t)(value + 128.0f);
+    }
 }
 
 int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t max_tokens,
@@ -63,7 +105,23 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
                            size_t active_batch, size_t query_heads, size_t tokens, const float* q,
                            const float* k, const float* v, double scale, size_t context_window, size_t window,
                            float* out, char* err, size_t err_len) {
-    if (slab_dtype != 0 && slab_dtype != 2) return fail(err, err_len, "kv attention: unsupported slab dtype");
+    return et_oracle_kv_attention_scaled(slab_dtype, k_slab, v_slab, NULL, NULL, max_tokens, kv_heads, width,
+                                         block_size, block_table, table_stride, cursors, advances, batch,
+                                         active_batch, query_heads, tokens, q, k, v, scale, context_window, window,
+                                         out, err, err_len);
+}
+
+int et_oracle_kv_attention_scaled(int slab_dtype, void* k_slab, void* v_slab, float* k_scales, float* v_scales,
+                                  size_t max_tokens, size_t kv_heads, size_t width, size_t block_size,
+                                  const uint32_t* block_table, size_t table_stride,
+                                  const uint32_t* cursors, const uint32_t* advances, size_t batch,
+                                  size_t active_batch, size_t query_heads, size_t tokens, const float* q,
+                                  const float* k, const float* v, double scale, size_t context_window,
+                                  size_t window, float* out, char* err, size_t err_len) {
+    if (slab_dtype != 0 && slab_dtype != 2 && slab_dtype != 3 && slab_dtype != 4)
+        return fail(err, err_len, "kv attention: unsupported slab dtype");
+    if (slab_dtype == 4 && (k_scales == NULL || v_scales == NULL))
+        return fail(err, err_len, "kv attention: the u8 tier needs its scale slabs");
     /* napi/mod.rs:3347-3360 */
     if (kv_heads == 0 || query_heads % kv_heads != 0)
         return fail(err, err_len, "kv attention: incompatible grouped-query q/k/v shapes");
@@ -91,12 +149,18 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
             const size_t position = cursor + token;
             const size_t row = (size_t)blocks[position / block_size] * block_size + position % block_size;
             if (row >= max_tokens) { free(weights); return fail(err, err_len, "kv attention: block outside the pool"); }
-            for (size_t head = 0; head < kv_heads; head++)
-                for (size_t column = 0; column < width; column++) {
-                    const size_t logical = ((b * kv_heads + head) * tokens + token) * width + column;
-                    slab_set(slab_dtype, k_slab, (row * kv_heads + head) * width + column, k[logical]);
-                    slab_set(slab_dtype, v_slab, (row * kv_heads + head) * width + column, v[logical]);
+            for (size_t head = 0; head < kv_heads; head++) {
+                const size_t logical_row = ((b * kv_heads + head) * tokens + token) * width;
+                if (slab_dtype == 4) {
+                    slab_set_row_u8((uint8_t*)k_slab, k_scales, row * kv_heads + head, k + logical_row, width);
+                    slab_set_row_u8((uint8_t*)v_slab, v_scales, row * kv_heads + head, v + logical_row, width);
+                    continue;
                 }
+                for (size_t column = 0; column < width; column++) {
+                    slab_set(slab_dtype, k_slab, (row * kv_heads + head) * width + column, k[logical_row + column]);
+                    slab_set(slab_dtype, v_slab, (row * kv_heads + head) * width + column, v[logical_row + column]);
+                }
+            }
         }
         /* then attend, :3476-3542: three passes in f64 per (head, query) */
         for (size_t head = 0; head < query_heads; head++) {
@@ -116,7 +180,7 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
                     double score = 0.0;
                     for (size_t column = 0; column < width; column++)
                         score += (double)q_row[column] *
-                                 (double)slab_get(slab_dtype, k_slab, (row * kv_heads + kv_head) * width + column);
+                                 (double)slab_get(slab_dtype, k_slab, k_scales, (row * kv_heads + kv_head) * width + column, width);
                     if (score * scale > maximum) maximum = score * scale;
                 }
                 /* The reference recomputes every score in the second pass and again per output column
@@ -134,7 +198,7 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
                     double score = 0.0;
                     for (size_t column = 0; column < width; column++)
                         score += (double)q_row[column] *
-                                 (double)slab_get(slab_dtype, k_slab, (row * kv_heads + kv_head) * width + column);
+                                 (double)slab_get(slab_dtype, k_slab, k_scales, (row * kv_heads + kv_head) * width + column, width);
                     weights[position - begin] = exp(score * scale - maximum);
                     denominator += weights[position - begin];
                 }
@@ -144,7 +208,7 @@ int et_oracle_kv_attention(int slab_dtype, void* k_slab, void* v_slab, size_t ma
                     for (size_t position = begin; position < end; position++) {
                         const size_t row = (size_t)blocks[position / block_size] * block_size + position % block_size;
                         result += weights[position - begin] *
-                                  (double)slab_get(slab_dtype, v_slab, (row * kv_heads + kv_head) * width + column);
+                                  (double)slab_get(slab_dtype, v_slab, v_scales, (row * kv_heads + kv_head) * width + column, width);
                     }
                     out_row[column] = (float)(result / denominator);
                 }

@@ -1,7 +1,8 @@
 """Paged key/value-cache attention on the GPU against the CPU oracle (oracle/et_oracle_kv.c).
 
-Bars: slabs after the call are bit-identical to the oracle's (f32 copies, f16 round-to-nearest-even);
-outputs agree to 1e-4 (f32 online softmax against the oracle's f64 three passes).
+Bars: slabs after the call are bit-identical to the oracle's (f32 copies, f16 / bf16
+round-to-nearest-even, the u8 tier's bytes and scales); outputs agree to 1e-4 (f32 online softmax
+against the oracle's f64 three passes over the same stored values).
 """
 import numpy as np
 import pytest
@@ -12,6 +13,22 @@ import oracle
 pytestmark = pytest.mark.gpu
 
 OUT_TOL = 1e-4
+ALL_DTYPES = [np.float32, np.float16, "bf16", "u8"]
+
+
+def dims_per_piece(dtype):
+    """Elements of a slab row in sixteen bytes."""
+    return {np.float32: 4, np.float16: 8, "bf16": 8, "u8": 16}[dtype]
+
+
+def random_slab(rng, shape, dtype):
+    values = rng.standard_normal(shape).astype(np.float32)
+    if dtype == "bf16":  # bfloat16 bits
+        return torch.from_numpy(values).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16), None
+    if dtype == "u8":    # bytes 1..255 and positive scales, as the write produces them
+        scales = (np.abs(values).max(-1) / np.float32(127.0) + np.float32(1e-12)).astype(np.float32)
+        return rng.integers(1, 256, shape).astype(np.uint8), scales
+    return values.astype(dtype), None
 
 
 def make_case(rng, *, slots, query_heads, kv_heads, width, block_size, contexts, tokens, advances, dtype,
@@ -23,12 +40,13 @@ def make_case(rng, *, slots, query_heads, kv_heads, width, block_size, contexts,
     total_blocks = slots * blocks_per_slot + spare_blocks
     max_tokens = total_blocks * block_size
     table = rng.permutation(total_blocks)[: slots * blocks_per_slot].reshape(slots, blocks_per_slot).astype(np.uint32)
-    k_slab = rng.standard_normal((max_tokens, kv_heads, width)).astype(np.float32).astype(dtype)
-    v_slab = rng.standard_normal((max_tokens, kv_heads, width)).astype(np.float32).astype(dtype)
+    k_slab, k_scales = random_slab(rng, (max_tokens, kv_heads, width), dtype)
+    v_slab, v_scales = random_slab(rng, (max_tokens, kv_heads, width), dtype)
     q = rng.standard_normal((slots, query_heads, tokens, width)).astype(np.float32)
     k = rng.standard_normal((slots, kv_heads, tokens, width)).astype(np.float32)
     v = rng.standard_normal((slots, kv_heads, tokens, width)).astype(np.float32)
-    return dict(k_slab=k_slab, v_slab=v_slab, table=table, cursors=contexts.astype(np.uint32),
+    return dict(k_slab=k_slab, v_slab=v_slab, k_scales=k_scales, v_scales=v_scales, table=table,
+                cursors=contexts.astype(np.uint32),
                 advances=advances.astype(np.uint32), q=q, k=k, v=v, block_size=block_size,
                 max_context=int((contexts + advances).max()))
 
@@ -36,30 +54,46 @@ def make_case(rng, *, slots, query_heads, kv_heads, width, block_size, contexts,
 def run_gpu(et, device, case, scale, *, window=0, context_window=0, active_batch=None, max_context=None,
             workspace=None):
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
-    k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+    bf16 = case["k_slab"].dtype == np.uint16
+
+    def slab(array):
+        return dev(array.view(np.int16)).view(torch.bfloat16) if bf16 else dev(array)
+
+    def back(tensor):
+        return tensor.view(torch.int16).cpu().numpy().view(np.uint16) if bf16 else tensor.cpu().numpy()
+
+    k_slab, v_slab = slab(case["k_slab"]), slab(case["v_slab"])
+    scales = [dev(case[name]) if case.get(name) is not None else None for name in ("k_scales", "v_scales")]
     layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)),
                        dev(case["cursors"].view(np.int32)), dev(case["advances"].view(np.int32)),
                        case["max_context"] if max_context is None else max_context,
-                       active_batch=active_batch, context_window=context_window)
+                       active_batch=active_batch, context_window=context_window, k_scales=scales[0],
+                       v_scales=scales[1])
     q = dev(case["q"])
     out = torch.full_like(q, float("nan"))
     et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, window, out, workspace=workspace)
-    return out.cpu().numpy(), k_slab.cpu().numpy(), v_slab.cpu().numpy(), layer
+    got_scales = [t.cpu().numpy() if t is not None else None for t in scales]
+    return out.cpu().numpy(), back(k_slab), back(v_slab), layer, got_scales
 
 
 def run_oracle(case, scale, *, window=0, context_window=0, active_batch=None):
     k_slab, v_slab = case["k_slab"].copy(), case["v_slab"].copy()
+    scales = [case[name].copy() if case.get(name) is not None else None for name in ("k_scales", "v_scales")]
     out = oracle.kv_attention(k_slab, v_slab, case["block_size"], case["table"], case["cursors"], case["advances"],
                               case["q"], case["k"], case["v"], scale, window=window,
-                              context_window=context_window, active_batch=active_batch)
-    return out, k_slab, v_slab
+                              context_window=context_window, active_batch=active_batch, k_scales=scales[0],
+                              v_scales=scales[1])
+    return out, k_slab, v_slab, scales
 
 
 def compare(got, want):
     out, k_slab, v_slab = got[:3]
-    ref_out, ref_k, ref_v = want
+    ref_out, ref_k, ref_v = want[:3]
     assert np.array_equal(k_slab.view(np.uint8), ref_k.view(np.uint8)), "K slab differs"
     assert np.array_equal(v_slab.view(np.uint8), ref_v.view(np.uint8)), "V slab differs"
+    if len(got) > 4 and got[4][0] is not None:
+        for mine, theirs in zip(got[4], want[3]):
+            assert np.array_equal(mine.view(np.uint32), theirs.view(np.uint32)), "scale slab differs"
     assert np.isfinite(out).all()
     error = np.abs(out - ref_out).max()
     assert error <= OUT_TOL, f"max |out - oracle| = {error}"
@@ -78,11 +112,11 @@ def test_the_reference_test_case(et, device):
     compare(got, run_oracle(case, 0.5))
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("lanes", [8, 16, 32])
 @pytest.mark.parametrize("group,kv_heads", [(1, 3), (2, 2), (4, 2), (8, 1), (3, 2), (12, 1)])
 def test_streaming_kernel_shapes(et, device, dtype, lanes, group, kv_heads):
-    width = lanes * (4 if dtype == np.float32 else 8)
+    width = lanes * dims_per_piece(dtype)
     rng = np.random.default_rng(1000 * lanes + 10 * group + kv_heads)
     case = make_case(rng, slots=3, query_heads=group * kv_heads, kv_heads=kv_heads, width=width, block_size=16,
                      contexts=[0, 37, 200], tokens=1, advances=[1, 1, 1], dtype=dtype)
@@ -92,12 +126,12 @@ def test_streaming_kernel_shapes(et, device, dtype, lanes, group, kv_heads):
     compare(got, run_oracle(case, scale))
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("lanes", [8, 16, 32])
 @pytest.mark.parametrize("group", [1, 4, 8])
 def test_eight_wave_workgroups_without_context_splits(et, device, dtype, lanes, group):
     # 256 rows of queries: one eight-wave workgroup per (slot, kv head), no partial records
-    width = lanes * (4 if dtype == np.float32 else 8)
+    width = lanes * dims_per_piece(dtype)
     rng = np.random.default_rng(7000 + 100 * lanes + group)
     slots, kv_heads = 32, 8
     contexts = rng.integers(0, 150, slots)
@@ -106,12 +140,13 @@ def test_eight_wave_workgroups_without_context_splits(et, device, dtype, lanes, 
                      contexts=contexts, tokens=1, advances=[1] * slots, dtype=dtype)
     scale = 1.0 / np.sqrt(width)
     got = run_gpu(et, device, case, scale)
-    assert et.kv_attention_kernel(got[3], group * kv_heads, 1) == "kv_attend"
-    assert et.kv_attention_workspace_bytes(got[3], group * kv_heads, 1) == 0
+    if not (dtype == "u8" and group == 8):  # sixteen values per piece: eight heads' merge area needs four waves
+        assert et.kv_attention_kernel(got[3], group * kv_heads, 1) == "kv_attend"
+        assert et.kv_attention_workspace_bytes(got[3], group * kv_heads, 1) == 0
     compare(got, run_oracle(case, scale))
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 @pytest.mark.parametrize("block_size", [1, 5, 16, 64])
 @pytest.mark.parametrize("tokens,advances", [(1, [1, 1, 1, 1]), (4, [4, 1, 3, 2])])
 def test_paging_chunks_and_ragged_advances(et, device, dtype, block_size, tokens, advances):
@@ -122,7 +157,8 @@ def test_paging_chunks_and_ragged_advances(et, device, dtype, block_size, tokens
     compare(got, run_oracle(case, 0.09))
 
 
-@pytest.mark.parametrize("width,dtype", [(4, np.float16), (20, np.float32), (96, np.float16), (200, np.float32)])
+@pytest.mark.parametrize("width,dtype", [(4, np.float16), (20, np.float32), (96, np.float16), (200, np.float32),
+                                         (40, "bf16"), (24, "u8"), (100, "u8")])
 def test_any_width_kernel(et, device, width, dtype):
     rng = np.random.default_rng(width)
     case = make_case(rng, slots=2, query_heads=6, kv_heads=3, width=width, block_size=8,
@@ -142,7 +178,7 @@ def test_sliding_windows(et, device, context_window, window, width):
     compare(got, run_oracle(case, 0.1, window=window, context_window=context_window))
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
 def test_long_context_is_split(et, device, dtype):
     rng = np.random.default_rng(77)
     case = make_case(rng, slots=2, query_heads=8, kv_heads=2, width=128, block_size=16,
@@ -227,7 +263,7 @@ def test_device_side_checks_report_the_reference_errors(et, device):
         run_gpu(et, device, case, 0.1)
 
 
-@pytest.mark.parametrize("dtype", [np.float16])
+@pytest.mark.parametrize("dtype", [np.float16, "u8"])
 def test_decode_batch_at_full_size(et, device, dtype):
     # 32 slots x 32 query heads over 8 kv heads of width 128, contexts around 2048, block size 16
     rng = np.random.default_rng(2048)
@@ -238,12 +274,14 @@ def test_decode_batch_at_full_size(et, device, dtype):
     got = run_gpu(et, device, case, scale)
     compare(got, run_oracle(case, scale))
     # size-independent property: with every key zero all scores are equal, the output is the mean of V
-    case["k_slab"][:] = 0
+    case["k_slab"][:] = 128 if dtype == "u8" else 0
     case["k"][:] = 0
-    out = run_gpu(et, device, case, scale)[0]
+    out, _, v_after, _, scales_after = run_gpu(et, device, case, scale)
     for b in (0, 31):
-        rows = [case["table"][b, p // 16] * 16 + p % 16 for p in range(contexts[b])]
-        values = np.concatenate([case["v_slab"][rows].astype(np.float64),
-                                 case["v"][b].astype(dtype).astype(np.float64).transpose(1, 0, 2)])
+        rows = [case["table"][b, p // 16] * 16 + p % 16 for p in range(contexts[b] + 1)]  # with the new row
+        if dtype == "u8":
+            values = (v_after[rows].astype(np.float64) - 128) * scales_after[1][rows][..., None].astype(np.float64)
+        else:
+            values = v_after[rows].astype(np.float64)
         mean = values.mean(axis=0)  # [kv_heads, width]
         assert np.abs(out[b, :, 0] - np.repeat(mean, 4, axis=0)).max() <= OUT_TOL

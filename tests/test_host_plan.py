@@ -209,8 +209,10 @@ def test_kv_attention_validation_follows_the_reference(et):
     flag.cancel()
     with pytest.raises(et.Cancelled, match="operation aborted"):
         et.kv_attention_into(layer, q, kv, kv, 1.0, None, out, cancelled=flag, stream=0)
-    with pytest.raises(et.QuantizedError, match="slabs must be f32 or f16"):
-        _kv_layer(et, torch, dtype=torch.bfloat16)
+    with pytest.raises(et.QuantizedError, match=r"kv pool: dtype must be f32, f16, bf16 or u8 \(int8-quantized\)"):
+        _kv_layer(et, torch, dtype=torch.float64)
+    with pytest.raises(et.QuantizedError, match="the u8 tier needs contiguous f32 scales"):
+        _kv_layer(et, torch, dtype=torch.uint8)
 
 
 def test_kv_attention_launch_shapes_and_status_wording(et):

@@ -163,3 +163,80 @@ def test_adding_one_vector_to_every_key_changes_nothing():
                                         v_rows[ctx].reshape(1, 2, 1, width), 0.7))
     assert np.allclose(outs[0], outs[1], rtol=0, atol=2e-6)
     assert not np.array_equal(outs[0], np.zeros_like(outs[0]))
+
+
+def test_f32_to_bf16_matches_torch_rounding():
+    import torch
+    rng = np.random.default_rng(1)
+    bits = rng.integers(0, 2**32, 30000, dtype=np.uint64).astype(np.uint32)
+    edge = np.array([0, 0x80000000, 0x7f800000, 0xff800000, 0x7fc00000, 0x7f800001, 0x3f808000, 0x3f818000,
+                     0x3f808001, 0x3f807fff, 0x7f7fffff, 0x7f7f8000, 0x00008000, 0x00018000, 0x00000001], np.uint32)
+    bits = np.concatenate([bits, edge])
+    values = bits.view(np.float32)
+    want = torch.from_numpy(values.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([oracle.f32_to_bf16_bits(x) for x in values], np.uint16)
+    nan = np.isnan(values)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all((got[nan] & 0x7f80) == 0x7f80) and np.all((got[nan] & 0x007f) != 0)
+    assert np.array_equal(got[nan] & 0x8000, (bits[nan] >> 16).astype(np.uint16) & 0x8000)
+
+
+def _pool_case(rng, dtype):
+    """One slot with 9 cached positions and 2 arriving ones, 2 kv heads of width 8, blocks of 4."""
+    heads, kv_heads, width, block, cached, new = 4, 2, 8, 4, 9, 2
+    q = rng.standard_normal((1, heads, new, width)).astype(np.float32)
+    k = rng.standard_normal((1, kv_heads, cached + new, width)).astype(np.float32)
+    v = rng.standard_normal((1, kv_heads, cached + new, width)).astype(np.float32)
+    table = np.array([[2, 0, 1]])
+    slabs = [np.zeros((12, kv_heads, width), dtype) for _ in range(2)]
+    scales = [np.zeros((12, kv_heads), np.float32) for _ in range(2)] if dtype == np.uint8 else [None, None]
+    # fill the cache through the oracle itself: one call that appends the first nine positions
+    oracle.kv_attention(slabs[0], slabs[1], block, table, [0], [cached], np.zeros((1, heads, cached, width), np.float32),
+                        k[:, :, :cached], v[:, :, :cached], 1.0, k_scales=scales[0], v_scales=scales[1])
+    out = oracle.kv_attention(slabs[0], slabs[1], block, table, [cached], [new], q, k[:, :, cached:], v[:, :, cached:],
+                              0.35, k_scales=scales[0], v_scales=scales[1])
+    return q, k, v, slabs, scales, out, table
+
+
+def test_reduced_precision_pools_track_the_f32_pool():
+    # the reference tests these tiers through a whole model (Inference.test.ts:509-550); here the
+    # attention over a bf16 / u8 pool is held against the f32 pool on the same inputs
+    outputs = {}
+    for dtype in (np.float32, np.float16, np.uint16, np.uint8):
+        outputs[np.dtype(dtype).name] = _pool_case(np.random.default_rng(5), dtype)[5]
+    assert np.abs(outputs["float16"] - outputs["float32"]).max() < 2e-3
+    assert np.abs(outputs["uint16"] - outputs["float32"]).max() < 2e-2   # bf16: 8 bits of mantissa
+    assert np.abs(outputs["uint8"] - outputs["float32"]).max() < 3e-2    # 127 steps per row
+    assert np.abs(outputs["uint8"] - outputs["float32"]).max() > 1e-5    # and it is not the f32 path
+
+
+def test_u8_tier_rows_scales_and_rounding():
+    rng = np.random.default_rng(6)
+    q, k, v, slabs, scales, out, table = _pool_case(rng, np.uint8)
+    block = 4
+    for slab, scale, source in ((slabs[0], scales[0], k), (slabs[1], scales[1], v)):
+        for position in range(11):
+            row = table[0, position // block] * block + position % block
+            for head in range(2):
+                x = source[0, head, position]
+                want_scale = np.float32(np.abs(x).max()) / np.float32(127.0) + np.float32(1e-12)
+                assert scale[row, head] == want_scale
+                ratio = (x / want_scale).astype(np.float32)
+                rounded = np.where(ratio >= 0, np.floor(ratio + np.float32(0.5)), np.ceil(ratio - np.float32(0.5)))
+                assert np.array_equal(slab[row, head], (np.clip(rounded, -127, 127) + 128).astype(np.uint8))
+                # dequantised values are within half a step of the input
+                back = (slab[row, head].astype(np.float32) - 128) * scale[row, head]
+                assert np.abs(back - x).max() <= 0.5 * scale[row, head] * (1 + 1e-6)
+    # a row of equal magnitudes stores +-127; halves round away from zero
+    slab = [np.zeros((4, 1, 4), np.uint8) for _ in range(2)]
+    scale = [np.zeros((4, 1), np.float32) for _ in range(2)]
+    row = np.array([[[[3.0, -3.0, 3.0, -3.0]]]], np.float32)
+    half = np.array([[[[127.0, 0.5, -0.5, 1.5]]]], np.float32)  # scale 1 + 1e-12 rounds to 1
+    oracle.kv_attention(slab[0], slab[1], 4, np.array([[0]]), [0], [1], np.zeros((1, 1, 1, 4), np.float32), row, half, 1.0,
+                        k_scales=scale[0], v_scales=scale[1])
+    assert slab[0][0, 0].tolist() == [255, 1, 255, 1] and scale[0][0, 0] == np.float32(3.0) / np.float32(127.0) + np.float32(1e-12)
+    assert slab[1][0, 0].tolist() == [255, 129, 127, 130]
+    # the attention output over one position is that dequantised value row
+    got = oracle.kv_attention(slab[0], slab[1], 4, np.array([[0]]), [1], [1], np.ones((1, 1, 1, 4), np.float32),
+                              row, half, 1.0, k_scales=scale[0], v_scales=scale[1], window=1)
+    assert np.allclose(got[0, 0, 0], (slab[1][1, 0].astype(np.float32) - 128) * scale[1][1, 0], rtol=1e-6)
