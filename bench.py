@@ -50,6 +50,9 @@ def parse_args():
                    help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
+    p.add_argument("--kv-dtype", choices=["f16", "bf16", "u8", "f32"], default="f16",
+                   help="kv_attention_decode / llama3_8b_batched_decode: element type of the key/value slabs "
+                        "(u8 = the int8-quantized tier with one f32 scale per row and head)")
     p.add_argument("--codec", default="q4_k", help="quantized_embedding_vocab: the table's codec (q2_k ... q6_k, q4_0, q8_0)")
     p.add_argument("--context", type=int, default=2048, help="kv_attention_decode / llama3_8b_batched_decode: "
                    "positions per slot")
@@ -171,6 +174,25 @@ def calibrate(args, et):
     }))
 
 
+def make_kv_slabs(torch, kv_dtype, max_tokens, kv_heads, width, device):
+    """Random key / value slabs of the given tier: (k_slab, v_slab, k_scales, v_scales, bytes per cached row of a head)."""
+    if kv_dtype == "u8":
+        slabs = [torch.randint(1, 256, (max_tokens, kv_heads, width), device=device, dtype=torch.uint8) for _ in range(2)]
+        scales = [torch.rand(max_tokens, kv_heads, device=device) * 0.02 + 0.005 for _ in range(2)]
+        return slabs[0], slabs[1], scales[0], scales[1], width + 4
+    dtype = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[kv_dtype]
+    slabs = [torch.randn(max_tokens, kv_heads, width, device=device, dtype=dtype) for _ in range(2)]
+    return slabs[0], slabs[1], None, None, width * slabs[0].element_size()
+
+
+def kv_slabs_to_host(np, torch, layer):
+    """numpy views of a layer's slabs for the oracle (bfloat16 as its bits)."""
+    def host(t):
+        return t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype == torch.bfloat16 else t.cpu().numpy()
+    scales = [t.cpu().numpy() if t is not None else None for t in (layer.k_scales, layer.v_scales)]
+    return host(layer.k_slab), host(layer.v_slab), scales[0], scales[1]
+
+
 def kv_decode(args, et):
     """Workload ``kv_attention_decode``: one decode step of paged key/value-cache attention for a
     Llama-3-8B-shaped layer - 32 slots, 32 query heads over 8 kv heads of width 128, f16 slabs in
@@ -201,9 +223,10 @@ def kv_decode(args, et):
     q, k, v = (torch.from_numpy(a).to(device) for a in (q_host, k_host, v_host))
     states = []
     for _ in range(layers):
-        k_slab = torch.randn(max_tokens, kv_heads, width, device=device, dtype=torch.float16)
-        v_slab = torch.randn(max_tokens, kv_heads, width, device=device, dtype=torch.float16)
-        states.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context))
+        k_slab, v_slab, k_scales, v_scales, row_bytes = make_kv_slabs(torch, args.kv_dtype, max_tokens, kv_heads,
+                                                                      width, device)
+        states.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context, k_scales=k_scales,
+                                 v_scales=v_scales))
     out = torch.empty_like(q)
     workspace = et.kv_attention_workspace(states[0], query_heads, 1)
     statuses = []
@@ -220,27 +243,27 @@ def kv_decode(args, et):
     torch.cuda.synchronize()
     et.kv_attention_status_check(states[0], 1, statuses[-1])
     check = 2
-    k_ref, v_ref = states[0].k_slab.cpu().numpy(), states[0].v_slab.cpu().numpy()
+    k_ref, v_ref, ks_ref, vs_ref = kv_slabs_to_host(np, torch, states[0])
     want = oracle.kv_attention(k_ref, v_ref, block, table_host[:check].view(np.uint32),
                                cursors_host[:check].view(np.uint32), advances_host[:check].view(np.uint32),
-                               q_host[:check], k_host[:check], v_host[:check], scale)
+                               q_host[:check], k_host[:check], v_host[:check], scale, k_scales=ks_ref, v_scales=vs_ref)
     err = float(np.abs(out.cpu().numpy()[:check] - want).max())
     assert err <= 1e-4, f"parity gate failed: max |err| {err:.4g}"
 
     ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
     seconds = ms * 1e-3
-    slab_bytes = 2 * slots * context * kv_heads * width * 2           # K and V rows read
-    small = 4 * (2 * q.numel() + 2 * k.numel()) + 2 * 2 * k.numel()  # q, out, new k / v in, new rows out
+    slab_bytes = 2 * slots * context * kv_heads * row_bytes         # K and V rows (and scales) read
+    small = 4 * (2 * q.numel() + 2 * k.numel()) + 2 * slots * kv_heads * row_bytes  # q, out, new k / v in, new rows out
     algorithmic = slab_bytes + small
     gbs = algorithmic / seconds / 1e9
     tokens_per_s = slots / seconds
     result = {
         "metric": "kv_attention_decode GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f16 slabs, f32 arithmetic", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": f"{args.kv_dtype} slabs, f32 arithmetic", "data": "synthetic",
         "config": {
             "workload": f"kv_attention_decode: {slots} slots x {query_heads} query heads / {kv_heads} kv heads x "
-                        f"width {width}, context {context}, f16 slabs, block {block}",
+                        f"width {width}, context {context}, {args.kv_dtype} slabs, block {block}",
             "slabs": "hot: one layer" if args.hot else f"cold: alternating over {layers} layers "
                                                        f"({layers * slab_bytes >> 20} MiB)",
             "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues",
@@ -250,7 +273,7 @@ def kv_decode(args, et):
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(("kv_attention_decode", context)),
+                     "traffic": MEASURED_TRAFFIC.get(("kv_attention_decode", context)) if args.kv_dtype == "f16" else None,
                      "kernel": et.kv_attention_kernel(states[0], query_heads, 1),
                      "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
     }
@@ -260,7 +283,8 @@ def kv_decode(args, et):
         while time.perf_counter() - t0 < args.cpu_seconds or calls == 0:
             oracle.kv_attention(k_ref, v_ref, block, table_host[:sample].view(np.uint32),
                                 cursors_host[:sample].view(np.uint32), advances_host[:sample].view(np.uint32),
-                                q_host[:sample], k_host[:sample], v_host[:sample], scale)
+                                q_host[:sample], k_host[:sample], v_host[:sample], scale, k_scales=ks_ref,
+                                v_scales=vs_ref)
             calls += 1
         elapsed = time.perf_counter() - t0
         per_step = elapsed / calls * (slots / sample)
@@ -514,9 +538,12 @@ def llama_decode(args, et):
     cursors_host = np.full(slots, context - 1, dtype=np.int32)
     advances_host = np.ones(slots, dtype=np.int32)
     table, cursors, advances = (torch.from_numpy(a).to(device) for a in (table_host, cursors_host, advances_host))
-    kv = [et.KvLayer(torch.randn(total_blocks * block, kv_heads, width, device=device, dtype=torch.float16),
-                     torch.randn(total_blocks * block, kv_heads, width, device=device, dtype=torch.float16),
-                     block, table, cursors, advances, context) for _ in range(layers)]
+    kv = []
+    for _ in range(layers):
+        k_slab, v_slab, k_scales, v_scales, kv_row_bytes = make_kv_slabs(torch, args.kv_dtype, total_blocks * block,
+                                                                         kv_heads, width, device)
+        kv.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context, k_scales=k_scales,
+                             v_scales=v_scales))
     kv_ws = et.kv_attention_workspace(kv[0], heads, 1)
     greedy_ws = torch.empty(et.greedy_workspace_bytes(slots, vocab), dtype=torch.uint8, device=device)
     embedding = torch.randn(vocab, hidden, device=device)
@@ -631,9 +658,11 @@ def llama_decode(args, et):
     k_ref = oracle.rotary(lin("wk", hh).reshape(2, kv_heads, 1, width), cursors_host[:2], 500000.0)
     v_ref = lin("wv", hh).reshape(2, kv_heads, 1, width)
     # the slabs already hold the rows this very step appended; the oracle writes the same values again
-    att = oracle.kv_attention(kv[0].k_slab.cpu().numpy(), kv[0].v_slab.cpu().numpy(), block,
+    slabs_host = kv_slabs_to_host(np, torch, kv[0])
+    att = oracle.kv_attention(slabs_host[0], slabs_host[1], block,
                               table_host[:2].view(np.uint32), cursors_host[:2].view(np.uint32),
-                              advances_host[:2].view(np.uint32), q_ref, k_ref, v_ref, scale)
+                              advances_host[:2].view(np.uint32), q_ref, k_ref, v_ref, scale, k_scales=slabs_host[2],
+                              v_scales=slabs_host[3])
     x1 = oracle.add(x0, lin("wo", att.reshape(2, hidden)))
     hh = oracle.rms_norm(x1, norms_host[0][1], 1e-5)
     want = oracle.add(x1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
@@ -661,7 +690,7 @@ def llama_decode(args, et):
     et.greedy_status_check(keep[-1])
     seconds = ms * 1e-3
     weight_bytes = layers * sum(host[n].size for n in shapes if n != "head") + host["head"].size
-    kv_bytes = layers * 2 * slots * context * kv_heads * width * 2
+    kv_bytes = layers * 2 * slots * context * kv_heads * kv_row_bytes
     algorithmic = weight_bytes + kv_bytes + slots * vocab * 4 * 2
     gbs = algorithmic / seconds / 1e9
     result = {
@@ -669,7 +698,7 @@ def llama_decode(args, et):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "int8" if args.mode == "int8" else "f32", "data": "synthetic",
         "config": {"workload": f"llama3_8b_batched_decode: {layers} layers, hidden {hidden}, {heads}/{kv_heads} heads x {width}, "
-                               f"ffn {ffn}, vocab {vocab}; Q4_K weights, f16 kv slabs in blocks of {block}; {slots} slots at "
+                               f"ffn {ffn}, vocab {vocab}; Q4_K weights, {args.kv_dtype} kv slabs in blocks of {block}; {slots} slots at "
                                f"context {context}; {'int8' if args.mode == 'int8' else 'f32'} activations",
                    "launch": "one HIP graph of the whole step, replayed K times",
                    "operators": "one quantisation per distinct input, residual sums in the contraction epilogues"
@@ -688,9 +717,10 @@ def llama_decode(args, et):
         q1 = oracle.rotary(lin("wq", hh).reshape(1, heads, 1, width), cursors_host[:1], 500000.0)
         k1 = oracle.rotary(lin("wk", hh).reshape(1, kv_heads, 1, width), cursors_host[:1], 500000.0)
         v1 = lin("wv", hh).reshape(1, kv_heads, 1, width)
-        a1 = oracle.kv_attention(kv[0].k_slab.cpu().numpy(), kv[0].v_slab.cpu().numpy(), block,
+        a1 = oracle.kv_attention(slabs_host[0], slabs_host[1], block,
                                  table_host[:1].view(np.uint32), cursors_host[:1].view(np.uint32),
-                                 advances_host[:1].view(np.uint32), q1, k1, v1, scale)
+                                 advances_host[:1].view(np.uint32), q1, k1, v1, scale, k_scales=slabs_host[2],
+                                 v_scales=slabs_host[3])
         y1 = oracle.add(one, lin("wo", a1.reshape(1, hidden)))
         hh = oracle.rms_norm(y1, norms_host[0][1], 1e-5)
         oracle.add(y1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))

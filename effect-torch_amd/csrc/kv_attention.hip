@@ -210,6 +210,7 @@ struct Piece<float> {
     static constexpr int kDims = 4;
     static constexpr int kElementBytes = 4;
     static constexpr bool kScaled = false;
+    using Raw = uint4;
     uint4 raw;
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = i == 0 ? raw.x : i == 1 ? raw.y : i == 2 ? raw.z : raw.w;
@@ -226,6 +227,7 @@ struct Piece<__half> {
     static constexpr int kDims = 8;
     static constexpr int kElementBytes = 2;
     static constexpr bool kScaled = false;
+    using Raw = uint4;
     uint4 raw;
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = (i >> 1) == 0 ? raw.x : (i >> 1) == 1 ? raw.y : (i >> 1) == 2 ? raw.z : raw.w;
@@ -247,6 +249,7 @@ struct Piece<Bf16> {
     static constexpr int kDims = 8;
     static constexpr int kElementBytes = 2;
     static constexpr bool kScaled = false;
+    using Raw = uint4;
     uint4 raw;
     __device__ __forceinline__ float get(int i) const {
         const uint32_t w = (i >> 1) == 0 ? raw.x : (i >> 1) == 1 ? raw.y : (i >> 1) == 2 ? raw.z : raw.w;
@@ -260,39 +263,36 @@ struct Piece<Bf16> {
         raw = make_uint4(pack(low.x, low.y), pack(low.z, low.w), pack(high.x, high.y), pack(high.z, high.w));
     }
 };
+// The u8 tier takes eight bytes per lane, not sixteen: a head of width 128 then spans sixteen lanes,
+// the shape the reduce-scatter softmax (attend_step_scatter) is built for.
 template <>
 struct Piece<U8> {
-    static constexpr int kDims = 16;
+    static constexpr int kDims = 8;
     static constexpr int kElementBytes = 1;
     static constexpr bool kScaled = true;
-    uint4 raw;
+    using Raw = uint2;
+    uint2 raw;
     float scale;  // of the row and head these bytes belong to
     __device__ __forceinline__ float get(int i) const {
-        const uint32_t w = (i >> 2) == 0 ? raw.x : (i >> 2) == 1 ? raw.y : (i >> 2) == 2 ? raw.z : raw.w;
+        const uint32_t w = (i >> 2) == 0 ? raw.x : raw.y;
         // (byte - 128) * scale, one rounding: -128 * scale is exact
         return fmaf(static_cast<float>((w >> (8 * (i & 3))) & 0xffu), scale, -128.0f * scale);
     }
     template <int LANES>
     __device__ __forceinline__ void from_input(const float* source) {
-        float values[16];
+        const float4 low = *reinterpret_cast<const float4*>(source);
+        const float4 high = *reinterpret_cast<const float4*>(source + 4);
+        const float values[8] = {low.x, low.y, low.z, low.w, high.x, high.y, high.z, high.w};
         float maximum = 0.f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float4 v = *reinterpret_cast<const float4*>(source + 4 * j);
-            values[4 * j] = v.x;
-            values[4 * j + 1] = v.y;
-            values[4 * j + 2] = v.z;
-            values[4 * j + 3] = v.w;
-        }
-#pragma unroll
-        for (int i = 0; i < 16; i++) maximum = fmaxf(maximum, fabsf(values[i]));
+        for (int i = 0; i < 8; i++) maximum = fmaxf(maximum, fabsf(values[i]));
         scale = u8_scale(group_max<LANES>(maximum));
-        uint32_t words[4];
+        uint32_t words[2];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < 2; j++)
             words[j] = u8_byte(values[4 * j], scale) | (u8_byte(values[4 * j + 1], scale) << 8) |
                        (u8_byte(values[4 * j + 2], scale) << 16) | (u8_byte(values[4 * j + 3], scale) << 24);
-        raw = make_uint4(words[0], words[1], words[2], words[3]);
+        raw = make_uint2(words[0], words[1]);
     }
 };
 
@@ -551,8 +551,8 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
             for (int u = 0; u < U; u++) {
                 // positions past the end read the last cached row again and are masked out below
                 const uint32_t row = row_of(min(step_begin + u * PPG + group, cached_end - 1));
-                kp[u].raw = *reinterpret_cast<const uint4*>(k_base + row * row_bytes);
-                vp[u].raw = *reinterpret_cast<const uint4*>(v_base + row * row_bytes);
+                kp[u].raw = *reinterpret_cast<const typename Piece<T>::Raw*>(k_base + row * row_bytes);
+                vp[u].raw = *reinterpret_cast<const typename Piece<T>::Raw*>(v_base + row * row_bytes);
                 if constexpr (Piece<T>::kScaled) {
                     kp[u].scale = a.k_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head];
                     vp[u].scale = a.v_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head];
@@ -596,8 +596,8 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
             const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
             const uint32_t row = base + within_block(a, position);
             if (base != kNoBlock && row < a.max_tokens) {
-                *reinterpret_cast<uint4*>(k_base + row * row_bytes) = kp[0].raw;
-                *reinterpret_cast<uint4*>(v_base + row * row_bytes) = vp[0].raw;
+                *reinterpret_cast<typename Piece<T>::Raw*>(k_base + row * row_bytes) = kp[0].raw;
+                *reinterpret_cast<typename Piece<T>::Raw*>(v_base + row * row_bytes) = vp[0].raw;
                 if constexpr (Piece<T>::kScaled) {
                     if (sub == 0) {
                         a.k_scales[static_cast<uint64_t>(row) * a.kv_heads + kv_head] = kp[0].scale;
@@ -805,15 +805,8 @@ __global__ void kv_merge_kernel(const KvArgs a) {
 template <typename T, int LPT, int G>
 hipError_t launch_streaming(const KvArgs& a, uint32_t workgroups, int waves, hipStream_t stream) {
     constexpr int U = G >= 8 ? 2 : 4;
-    // (kv_attention_shape never asks for eight waves of the u8 tier with groups of eight heads: the
-    // merge area of 16-value pieces would not fit LDS)
-    if constexpr (!(std::is_same<T, U8>::value && G >= 8)) {
-        if (waves == 8) {
-            hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
-            return hipGetLastError();
-        }
-    }
-    if (waves == 8) return hipErrorInvalidValue;
+    if (waves == 8)
+        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
     else
         hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4>), dim3(workgroups), dim3(256), 0, stream, a);
     return hipGetLastError();
@@ -839,10 +832,8 @@ hipError_t launch_streaming_width(const KvArgs& a, int g, uint32_t workgroups, i
 }
 
 // Query heads of one kv head served together by the streaming kernel; 0 = not covered.
-// Elements of a slab row in sixteen bytes.
-uint32_t piece_dims(const KvAttention& p) {
-    return p.slab_dtype == ET_DTYPE_F32 ? 4 : p.slab_dtype == ET_DTYPE_U8 ? 16 : 8;
-}
+// Elements of a slab row one lane takes (sixteen bytes; eight for the u8 tier).
+uint32_t piece_dims(const KvAttention& p) { return p.slab_dtype == ET_DTYPE_F32 ? 4 : 8; }
 
 int streaming_group(const KvAttention& p) {
     const uint32_t dims = piece_dims(p);
@@ -876,7 +867,7 @@ KvLaunchShape kv_attention_shape(const KvAttention& p) {
     // slots x 8 kv heads at context 2048: 512 x 4 waves 58.9 us, 1024 x 4 waves 63.7, 256 x 8 waves
     // without any split - no partial records, no merge launch - 55.6). Eight waves need enough rows
     // of queries to go round without splitting.
-    shape.waves = shape.streaming && rows >= 128 && !(p.slab_dtype == ET_DTYPE_U8 && g >= 8) ? 8 : 4;
+    shape.waves = shape.streaming && rows >= 128 ? 8 : 4;
     const uint64_t step = shape.streaming ? positions_per_step(p, g, shape.waves) : 64;
     uint64_t splits = 1;
     const uint64_t wanted = shape.streaming ? (shape.waves == 8 ? 256 : 512) : 4096;
