@@ -71,20 +71,27 @@ constexpr int vmcnt_only(int n) {
 // A row's share of a stage, as it lies in memory: a Q4_K super-block is d, dmin, scales[12], qs[128];
 // a Q5_K one d, dmin, scales[12], qh[32] (the fifth bits: bit g of qh[c] belongs to column c of
 // sub-block g), qs[128] (crates/runtime-cpu/src/quantized.rs:180-234).
-// A Q6_K super-block is ql[128], qh[64], sixteen int8 scales (one per 16 columns), d: 210 bytes, so
-// the stages of a row start on 2-byte boundaries. Its LDS row is 224 bytes: chunks 0..12 are bytes
-// 0..207 of the stage, chunk 13 is bytes 194..209 (d at offset 222) so that no copy reads past the
-// stage (crates/runtime-cpu/src/quantized.rs:238-261).
+// Super-blocks whose size is not a multiple of sixteen (Q6_K: 210 bytes = ql[128], qh[64], sixteen int8
+// scales, d; Q3_K: 110 = hmask[32], qs[64], scales[12], d; Q2_K: 84 = scales[16], qs[64], d, dmin;
+// crates/runtime-cpu/src/quantized.rs:117-176, 238-261) get an LDS row of the next multiple: every
+// 16-byte chunk holds the stage's bytes at the same offset except the last one, which is taken from the
+// stage's last sixteen bytes - so no copy reads past the stage (or the weight buffer). Q3_K and Q6_K
+// stages start on 2-byte boundaries; global_load_lds takes such sources, more slowly.
 template <int CODEC>
 struct Codec {
-    static_assert(CODEC == kQ4_K || CODEC == kQ5_K || CODEC == kQ6_K, "the K-quants with a half-float form");
-    static constexpr uint32_t kStageBytes = CODEC == kQ6_K ? 210u : CODEC == kQ5_K ? 176u : 144u;  // in memory
-    static constexpr uint32_t kRowBytes = CODEC == kQ6_K ? 224u : kStageBytes;                     // in LDS
-    static constexpr uint32_t kQuantsAt = CODEC == kQ5_K ? 48u : 16u;
+    static_assert(CODEC == kQ2_K || CODEC == kQ3_K || CODEC == kQ4_K || CODEC == kQ5_K || CODEC == kQ6_K,
+                  "the K-quants");
+    static constexpr uint32_t kStageBytes = block_bytes(CODEC);            // in memory
+    static constexpr uint32_t kRowBytes = (kStageBytes + 15u) / 16u * 16u;  // in LDS
+    static constexpr uint32_t kQuantsAt = CODEC == kQ5_K ? 48u : 16u;       // Q4_K / Q5_K
+    // where the stage's last sixteen bytes lie in the LDS row: d (and dmin) are read from there
+    static constexpr uint32_t kTailAt = kRowBytes - 16u, kTailFrom = kStageBytes - 16u;
     // byte of the stage that LDS byte `within` (a multiple of 16) of the row holds
     static __device__ __forceinline__ uint32_t source_of(uint32_t within) {
-        return CODEC == kQ6_K && within == 208u ? 194u : within;
+        return kRowBytes != kStageBytes && within == kTailAt ? kTailFrom : within;
     }
+    // LDS offset of stage byte `at` of the tail
+    static constexpr uint32_t in_tail(uint32_t at) { return kTailAt + (at - kTailFrom); }
 };
 
 template <int CODEC, int RG, int AX, int AW>
@@ -142,6 +149,29 @@ struct Group {
     uint32_t count;
     uint32_t row_tiles;  // of all members together
 };
+
+// Eight bytes as eight half floats, (n - OFFSET) * scale in two exact steps (for offsets whose product
+// with the scale a half float does not hold: 1028 * 31).
+template <int OFFSET>
+__device__ __forceinline__ v8h bytes_minus_times(uint32_t first, uint32_t second, v2h scale) {
+#pragma clang fp contract(off)
+    const v2h offset = {static_cast<_Float16>(1024.0f + OFFSET), static_cast<_Float16>(1024.0f + OFFSET)};
+    union {
+        uint32_t word[4];
+        v2h pair[4];
+        v8h all;
+    } u;
+    u.word[0] = __builtin_amdgcn_perm(0x64646464u, first, 0x04010400u);
+    u.word[1] = __builtin_amdgcn_perm(0x64646464u, first, 0x04030402u);
+    u.word[2] = __builtin_amdgcn_perm(0x64646464u, second, 0x04010400u);
+    u.word[3] = __builtin_amdgcn_perm(0x64646464u, second, 0x04030402u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const v2h centred = u.pair[i] - offset;
+        u.pair[i] = centred * scale;
+    }
+    return u.all;
+}
 
 template <int CODEC, int RG, int AX, int AW>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
@@ -256,12 +286,95 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const uint32_t b_base = wave_k * NB;
         const uint8_t* row_in_slot = region + (wave_n * 32u + in_half) * kRowBytes;  // this lane's weight row
 
+        if constexpr (CODEC == kQ3_K) {
+            // value = d * (sc - 32) * (v - 4), v = two bits of qs | the hmask bit << 2, a 6-bit scale per 16
+            // columns; |(sc - 32) * (v - 4)| <= 128 is exact in a half float. No minimum term.
+            const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + Codec<CODEC>::in_tail(108u)));
+            const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
+            const uint4 hm = *reinterpret_cast<const uint4*>(row_in_slot + 16u * half);  // hmask of these columns
+            v16f p_lo = zero, p_hi = zero;
+#pragma unroll
+            for (int bb = 0; bb < NB; bb++) {
+                const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
+                const uint4 qs = *reinterpret_cast<const uint4*>(row_in_slot + 32u + 32u * n + 16u * half);
+                // scale of group 8 n + 2 t + half: nibble n of packed[2 t + half], top bits from packed[8 + ..]
+                const uint32_t low_byte = row_in_slot[Codec<CODEC>::in_tail(96u) + 2u * t + half];
+                const uint32_t high_byte = row_in_slot[Codec<CODEC>::in_tail(104u) + 2u * (t & 1u) + half];
+                const int sc = static_cast<int>(((low_byte >> (4u * n)) & 15u) |
+                                                (((high_byte >> (2u * (2u * n + (t >> 1)))) & 3u) << 4)) - 32;
+                const uint32_t bit = 4u * n + t;
+                const uint32_t w0 = ((qs.x >> (2u * t)) & 0x03030303u) | (((hm.x >> bit) & 0x01010101u) << 2),
+                               w1 = ((qs.y >> (2u * t)) & 0x03030303u) | (((hm.y >> bit) & 0x01010101u) << 2),
+                               w2 = ((qs.z >> (2u * t)) & 0x03030303u) | (((hm.z >> bit) & 0x01010101u) << 2),
+                               w3 = ((qs.w >> (2u * t)) & 0x03030303u) | (((hm.w >> bit) & 0x01010101u) << 2);
+                const _Float16 sc_h = static_cast<_Float16>(static_cast<float>(sc));
+                const v2h sc2 = {sc_h, sc_h};
+                const v8h b0 = bytes_minus_times<4>(w0, w1, sc2), b1 = bytes_minus_times<4>(w2, w3, sc2);
+                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
+                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
+                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
+                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
+                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
+                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
+                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
+                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
+            }
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+                                                                 zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
+            continue;
+        }
+        if constexpr (CODEC == kQ2_K) {
+            // value = d * sc * v - dmin * mn with a 4-bit scale and minimum per 16 columns. The minima ride
+            // on the matrix cores too: a weight operand that is mn in all sixteen columns sums the
+            // activations of the run times mn (acc_min is then the second pair of accumulators).
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(row_in_slot + Codec<CODEC>::in_tail(80u));
+            const float d_block = half_bits_to_float(dd & 0xffffu), dmin_block = half_bits_to_float(dd >> 16);
+            const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
+            v16f p_lo = zero, p_hi = zero, m_lo = zero, m_hi = zero;
+#pragma unroll
+            for (int bb = 0; bb < NB; bb++) {
+                const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
+                const uint4 qs = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 32u * n + 16u * half);
+                const uint32_t both = row_in_slot[2u * b + half];  // scales[8 n + 2 t + half]
+                const uint32_t w0 = (qs.x >> (2u * t)) & 0x03030303u, w1 = (qs.y >> (2u * t)) & 0x03030303u,
+                               w2 = (qs.z >> (2u * t)) & 0x03030303u, w3 = (qs.w >> (2u * t)) & 0x03030303u;
+                const _Float16 sc_h = static_cast<_Float16>(static_cast<float>(both & 15u));
+                const _Float16 mn_h = static_cast<_Float16>(static_cast<float>(both >> 4));
+                const v2h sc2 = {sc_h, sc_h};
+                const v8h b0 = nibbles_times(w0, w1, sc2), b1 = nibbles_times(w2, w3, sc2);
+                const v8h bm = {mn_h, mn_h, mn_h, mn_h, mn_h, mn_h, mn_h, mn_h};
+                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
+                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
+                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
+                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
+                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
+                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
+                m_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bm, m_lo, 0, 0, 0);
+                m_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bm, m_hi, 0, 0, 0);
+                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
+                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
+                m_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bm, m_lo, 0, 0, 0);
+                m_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bm, m_hi, 0, 0, 0);
+            }
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+                                                                 zero, 0, 0, 0);
+            const v16f sm = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? dmin_block : 0.f,
+                                                                 zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
+                acc_min[r] = fmaf(fmaf(4096.0f, m_hi[r], m_lo[r]), sm[r], acc_min[r]);
+            }
+            continue;
+        }
         if constexpr (CODEC == kQ6_K) {
             // value = d * sc * (q - 32) with an int8 scale per 16 columns: a lane half's sixteen columns
             // of a 32-column block are one such run. sc * (q - 32) reaches 4096, too wide for a half
             // float, so sc = 16 * s_hi + s_lo (s_lo 0..15, s_hi -8..7) and both parts are contracted:
             // four accumulators, (X_lo, X_hi) x (s_lo, s_hi), joined once per stage.
-            const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + 222u));
+            const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + Codec<CODEC>::in_tail(208u)));
             const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
             v16f p_ll = zero, p_lh = zero, p_hl = zero, p_hh = zero;  // activation half, scale part
 #pragma unroll
@@ -458,7 +571,8 @@ __global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, co
 }  // namespace
 
 bool gemm_h16_supported(int32_t codec, uint64_t columns) {
-    return (codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) && columns % 256 == 0 && columns > 0;
+    return (codec == kQ2_K || codec == kQ3_K || codec == kQ4_K || codec == kQ5_K || codec == kQ6_K) &&
+           columns % 256 == 0 && columns > 0;
 }
 
 GemmGroupGeometry gemm_h16_group_geometry(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
@@ -553,6 +667,16 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     // weight lead: what the activation ring (three slots of 34 KiB) leaves of LDS
     if (codec == kQ6_K)  // 64-row tiles only (gemm_h16_group_geometry): 128 rows of 224 bytes leave no room for a ring
         return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+    if (codec == kQ2_K || codec == kQ3_K) {  // rows of 96 / 112 bytes per stage: room for the longest lead
+        if (codec == kQ2_K) {
+            if (g.tile_rows == 128)
+                return launch_group<kQ2_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+            return launch_group<kQ2_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        }
+        if (g.tile_rows == 128)
+            return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+    }
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
             return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);

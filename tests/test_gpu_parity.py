@@ -208,12 +208,12 @@ def test_linear_matches_oracle(et, device, codec, rows, columns, vectors):
     close(got, exact, oracle_noise=0)
 
 
-@pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q5_K, oracle.Q6_K, oracle.Q8_0, oracle.Q4_0])
+@pytest.mark.parametrize("codec", [oracle.Q2_K, oracle.Q3_K, oracle.Q4_K, oracle.Q5_K, oracle.Q6_K, oracle.Q8_0, oracle.Q4_0])
 @pytest.mark.parametrize("vectors,rows,columns", [(7, 129, 256), (12, 64, 2304), (33, 1, 512), (65, 300, 1024),
                                                   (100, 130, 4096), (130, 257, 768), (200, 63, 256)])
 def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, rows, columns):
     # seven or more vectors: fixed-point activations on the matrix cores (two 12-bit halves as half
-    # floats for Q4_K, Q5_K and Q6_K, three byte limbs for the 32-wide codecs); ragged tiles on both sides, one and
+    # floats for the K-quants, three byte limbs for the 32-wide codecs); ragged tiles on both sides, one and
     # several stages of 256 columns, ring turns with padding stages
     rng = np.random.default_rng(codec * 11 + vectors + rows + columns)
     weight = synth.random_weight(codec, rows, columns, rng)
@@ -222,10 +222,11 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
     bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   None, et.GgmlQuant(codec), (rows, columns))
-    family = "quantize_halves+gemm_h16" if codec in (oracle.Q4_K, oracle.Q5_K, oracle.Q6_K) else "quantize_limbs+gemm_i8"
+    k_quants = (oracle.Q2_K, oracle.Q3_K, oracle.Q4_K, oracle.Q5_K, oracle.Q6_K)
+    family = "quantize_halves+gemm_h16" if codec in k_quants else "quantize_limbs+gemm_i8"
     assert plan.kernel in (family, family + "+reduce")
     got = run_linear(et, device, codec, rows, columns, x, weight, bias)
-    if codec not in (oracle.Q4_K, oracle.Q5_K, oracle.Q6_K):
+    if codec not in k_quants:
         # a width that is not a whole number of 256-column stages stays on the GEMV kernels
         odd = columns + 32
         weight_odd = synth.random_weight(codec, rows, odd, rng)
@@ -246,12 +247,14 @@ def test_linear_many_vectors_f32_matrix_core_tiles(et, device, codec, vectors, r
 @pytest.mark.parametrize("codec,vectors,rows,columns", [(oracle.Q4_K, 32, 1024, 4096), (oracle.Q4_K, 32, 4096, 4096),
                                                         (oracle.Q4_K, 32, 4096, 14336), (oracle.Q5_K, 32, 4096, 4096),
                                                         (oracle.Q5_K, 64, 14336, 4096), (oracle.Q6_K, 32, 1024, 4096),
-                                                        (oracle.Q6_K, 32, 4096, 14336), (oracle.Q8_0, 40, 700, 2304),
+                                                        (oracle.Q6_K, 32, 4096, 14336), (oracle.Q3_K, 32, 4096, 4096),
+                                                        (oracle.Q2_K, 64, 14336, 4096), (oracle.Q2_K, 32, 1024, 4096),
+                                                        (oracle.Q8_0, 40, 700, 2304),
                                                         (oracle.Q4_0, 9, 65, 1280)])
 def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vectors, rows, columns):
     # decode-batch shapes: far fewer 64-row tiles than compute units, so the stages of K are shared
     # out over several workgroups per tile and summed by a second kernel, in a fixed order
-    if codec in (oracle.Q5_K, oracle.Q6_K) and mode == "INT8":
+    if codec in (oracle.Q2_K, oracle.Q3_K, oracle.Q5_K, oracle.Q6_K) and mode == "INT8":
         pytest.skip("the int8-activation mode has no kernel for this codec")
     rng = np.random.default_rng(rows + columns + vectors)
     weight = synth.random_weight(codec, rows, columns, rng)
@@ -260,11 +263,11 @@ def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vecto
     act = et.ActivationMode[mode]
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   torch.zeros(rows), et.GgmlQuant(codec), (rows, columns), act)
-    if (codec, rows) == (oracle.Q5_K, 14336):
+    if rows == 14336:
         assert plan.kernel == "quantize_halves+gemm_h16"  # 128-row tiles fill the device: no K shares
     else:
-        assert plan.kernel.endswith("+gemm_h16+reduce" if mode == "F32" and codec in (oracle.Q4_K, oracle.Q5_K, oracle.Q6_K)
-                                    else "+gemm_i8+reduce")
+        assert plan.kernel.endswith("+gemm_i8+reduce" if mode == "INT8" or codec in (oracle.Q8_0, oracle.Q4_0)
+                                    else "+gemm_h16+reduce")
     got = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
     again = run_linear(et, device, codec, rows, columns, x, weight, bias, act)
     assert np.array_equal(got, again)  # the same bits on every run

@@ -54,8 +54,9 @@ def test_linear_plan_shapes(et):
     assert plan5.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce")
     plan6 = et.linear_requirements(torch.zeros(10, 512), _w(7, 420), None, et.GgmlQuant.Q6_K, (7, 512))
     assert plan6.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce")
-    plan3 = et.linear_requirements(torch.zeros(10, 512), _w(7, 220), None, et.GgmlQuant.Q3_K, (7, 512))
-    assert plan3.kernel == "gemv_limb"  # no batch kernel for Q2_K / Q3_K: repeated two-vector launches
+    for codec, row_bytes in ((et.GgmlQuant.Q3_K, 220), (et.GgmlQuant.Q2_K, 168)):
+        batch = et.linear_requirements(torch.zeros(10, 512), _w(7, row_bytes), None, codec, (7, 512))
+        assert batch.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce")
     plan8 = et.linear_requirements(torch.zeros(10, 512), _w(7, 544), None, et.GgmlQuant.Q8_0, (7, 512))
     assert plan8.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
     for few in (3, 6):
