@@ -28,21 +28,31 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
     return static_cast<float>(cvt.h);
 }
 
+// Little-endian loads at any address (blocks of 18, 34, 110 or 210 bytes are not dword aligned): one
+// instruction each instead of a load per byte.
+typedef uint16_t __attribute__((aligned(1))) Unaligned16;
+typedef uint32_t __attribute__((aligned(1))) Unaligned32;
+__device__ __forceinline__ uint32_t load16(const uint8_t* at) { return *reinterpret_cast<const Unaligned16*>(at); }
+__device__ __forceinline__ uint32_t load32(const uint8_t* at) { return *reinterpret_cast<const Unaligned32*>(at); }
+__device__ __forceinline__ uint32_t byte_of(uint32_t word, int i) { return (word >> (8 * i)) & 0xffu; }
+
 __device__ __forceinline__ float f16_at(const uint8_t* block, uint32_t offset) {
-    return f16_bits_to_f32(static_cast<uint32_t>(block[offset]) |
-                           (static_cast<uint32_t>(block[offset + 1]) << 8));
+    return f16_bits_to_f32(load16(block + offset));
 }
 
-// crates/runtime-cpu/src/quantized.rs:77-86
+// crates/runtime-cpu/src/quantized.rs:77-86; `scales` = the twelve packed bytes
 __device__ __forceinline__ void scale_min_k4(uint32_t index, const uint8_t* scales, uint32_t& scale,
                                              uint32_t& min) {
+    const uint32_t shift = 8u * (index & 3u);
+    const uint32_t s0 = (load32(scales) >> shift) & 0xffu;      // scales[index & 3]
+    const uint32_t s1 = (load32(scales + 4) >> shift) & 0xffu;  // scales[4 + (index & 3)]
     if (index < 4) {
-        scale = scales[index] & 63u;
-        min = scales[index + 4] & 63u;
+        scale = s0 & 63u;
+        min = s1 & 63u;
     } else {
-        scale = (scales[index + 4] & 0x0fu) | ((static_cast<uint32_t>(scales[index - 4]) >> 6) << 4);
-        min = (static_cast<uint32_t>(scales[index + 4]) >> 4) |
-              ((static_cast<uint32_t>(scales[index]) >> 6) << 4);
+        const uint32_t s2 = (load32(scales + 8) >> shift) & 0xffu;  // scales[8 + (index & 3)]
+        scale = (s2 & 0x0fu) | ((s0 >> 6) << 4);
+        min = (s2 >> 4) | ((s1 >> 6) << 4);
     }
 }
 
@@ -54,8 +64,9 @@ __device__ __forceinline__ void decode4(const uint8_t* block, uint32_t e, float 
 template <>
 __device__ __forceinline__ void decode4<kQ8_0>(const uint8_t* block, uint32_t e, float out[4]) {
     const float d = f16_at(block, 0);
+    const uint32_t q = load32(block + 2 + e);
 #pragma unroll
-    for (int i = 0; i < 4; i++) out[i] = d * static_cast<float>(static_cast<int8_t>(block[2 + e + i]));
+    for (int i = 0; i < 4; i++) out[i] = d * static_cast<float>(static_cast<int8_t>(byte_of(q, i)));
 }
 
 template <>
@@ -63,9 +74,10 @@ __device__ __forceinline__ void decode4<kQ4_0>(const uint8_t* block, uint32_t e,
     const float d = f16_at(block, 0);
     const bool high = e >= 16;
     const uint32_t j = high ? e - 16 : e;
+    const uint32_t q = load32(block + 2 + j);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t byte = block[2 + j + i];
+        const uint32_t byte = byte_of(q, i);
         const int nib = static_cast<int>(high ? (byte >> 4) : (byte & 0x0fu)) - 8;
         out[i] = d * static_cast<float>(nib);
     }
@@ -80,10 +92,10 @@ __device__ __forceinline__ void decode4<kQ2_K>(const uint8_t* block, uint32_t e,
     const float d = f16_at(block, 80), dmin = f16_at(block, 82);
     const float dl = d * static_cast<float>(scale & 0x0fu);
     const float ml = dmin * static_cast<float>(scale >> 4);
-    const uint8_t* q = block + 16 + half * 32 + q_offset + i0;
+    const uint32_t q = load32(block + 16 + half * 32 + q_offset + i0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const float prod = dl * static_cast<float>((static_cast<uint32_t>(q[i]) >> shift) & 3u);
+        const float prod = dl * static_cast<float>((byte_of(q, i) >> shift) & 3u);
         out[i] = prod - ml;
     }
 }
@@ -100,12 +112,12 @@ __device__ __forceinline__ void decode4<kQ3_K>(const uint8_t* block, uint32_t e,
     const int scale = static_cast<int>(low | (high << 4)) - 32;
     const float d = f16_at(block, 108);
     const float dl = d * static_cast<float>(scale);
-    const uint8_t* q = block + 32 + half * 32 + q_offset + i0;
-    const uint8_t* hm = block + q_offset + i0;
+    const uint32_t q = load32(block + 32 + half * 32 + q_offset + i0);
+    const uint32_t hm = load32(block + q_offset + i0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int low_quant = static_cast<int>((static_cast<uint32_t>(q[i]) >> shift) & 3u);
-        const int high_quant = (hm[i] & mask) == 0 ? 4 : 0;
+        const int low_quant = static_cast<int>((byte_of(q, i) >> shift) & 3u);
+        const int high_quant = (byte_of(hm, i) & mask) == 0 ? 4 : 0;
         out[i] = dl * static_cast<float>(low_quant - high_quant);
     }
 }
@@ -119,10 +131,10 @@ __device__ __forceinline__ void decode4<kQ4_K>(const uint8_t* block, uint32_t e,
     const float d = f16_at(block, 0), dmin = f16_at(block, 2);
     const float dl = d * static_cast<float>(scale);
     const float ml = dmin * static_cast<float>(min);
-    const uint8_t* q = block + 16 + pair * 32 + i0;
+    const uint32_t q = load32(block + 16 + pair * 32 + i0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t byte = q[i];
+        const uint32_t byte = byte_of(q, i);
         const uint32_t quant = side == 0 ? (byte & 0x0fu) : (byte >> 4);
         const float prod = dl * static_cast<float>(quant);
         out[i] = prod - ml;
@@ -138,14 +150,14 @@ __device__ __forceinline__ void decode4<kQ5_K>(const uint8_t* block, uint32_t e,
     const float d = f16_at(block, 0), dmin = f16_at(block, 2);
     const float dl = d * static_cast<float>(scale);
     const float ml = dmin * static_cast<float>(min);
-    const uint8_t* high = block + 16 + i0;
-    const uint8_t* ql = block + 48 + pair * 32 + i0;
+    const uint32_t high = load32(block + 16 + i0);
+    const uint32_t ql = load32(block + 48 + pair * 32 + i0);
     const uint32_t mask = 1u << group;  // 1 << (pair*2 + side)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t byte = ql[i];
+        const uint32_t byte = byte_of(ql, i);
         const uint32_t low_quant = side == 0 ? (byte & 0x0fu) : (byte >> 4);
-        const uint32_t quant = low_quant + ((high[i] & mask) == 0 ? 0u : 16u);
+        const uint32_t quant = low_quant + ((byte_of(high, i) & mask) == 0 ? 0u : 16u);
         const float prod = dl * static_cast<float>(quant);
         out[i] = prod - ml;
     }
@@ -155,18 +167,17 @@ template <>
 __device__ __forceinline__ void decode4<kQ6_K>(const uint8_t* block, uint32_t e, float out[4]) {
     // e = half*128 + quarter*32 + index
     const uint32_t half = e >> 7, quarter = (e >> 5) & 3u, i0 = e & 31u;
-    const uint8_t* ql = block + half * 64;
-    const uint8_t* qh = block + 128 + half * 32;
+    const uint32_t ql = load32(block + half * 64 + i0 + ((quarter & 1u) ? 32u : 0u));
+    const uint32_t qh = load32(block + 128 + half * 32 + i0);
     const uint32_t scale_index = half * 8u + (i0 >> 4) + quarter * 2u;
     const int scale = static_cast<int8_t>(block[192 + scale_index]);
     const float d = f16_at(block, 208);
     const float ds = d * static_cast<float>(scale);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t index = i0 + i;
-        const uint32_t lo = ql[index + ((quarter & 1u) ? 32u : 0u)];
+        const uint32_t lo = byte_of(ql, i);
         const uint32_t nib = (quarter & 2u) ? (lo >> 4) : (lo & 0x0fu);
-        const uint32_t hi2 = (static_cast<uint32_t>(qh[index]) >> (2u * quarter)) & 3u;
+        const uint32_t hi2 = (byte_of(qh, i) >> (2u * quarter)) & 3u;
         const int quant = static_cast<int>(nib | (hi2 << 4)) - 32;
         out[i] = ds * static_cast<float>(quant);
     }
