@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published (5.0 POP/s)
+F16_PEAK_TFLOPS = 2500.0       # MI355X dense fp16 MFMA, published (2.5 PFLOP/s)
 ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
@@ -47,7 +48,8 @@ def parse_args():
     p.add_argument("--steps", type=int, default=2000)
     p.add_argument("--warmup", type=int, default=200)
     p.add_argument("--workload", default="q4_k_gemv_14336x4096",
-                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, kv_attention_decode")
+                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,f16,f16_16x16}, "
+                        "kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
     p.add_argument("--kv-dtype", choices=["f16", "bf16", "u8", "f32"], default="f16",
@@ -171,6 +173,41 @@ def calibrate(args, et):
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": moved, "avg_launch_us": round(ms * 1e3, 3)},
+    }))
+
+
+def calibrate_mfma(args, et):
+    """Loops of one matrix-core instruction that touch no memory (``calibrate_mfma_i8``, ``_i8_scaled``,
+    ``_i8_scaled_bf16``, ``_f16``, ``_f16_16x16``): what the matrix cores of this device sustain, next to the published peak.
+    ``_i8_scaled`` adds the f32 epilogue of a contraction whose operands both carry a scale per 32
+    columns: the ceiling of that arithmetic whatever feeds it."""
+    import torch
+
+    kind = args.workload[len("calibrate_mfma_"):]
+    if kind not in et.MFMA_OPERATIONS:
+        sys.exit(f"unknown workload {args.workload}; kinds: {sorted(et.MFMA_OPERATIONS)}")
+    device = torch.device("cuda:0")
+    workgroups, iterations = 512, 2000  # two workgroups of four waves per compute unit: two waves per SIMD
+    sink = torch.zeros(256 * workgroups, dtype=torch.float32, device=device)
+    step = lambda i: et.calibration_mfma(kind, iterations, sink)  # noqa: E731
+    ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+    torch.cuda.synchronize()
+    expected = {"i8": 32.0, "i8_scaled": 16.0, "i8_scaled_bf16": 16.0, "f16": 16.0, "f16_16x16": 32.0}[kind] * iterations * \
+        (16 if kind == "f16_16x16" else 64)
+    assert torch.all(sink == expected), (float(sink[0]), expected)
+    operations = et.MFMA_OPERATIONS[kind] * 4 * iterations * 4 * workgroups
+    tops = operations / (ms * 1e-3) / 1e12
+    peak = INT8_PEAK_TOPS if kind.startswith("i8") else F16_PEAK_TFLOPS
+    print(json.dumps({
+        "metric": f"{args.workload} TOP/s", "value": round(tops, 1), "unit": "TOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8" if kind.startswith("i8") else "f16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {workgroups} workgroups of four waves, {iterations} rounds of four "
+                               "independent instructions per wave, no memory traffic",
+                   "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues"},
+        "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(tops / peak, 4), "traffic": None},
     }))
 
 
@@ -860,6 +897,8 @@ def main():
 
     if args.workload in ("calibrate_read", "calibrate_copy"):
         return calibrate(args, et)
+    if args.workload.startswith("calibrate_mfma_"):
+        return calibrate_mfma(args, et)
     if args.workload in DECODE_OPS:
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return decode_op(args, et)

@@ -14,7 +14,9 @@ from .quantized import (  # noqa: F401
     QuantizedRequirements,
     LinearGroup,
     RawLinear,
+    MFMA_OPERATIONS,
     calibration_copy,
+    calibration_mfma,
     calibration_read,
     dequantize_rows,
     embedding_into,

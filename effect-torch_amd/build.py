@@ -34,7 +34,8 @@ SOURCES = {
     "gemm_h16.hip": [],
     "kv_attention.hip": [],
     "decode_ops.hip": ["-ffp-contract=off"],
-    "calibrate.hip": [],
+    # matrix-core results straight into VGPRs, as in the batch kernels (no accumulation-register moves)
+    "calibrate.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "quantized.cpp": [],
     "kv_cache.cpp": [],
     "decode_host.cpp": [],

@@ -712,6 +712,22 @@ int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* st
     });
 }
 
+int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgroups, float* sink, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (sink == nullptr || workgroups == 0 || workgroups > 65536 || iterations == 0 || iterations > (1u << 20) ||
+            kind < ET_MFMA_I8 || kind > ET_MFMA_I8_SCALED_BF16) {
+            *error = "calibration_mfma: kind 0..4, 1 <= iterations <= 2^20, 1 <= workgroups <= 65536, sink non-NULL";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status = et::calibration_mfma(kind, iterations, workgroups, sink, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("calibration_mfma: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
 const char* et_hip_last_error(void) { return g_last_error.c_str(); }
 
 }  // extern "C"

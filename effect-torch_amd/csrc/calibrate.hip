@@ -1,9 +1,13 @@
-// Measurement aids: a plain streaming read and a plain copy of known size.
+// Measurement aids: a plain streaming read, a plain copy of known size, and loops of matrix-core
+// instructions that touch no memory.
 //
 // They give (a) the HBM bandwidth this device actually delivers to a kernel of
 // the same footprint as a GEMV (the practical ceiling the dequant-GEMV is
-// compared with, next to the published peak) and (b) a reference reading for
-// hardware counters (FETCH_SIZE / WRITE_SIZE per byte actually moved).
+// compared with, next to the published peak), (b) a reference reading for
+// hardware counters (FETCH_SIZE / WRITE_SIZE per byte actually moved) and (c) the rate the
+// matrix cores sustain on this device for the instructions the batch kernels use, alone and with
+// the f32 block-scale epilogue of an int8 contraction whose operands both carry a scale per 32
+// columns - the ceiling that arithmetic has whatever feeds it.
 // Nothing on the operator path uses them; the reference has no counterpart.
 #include <hip/hip_runtime.h>
 
@@ -46,7 +50,146 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src
     for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < quads; i += stride) dst[i] = src[i];
 }
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// Every wave runs `iterations` rounds of four independent instructions of one kind and leaves the
+// sum of what it accumulated in sink[thread]. Operands are all ones, so the sums are known:
+//   kMfmaI8        v_mfma_i32_32x32x32_i8, accumulating: every element ends at 32 * iterations
+//   kMfmaI8Scaled  the same instruction from zero, then per element one convert and one multiply-add
+//                  with a tile of scale products that v_mfma_f32_32x32x2f32 makes from a scale per
+//                  vector and a scale per row (the epilogue of gemm_i8.hip); element = 32 * 0.5 * iterations
+//   kMfmaF16       v_mfma_f32_32x32x16_f16, accumulating: 16 * iterations
+//   kMfmaF16Small  v_mfma_f32_16x16x32_f16, accumulating: 32 * iterations
+//   kMfmaI8ScaledBf16  kMfmaI8Scaled with the scale products from a bfloat16 instruction (see below)
+template <int KIND>
+__global__ __launch_bounds__(256) void mfma_kernel(float* __restrict__ sink, uint32_t iterations) {
+    float total = 0.f;
+    if constexpr (KIND == kMfmaI8) {
+        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+        v16i c[4] = {};
+        for (uint32_t it = 0; it < iterations; it++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) c[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ones, ones, c[k], 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += static_cast<float>(c[k][r]);
+    } else if constexpr (KIND == kMfmaI8Scaled) {
+        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+        v16i zero_i = {};
+        v16f zero_f = {};
+        float acc[4][16] = {};
+        // only the k = 0 half of the lanes carries a value of the rank-1 product
+        const float row_scale = threadIdx.x % 64 < 32 ? 0.5f : 0.f;
+        float vector_scale[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+        v4i a[4] = {ones, ones, ones, ones};
+        for (uint32_t it = 0; it < iterations; it++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                // Operands that the compiler cannot prove equal or constant keep four instructions of
+                // each kind inside the loop: an empty asm statement per operand, values unchanged.
+                asm volatile("" : "+v"(vector_scale[k]));
+                asm volatile("" : "+v"(a[k]));
+                const v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[k], ones, zero_i, 0, 0, 0);
+                const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(vector_scale[k], row_scale, zero_f, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[k][r] = fmaf(static_cast<float>(c[r]), sd[r], acc[k][r]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += acc[k][r];
+    } else if constexpr (KIND == kMfmaI8ScaledBf16) {
+        // The same arithmetic with the tile of scale products from v_mfma_f32_32x32x16_bf16 (half the
+        // matrix-core time of the f32 instruction): the vector's scale as three bfloat16 pieces (exact:
+        // 3 x 8 bits), the row's half-float scale as two (8 + 3 bits), their six products in six of
+        // the sixteen K slots, every product exact in the f32 accumulator.
+        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+        v16i zero_i = {};
+        v16f zero_f = {};
+        float acc[4][16] = {};
+        const bool first_half = threadIdx.x % 64 < 32;
+        float vector_scale[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+        const float row_value = 0.5f;
+        const uint32_t d0 = __float_as_uint(row_value) & 0xffff0000u;
+        const uint32_t d1 = __float_as_uint(row_value - __uint_as_float(d0)) >> 16;
+        union {
+            uint4 words;
+            v8bf values;
+        } row_operand, vector_operand;
+        // K slots 0..5 of the first lane half: (d0, d1, d0, d1, d0, d1) against (s0, s0, s1, s1, s2, s2)
+        const uint32_t d_pair = first_half ? (d0 >> 16) | (d1 << 16) : 0u;
+        row_operand.words = make_uint4(d_pair, d_pair, d_pair, 0u);
+        v4i a[4] = {ones, ones, ones, ones};
+        for (uint32_t it = 0; it < iterations; it++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                asm volatile("" : "+v"(vector_scale[k]));
+                asm volatile("" : "+v"(a[k]));
+                const float s = first_half ? vector_scale[k] : 0.f;
+                const uint32_t s0 = __float_as_uint(s) & 0xffff0000u;
+                const float rest = s - __uint_as_float(s0);
+                const uint32_t s1 = __float_as_uint(rest) & 0xffff0000u;
+                const uint32_t s2 = __float_as_uint(rest - __uint_as_float(s1)) >> 16;
+                vector_operand.words = make_uint4((s0 >> 16) | s0, (s1 >> 16) | s1, s2 | (s2 << 16), 0u);
+                const v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[k], ones, zero_i, 0, 0, 0);
+                const v16f sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_operand.values, row_operand.values, zero_f, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[k][r] = fmaf(static_cast<float>(c[r]), sd[r], acc[k][r]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += acc[k][r];
+    } else if constexpr (KIND == kMfmaF16) {
+        v8h ones;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ones[i] = static_cast<_Float16>(1.0f);
+        v16f c[4] = {};
+        for (uint32_t it = 0; it < iterations; it++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) c[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, ones, c[k], 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += c[k][r];
+    } else {
+        v8h ones;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ones[i] = static_cast<_Float16>(1.0f);
+        v4f c[4] = {};
+        for (uint32_t it = 0; it < iterations; it++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) c[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, ones, c[k], 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) total += c[k][r];
+    }
+    sink[blockIdx.x * 256u + threadIdx.x] = total;
+}
+
 }  // namespace
+
+hipError_t calibration_mfma(int kind, uint32_t iterations, uint32_t workgroups, float* sink, hipStream_t stream) {
+    const dim3 grid(workgroups), block(256);
+    switch (kind) {
+        case kMfmaI8: hipLaunchKernelGGL(mfma_kernel<kMfmaI8>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaI8Scaled: hipLaunchKernelGGL(mfma_kernel<kMfmaI8Scaled>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaF16: hipLaunchKernelGGL(mfma_kernel<kMfmaF16>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaF16Small: hipLaunchKernelGGL(mfma_kernel<kMfmaF16Small>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaI8ScaledBf16: hipLaunchKernelGGL(mfma_kernel<kMfmaI8ScaledBf16>, grid, block, 0, stream, sink, iterations); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
 
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             hipStream_t stream) {

@@ -200,10 +200,14 @@ hipError_t argmax_rows(const float* logits, uint64_t rows, uint64_t columns, uin
 hipError_t gather_rows(const void* table, uint64_t table_rows, uint64_t row_bytes, const void* indexes,
                        int index_is_i64, uint64_t count, void* out, void* status, hipStream_t stream);
 
-// ---- calibrate.hip: measurement aids (plain read / copy of known size) -------
+// ---- calibrate.hip: measurement aids (plain read / copy of known size, matrix-core loops) -------
 // sink must hold 4 * `workgroups` words; bytes < 2^36.
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             hipStream_t stream);
 hipError_t calibration_copy(const void* src, void* dst, uint64_t bytes, hipStream_t stream);
+// Loops of matrix-core instructions without memory traffic: four waves per workgroup, four
+// independent instructions per wave and round; sink gets one float per thread (256 * workgroups).
+enum : int { kMfmaI8 = 0, kMfmaI8Scaled = 1, kMfmaF16 = 2, kMfmaF16Small = 3, kMfmaI8ScaledBf16 = 4 };
+hipError_t calibration_mfma(int kind, uint32_t iterations, uint32_t workgroups, float* sink, hipStream_t stream);
 
 }  // namespace et

@@ -415,3 +415,16 @@ def calibration_copy(src: torch.Tensor, dst: torch.Tensor, stream=None) -> None:
     """Plain copy ``dst <- src`` (measurement aid, ``et_hip_calibration_copy``)."""
     _check(N.lib().et_hip_calibration_copy(src.data_ptr(), dst.data_ptr(),
                                            src.numel() * src.element_size(), _stream_handle(stream)))
+
+
+MFMA_KINDS = {"i8": 0, "i8_scaled": 1, "f16": 2, "f16_16x16": 3, "i8_scaled_bf16": 4}
+MFMA_OPERATIONS = {"i8": 65536, "i8_scaled": 65536, "f16": 32768, "f16_16x16": 16384, "i8_scaled_bf16": 65536}
+
+
+def calibration_mfma(kind: str, iterations: int, sink: torch.Tensor, stream=None) -> None:
+    """Rounds of four independent matrix-core instructions per wave, no memory traffic (measurement
+    aid, ``et_hip_calibration_mfma``); ``sink`` is f32 with 256 elements per workgroup."""
+    if sink.dtype != torch.float32 or sink.numel() % 256 != 0 or sink.numel() == 0:
+        raise ValueError("calibration_mfma: sink must be f32 with a multiple of 256 elements")
+    _check(N.lib().et_hip_calibration_mfma(MFMA_KINDS[kind], iterations, sink.numel() // 256, sink.data_ptr(),
+                                           _stream_handle(stream)))

@@ -642,3 +642,18 @@ def test_group_launch_of_contractions_sharing_their_input(et, device):
         et.LinearGroup([plans[0], et.RawLinear(et.GgmlQuant.Q4_K, 64, 512, vectors)])
     with pytest.raises(et.QuantizedError, match="no group launch"):
         et.LinearGroup([et.RawLinear(et.GgmlQuant.Q4_K, 64, columns, 2)])
+
+
+# --------------------------------------------------------------------------- measurement aids
+
+@pytest.mark.parametrize("kind,per_round,elements", [("i8", 32.0, 64), ("i8_scaled", 16.0, 64), ("i8_scaled_bf16", 16.0, 64), ("f16", 16.0, 64),
+                                                      ("f16_16x16", 32.0, 16)])
+def test_matrix_core_calibration_loops_sum_what_they_should(et, device, kind, per_round, elements):
+    """All operands are ones, so every accumulator element ends at a known integer: K ones per round
+    (times the scale product 0.5 for the scaled kind); a thread reports the sum of its elements."""
+    rounds, workgroups = 37, 3
+    sink = torch.full((256 * workgroups,), float("nan"), device=device)
+    et.calibration_mfma(kind, rounds, sink)
+    assert torch.all(sink == per_round * rounds * elements), (float(sink[0]), per_round * rounds * elements)
+    with pytest.raises(et.QuantizedError, match="calibration_mfma"):
+        et.calibration_mfma(kind, 0, sink)
