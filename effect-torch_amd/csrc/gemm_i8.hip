@@ -67,6 +67,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 constexpr int kStageBlocks = 8;  // 32-column blocks per stage
 constexpr int kConsumers = 8;    // waves that run the MFMAs: two per SIMD
@@ -94,6 +95,35 @@ __device__ __forceinline__ void q4k_scale_min(const uint4& header, uint32_t g, f
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
 constexpr int vmcnt_only(int n) {
     return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8);
+}
+
+// The tile of scale products s[m] * d[n] from v_mfma_f32_32x32x16_bf16, which takes half the
+// matrix-core time of the f32 instruction: a half-float row scale is exactly two bfloat16 pieces
+// (8 + 3 bits), an f32 vector scale exactly three, and their six products - each exact in the f32
+// accumulator - fill K slots 0..5 of the first lane half: rows (d0, d1, d0, d1, d0, d1) against
+// vectors (s0, s0, s1, s1, s2, s2). The second lane half holds zeros on the row side, so the vector
+// side needs no mask there (scales are finite).
+union ScaleOperand {
+    uint4 words;
+    v8bf values;
+};
+__device__ __forceinline__ ScaleOperand row_scale_pieces(float d, bool first_half) {
+    const uint32_t d0 = __float_as_uint(d) & 0xffff0000u;
+    const uint32_t d1 = __float_as_uint(d - __uint_as_float(d0)) >> 16;  // exact: at most three bits left
+    const uint32_t pair = first_half ? (d0 >> 16) | (d1 << 16) : 0u;
+    ScaleOperand operand;
+    operand.words = make_uint4(pair, pair, pair, 0u);
+    return operand;
+}
+__device__ __forceinline__ ScaleOperand vector_scale_pieces(float s) {
+    const uint32_t s0 = __float_as_uint(s) & 0xffff0000u;
+    const float rest = s - __uint_as_float(s0);
+    const uint32_t s1 = __float_as_uint(rest) & 0xffff0000u;
+    const uint32_t s2 = __float_as_uint(rest - __uint_as_float(s1));  // at most eight bits: its top half is exact
+    ScaleOperand operand;
+    operand.words = make_uint4(__builtin_amdgcn_perm(s0, s0, 0x07060706u), __builtin_amdgcn_perm(s1, s1, 0x07060706u),
+                               __builtin_amdgcn_perm(s2, s2, 0x07060706u), 0u);
+    return operand;
 }
 
 // Weight slot in LDS: the stage's bytes of the workgroup's 64 rows, row after row exactly as in
@@ -296,6 +326,10 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         // B operands (16 int8 weights of row n, this lane's half of the block) and block scales
         v4i bw[NB];
         float w_scale[NB];
+        // Half-float row scales (Q8_0, Q4_0) go through the bfloat16 instruction; d * sc of Q4_K has
+        // seventeen bits and stays on the f32 one.
+        constexpr bool kPieces = CODEC != kQ4_K;
+        ScaleOperand w_pieces[NB];
 #pragma unroll
         for (int bb = 0; bb < NB; bb++) {
             const uint32_t b = b_base + bb;  // block inside the stage
@@ -340,6 +374,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 }
             }
             // rank-1 operand: only the k = 0 half of the lanes carries a value
+            if constexpr (kPieces) w_pieces[bb] = row_scale_pieces(w_scale[bb], half == 0);
             w_scale[bb] = half == 0 ? w_scale[bb] : 0.f;
         }
 
@@ -382,8 +417,12 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             const int bb = step / MT;
             // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1
             // product in the MFMA result layout.
-            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale_next : 0.f, w_scale[bb],
-                                                                 zero_f, 0, 0, 0);
+            v16f sd;
+            if constexpr (kPieces)
+                sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_scale_pieces(x_scale_next).values, w_pieces[bb].values,
+                                                             zero_f, 0, 0, 0);
+            else
+                sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale_next : 0.f, w_scale[bb], zero_f, 0, 0, 0);
             v16i c[LIMBS];
 #pragma unroll
             for (int l = 0; l < LIMBS; l++)
