@@ -100,29 +100,26 @@ constexpr int vmcnt_only(int n) {
 // The tile of scale products s[m] * d[n] from v_mfma_f32_32x32x16_bf16, which takes half the
 // matrix-core time of the f32 instruction: a half-float row scale is exactly two bfloat16 pieces
 // (8 + 3 bits), an f32 vector scale exactly three, and their six products - each exact in the f32
-// accumulator - fill K slots 0..5 of the first lane half: rows (d0, d1, d0, d1, d0, d1) against
-// vectors (s0, s0, s1, s1, s2, s2). The second lane half holds zeros on the row side, so the vector
-// side needs no mask there (scales are finite).
+// accumulator - fill six of the eight K slots of the first lane half: rows (d0, d0, d0, 0, d1, d1,
+// d1, 0) against vectors (s0, s1, s2, 0, s0, s1, s2, 0). The second lane half holds zeros on the
+// row side, so the vector side needs no mask there (scales are finite). The quantiser stores the
+// vector pieces next to the scale (kernels.h: pieces[b][m]); kernels that use them copy the pieces
+// into LDS in place of the two f32 tables.
 union ScaleOperand {
     uint4 words;
     v8bf values;
 };
 __device__ __forceinline__ ScaleOperand row_scale_pieces(float d, bool first_half) {
-    const uint32_t d0 = __float_as_uint(d) & 0xffff0000u;
-    const uint32_t d1 = __float_as_uint(d - __uint_as_float(d0)) >> 16;  // exact: at most three bits left
-    const uint32_t pair = first_half ? (d0 >> 16) | (d1 << 16) : 0u;
+    const uint32_t d0 = __float_as_uint(d) >> 16;  // top sixteen bits: the bfloat16 below d
+    const uint32_t d1 = __float_as_uint(d - __uint_as_float(d0 << 16)) >> 16;  // exact: at most three bits left
     ScaleOperand operand;
-    operand.words = make_uint4(pair, pair, pair, 0u);
+    operand.words = first_half ? make_uint4(d0 | (d0 << 16), d0, d1 | (d1 << 16), d1) : make_uint4(0u, 0u, 0u, 0u);
     return operand;
 }
-__device__ __forceinline__ ScaleOperand vector_scale_pieces(float s) {
-    const uint32_t s0 = __float_as_uint(s) & 0xffff0000u;
-    const float rest = s - __uint_as_float(s0);
-    const uint32_t s1 = __float_as_uint(rest) & 0xffff0000u;
-    const uint32_t s2 = __float_as_uint(rest - __uint_as_float(s1));  // at most eight bits: its top half is exact
+// `pieces` as the quantiser stores them: (s0 | s1 << 16, s2).
+__device__ __forceinline__ ScaleOperand vector_scale_pieces(const uint2& pieces) {
     ScaleOperand operand;
-    operand.words = make_uint4(__builtin_amdgcn_perm(s0, s0, 0x07060706u), __builtin_amdgcn_perm(s1, s1, 0x07060706u),
-                               __builtin_amdgcn_perm(s2, s2, 0x07060706u), 0u);
+    operand.words = make_uint4(pieces.x, pieces.y, pieces.x, pieces.y);
     return operand;
 }
 
@@ -151,7 +148,7 @@ template <int CODEC, int MT, int LIMBS, int AX, int AW>
 struct Shape {
     using W = WeightLayout<CODEC>;
     static constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);        // in memory, padded
-    static constexpr uint32_t kTile = LIMBS * 8192u + 2048u;          // in LDS: operands and both tables
+    static constexpr uint32_t kTile = LIMBS * 8192u + 2048u;          // in LDS: operands and the two f32 tables or the pieces
     // Two rings: activations come from L2 (every workgroup reads the same blobs) and need little
     // lead; weights come from HBM and need as much as LDS allows.
     static constexpr int kActivationDepth = AX + 1, kWeightDepth = AW + 1;
@@ -217,8 +214,10 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 if (job >= static_cast<uint32_t>(S::kActivationJobs)) job -= S::kActivationJobs;
                 const uint32_t t = job / (S::kTile / 1024u), within = job % (S::kTile / 1024u);
                 const uint32_t tile = min(tile0 + t, vector_tiles - 1u);
+                // codecs with bfloat16 scale products take the pieces table in place of the two f32 tables
+                const uint32_t from = CODEC != kQ4_K && within >= static_cast<uint32_t>(LIMBS) * 8u ? within + 2u : within;
                 const uint8_t* src = tiles + (static_cast<uint64_t>(first_stage + s) * vector_tiles + tile) * S::kBlob +
-                                     within * 1024u + lane * 16u;
+                                     from * 1024u + lane * 16u;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
             }
@@ -384,10 +383,13 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         // step's (its results are double-buffered), with three limbs its own (three results of
         // sixteen registers each leave no room for a second set).
         constexpr int kSteps = NB * MT;
-        const auto read_step = [&](int step, v4i (&a)[LIMBS], float& x_scale) {
+        const auto read_step = [&](int step, v4i (&a)[LIMBS], float& x_scale, uint2& x_pieces) {
             const uint32_t b = b_base + step / MT;
             const uint8_t* blob = slot + (step % MT) * S::kTile;
-            x_scale = *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
+            if constexpr (kPieces)
+                x_pieces = *reinterpret_cast<const uint2*>(blob + LIMBS * 8192u + b * 256u + (lane & 31u) * 8u);
+            else
+                x_scale = *reinterpret_cast<const float*>(blob + LIMBS * 8192u + b * 128u + (lane & 31u) * 4u);
             const uint8_t* chunk = blob + (2u * b + half) * 512u + (lane & 31u) * 16u;
 #pragma unroll
             for (int l = 0; l < LIMBS; l++) a[l] = *reinterpret_cast<const v4i*>(chunk + l * 8192u);
@@ -408,8 +410,9 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             }
         };
         v4i a_next[LIMBS];
-        float x_scale_next;
-        read_step(0, a_next, x_scale_next);
+        float x_scale_next = 0.f;
+        uint2 x_pieces_next = make_uint2(0u, 0u);
+        read_step(0, a_next, x_scale_next, x_pieces_next);
         v16f sd_previous;
         v16i c_previous[LIMBS];
 #pragma unroll
@@ -419,7 +422,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             // product in the MFMA result layout.
             v16f sd;
             if constexpr (kPieces)
-                sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_scale_pieces(x_scale_next).values, w_pieces[bb].values,
+                sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_scale_pieces(x_pieces_next).values, w_pieces[bb].values,
                                                              zero_f, 0, 0, 0);
             else
                 sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale_next : 0.f, w_scale[bb], zero_f, 0, 0, 0);
@@ -427,7 +430,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 #pragma unroll
             for (int l = 0; l < LIMBS; l++)
                 c[l] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[l], bw[bb], zero_i, 0, 0, 0);
-            if (step + 1 < kSteps) read_step(step + 1, a_next, x_scale_next);
+            if (step + 1 < kSteps) read_step(step + 1, a_next, x_scale_next, x_pieces_next);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (LIMBS == 1) {
                 if (step > 0) epilogue(step - 1, sd_previous, c_previous);

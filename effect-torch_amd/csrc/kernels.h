@@ -60,7 +60,9 @@ hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 //   limb l, 16-column chunk c (0..15), vector m (0..31): 16 int8 at  l*8192 + c*512 + m*16
 //   scale[block b (0..7)][m] f32 at  limbs*8192 + b*128 + m*4
 //   xsum [b][m] f32 (scale * integer block sum) at  limbs*8192 + 1024 + b*128 + m*4
-// and padding up to a multiple of 4096 bytes.
+//   pieces[b][m]: the scale as three bfloat16 values whose sum it is exactly, (s0 | s1 << 16, s2),
+//                 8 bytes at  limbs*8192 + 2048 + b*256 + m*8
+// in all a multiple of 4096 bytes.
 // limbs = 1: int8 activations, scale = max|x| / 127.
 // limbs = 3: 24-bit fixed point in three balanced signed bytes, scale = max|x| / (127 * 65536).
 // limbs = 2 is the layout of gemm_h16: 24-bit fixed point per vector and 256-column stage in two

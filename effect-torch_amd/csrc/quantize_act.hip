@@ -112,6 +112,13 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
                 const uint32_t block = (quad & 63u) >> 3;
                 tables[block * 32u + (v & 31u)] = unit;
                 tables[256u + block * 32u + (v & 31u)] = unit * static_cast<float>(total_q);
+                // The scale once more as three bfloat16 pieces whose sum it is exactly (8 bits each),
+                // for the kernels that make their scale products on the bfloat16 matrix instruction.
+                const uint32_t s0 = __float_as_uint(unit) & 0xffff0000u;
+                const float rest = unit - __uint_as_float(s0);
+                const uint32_t s1 = __float_as_uint(rest) & 0xffff0000u;
+                const uint32_t s2 = __float_as_uint(rest - __uint_as_float(s1));
+                reinterpret_cast<uint2*>(tables + 512u)[block * 32u + (v & 31u)] = make_uint2((s0 >> 16) | s1, s2 >> 16);
             }
         } else {
             static_assert(TILED || LIMBS == 1, "the row-major layout is the int8 one");
