@@ -272,15 +272,11 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     const uint32_t wave_k = wave / kRowGroups;  // share of the stage's blocks
     const uint32_t n0 = row0 + wave_n * 32u;
     const uint32_t m0 = tile0 * 32u;
-    float acc[MT][16];
-    v16f acc_min[MT];
+    v16f acc[MT];  // a matrix-core register tile: the Q4_K min term accumulates into it directly
 #pragma unroll
     for (int t = 0; t < MT; t++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            acc[t][r] = 0.f;
-            acc_min[t][r] = 0.f;
-        }
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
     v16i zero_i;
     v16f zero_f;
 #pragma unroll
@@ -305,7 +301,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
             dmin_block = half_bits_to_float(header.x >> 16);
         }
         if constexpr (CODEC == kQ4_K) {
-            // min term: acc_min[m, n] += sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
+            // min term: acc[m, n] -= sum_g (dmin * m_g)[n] * xsum[m, g]; K = 2 per MFMA,
             // lane half h supplies sub-block 2j + h. First in the stage: its LDS reads go out with
             // the other operands' and its MFMAs run under the first steps.
 #pragma unroll
@@ -313,12 +309,12 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
                 const uint32_t g = b_base + 2u * jj + half;
                 float sc, mn;
                 q4k_scale_min(header, g, sc, mn);
-                const float b_operand = dmin_block * mn;
+                const float b_operand = -(dmin_block * mn);
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const float a_operand = *reinterpret_cast<const float*>(
                         slot + t * S::kTile + LIMBS * 8192u + 1024u + g * 128u + (lane & 31u) * 4u);
-                    acc_min[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc_min[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_operand, b_operand, acc[t], 0, 0, 0);
                 }
             }
         }
@@ -452,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         for (int t = 0; t < MT; t++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float value = CODEC == kQ4_K ? acc[t][r] - acc_min[t][r] : acc[t][r];
+                const float value = acc[t][r];
                 exchange[((((wave_k - 1u) * kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane] = value;
             }
     }
@@ -464,7 +460,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     for (int t = 0; t < MT; t++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            float value = CODEC == kQ4_K ? acc[t][r] - acc_min[t][r] : acc[t][r];
+            float value = acc[t][r];
 #pragma unroll
             for (int k = 1; k < kSplit; k++)
                 value += exchange[((((k - 1) * kRowGroups + wave_n) * MT + t) * 16 + r) * 64 + lane];
@@ -585,7 +581,9 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
     // Activations: 26 KiB per stage and 32-vector tile with three limbs, 10 KiB with one; two
     // stages of lead. The weight ring (9 to 20 KiB per stage) takes the rest of LDS.
     // One 32-vector tile per workgroup with three limbs: two tiles of three-limb results do not
-    // fit in registers. Q4_K carries a second accumulator (the min term): at most two tiles.
+    // fit in registers. With one limb four tiles share the weight operands of a step; Q4_K stays at
+    // two (four measured slower: 14336 x 4096 with 512 vectors 226 against 170 us - its min-term
+    // instructions and a single stage of activation lead).
     // (tiles_per_workgroup() below states the same choice for the launch geometry.)
     if (limbs == 3)
         return launch_shape<CODEC, 1, 3, 2>(weight, tiles, out, rows, columns, vectors, stream);
@@ -593,8 +591,7 @@ hipError_t launch_codec(int limbs, const uint8_t* weight, const uint8_t* tiles, 
         return launch_shape<CODEC, 1, 1, 2>(weight, tiles, out, rows, columns, vectors, stream);
     if (vectors <= 64 || CODEC == kQ4_K)
         return launch_shape<CODEC, 2, 1, 2>(weight, tiles, out, rows, columns, vectors, stream);
-    return launch_shape<CODEC, (CODEC == kQ4_K ? 2 : 4), 1, (CODEC == kQ4_K ? 2 : 1)>(weight, tiles, out, rows, columns,
-                                                                                vectors, stream);
+    return launch_shape<CODEC, 4, 1, 1>(weight, tiles, out, rows, columns, vectors, stream);
 }
 
 uint32_t tiles_per_workgroup(int32_t codec, int limbs, uint64_t vectors) {
