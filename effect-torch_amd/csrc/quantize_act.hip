@@ -206,34 +206,49 @@ __global__ __launch_bounds__(64) void quantize_halves_kernel(const float* __rest
     }
 }
 
-// The activations are rms_norm(x) * weight, with rms_norm_kernel's arithmetic: one workgroup of 256
-// per vector finds the row's scale, then wave w quantises stages w, w + 4, ... - float4 number
-// threadIdx.x + 256 j of the row is lane threadIdx.x % 64 of stage threadIdx.x / 64 + 4 j.
-__global__ __launch_bounds__(256) void quantize_halves_rms_kernel(const float* __restrict__ x, uint64_t x_row_stride,
-                                                                  const float* __restrict__ weight, double eps,
-                                                                  uint32_t vectors, uint32_t columns,
-                                                                  uint8_t* __restrict__ tiles) {
+// The activations are rms_norm(x) * weight, with rms_norm_kernel's arithmetic and summation order
+// (rms_row_scale in decode_math.h: thread t of 256 adds the squares of float4 number t, t + 256, ...
+// in that order, the waves' sums meet as ((0 + 1) + (2 + 3))). One workgroup of sixteen waves per
+// vector, so that a row of 4096 columns is quantised in one pass, a stage per wave: thread T holds
+// float4 number T; the squares go through LDS to the first 256 threads, which add them in
+// rms_row_scale's order.
+constexpr uint32_t kRmsThreads = 1024;
+__global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+                                                                         const float* __restrict__ weight, double eps,
+                                                                         uint32_t vectors, uint32_t columns,
+                                                                         uint8_t* __restrict__ tiles) {
+    __shared__ double squares[kRmsThreads];
     __shared__ double partial[4];
     const uint32_t v = blockIdx.x;
-    const float* in = x + v * x_row_stride;
-    float4 held[kRmsHeld];
-    const double scale = rms_row_scale(in, columns, eps, held, partial);
+    const float4* in = reinterpret_cast<const float4*>(x + v * x_row_stride);
+    const uint32_t quads = columns / 4;
+    const auto square_sum = [](const float4& f) {
+        return (static_cast<double>(f.x) * f.x + static_cast<double>(f.y) * f.y) +
+               (static_cast<double>(f.z) * f.z + static_cast<double>(f.w) * f.w);
+    };
+    const float4 held = threadIdx.x < quads ? in[threadIdx.x] : make_float4(0.f, 0.f, 0.f, 0.f);
+    squares[threadIdx.x] = square_sum(held);
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        double sum = 0.0;
+#pragma unroll
+        for (int j = 0; j < kRmsHeld; j++) sum += squares[threadIdx.x + 256 * j];
+        for (uint32_t i = threadIdx.x + 256 * kRmsHeld; i < quads; i += 256) sum += square_sum(in[i]);
+        sum = wave_sum(sum);
+        if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = sum;
+    }
+    __syncthreads();
+    const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
+    const double scale = 1.0 / sqrt(mean_square + eps);
     const uint32_t vector_tiles = (vectors + 31u) >> 5, stages = columns >> 8;
     const uint32_t wave = threadIdx.x >> 6, quad = threadIdx.x & 63u;
     const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
-#pragma unroll
-    for (int j = 0; j < kRmsHeld; j++) {
-        const uint32_t stage = wave + 4u * j;  // uniform in the wave
-        if (stage < stages) {
-            const uint32_t i = threadIdx.x + 256u * j;
-            quantize_halves_store(rms_four(held[j], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
-                                  v, stage, quad, vector_tiles, tiles);
-        }
-    }
-    for (uint32_t stage = wave + 4u * kRmsHeld; stage < stages; stage += 4u) {
+    if (wave < stages)
+        quantize_halves_store(rms_four(held, scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[threadIdx.x] : ones),
+                              v, wave, quad, vector_tiles, tiles);
+    for (uint32_t stage = wave + kRmsThreads / 64u; stage < stages; stage += kRmsThreads / 64u) {
         const uint32_t i = 64u * stage + quad;
-        quantize_halves_store(rms_four(reinterpret_cast<const float4*>(in)[i], scale,
-                                       weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
+        quantize_halves_store(rms_four(in[i], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
                               v, stage, quad, vector_tiles, tiles);
     }
 }
@@ -303,7 +318,7 @@ hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const 
                                    uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream) {
     if (columns % 256 != 0 || vectors > 0x7fffffffull) return hipErrorInvalidValue;
     if (vectors == 0 || columns == 0) return hipSuccess;
-    hipLaunchKernelGGL(quantize_halves_rms_kernel, dim3(static_cast<uint32_t>(vectors)), dim3(256), 0, stream, x,
+    hipLaunchKernelGGL(quantize_halves_rms_kernel, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream, x,
                        x_row_stride, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
 }
