@@ -568,6 +568,7 @@ def llama_decode(args, et):
     fused = not args.unfused
     shared_hidden = torch.empty(max(plans["wq"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
     shared_ffn = torch.empty(max(plans["down"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
+    shared_attended = torch.empty(max(plans["wo"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
 
     blocks_per_slot = -(-context // block)
     total_blocks = slots * blocks_per_slot
@@ -605,10 +606,16 @@ def llama_decode(args, et):
         group_ws = torch.empty(max(qkv_group.workspace_bytes, ffn_group.workspace_bytes, 16), dtype=torch.uint8,
                                device=device)
 
-    def layer_step(index):
+    # (following plan, its norm weight) after a layer's down projection: the next layer's attention
+    # norm, or the final norm in front of the output head
+    after_down = lambda index: (plans["wq"], norms[index + 1][0]) if index + 1 < layers else (plans["head"], final_norm)  # noqa: E731
+
+    def layer_step(index, prepared_by_previous=False):
         w, kvl = weights[index], kv[index]
         if on_the_fly:
-            plans["wq"].prepare_input_rms_norm(x, norms[index][0], 1e-5, shared_hidden)
+            # the layer before has left this norm's prepared input behind (enqueue_prepared_then_norm)
+            if not prepared_by_previous:
+                plans["wq"].prepare_input_rms_norm(x, norms[index][0], 1e-5, shared_hidden)
         else:
             et.rms_norm_into(x, norms[index][0], 1e-5, h)
         if fused:
@@ -631,15 +638,18 @@ def llama_decode(args, et):
             et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
         keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
                                          workspace=kv_ws, synchronize=False))
-        if fused:
+        if on_the_fly:
+            # x += attended Wo, then the ffn norm inside the quantiser, in the launch that sums Wo's K shares
+            plans["wo"].prepare_input(attended, shared_attended)
+            plans["wo"].enqueue_prepared_then_norm(shared_attended, w["wo"], None, x, linear_ws, plans["gate"],
+                                                   norms[index][1], 1e-5, shared_hidden, residual=x)
+        elif fused:
             plans["wo"].prepare_input(attended, shared_hidden)
             plans["wo"].enqueue_prepared(shared_hidden, w["wo"], None, x, linear_ws, residual=x)
         else:
             plans["wo"].enqueue(attended, w["wo"], None, projected, linear_ws)
             et.add_into(x, projected, x)
-        if on_the_fly:
-            plans["gate"].prepare_input_rms_norm(x, norms[index][1], 1e-5, shared_hidden)
-        else:
+        if not on_the_fly:
             et.rms_norm_into(x, norms[index][1], 1e-5, h)
         if fused:
             if on_the_fly:
@@ -655,9 +665,12 @@ def llama_decode(args, et):
             plans["down"].prepare_input_silu_mul(gate, up, shared_ffn)
         else:
             et.silu_mul_into(gate, up, gate)
-        if fused:
-            if not on_the_fly:
-                plans["down"].prepare_input(gate, shared_ffn)
+        if on_the_fly:
+            following, norm_weight = after_down(index)
+            plans["down"].enqueue_prepared_then_norm(shared_ffn, w["down"], None, x, linear_ws, following, norm_weight,
+                                                     1e-5, shared_hidden, residual=x)
+        elif fused:
+            plans["down"].prepare_input(gate, shared_ffn)
             plans["down"].enqueue_prepared(shared_ffn, w["down"], None, x, linear_ws, residual=x)
         else:
             plans["down"].enqueue(gate, w["down"], None, down, linear_ws)
@@ -667,9 +680,8 @@ def llama_decode(args, et):
         keep.clear()
         keep.append(et.gather_rows_into(embedding, tokens.view(torch.uint32), x, synchronize=False))
         for index in range(layers):
-            layer_step(index)
+            layer_step(index, prepared_by_previous=on_the_fly and index > 0)
         if on_the_fly:
-            plans["head"].prepare_input_rms_norm(x, final_norm, 1e-5, shared_hidden)
             plans["head"].enqueue_prepared(shared_hidden, base["head"], None, logits, linear_ws)
         else:
             et.rms_norm_into(x, final_norm, 1e-5, h)

@@ -120,6 +120,8 @@ SIGNATURES = {
                                                             _vp, _vp]),
     "et_hip_linear_prepare_input_from": (ctypes.c_int, [_vp, ctypes.POINTER(EtPrepareSource), _vp, _u64, _vp]),
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
+    "et_hip_linear_enqueue_prepared_then_norm": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp,
+                                                                ctypes.c_double, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
     "et_hip_embedding_plan_destroy": (None, [_vp]),
     "et_hip_embedding_plan_output_rank": (_i32, [_vp]),

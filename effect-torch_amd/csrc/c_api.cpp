@@ -251,6 +251,23 @@ int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepa
     });
 }
 
+int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
+                                             const uint8_t* weight, const float* bias, const float* residual,
+                                             float* y, void* workspace, uint64_t workspace_bytes,
+                                             const et_linear_plan* next, const float* norm_weight, double eps,
+                                             void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                             const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr || next == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_enqueue_prepared_then_norm(*plan, prepared, weight, bias, residual, y, workspace,
+                                                                workspace_bytes, *next, norm_weight, eps, next_prepared,
+                                                                next_prepared_bytes, stream, cancel, error);
+    });
+}
+
 int et_hip_embedding_requirements(const et_tensor* indexes, const et_tensor* weight, int32_t codec,
                                   uint64_t rows, uint64_t columns, et_embedding_plan** out) {
     return guarded([&](std::string* error) -> int {

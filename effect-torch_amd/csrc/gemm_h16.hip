@@ -610,7 +610,7 @@ uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint3
 namespace {
 template <int CODEC, int RG, int AX, int AW>
 hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
-                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream) {
+                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares) {
     using S = Shape<CODEC, RG, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW>;
@@ -641,7 +641,7 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, group, tiles,
                        vector_tiles, columns, vectors, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
-    if (k_splits > 1) {
+    if (k_splits > 1 && !leave_shares) {
         const uint64_t items = row_tiles * S::kRows * vectors / 4;
         hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
                            group, partials, vectors, k_splits, S::kRows);
@@ -650,8 +650,14 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
 }
 }  // namespace
 
+GemmShares gemm_h16_shares_layout(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors) {
+    const GemmGroupGeometry g = gemm_h16_group_geometry(codec, &rows, 1, columns, vectors);
+    return GemmShares{g.k_splits, g.row_tiles * g.tile_rows};
+}
+
 hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
-                          float* partials, uint64_t columns64, uint64_t vectors64, hipStream_t stream) {
+                          float* partials, uint64_t columns64, uint64_t vectors64, hipStream_t stream,
+                          bool leave_shares) {
     if (!gemm_h16_supported(codec, columns64)) return hipErrorInvalidValue;
     if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
     const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
@@ -666,31 +672,31 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     }
     // weight lead: what the activation ring (three slots of 34 KiB) leaves of LDS
     if (codec == kQ6_K)  // 64-row tiles only (gemm_h16_group_geometry): 128 rows of 224 bytes leave no room for a ring
-        return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
     if (codec == kQ2_K || codec == kQ3_K) {  // rows of 96 / 112 bytes per stage: room for the longest lead
         if (codec == kQ2_K) {
             if (g.tile_rows == 128)
-                return launch_group<kQ2_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
-            return launch_group<kQ2_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+                return launch_group<kQ2_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+            return launch_group<kQ2_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
         }
         if (g.tile_rows == 128)
-            return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
-        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+            return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
     }
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
-            return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
-        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+            return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
     }
     if (g.tile_rows == 128)
-        return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
-    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream);
+        return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream) {
     const GemmMember one = {weight, out.bias, out.residual, out.y, rows};
-    return gemm_h16_group(codec, &one, 1, tiles, out.partials, columns, vectors, stream);
+    return gemm_h16_group(codec, &one, 1, tiles, out.partials, columns, vectors, stream, out.leave_shares);
 }
 
 }  // namespace et

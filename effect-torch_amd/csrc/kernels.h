@@ -84,6 +84,13 @@ hipError_t quantize_tiles_silu_mul(const float* gate, const float* up, uint64_t 
                                    uint64_t columns, uint8_t* tiles, hipStream_t stream);
 hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const float* weight, double eps,
                                    uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream);
+// The same with x = y computed in the same launch from the unsummed K shares of a contraction:
+// y[m, n] = shares in share order (+ bias[n]) (+ residual[m, n], which may be y itself), written to
+// y [vectors, columns] - the bytes reduce_group_kernel writes - and then normed and quantised.
+hipError_t quantize_tiles_rms_norm_of_shares(const float* shares, uint32_t share_count, uint64_t launch_rows,
+                                             const float* bias, const float* residual, float* y, const float* weight,
+                                             double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles,
+                                             hipStream_t stream);
 
 // ---- gemm_i8.hip: matrix-core contraction over quantised activation tiles ---------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
@@ -98,6 +105,9 @@ struct GemmOutput {
     const float* residual;  // [vectors, rows] added to the result, or null; may be y itself
     float* y;               // [vectors, rows]
     float* partials;        // see gemm_i8_k_splits, or null
+    // gemm_h16 only: leave the K shares in `partials` unsummed ([share][vector][launch row], see
+    // gemm_h16_shares_layout) for a consumer that sums them itself; bias, residual and y are then unused.
+    bool leave_shares = false;
 };
 hipError_t gemm_i8(int32_t codec, int limbs, const uint8_t* weight, const uint8_t* tiles,
                    const GemmOutput& out, uint64_t rows, uint64_t columns, uint64_t vectors,
@@ -134,7 +144,15 @@ GemmGroupGeometry gemm_h16_group_geometry(int32_t codec, const uint64_t* rows, u
 uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
                                       uint64_t vectors);
 hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
-                          float* partials, uint64_t columns, uint64_t vectors, hipStream_t stream);
+                          float* partials, uint64_t columns, uint64_t vectors, hipStream_t stream,
+                          bool leave_shares = false);
+// Where a one-matrix launch with K shares leaves them: share k, vector m, row n at
+// partials[(k * vectors + m) * launch_rows + n].
+struct GemmShares {
+    uint32_t count;        // 1: the launch does not share K
+    uint64_t launch_rows;  // rows rounded up to whole tiles
+};
+GemmShares gemm_h16_shares_layout(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors);
 
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch

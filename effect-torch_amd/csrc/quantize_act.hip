@@ -213,7 +213,20 @@ __global__ __launch_bounds__(64) void quantize_halves_kernel(const float* __rest
 // float4 number T; the squares go through LDS to the first 256 threads, which add them in
 // rms_row_scale's order.
 constexpr uint32_t kRmsThreads = 1024;
-__global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+// The unsummed K shares of a contraction, for the variant that sums them itself: the row it norms is
+// y[m, :] = share 0 + share 1 + ... (+ bias) (+ residual[m, :]) in reduce_group_kernel's order, and it
+// writes that row to y before it reads it (residual may be y: a float4 is read, then written, by one
+// thread).
+struct ShareSource {
+    const float* shares;     // [count][vectors][launch_rows]
+    uint32_t count;
+    uint64_t launch_rows, share_stride;
+    const float* bias;       // [columns] or null
+    const float* residual;   // [vectors, columns] or null
+};
+template <bool SHARES>
+__global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const float* x, uint64_t x_row_stride,
+                                                                         const ShareSource source,
                                                                          const float* __restrict__ weight, double eps,
                                                                          uint32_t vectors, uint32_t columns,
                                                                          uint8_t* __restrict__ tiles) {
@@ -226,7 +239,35 @@ __global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const 
         return (static_cast<double>(f.x) * f.x + static_cast<double>(f.y) * f.y) +
                (static_cast<double>(f.z) * f.z + static_cast<double>(f.w) * f.w);
     };
-    const float4 held = threadIdx.x < quads ? in[threadIdx.x] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 held = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (SHARES) {
+        // x is y: every float4 of the row is summed and written once, number T, T + 1024, ... by thread T
+        float4* row = reinterpret_cast<float4*>(const_cast<float*>(x) + v * x_row_stride);
+        for (uint32_t i = threadIdx.x; i < quads; i += kRmsThreads) {
+            const float* first = source.shares + v * source.launch_rows + 4u * i;
+            float4 total = *reinterpret_cast<const float4*>(first);
+            for (uint32_t k = 1; k < source.count; k++) {
+                const float4 part = *reinterpret_cast<const float4*>(first + k * source.share_stride);
+                total.x += part.x;
+                total.y += part.y;
+                total.z += part.z;
+                total.w += part.w;
+            }
+            if (source.bias != nullptr) {
+                const float4 b = reinterpret_cast<const float4*>(source.bias)[i];
+                total = make_float4(total.x + b.x, total.y + b.y, total.z + b.z, total.w + b.w);
+            }
+            if (source.residual != nullptr) {
+                const float4 r = reinterpret_cast<const float4*>(source.residual + v * static_cast<uint64_t>(columns))[i];
+                total = make_float4(total.x + r.x, total.y + r.y, total.z + r.z, total.w + r.w);
+            }
+            row[i] = total;
+            if (i == threadIdx.x) held = total;
+        }
+        if (quads > kRmsThreads) __syncthreads();  // the passes below read what other threads wrote
+    } else {
+        if (threadIdx.x < quads) held = in[threadIdx.x];
+    }
     squares[threadIdx.x] = square_sum(held);
     __syncthreads();
     if (threadIdx.x < 256) {
@@ -318,8 +359,22 @@ hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const 
                                    uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream) {
     if (columns % 256 != 0 || vectors > 0x7fffffffull) return hipErrorInvalidValue;
     if (vectors == 0 || columns == 0) return hipSuccess;
-    hipLaunchKernelGGL(quantize_halves_rms_kernel, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream, x,
-                       x_row_stride, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
+    hipLaunchKernelGGL(quantize_halves_rms_kernel<false>, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream,
+                       x, x_row_stride, ShareSource{}, weight, eps, static_cast<uint32_t>(vectors),
+                       static_cast<uint32_t>(columns), tiles);
+    return hipGetLastError();
+}
+
+hipError_t quantize_tiles_rms_norm_of_shares(const float* shares, uint32_t share_count, uint64_t launch_rows,
+                                             const float* bias, const float* residual, float* y, const float* weight,
+                                             double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles,
+                                             hipStream_t stream) {
+    if (columns % 256 != 0 || vectors > 0x7fffffffull || share_count == 0 || launch_rows < columns || launch_rows % 4 != 0)
+        return hipErrorInvalidValue;
+    if (vectors == 0 || columns == 0) return hipSuccess;
+    const ShareSource source = {shares, share_count, launch_rows, launch_rows * vectors, bias, residual};
+    hipLaunchKernelGGL(quantize_halves_rms_kernel<true>, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream,
+                       y, columns, source, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
 }
 

@@ -478,6 +478,63 @@ int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, co
     return ET_OK;
 }
 
+int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* prepared, const uint8_t* weight,
+                                      const float* bias, const float* residual, float* y, void* workspace,
+                                      uint64_t workspace_bytes, const et_linear_plan& next, const float* norm_weight,
+                                      double eps, void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                      const volatile int32_t* cancel, std::string* error) {
+    if (next.columns != plan.rows || next.vectors != plan.vectors)
+        return fail(error, ET_ERR_INVALID,
+                    "quantized_linear: the next contraction must take this one's result: " + std::to_string(plan.vectors) +
+                        " x " + std::to_string(plan.rows) + " against " + std::to_string(next.vectors) + " x " +
+                        std::to_string(next.columns));
+    if (!fused_prepare(next))
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "quantized_linear: this plan's prepared input cannot be computed from an operator on the fly");
+    if (!(eps == eps)) return fail(error, ET_ERR_INVALID, "quantized_linear: rms norm epsilon is not a number");
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (y == nullptr || !aligned(y) || !aligned(residual) || !aligned(bias) || !aligned(norm_weight) || !aligned(next_prepared))
+        return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
+    if (next_prepared == nullptr || next_prepared_bytes < prepared_input_bytes(next))
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: prepared-input buffer of " + std::to_string(next_prepared_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(prepared_input_bytes(next)) +
+                                                 " required");
+    // Only a gemm_h16 launch with K shares has a second launch to fold the norm into; every other
+    // plan runs the two steps one after the other.
+    const bool shares = plan.kernel == LinearKernel::kGemmHalf && plan.k_splits > 1;
+    if (!shares) {
+        if (int status = linear_enqueue_prepared(plan, prepared, weight, bias, residual, y, workspace, workspace_bytes, stream,
+                                                 cancel, error))
+            return status;
+        et_prepare_source source = {};
+        source.kind = ET_PREPARE_RMS_NORM;
+        source.x = y;
+        source.x_row_stride = plan.rows;
+        source.second = norm_weight;
+        source.eps = eps;
+        return linear_prepare_input_from(next, source, next_prepared, next_prepared_bytes, stream, error);
+    }
+    if ((bias != nullptr) != plan.has_bias)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias does not match the immutable plan");
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (prepared == nullptr || weight == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: NULL operand");
+    if (workspace == nullptr || workspace_bytes < plan.workspace_bytes)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                                                 " bytes is smaller than the planned " + std::to_string(plan.workspace_bytes));
+    float* partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + plan.partial_offset);
+    const GemmShares layout = gemm_h16_shares_layout(plan.codec, plan.rows, plan.columns, plan.vectors);
+    if (layout.count != plan.k_splits) return fail(error, ET_ERR_EXECUTION, "quantized_linear: K shares do not match the plan");
+    GemmOutput out = {bias, residual, y, partials};
+    out.leave_shares = true;
+    if (hipError_t status = contract_tiles(plan, weight, static_cast<const uint8_t*>(prepared), out, as_stream(stream)))
+        return hip_failure(error, "quantized_linear", status);
+    if (hipError_t status = quantize_tiles_rms_norm_of_shares(partials, layout.count, layout.launch_rows, bias, residual, y,
+                                                              norm_weight, eps, plan.vectors, plan.rows,
+                                                              static_cast<uint8_t*>(next_prepared), as_stream(stream)))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
 int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
                    const uint8_t* weight, const float* bias, float* y, void* workspace,
                    uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,

@@ -111,6 +111,13 @@ int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t c
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                             const volatile int32_t* cancel, std::string* error);
+// linear_enqueue_prepared, then the prepared input of rms_norm(y) * norm_weight for `next` (see
+// et_hip_linear_enqueue_prepared_then_norm in et_hip.h).
+int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* prepared, const uint8_t* weight,
+                                      const float* bias, const float* residual, float* y, void* workspace,
+                                      uint64_t workspace_bytes, const et_linear_plan& next, const float* norm_weight,
+                                      double eps, void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                      const volatile int32_t* cancel, std::string* error);
 
 int embedding_requirements(const TensorView& indexes, const TensorView& weight, int32_t codec,
                            uint64_t rows, uint64_t columns, et_embedding_plan* plan,

@@ -375,6 +375,24 @@ class RawLinear:
             bias.data_ptr() if bias is not None else None, residual.data_ptr() if residual is not None else None,
             y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
 
+    def enqueue_prepared_then_norm(self, prepared: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                                   y: torch.Tensor, workspace: Optional[torch.Tensor], following: "RawLinear",
+                                   norm_weight: Optional[torch.Tensor], eps: float, next_prepared: torch.Tensor,
+                                   residual: Optional[torch.Tensor] = None, stream=None,
+                                   cancelled: Optional[CancellationFlag] = None) -> None:
+        """:meth:`enqueue_prepared`, then ``next_prepared`` = the prepared input of
+        ``rms_norm(y) * norm_weight`` for ``following`` (``et_hip_linear_enqueue_prepared_then_norm``):
+        the same bytes as the two calls, one launch less where this plan shares K over workgroups."""
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+        _check(N.lib().et_hip_linear_enqueue_prepared_then_norm(
+            self.requirements._handle, prepared.data_ptr(), weight.data_ptr(),
+            bias.data_ptr() if bias is not None else None, residual.data_ptr() if residual is not None else None,
+            y.data_ptr(), ws_ptr, ws_bytes, following.requirements._handle,
+            norm_weight.data_ptr() if norm_weight is not None else None, float(eps), next_prepared.data_ptr(),
+            next_prepared.numel() * next_prepared.element_size(), _stream_handle(stream),
+            cancelled.ptr if cancelled is not None else None))
+
 
 class LinearGroup:
     """Up to four :class:`RawLinear` plans of the same columns and vectors that run from one prepared

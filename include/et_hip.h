@@ -213,6 +213,22 @@ int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepa
                                    float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                                    const volatile int32_t* cancel);
 
+/* et_hip_linear_enqueue_prepared, then the prepared input of rms_norm(y) * norm_weight for the
+ * contraction that comes next (`next`: columns = this plan's rows, the same vectors,
+ * et_hip_linear_plan_fused_prepare(next) != 0) - the residual stream of a transformer layer: y = x W
+ * + residual, then the next block's norm. y and next_prepared receive the bytes of
+ * et_hip_linear_enqueue_prepared followed by et_hip_linear_prepare_input_from(ET_PREPARE_RMS_NORM).
+ * Where this plan shares K over workgroups, the launch that would only sum the shares sums them,
+ * writes y, norms and quantises: one launch less. Other plans run the two steps one after the
+ * other. norm_weight: [rows] f32 or NULL. No counterpart in the reference, whose executor runs one
+ * operator at a time. */
+int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
+                                             const uint8_t* weight, const float* bias, const float* residual,
+                                             float* y, void* workspace, uint64_t workspace_bytes,
+                                             const et_linear_plan* next, const float* norm_weight, double eps,
+                                             void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                             const volatile int32_t* cancel);
+
 /* ---- quantized_embedding (= bit-exact dequantisation of selected rows) ---- */
 
 /* Plan step = embedding_requirements (crates/runtime-cpu/src/quantized.rs:340-365).

@@ -644,6 +644,50 @@ def test_group_launch_of_contractions_sharing_their_input(et, device):
         et.LinearGroup([et.RawLinear(et.GgmlQuant.Q4_K, 64, columns, 2)])
 
 
+def test_contraction_then_norm_prepared_input_in_the_reduction_launch(et, device):
+    # y = W x + residual, then the next block's norm inside the quantiser: where the contraction shares
+    # K over workgroups the launch that sums the shares also writes y, norms and quantises - the same
+    # bytes as the two calls, for y and for the prepared input
+    rng = np.random.default_rng(91)
+    vectors = 33
+    # (rows, columns, bias, K shares?) - 14336 rows fill the device without shares: the two steps in turn
+    for rows, columns, with_bias, shares in ((4096, 4096, False, True), (4096, 14336, True, True),
+                                            (2560, 1024, False, True), (14336, 4096, False, False)):
+        plan = et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors, with_bias)
+        following = et.RawLinear(et.GgmlQuant.Q4_K, 64, rows, vectors)
+        assert ("reduce" in plan.requirements.kernel) == shares
+        weight = to_dev(synth.random_weight(oracle.Q4_K, rows, columns, rng), device)
+        x = to_dev(synth.random_activations(vectors, columns, rng), device)
+        bias = to_dev(rng.standard_normal(rows).astype(np.float32), device) if with_bias else None
+        norm_weight = to_dev(rng.standard_normal(rows).astype(np.float32), device)
+        stream_in = to_dev(rng.standard_normal((vectors, rows)).astype(np.float32), device)
+        prepared = torch.empty(plan.prepared_input_bytes, dtype=torch.uint8, device=device)
+        plan.prepare_input(x, prepared)
+        workspace = torch.empty(max(plan.requirements.workspace_bytes, 16), dtype=torch.uint8, device=device)
+        for w in (norm_weight, None):
+            # in place, as a residual stream is updated
+            y_two, y_one = stream_in.clone(), stream_in.clone()
+            next_two, next_one = (torch.zeros(following.prepared_input_bytes, dtype=torch.uint8, device=device)
+                                  for _ in range(2))
+            plan.enqueue_prepared(prepared, weight, bias, y_two, workspace, residual=y_two)
+            following.prepare_input_rms_norm(y_two, w, 1e-5, next_two)
+            plan.enqueue_prepared_then_norm(prepared, weight, bias, y_one, workspace, following, w, 1e-5, next_one,
+                                            residual=y_one)
+            assert torch.equal(y_two, y_one)
+            assert torch.equal(next_two, next_one)
+        # without a residual, into a fresh y
+        y_two, y_one = torch.empty((vectors, rows), device=device), torch.full((vectors, rows), float("nan"), device=device)
+        plan.enqueue_prepared(prepared, weight, bias, y_two, workspace)
+        following.prepare_input_rms_norm(y_two, norm_weight, 1e-5, next_two)
+        plan.enqueue_prepared_then_norm(prepared, weight, bias, y_one, workspace, following, norm_weight, 1e-5, next_one)
+        assert torch.equal(y_two, y_one) and torch.equal(next_two, next_one)
+    # the next contraction must take this one's result, and be able to prepare from an operator
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, 4096, 4096, vectors)
+    with pytest.raises(et.QuantizedError, match="must take this one's result"):
+        plan.enqueue_prepared_then_norm(prepared, weight, None, y_one, workspace, et.RawLinear(et.GgmlQuant.Q4_K, 64, 512, vectors),
+                                        None, 1e-5, next_one)
+
+
 # --------------------------------------------------------------------------- measurement aids
 
 @pytest.mark.parametrize("kind,per_round,elements", [("i8", 32.0, 64), ("i8_scaled", 16.0, 64), ("i8_scaled_bf16", 16.0, 64), ("f16", 16.0, 64),
