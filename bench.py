@@ -620,7 +620,9 @@ def llama_decode(args, et):
             et.rms_norm_into(x, norms[index][0], 1e-5, h)
         if fused:
             if on_the_fly:
-                qkv_group.enqueue_prepared(shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v], group_ws)
+                # q and k rotated at the slots' cursors in the launch that sums the group's K shares
+                qkv_group.enqueue_prepared_then_rotary(shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v], group_ws,
+                                                       (0, 1), cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, width)
             else:
                 plans["wq"].prepare_input(h, shared_hidden)
                 plans["wq"].enqueue_prepared(shared_hidden, w["wq"], None, q, linear_ws)
@@ -631,7 +633,9 @@ def llama_decode(args, et):
             plans["wk"].enqueue(h, w["wk"], None, k, linear_ws)
             plans["wv"].enqueue(h, w["wv"], None, v, linear_ws)
         q4, k4, v4 = q.view(slots, heads, 1, width), k.view(slots, kv_heads, 1, width), v.view(slots, kv_heads, 1, width)
-        if fused:
+        if on_the_fly:
+            pass  # rotated above
+        elif fused:
             et.rotary_pair_into(q4, k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4, k4)
         else:
             et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)

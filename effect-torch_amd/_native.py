@@ -49,6 +49,20 @@ class EtPrepareSource(ctypes.Structure):
 PREPARE_PLAIN, PREPARE_RMS_NORM, PREPARE_SILU_MUL = 0, 1, 2
 
 
+class EtRotaryAfter(ctypes.Structure):
+    """``et_rotary_after`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("members", ctypes.c_uint32),
+        ("offsets", ctypes.c_void_p),
+        ("offsets_len", ctypes.c_uint64),
+        ("theta", ctypes.c_double),
+        ("sign", ctypes.c_double),
+        ("layout", ctypes.c_int32),
+        ("head_dim", ctypes.c_uint64),
+    ]
+
+
 class EtKvLayer(ctypes.Structure):
     """``et_kv_layer`` of include/et_hip.h."""
 
@@ -120,6 +134,8 @@ SIGNATURES = {
                                                             _vp, _vp]),
     "et_hip_linear_prepare_input_from": (ctypes.c_int, [_vp, ctypes.POINTER(EtPrepareSource), _vp, _u64, _vp]),
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
+    "et_hip_linear_enqueue_prepared_group_then_rotary": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp,
+                                                                        _u64, ctypes.POINTER(EtRotaryAfter), _vp, _vp]),
     "et_hip_linear_enqueue_prepared_then_norm": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp,
                                                                 ctypes.c_double, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),

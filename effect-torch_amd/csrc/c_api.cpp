@@ -251,6 +251,23 @@ int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepa
     });
 }
 
+int et_hip_linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans, uint32_t count,
+                                                     const void* prepared, const uint8_t* const* weights,
+                                                     const float* const* biases, const float* const* residuals,
+                                                     float* const* ys, void* workspace, uint64_t workspace_bytes,
+                                                     const et_rotary_after* rotary, void* stream,
+                                                     const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (rotary == nullptr) {
+            *error = "rotary: NULL descriptor";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_enqueue_prepared_group_then_rotary(plans, count, prepared, weights, biases, residuals,
+                                                                        ys, workspace, workspace_bytes, *rotary, stream,
+                                                                        cancel, error);
+    });
+}
+
 int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
                                              const uint8_t* weight, const float* bias, const float* residual,
                                              float* y, void* workspace, uint64_t workspace_bytes,

@@ -56,6 +56,21 @@ __device__ __forceinline__ float4 rms_four(const float4& v, double scale, const 
                        rms_one(v.w, scale, w.w));
 }
 
+// One pair of rotary_forward_into_impl (crates/runtime-cpu/src/composed.rs:2683-2729): position =
+// offset + step, angle = sign * position * theta^(-2 index / head_dim), everything in f64, each
+// result rounded once.
+__device__ __forceinline__ void rotate_pair(float a_in, float b_in, uint32_t offset, uint32_t step, uint32_t index,
+                                            uint32_t head_dim, double theta, double sign, float& lo, float& hi) {
+#pragma clang fp contract(off)  // every product and sum rounded on its own, whatever the file's setting
+    const double angle = sign * static_cast<double>(static_cast<uint64_t>(offset) + step) *
+                         pow(theta, -2.0 * static_cast<double>(index) / static_cast<double>(head_dim));
+    double s, c;
+    sincos(angle, &s, &c);
+    const double a = a_in, b = b_in;
+    lo = static_cast<float>(a * c - b * s);
+    hi = static_cast<float>(b * c + a * s);
+}
+
 // Tensor.silu (packages/core/src/Tensor.ts:1537-1540) times the up projection. Tensor.sigmoid is
 // tanh(x / 2) / 2 + 1 / 2, every step rounded to f32 (Tensor.ts:1240-1245).
 __device__ __forceinline__ float silu_mul_one(float gate, float up) {

@@ -84,16 +84,13 @@ __global__ __launch_bounds__(256) void rotary_kernel(RotaryTensor first, RotaryT
     const uint32_t step = static_cast<uint32_t>(row_step % steps);
     const uint64_t row = row_step / steps;
     const uint32_t offset = offsets_len == 1 ? offsets[0] : offsets[row / rows_per_batch];
-    const double angle = sign * static_cast<double>(static_cast<uint64_t>(offset) + step) *
-                         pow(theta, -2.0 * static_cast<double>(index) / static_cast<double>(head_dim));
-    double s, c;
-    sincos(angle, &s, &c);
     const uint64_t base = row_step * head_dim;
     const uint64_t lo = interleaved ? base + 2 * index : base + index;
     const uint64_t hi = interleaved ? base + 2 * index + 1 : base + half + index;
-    const double a = x[lo], b = x[hi];
-    out[lo] = static_cast<float>(a * c - b * s);
-    out[hi] = static_cast<float>(b * c + a * s);
+    float rotated_lo, rotated_hi;
+    rotate_pair(x[lo], x[hi], offset, step, index, head_dim, theta, sign, rotated_lo, rotated_hi);
+    out[lo] = rotated_lo;
+    out[hi] = rotated_hi;
 }
 
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,

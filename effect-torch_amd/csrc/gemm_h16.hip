@@ -25,6 +25,7 @@
 
 #include <cstdint>
 
+#include "decode_math.h"
 #include "et_codecs.h"
 #include "gemv_common.h"
 #include "kernels.h"
@@ -568,6 +569,53 @@ __global__ __launch_bounds__(256) void reduce_group_kernel(const Group group, co
     }
 }
 
+// reduce_group_kernel with a rotary embedding behind the sums of the members it names: a thread sums
+// the two elements of one rotary pair (of any two neighbouring rows for the other members), adds bias
+// and residual as reduce_group_kernel does, rotates with rotary_kernel's arithmetic and stores - the
+// bytes of the reduction followed by the rotary launch.
+__global__ __launch_bounds__(256) void reduce_group_rotary_kernel(const Group group, const float* __restrict__ partials,
+                                                                  uint32_t vectors, uint32_t k_splits, uint32_t kRows,
+                                                                  const GemmRotary rotary) {
+    const uint64_t launch_rows = static_cast<uint64_t>(group.row_tiles) * kRows;
+    const uint64_t item = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= launch_rows / 2 * vectors) return;
+    const uint32_t m = static_cast<uint32_t>(item / (launch_rows / 2));
+    const uint32_t launch_row = static_cast<uint32_t>(item - m * (launch_rows / 2)) * 2u;
+    const uint32_t row_tile = launch_row / kRows;
+    uint32_t which = 0;
+    for (uint32_t i = 1; i < group.count; i++)
+        if (row_tile >= group.member[i].first_tile) which = i;
+    const Member& member = group.member[which];
+    const uint32_t first_row = member.first_tile * kRows;
+    const uint32_t n = launch_row - first_row;  // even
+    if (n >= member.rows) return;
+    const bool rotate = (rotary.members >> which) & 1u;
+    const uint32_t half = rotary.head_dim / 2;
+    uint32_t lo = n, hi = n + 1u, index = 0;
+    if (rotate) {
+        const uint32_t pair = n / 2u, head = pair / half;
+        index = pair - head * half;
+        lo = rotary.interleaved ? head * rotary.head_dim + 2u * index : head * rotary.head_dim + index;
+        hi = rotary.interleaved ? lo + 1u : lo + half;
+    }
+    const uint64_t share_stride = launch_rows * vectors;
+    const auto summed = [&](uint32_t row) {
+        const float* first = partials + m * launch_rows + first_row + row;
+        float total = first[0];
+        for (uint32_t k = 1; k < k_splits; k++) total += first[k * share_stride];
+        const float with_bias = member.bias != nullptr ? total + member.bias[row] : total;
+        return member.residual != nullptr ? with_bias + member.residual[static_cast<uint64_t>(m) * member.rows + row]
+                                          : with_bias;
+    };
+    float value_lo = summed(lo), value_hi = hi < member.rows ? summed(hi) : 0.f;
+    if (rotate) {
+        const uint32_t offset = rotary.offsets_len == 1 ? rotary.offsets[0] : rotary.offsets[m];
+        rotate_pair(value_lo, value_hi, offset, 0u, index, rotary.head_dim, rotary.theta, rotary.sign, value_lo, value_hi);
+    }
+    member.y[static_cast<uint64_t>(m) * member.rows + lo] = value_lo;
+    if (hi < member.rows) member.y[static_cast<uint64_t>(m) * member.rows + hi] = value_hi;
+}
+
 }  // namespace
 
 bool gemm_h16_supported(int32_t codec, uint64_t columns) {
@@ -610,7 +658,8 @@ uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint3
 namespace {
 template <int CODEC, int RG, int AX, int AW>
 hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
-                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares) {
+                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares,
+                        const GemmRotary* rotary) {
     using S = Shape<CODEC, RG, AX, AW>;
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW>;
@@ -641,7 +690,11 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, group, tiles,
                        vector_tiles, columns, vectors, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
-    if (k_splits > 1 && !leave_shares) {
+    if (k_splits > 1 && !leave_shares && rotary != nullptr) {
+        const uint64_t pairs = row_tiles * S::kRows / 2 * vectors;
+        hipLaunchKernelGGL(reduce_group_rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0,
+                           stream, group, partials, vectors, k_splits, S::kRows, *rotary);
+    } else if (k_splits > 1 && !leave_shares) {
         const uint64_t items = row_tiles * S::kRows * vectors / 4;
         hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
                            group, partials, vectors, k_splits, S::kRows);
@@ -657,7 +710,7 @@ GemmShares gemm_h16_shares_layout(int32_t codec, uint64_t rows, uint64_t columns
 
 hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
                           float* partials, uint64_t columns64, uint64_t vectors64, hipStream_t stream,
-                          bool leave_shares) {
+                          bool leave_shares, const GemmRotary* rotary) {
     if (!gemm_h16_supported(codec, columns64)) return hipErrorInvalidValue;
     if (count == 0 || count > kGemmGroupMost || columns64 % 256 != 0 || columns64 == 0) return hipErrorInvalidValue;
     const uint32_t columns = static_cast<uint32_t>(columns64), vectors = static_cast<uint32_t>(vectors64);
@@ -667,30 +720,32 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
         rows[i] = members[i].rows;
     }
     GemmGroupGeometry g = gemm_h16_group_geometry(codec, rows, count, columns, vectors);
+    // the rotary rides on the launch that sums K shares: without shares the caller rotates itself
+    if (rotary != nullptr && (g.k_splits == 1 || partials == nullptr)) return hipErrorInvalidValue;
     if (partials == nullptr && g.k_splits > 1) {  // nowhere to keep shares: 64-row workgroups, whole K each
         g = GemmGroupGeometry{64, 0, 1};
     }
     // weight lead: what the activation ring (three slots of 34 KiB) leaves of LDS
     if (codec == kQ6_K)  // 64-row tiles only (gemm_h16_group_geometry): 128 rows of 224 bytes leave no room for a ring
-        return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+        return launch_group<kQ6_K, 2, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
     if (codec == kQ2_K || codec == kQ3_K) {  // rows of 96 / 112 bytes per stage: room for the longest lead
         if (codec == kQ2_K) {
             if (g.tile_rows == 128)
-                return launch_group<kQ2_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
-            return launch_group<kQ2_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+                return launch_group<kQ2_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+            return launch_group<kQ2_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
         }
         if (g.tile_rows == 128)
-            return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
-        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+            return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
     }
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
-            return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
-        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+            return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
     }
     if (g.tile_rows == 128)
-        return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
-    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares);
+        return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,

@@ -143,9 +143,20 @@ GemmGroupGeometry gemm_h16_group_geometry(int32_t codec, const uint64_t* rows, u
                                           uint64_t vectors);
 uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint32_t count, uint64_t columns,
                                       uint64_t vectors);
+// A rotary embedding applied to some members of a group launch in the launch that sums their K
+// shares: member i with bit i of `members` set is [vectors, rows / head_dim heads, 1 step, head_dim]
+// at positions offsets[0] or offsets[vector] (rotary_kernel's arithmetic, decode_math.h).
+struct GemmRotary {
+    uint32_t members;
+    const uint32_t* offsets;
+    uint32_t offsets_len;
+    double theta, sign;
+    int interleaved;
+    uint32_t head_dim;
+};
 hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t count, const uint8_t* tiles,
                           float* partials, uint64_t columns, uint64_t vectors, hipStream_t stream,
-                          bool leave_shares = false);
+                          bool leave_shares = false, const GemmRotary* rotary = nullptr);
 // Where a one-matrix launch with K shares leaves them: share k, vector m, row n at
 // partials[(k * vectors + m) * launch_rows + n].
 struct GemmShares {

@@ -454,6 +454,72 @@ int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t c
     return ET_OK;
 }
 
+int linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                              const uint8_t* const* weights, const float* const* biases,
+                                              const float* const* residuals, float* const* ys, void* workspace,
+                                              uint64_t workspace_bytes, const et_rotary_after& rotary, void* stream,
+                                              const volatile int32_t* cancel, std::string* error) {
+    if (int rc = check_group(plans, count, error)) return rc;
+    if (rotary.layout != ET_ROTARY_HALF_SPLIT && rotary.layout != ET_ROTARY_INTERLEAVED_PAIRS)
+        return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(rotary.layout));
+    const uint64_t vectors = plans[0]->vectors;
+    if (rotary.head_dim == 0 || rotary.head_dim % 2 != 0 || rotary.head_dim > 0xffffffffull)
+        return fail(error, ET_ERR_UNSUPPORTED, "rotary: expected a float rank >= 2 tensor with even head dimension");
+    if (rotary.offsets_len != 1 && rotary.offsets_len != vectors)
+        return fail(error, ET_ERR_UNSUPPORTED, "rotary embedding: " + std::to_string(rotary.offsets_len) +
+                                                   " offsets for batch " + std::to_string(vectors));
+    if (rotary.members >> count != 0) return fail(error, ET_ERR_INVALID, "rotary: the group has no such member");
+    for (uint32_t i = 0; i < count; i++)
+        if (((rotary.members >> i) & 1u) && plans[i]->rows % rotary.head_dim != 0)
+            return fail(error, ET_ERR_UNSUPPORTED, "rotary: " + std::to_string(plans[i]->rows) +
+                                                       " rows are not whole heads of " + std::to_string(rotary.head_dim));
+    if (rotary.members != 0 && vectors != 0 && rotary.offsets == nullptr)
+        return fail(error, ET_ERR_INVALID, "rotary: NULL device pointer");
+    uint64_t rows[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) rows[i] = plans[i]->rows;
+    const bool shares =
+        gemm_h16_group_geometry(plans[0]->codec, rows, count, plans[0]->columns, vectors).k_splits > 1 && rotary.members != 0;
+    if (!shares) {
+        // no second launch to ride on: the group, then the rotary launches
+        if (int rc = linear_enqueue_prepared_group(plans, count, prepared, weights, biases, residuals, ys, workspace,
+                                                   workspace_bytes, stream, cancel, error))
+            return rc;
+        for (uint32_t i = 0; i < count && vectors != 0; i++)
+            if ((rotary.members >> i) & 1u)
+                if (hipError_t status = et::rotary(ys[i], rotary.offsets, static_cast<uint32_t>(rotary.offsets_len), rotary.theta,
+                                                   rotary.sign, rotary.layout == ET_ROTARY_INTERLEAVED_PAIRS, ys[i], vectors,
+                                                   vectors * (plans[i]->rows / rotary.head_dim), 1, rotary.head_dim,
+                                                   as_stream(stream)))
+                    return hip_failure(error, "rotary", status);
+        return ET_OK;
+    }
+    if (weights == nullptr || ys == nullptr || prepared == nullptr)
+        return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+    GemmMember members[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) {
+        const float* bias = biases != nullptr ? biases[i] : nullptr;
+        if ((bias != nullptr) != plans[i]->has_bias)
+            return fail(error, ET_ERR_EXECUTION, "quantized_linear: bias presence does not match the immutable plan");
+        if (weights[i] == nullptr || ys[i] == nullptr)
+            return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+        members[i] = GemmMember{weights[i], bias, residuals != nullptr ? residuals[i] : nullptr, ys[i], plans[i]->rows};
+    }
+    if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    if (vectors == 0) return ET_OK;
+    const uint64_t need = group_partial_bytes(plans, count);
+    if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(need) + " the group needs");
+    const GemmRotary after = {rotary.members, rotary.offsets, static_cast<uint32_t>(rotary.offsets_len), rotary.theta,
+                              rotary.sign, rotary.layout == ET_ROTARY_INTERLEAVED_PAIRS,
+                              static_cast<uint32_t>(rotary.head_dim)};
+    if (hipError_t status = gemm_h16_group(plans[0]->codec, members, count, static_cast<const uint8_t*>(prepared),
+                                           static_cast<float*>(workspace), plans[0]->columns, vectors, as_stream(stream),
+                                           false, &after))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                             const volatile int32_t* cancel, std::string* error) {

@@ -108,6 +108,13 @@ int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t c
                                   uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel,
                                   std::string* error);
 // y = W x (+ bias) (+ residual, which may be y itself) from a prepared input.
+// linear_enqueue_prepared_group, then a rotary embedding of the members named by `rotary.members`
+// (see et_hip_linear_enqueue_prepared_group_then_rotary in et_hip.h).
+int linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                              const uint8_t* const* weights, const float* const* biases,
+                                              const float* const* residuals, float* const* ys, void* workspace,
+                                              uint64_t workspace_bytes, const et_rotary_after& rotary, void* stream,
+                                              const volatile int32_t* cancel, std::string* error);
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                             const volatile int32_t* cancel, std::string* error);

@@ -421,6 +421,35 @@ class LinearGroup:
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
 
+    def enqueue_prepared_then_rotary(self, prepared: torch.Tensor, weights: Sequence[torch.Tensor],
+                                     ys: Sequence[torch.Tensor], workspace: Optional[torch.Tensor],
+                                     rotate: Sequence[int], offsets: torch.Tensor, theta: float, sign: float, layout: int,
+                                     head_dim: int, biases=None, residuals=None, stream=None,
+                                     cancelled: Optional[CancellationFlag] = None) -> None:
+        """:meth:`enqueue_prepared`, then the rotary embedding in place on the results of the members
+        listed in ``rotate`` (``[vectors, rows / head_dim, 1, head_dim]`` at ``offsets``), in the launch
+        that sums the K shares where there is one (``et_hip_linear_enqueue_prepared_group_then_rotary``)."""
+        _group_then_rotary(self, prepared, weights, ys, workspace, rotate, offsets, theta, sign, layout, head_dim,
+                           biases, residuals, stream, cancelled)
+
+
+def _group_then_rotary(group: "LinearGroup", prepared, weights, ys, workspace, rotate, offsets, theta, sign, layout,
+                       head_dim, biases, residuals, stream, cancelled) -> None:
+    count = len(group.plans)
+    pointers = lambda tensors: (ctypes.c_void_p * count)(  # noqa: E731
+        *[t.data_ptr() if t is not None else None for t in tensors])
+    if offsets.dtype not in (torch.uint32, torch.int32) or not offsets.is_contiguous():
+        raise ValueError("rotary offsets must be a contiguous u32 device tensor")
+    after = N.EtRotaryAfter(sum(1 << i for i in rotate), offsets.data_ptr(), offsets.numel(), float(theta), float(sign),
+                            int(layout), int(head_dim))
+    _check(N.lib().et_hip_linear_enqueue_prepared_group_then_rotary(
+        group._handles, count, prepared.data_ptr(), pointers(weights),
+        pointers(biases) if biases is not None else None,
+        pointers(residuals) if residuals is not None else None, pointers(ys),
+        workspace.data_ptr() if workspace is not None else None,
+        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+        ctypes.byref(after), _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
+
 
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""

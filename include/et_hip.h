@@ -358,6 +358,27 @@ int et_hip_rotary_pair_into(const et_tensor* x, const et_tensor* second, const u
                             uint64_t offsets_len, double theta, double sign, int32_t layout,
                             const et_tensor* destination, const et_tensor* second_destination,
                             void* stream);
+/* et_hip_linear_enqueue_prepared_group, then et_hip_rotary_into in place on the results of the
+ * members whose bit is set in `members` (bit i = plans[i]), each seen as [vectors, rows / head_dim,
+ * 1, head_dim] at offsets[0] or offsets[vector] - the q and k projections of a decode step at the
+ * slots' cursors. The ys receive the bytes of the two steps. Where the group shares K over
+ * workgroups, the launch that sums the shares also rotates (one launch less); other groups run the
+ * steps one after the other. No counterpart in the reference, whose executor runs one operator at a
+ * time. */
+typedef struct et_rotary_after {
+    uint32_t members;
+    const uint32_t* offsets;   /* DEVICE array of 1 or `vectors` u32 */
+    uint64_t offsets_len;
+    double theta, sign;
+    int32_t layout;            /* et_rotary_layout */
+    uint64_t head_dim;
+} et_rotary_after;
+int et_hip_linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans, uint32_t count,
+                                                     const void* prepared, const uint8_t* const* weights,
+                                                     const float* const* biases, const float* const* residuals,
+                                                     float* const* ys, void* workspace, uint64_t workspace_bytes,
+                                                     const et_rotary_after* rotary, void* stream,
+                                                     const volatile int32_t* cancel);
 
 /* out = a + b, f32, same shapes (the residual connections; the reference's binary
  * add without broadcasting, crates/runtime-cpu/src/ops.rs). `destination` may be `a`. */

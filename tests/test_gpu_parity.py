@@ -688,6 +688,53 @@ def test_contraction_then_norm_prepared_input_in_the_reduction_launch(et, device
                                         None, 1e-5, next_one)
 
 
+def test_group_launch_then_rotary_in_the_reduction_launch(et, device):
+    # q / k / v of a decode step: the launch that sums the group's K shares also rotates q and k at the
+    # slots' cursors - the bytes of the group launch followed by the rotary launch
+    rng = np.random.default_rng(92)
+    vectors, columns, head_dim = 32, 4096, 128
+    sizes = (4096, 1024, 1024)
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors) for rows in sizes]
+    group = et.LinearGroup(plans)
+    assert group.workspace_bytes > 0  # K shares
+    weights = [to_dev(synth.random_weight(oracle.Q4_K, rows, columns, rng), device) for rows in sizes]
+    x = to_dev(synth.random_activations(vectors, columns, rng), device)
+    prepared = torch.empty(plans[0].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[0].prepare_input(x, prepared)
+    workspace = torch.empty(group.workspace_bytes, dtype=torch.uint8, device=device)
+    cursors = to_dev(rng.integers(0, 4000, vectors).astype(np.uint32), device)
+    for layout in (et.RotaryLayout.HALF_SPLIT, et.RotaryLayout.INTERLEAVED_PAIRS):
+        for offsets in (cursors, cursors[:1].contiguous()):
+            two = [torch.empty((vectors, rows), device=device) for rows in sizes]
+            one = [torch.full((vectors, rows), float("nan"), device=device) for rows in sizes]
+            group.enqueue_prepared(prepared, weights, two, workspace)
+            q4, k4 = two[0].view(vectors, 32, 1, head_dim), two[1].view(vectors, 8, 1, head_dim)
+            et.rotary_pair_into(q4, k4, offsets, 500000.0, 1.0, layout, q4, k4)
+            group.enqueue_prepared_then_rotary(prepared, weights, one, workspace, (0, 1), offsets, 500000.0, 1.0, layout,
+                                               head_dim)
+            for a, b in zip(two, one):
+                assert torch.equal(a, b)
+    # a group without K shares runs the two steps in turn: the same bytes
+    big = [et.RawLinear(et.GgmlQuant.Q4_K, 14336, columns, vectors) for _ in range(2)]
+    pair = et.LinearGroup(big)
+    assert pair.workspace_bytes == 0
+    big_weights = [to_dev(synth.random_weight(oracle.Q4_K, 14336, columns, rng), device) for _ in range(2)]
+    two = [torch.empty((vectors, 14336), device=device) for _ in range(2)]
+    one = [torch.empty((vectors, 14336), device=device) for _ in range(2)]
+    pair.enqueue_prepared(prepared, big_weights, two)
+    first = two[0].view(vectors, 112, 1, head_dim)
+    et.rotary_into(first, cursors, 10000.0, -1.0, et.RotaryLayout.HALF_SPLIT, first)
+    pair.enqueue_prepared_then_rotary(prepared, big_weights, one, None, (0,), cursors, 10000.0, -1.0,
+                                      et.RotaryLayout.HALF_SPLIT, head_dim)
+    assert torch.equal(two[0], one[0]) and torch.equal(two[1], one[1])
+    with pytest.raises(et.QuantizedError, match="not whole heads"):
+        group.enqueue_prepared_then_rotary(prepared, weights, one, workspace, (0,), cursors, 500000.0, 1.0,
+                                           et.RotaryLayout.HALF_SPLIT, 96)
+    with pytest.raises(et.QuantizedError, match="offsets for batch"):
+        group.enqueue_prepared_then_rotary(prepared, weights, one, workspace, (0,), cursors[:5].contiguous(), 500000.0, 1.0,
+                                           et.RotaryLayout.HALF_SPLIT, head_dim)
+
+
 # --------------------------------------------------------------------------- measurement aids
 
 @pytest.mark.parametrize("kind,per_round,elements", [("i8", 32.0, 64), ("i8_scaled", 16.0, 64), ("i8_scaled_bf16", 16.0, 64), ("f16", 16.0, 64),
