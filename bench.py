@@ -640,11 +640,16 @@ def llama_decode(args, et):
         else:
             et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)
             et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
-        keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
-                                         workspace=kv_ws, synchronize=False))
+        if on_the_fly:
+            # the attention kernel quantises its result for Wo in its epilogue
+            keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
+                                             workspace=kv_ws, synchronize=False, prepared_for=plans["wo"],
+                                             prepared=shared_attended))
+        else:
+            keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
+                                             workspace=kv_ws, synchronize=False))
         if on_the_fly:
             # x += attended Wo, then the ffn norm inside the quantiser, in the launch that sums Wo's K shares
-            plans["wo"].prepare_input(attended, shared_attended)
             plans["wo"].enqueue_prepared_then_norm(shared_attended, w["wo"], None, x, linear_ws, plans["gate"],
                                                    norms[index][1], 1e-5, shared_hidden, residual=x)
         elif fused:

@@ -148,6 +148,8 @@ SIGNATURES = {
     "et_hip_dequantize_rows": (ctypes.c_int, [_i32, _u64, _u64, _vp, _vp, _vp]),
     "et_hip_kv_attention_workspace_bytes": (_u64, [_KV, _u64, _u64]),
     "et_hip_kv_attention_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp, _vp]),
+    "et_hip_kv_attention_prepared_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp,
+                                                         _vp, _u64, _vp, _vp]),
     "et_hip_kv_attention_status_check": (ctypes.c_int, [_KV, _u64, _vp]),
     "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
     "et_hip_rms_norm_into": (ctypes.c_int, [_T, _T, ctypes.c_double, _T, _vp]),

@@ -419,6 +419,27 @@ int et_hip_kv_attention_into(const et_kv_layer* layer, const et_tensor* q, const
     });
 }
 
+int et_hip_kv_attention_prepared_into(const et_kv_layer* layer, const et_tensor* q, const et_tensor* k,
+                                      const et_tensor* v, double scale, uint64_t window,
+                                      const et_tensor* destination, void* workspace, uint64_t workspace_bytes,
+                                      void* status, const et_linear_plan* consumer, void* prepared,
+                                      uint64_t prepared_bytes, void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (layer == nullptr || consumer == nullptr) {
+            *error = "kv attention: layer or plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        TensorView qv, kv, vv, dst;
+        if (!TensorView::from_c(q, &qv, error) || !TensorView::from_c(k, &kv, error) ||
+            !TensorView::from_c(v, &vv, error) || !TensorView::from_c(destination, &dst, error)) {
+            *error = "kv attention: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::kv::attention_into(*layer, qv, kv, vv, scale, window, dst, workspace, workspace_bytes, status,
+                                      stream, cancel, error, consumer, prepared, prepared_bytes);
+    });
+}
+
 int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens, const void* status_host) {
     return guarded([&](std::string* error) -> int {
         if (layer == nullptr || status_host == nullptr) {

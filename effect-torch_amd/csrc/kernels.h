@@ -195,6 +195,10 @@ struct KvAttention {
     double scale;
     float* out;                   // like q
     void* status;                 // 8 bytes per slot, written by the call
+    // Optional (tokens == 1): `out` seen as activations [batch, query_heads * width], quantised into
+    // gemm_h16's tiles (quantize_tiles with two halves) - by the attention kernel itself where one
+    // workgroup holds whole 256-column stages of a row, by a quantiser launch otherwise.
+    uint8_t* prepared = nullptr;
 };
 struct KvLaunchShape {
     bool streaming;

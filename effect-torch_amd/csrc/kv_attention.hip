@@ -28,6 +28,7 @@
 
 #include "et_hip.h"
 #include "kernels.h"
+#include "quantize_halves.h"
 
 namespace et {
 namespace {
@@ -62,6 +63,8 @@ struct KvArgs {
     uint32_t table_stride, active_batch, query_heads, tokens, context_window, window;
     uint32_t splits, max_context;
     float scale_log2;  // scale * log2(e)
+    uint8_t* prepared;       // see KvAttention::prepared; null = none, or a quantiser launch follows
+    uint32_t vector_tiles;   // of the prepared activations: ceil(batch / 32)
 };
 
 struct Span {
@@ -629,6 +632,11 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
     }
     __syncthreads();
     const uint32_t width = LPT * DPL;
+    // The G heads of this workgroup are G * width neighbouring columns of the slot's row of activations
+    // for the contraction that follows; where they are whole 256-column stages the rows' tiles are
+    // quantised here, from the values just stored (a skipped slot: from what the destination holds).
+    __shared__ __attribute__((aligned(16))) float row_part[G * width];
+    const bool quantise = a.prepared != nullptr && (G * width) % 256 == 0;
     for (uint32_t item = threadIdx.x; item < G * width; item += kThreads) {
         const uint32_t g = item / width, column = item % width;
         float top = kLowest;
@@ -641,7 +649,9 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
         }
         const uint64_t query = (static_cast<uint64_t>(slot) * a.query_heads + head0 + g) * a.tokens + token;
         if (a.splits == 1) {
-            if (s.ok) a.out[query * width + column] = value / total;
+            const float result = value / total;
+            if (s.ok) a.out[query * width + column] = result;
+            if (quantise) row_part[item] = s.ok ? result : a.out[query * width + column];
         } else {
             float* record = a.partial + (query * a.splits + split) * (width + 2);
             record[2 + column] = value;
@@ -649,6 +659,14 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
                 record[0] = top;
                 record[1] = total;
             }
+        }
+    }
+    if (quantise && a.splits == 1) {  // uniform: the launcher sets `prepared` only for one token per slot
+        __syncthreads();
+        const uint32_t wave = threadIdx.x >> 6, quad = threadIdx.x & 63u;
+        if (wave < G * width / 256u) {
+            const float4 in = *reinterpret_cast<const float4*>(&row_part[wave * 256u + 4u * quad]);
+            quantize_halves_store(in, slot, (head0 * width) / 256u + wave, quad, a.vector_tiles, a.prepared);
         }
     }
 }
@@ -922,6 +940,18 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
     const KvLaunchShape shape = kv_attention_shape(p);
     a.splits = shape.splits;
     a.partial = static_cast<float*>(workspace);
+    // The streaming kernel quantises the rows itself when it writes them in one piece (no context
+    // splits), every slot is active and its heads are whole stages; else a quantiser launch follows.
+    const bool fused_tiles = p.prepared != nullptr && p.tokens == 1 && shape.streaming && shape.splits == 1 &&
+                             p.active_batch == p.batch &&
+                             (static_cast<uint64_t>(streaming_group(p)) * p.width) % 256 == 0;
+    a.prepared = fused_tiles ? p.prepared : nullptr;
+    a.vector_tiles = (p.batch + 31u) / 32u;
+    const auto finish = [&](hipError_t error) -> hipError_t {
+        if (error != hipSuccess || p.prepared == nullptr || fused_tiles || p.batch == 0) return error;
+        const uint64_t columns = static_cast<uint64_t>(p.query_heads) * p.width;
+        return quantize_tiles(p.out, columns, p.batch, columns, 2, p.prepared, stream);
+    };
 
     // out.fill(0.0) for the slots that are not active (napi/mod.rs:3371); their status words too.
     const uint64_t per_slot = static_cast<uint64_t>(p.query_heads) * p.tokens * p.width;
@@ -931,7 +961,7 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
                            p.out + p.active_batch * per_slot, count, a.status + p.active_batch,
                            p.batch - p.active_batch);
     }
-    if (p.active_batch == 0) return hipGetLastError();
+    if (p.active_batch == 0) return finish(hipGetLastError());
 
     hipError_t error;
     if (shape.streaming) {
@@ -960,7 +990,7 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
         hipLaunchKernelGGL(kv_merge_kernel, dim3(static_cast<uint32_t>(queries)), dim3(threads), 0, stream, a);
         error = hipGetLastError();
     }
-    return error;
+    return finish(error);
 }
 
 }  // namespace et

@@ -92,7 +92,8 @@ const char* kernel_name(const et_kv_layer& layer, uint64_t query_heads, uint64_t
 int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, const quantized::TensorView& k,
                    const quantized::TensorView& v, double scale, uint64_t window,
                    const quantized::TensorView& destination, void* workspace, uint64_t workspace_bytes,
-                   void* status, void* stream, const volatile int32_t* cancel, std::string* error) {
+                   void* status, void* stream, const volatile int32_t* cancel, std::string* error,
+                   const et_linear_plan* consumer, void* prepared, uint64_t prepared_bytes) {
     // napi/mod.rs:3331-3344
     const size_t rank = q.shape.size();
     if (rank < 4 || q.dtype != ET_DTYPE_F32 || k.dtype != ET_DTYPE_F32 || v.dtype != ET_DTYPE_F32 ||
@@ -150,6 +151,24 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
     p.out = const_cast<float*>(static_cast<const float*>(destination.data)) + destination.offset;
     p.scale = scale;
     p.status = status;
+    if (consumer != nullptr) {
+        // the result as the activations of the contraction that follows: one row per slot
+        if (tokens != 1 || consumer->columns != query_heads * width || consumer->vectors != batch)
+            return fail(error, ET_ERR_UNSUPPORTED,
+                        "kv attention: the prepared input of a contraction takes one token per slot and [" +
+                            std::to_string(batch) + ", " + std::to_string(query_heads * width) + "] activations");
+        if (!quantized::fused_prepare(*consumer))
+            return fail(error, ET_ERR_UNSUPPORTED,
+                        "quantized_linear: this plan's prepared input cannot be computed from an operator on the fly");
+        if (prepared == nullptr || reinterpret_cast<uintptr_t>(prepared) % 16 != 0 ||
+            prepared_bytes < quantized::prepared_input_bytes(*consumer))
+            return fail(error, ET_ERR_EXECUTION, "quantized_linear: prepared-input buffer of " + std::to_string(prepared_bytes) +
+                                                     " bytes is smaller than the " +
+                                                     std::to_string(quantized::prepared_input_bytes(*consumer)) + " required");
+        if (reinterpret_cast<uintptr_t>(p.out) % 16 != 0)
+            return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
+        p.prepared = static_cast<uint8_t*>(prepared);
+    }
     const KvLaunchShape shape = kv_attention_shape(p);
     if (shape.streaming) {
         // the streaming kernel moves 16 bytes per lane

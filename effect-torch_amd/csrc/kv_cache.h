@@ -18,7 +18,8 @@ int workspace_bytes(const et_kv_layer& layer, uint64_t query_heads, uint64_t tok
 int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, const quantized::TensorView& k,
                    const quantized::TensorView& v, double scale, uint64_t window,
                    const quantized::TensorView& destination, void* workspace, uint64_t workspace_bytes,
-                   void* status, void* stream, const volatile int32_t* cancel, std::string* error);
+                   void* status, void* stream, const volatile int32_t* cancel, std::string* error,
+                   const et_linear_plan* consumer = nullptr, void* prepared = nullptr, uint64_t prepared_bytes = 0);
 int status_check(const et_kv_layer& layer, uint64_t tokens, const void* status_host, std::string* error);
 const char* kernel_name(const et_kv_layer& layer, uint64_t query_heads, uint64_t tokens);
 

@@ -90,11 +90,15 @@ def kv_attention_status_check(layer: KvLayer, tokens: int, status: torch.Tensor)
 def kv_attention_into(layer: KvLayer, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
                       window: Optional[int], destination: torch.Tensor, *,
                       workspace: Optional[torch.Tensor] = None, cancelled: Optional[CancellationFlag] = None,
-                      stream=None, synchronize: bool = True) -> Optional[torch.Tensor]:
+                      stream=None, synchronize: bool = True, prepared_for=None,
+                      prepared: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """kv_attention_into (napi/mod.rs:3320-3544): appends the new rows of ``k`` / ``v`` to the slabs,
     then attends. With ``synchronize`` (default) the stream is drained and a failed per-slot check
     raises the reference's error here; otherwise the device status block is returned for
-    :func:`kv_attention_status_check` after the caller's own fence."""
+    :func:`kv_attention_status_check` after the caller's own fence.
+
+    ``prepared_for`` (a :class:`RawLinear` whose activations are the result, one token per slot) and
+    ``prepared``: also leaves that plan's prepared input behind (``et_hip_kv_attention_prepared_into``)."""
     struct = layer.struct()
     tokens = q.shape[-2] if q.dim() >= 2 else 0
     heads = q.shape[-3] if q.dim() >= 3 else 0
@@ -105,11 +109,19 @@ def kv_attention_into(layer: KvLayer, q: torch.Tensor, k: torch.Tensor, v: torch
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=destination.device)
     status = torch.empty(8 * max(layer.cursors.numel(), 1), dtype=torch.uint8, device=destination.device)
     descs = (_desc(q), _desc(k), _desc(v), _desc(destination))
-    _check(N.lib().et_hip_kv_attention_into(ctypes.byref(struct), _ref(descs[0]), _ref(descs[1]), _ref(descs[2]),
-                                            float(scale), int(window or 0), _ref(descs[3]),
-                                            workspace.data_ptr(), workspace.numel(), status.data_ptr(),
-                                            _stream_handle(stream),
-                                            cancelled.ptr if cancelled is not None else None))
+    if prepared_for is not None:
+        _check(N.lib().et_hip_kv_attention_prepared_into(
+            ctypes.byref(struct), _ref(descs[0]), _ref(descs[1]), _ref(descs[2]), float(scale), int(window or 0),
+            _ref(descs[3]), workspace.data_ptr(), workspace.numel(), status.data_ptr(),
+            prepared_for.requirements._handle, prepared.data_ptr() if prepared is not None else None,
+            prepared.numel() * prepared.element_size() if prepared is not None else 0, _stream_handle(stream),
+            cancelled.ptr if cancelled is not None else None))
+    else:
+        _check(N.lib().et_hip_kv_attention_into(ctypes.byref(struct), _ref(descs[0]), _ref(descs[1]), _ref(descs[2]),
+                                                float(scale), int(window or 0), _ref(descs[3]),
+                                                workspace.data_ptr(), workspace.numel(), status.data_ptr(),
+                                                _stream_handle(stream),
+                                                cancelled.ptr if cancelled is not None else None))
     if not synchronize:
         return status
     kv_attention_status_check(layer, tokens, status)

@@ -321,6 +321,19 @@ int et_hip_kv_attention_into(const et_kv_layer* layer, const et_tensor* q, const
                              const et_tensor* destination, void* workspace,
                              uint64_t workspace_bytes, void* status, void* stream,
                              const volatile int32_t* cancel);
+/* et_hip_kv_attention_into for one token per slot, then the prepared input of the contraction that
+ * takes the result as its activations (`consumer`: et_hip_linear_plan_fused_prepare != 0, vectors =
+ * slots, columns = query_heads * head_dim - the output projection of a decode step): destination and
+ * `prepared` receive the bytes of et_hip_kv_attention_into followed by et_hip_linear_prepare_input.
+ * Where a workgroup of the attention kernel holds whole 256-column stages of a row and the context is
+ * not split, it quantises them in its epilogue (one launch less); otherwise the quantiser launch
+ * follows. No counterpart in the reference, whose executor runs one operator at a time. */
+int et_hip_kv_attention_prepared_into(const et_kv_layer* layer, const et_tensor* q, const et_tensor* k,
+                                      const et_tensor* v, double scale, uint64_t window,
+                                      const et_tensor* destination, void* workspace,
+                                      uint64_t workspace_bytes, void* status, const et_linear_plan* consumer,
+                                      void* prepared, uint64_t prepared_bytes, void* stream,
+                                      const volatile int32_t* cancel);
 /* After the stream has completed and `status` has been copied to the host: 0, or
  * ET_ERR_EXECUTION with the reference's message for the first failing slot, e.g.
  * "kv attention: advance {a} out of range for chunk length {tokens}"

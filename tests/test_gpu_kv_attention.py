@@ -284,3 +284,56 @@ def test_decode_batch_at_full_size(et, device, dtype):
             values = v_after[rows].astype(np.float64)
         mean = values.mean(axis=0)  # [kv_heads, width]
         assert np.abs(out[b, :, 0] - np.repeat(mean, 4, axis=0)).max() <= OUT_TOL
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, "u8"])
+@pytest.mark.parametrize("slots,kv_heads,group,width,contexts_top", [
+    (32, 8, 4, 128, 150),    # eight-wave workgroups, four heads = two stages each: quantised in the epilogue
+    (33, 8, 8, 64, 150),     # eight heads of 64 = two stages; a ragged last tile of vectors
+    (32, 8, 1, 128, 150),    # one head = half a stage: the quantiser launch follows
+    (8, 2, 4, 128, 3000),    # few rows: context splits + merge, then the quantiser launch
+])
+def test_prepared_input_of_the_next_contraction_from_the_attention_launch(et, device, dtype, slots, kv_heads, group,
+                                                                          width, contexts_top):
+    # the result as the activations of the output projection: the same bytes as kv_attention_into
+    # followed by prepare_input, for the destination, the slabs and the prepared tiles
+    rng = np.random.default_rng(9100 + slots + group)
+    heads = group * kv_heads
+    contexts = rng.integers(0, contexts_top, slots)
+    case = make_case(rng, slots=slots, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=contexts, tokens=1, advances=[1] * slots, dtype=dtype)
+    scale = 1.0 / np.sqrt(width)
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, 64, heads * width, slots)
+    assert plan.fused_prepare
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    results = []
+    for fused in (False, True):
+        k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+        scales = [dev(case[name]) if case.get(name) is not None else None for name in ("k_scales", "v_scales")]
+        layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)),
+                           dev(case["cursors"].view(np.int32)), dev(case["advances"].view(np.int32)),
+                           case["max_context"], k_scales=scales[0], v_scales=scales[1])
+        q = dev(case["q"])
+        out = torch.full_like(q, float("nan"))
+        prepared = torch.zeros(plan.prepared_input_bytes, dtype=torch.uint8, device=device)
+        if fused:
+            et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, 0, out, prepared_for=plan,
+                                 prepared=prepared)
+        else:
+            et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, 0, out)
+            plan.prepare_input(out.view(slots, heads * width), prepared)
+        results.append((out, k_slab, v_slab, prepared))
+    for two, one in zip(*results):
+        assert torch.equal(two, one)
+    # more than one token per slot has no such rows
+    case = make_case(rng, slots=4, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=[5, 6, 7, 8], tokens=2, advances=[2] * 4, dtype=dtype)
+    layer = et.KvLayer(dev(case["k_slab"]), dev(case["v_slab"]), 16, dev(case["table"].view(np.int32)),
+                       dev(case["cursors"].view(np.int32)), dev(case["advances"].view(np.int32)), case["max_context"],
+                       k_scales=dev(case["k_scales"]) if case["k_scales"] is not None else None,
+                       v_scales=dev(case["v_scales"]) if case["v_scales"] is not None else None)
+    q = dev(case["q"])
+    with pytest.raises(et.QuantizedError, match="one token per slot"):
+        et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, 0, torch.empty_like(q),
+                             prepared_for=et.RawLinear(et.GgmlQuant.Q4_K, 64, heads * width, 4),
+                             prepared=torch.zeros(1 << 20, dtype=torch.uint8, device=device))
