@@ -164,6 +164,7 @@ struct ShareSource {
     uint64_t launch_rows, share_stride;
     const float* bias;       // [columns] or null
     const float* residual;   // [vectors, columns] or null
+    float* y;                // [vectors, columns]: the summed rows, written before they are normed
 };
 template <bool SHARES>
 __global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const float* x, uint64_t x_row_stride,
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const 
     float4 held = make_float4(0.f, 0.f, 0.f, 0.f);
     if constexpr (SHARES) {
         // x is y: every float4 of the row is summed and written once, number T, T + 1024, ... by thread T
-        float4* row = reinterpret_cast<float4*>(const_cast<float*>(x) + v * x_row_stride);
+        float4* row = reinterpret_cast<float4*>(source.y + v * x_row_stride);
         for (uint32_t i = threadIdx.x; i < quads; i += kRmsThreads) {
             const float* first = source.shares + v * source.launch_rows + 4u * i;
             float4 total = *reinterpret_cast<const float4*>(first);
@@ -313,7 +314,7 @@ hipError_t quantize_tiles_rms_norm_of_shares(const float* shares, uint32_t share
     if (columns % 256 != 0 || vectors > 0x7fffffffull || share_count == 0 || launch_rows < columns || launch_rows % 4 != 0)
         return hipErrorInvalidValue;
     if (vectors == 0 || columns == 0) return hipSuccess;
-    const ShareSource source = {shares, share_count, launch_rows, launch_rows * vectors, bias, residual};
+    const ShareSource source = {shares, share_count, launch_rows, launch_rows * vectors, bias, residual, y};
     hipLaunchKernelGGL(quantize_halves_rms_kernel<true>, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream,
                        y, columns, source, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
