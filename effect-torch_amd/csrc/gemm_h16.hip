@@ -23,6 +23,7 @@
 // global_load_lds copies into LDS rings, one s_barrier per stage.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "decode_math.h"
@@ -674,15 +675,15 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
     if (row_tiles > 0x00ffffffull) return hipErrorInvalidValue;
     group.row_tiles = static_cast<uint32_t>(row_tiles);
     // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
-    static bool allowed[64] = {};
+    static std::atomic<bool> allowed[64] = {};  // callers may enqueue from several threads; setting twice is harmless
     int device = 0;
     if (hipError_t status = hipGetDevice(&device)) return status;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    if (!allowed[device]) {
+    if (!allowed[device].load(std::memory_order_acquire)) {
         if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes))
             return status;
-        allowed[device] = true;
+        allowed[device].store(true, std::memory_order_release);
     }
     const uint32_t vector_tiles = (vectors + 31u) / 32u;
     const uint64_t grid = ((row_tiles + 7u) / 8u) * 8u * vector_tiles * k_splits;

@@ -55,6 +55,7 @@
 // and every result register row is stored as 128 contiguous bytes of y.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "et_codecs.h"
@@ -527,16 +528,16 @@ hipError_t launch(const uint8_t* weight, const uint8_t* tiles, const GemmOutput&
     static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
     const auto kernel = gemm_i8_kernel<CODEC, MT, LIMBS, AX, AW>;
     // More than 64 KiB of dynamic LDS has to be allowed once per kernel and device.
-    static bool allowed[64] = {};
+    static std::atomic<bool> allowed[64] = {};  // callers may enqueue from several threads; setting twice is harmless
     int device = 0;
     if (hipError_t status = hipGetDevice(&device)) return status;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    if (!allowed[device]) {
+    if (!allowed[device].load(std::memory_order_acquire)) {
         if (hipError_t status =
                 hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes))
             return status;
-        allowed[device] = true;
+        allowed[device].store(true, std::memory_order_release);
     }
     const uint32_t vector_tiles = (vectors + 31u) / 32u;
     const uint32_t vector_groups = (vector_tiles + MT - 1) / MT;
