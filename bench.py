@@ -528,7 +528,7 @@ def quantized_embedding(args, et):
 
 
 def llama_decode(args, et):
-    """Workload ``llama3_8b_batched_decode`` (BASELINE config 4): one decode step of a Llama-3-8B-shaped
+    """Workload ``llama3_8b_batched_decode`` (the end-to-end batched-decode configuration): one decode step of a Llama-3-8B-shaped
     model for 32 slots at context 2048, every operator through the C ABI - per layer RMS norm, the
     q / k / v / o and gate / up / down contractions on Q4_K weights (M = 32, f32 activations), rotary
     on q and k at the slots' cursors, paged key/value-cache attention over f16 slabs, SiLU * up and the
