@@ -737,7 +737,8 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
         }
         if (g.tile_rows == 128)
             return launch_group<kQ3_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
-        return launch_group<kQ3_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+        // as for Q4_K: three stages of activation lead, one of weights (14336 x 4096 with 32 vectors 28.0 -> 25.9 us)
+        return launch_group<kQ3_K, 2, 3, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
     }
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
