@@ -662,7 +662,7 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
                         uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares,
                         const GemmRotary* rotary) {
     using S = Shape<CODEC, RG, AX, AW>;
-    static_assert(S::kLdsBytes <= 156 * 1024, "LDS of a gfx950 CU (160 KiB), with a margin");
+    static_assert(S::kLdsBytes <= 160 * 1024, "LDS of a gfx950 CU: 160 KiB, all of it dynamic here");
     const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW>;
     Group group = {};
     group.count = count;
@@ -743,7 +743,8 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     if (codec == kQ5_K) {
         if (g.tile_rows == 128)
             return launch_group<kQ5_K, 4, 2, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
-        return launch_group<kQ5_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+        // three stages of activation lead, one of weights: 158 KiB (14336 x 4096 with 32 vectors 29.9 -> 28.7 us)
+        return launch_group<kQ5_K, 2, 3, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
     }
     if (g.tile_rows == 128)
         return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
