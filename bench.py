@@ -35,11 +35,74 @@ F16_PEAK_TFLOPS = 2500.0       # MI355X dense fp16 MFMA, published (2.5 PFLOP/s)
 ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
-# counters' reading for a plain copy of known size. These cannot be collected from inside this
-# script; the runs and their figures are in profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md.
-MEASURED_TRAFFIC = {("q4_k_gemv_14336x4096", 1, "f32"): 33338900,
-                    # attend kernel; profiles/kv_attend_decode_32slots_ctx2048_f16.md
-                    ("kv_attention_decode", 2048): 270009600}
+# counters' reading for a plain copy of known size. The counters cannot be collected from inside
+# this script, so each figure is tied to the kernel it was taken from: the kernel's name as the
+# planner reports it and the SHA-256 of the source file that defines it at the time of the profile.
+# When either differs from what runs now, `roofline.traffic` is null until the profile is re-taken.
+MEASURED_TRAFFIC = {
+    ("q4_k_gemv_14336x4096", 1, "f32"): {
+        "bytes": 33338900, "kernel": "gemv_limb", "source": "gemv_limb.hip",
+        "sha256": "", "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
+    ("kv_attention_decode", 2048): {
+        "bytes": 270009600, "kernel": "kv_attend", "source": "kv_attention.hip",
+        "sha256": "", "profile": "profiles/kv_attend_decode_32slots_ctx2048_f16.md"},
+}
+
+
+def measured_traffic(key, kernel_name):
+    """The profiled HBM bytes per launch of `key`, or None when the kernel that runs now is not the
+    one that was profiled (another kernel name, or its source file has changed since)."""
+    import hashlib
+
+    entry = MEASURED_TRAFFIC.get(key)
+    if entry is None or not str(kernel_name).startswith(entry["kernel"]):
+        return None
+    path = os.path.join(ROOT, "effect-torch_amd", "csrc", entry["source"])
+    try:
+        with open(path, "rb") as source:
+            digest = hashlib.sha256(source.read()).hexdigest()
+    except OSError:
+        return None
+    return entry["bytes"] if digest == entry["sha256"] else None
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as info:
+            for line in info:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
+class pinned_to_one_core:
+    """Pins this process to one host core for the CPU baseline (the reference's loop is single
+    threaded) and restores the affinity afterwards."""
+
+    def __enter__(self):
+        self.before = None
+        self.core = None
+        try:
+            self.before = os.sched_getaffinity(0)
+            self.core = max(self.before)  # the highest allowed core: least likely to serve interrupts
+            os.sched_setaffinity(0, {self.core})
+        except (AttributeError, OSError):
+            self.before = None
+        return self
+
+    def __exit__(self, *exc):
+        if self.before is not None:
+            try:
+                os.sched_setaffinity(0, self.before)
+            except OSError:
+                pass
+        return False
+
+    def describe(self):
+        where = f"pinned to core {self.core}" if self.before is not None else "not pinned"
+        return f"{where} of {cpu_model()}"
 
 
 def parse_args():
@@ -88,10 +151,12 @@ def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
         sample_rows, calls = max(16, int(seconds / (per_row_vector * vectors))), 1
         sample_rows = min(sample_rows, rows)
     y = np.zeros((vectors, rows), dtype=np.float32)
-    t0 = time.perf_counter()
-    for _ in range(calls):
-        oracle.linear_rows(codec, rows, columns, x, weight, None, 0, sample_rows, out=y)
-    elapsed = time.perf_counter() - t0
+    with pinned_to_one_core() as pin:
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            oracle.linear_rows(codec, rows, columns, x, weight, None, 0, sample_rows, out=y)
+        elapsed = time.perf_counter() - t0
+        pinned = pin.describe()
     seconds_per_call = elapsed / calls * (rows / sample_rows)
     what = (f"{calls} full call(s) of the same workload" if sample_rows == rows else
             f"rows 0..{sample_rows} of {rows} of one call, scaled by {rows / sample_rows:.1f}")
@@ -101,13 +166,23 @@ def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
         "cores": 1,
         "kind": "port",
         "sample": f"{what}; {elapsed:.1f} s of CPU work; f32 activations, scalar C restatement of the "
-                  f"reference's single-threaded loop ({seconds_per_call * 1e3:.1f} ms per call)",
+                  f"reference's single-threaded loop ({seconds_per_call * 1e3:.1f} ms per call); {pinned}",
     }
 
 
+MIN_REPETITIONS = 5       # timed replays of the K steps; the median is reported
+TIMED_WINDOW_MS = 20.0    # short replays are repeated until about this much device time is covered
+MAX_REPETITIONS = 400
+LAST_TIMING = {}
+
+
 def time_steps(step, steps, warmup, use_graph):
-    """Warm up, then time exactly `steps` calls of step(i) on torch's current stream
-    (a HIP graph replay unless disabled); returns (ms per step, graph used, wall seconds)."""
+    """Warm up, then time `steps` calls of step(i) on torch's current stream (one HIP graph of the K
+    steps unless disabled), repeated: every repetition is bracketed by its own pair of HIP events on
+    that stream, the repetitions run back to back, and the MEDIAN over them is reported. A K-step
+    replay shorter than the timed window is repeated more often (at least MIN_REPETITIONS times), so
+    that a short run is not one sample taken while the device clocks still ramp.
+    Returns (ms per step, graph used, wall seconds); LAST_TIMING holds repetitions / min / max."""
     import torch
 
     stream = torch.cuda.current_stream()
@@ -127,20 +202,45 @@ def time_steps(step, steps, warmup, use_graph):
             print(f"HIP graph capture failed ({exc}); timing plain enqueues", file=sys.stderr)
             graph = None
             torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
+
+    def run_once():
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                step(i)
+
+    def timed(repetitions):
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                  for _ in range(repetitions)]
+        torch.cuda.synchronize()
+        for start, stop in events:
+            start.record(stream)
+            run_once()
+            stop.record(stream)
+        torch.cuda.synchronize()
+        return [start.elapsed_time(stop) for start, stop in events]
+
+    probe = timed(1)[0]
+    repetitions = int(min(MAX_REPETITIONS, max(MIN_REPETITIONS, -(-TIMED_WINDOW_MS // max(probe, 1e-3)))))
     wall0 = time.perf_counter()
-    start.record(stream)
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(steps):
-            step(i)
-    stop.record(stream)
-    torch.cuda.synchronize()
+    samples = sorted(timed(repetitions))
     wall = time.perf_counter() - wall0
-    return start.elapsed_time(stop) / steps, graph is not None, wall
+    median = samples[len(samples) // 2] if len(samples) % 2 else 0.5 * (samples[len(samples) // 2 - 1] +
+                                                                         samples[len(samples) // 2])
+    LAST_TIMING.clear()
+    LAST_TIMING.update({"repetitions": repetitions, "ms_per_step_min": round(samples[0] / steps, 6),
+                        "ms_per_step_max": round(samples[-1] / steps, 6),
+                        "timing": f"median of {repetitions} timed replays of the {steps} steps, one HIP event pair each"})
+    return median / steps, graph is not None, wall
+
+
+def with_timing(result):
+    """Adds the repetition record of the last time_steps() call to a result line."""
+    for key in ("repetitions", "ms_per_step_min", "ms_per_step_max"):
+        result[key] = LAST_TIMING.get(key)
+    result.setdefault("config", {})["timing"] = LAST_TIMING.get("timing")
+    return result
 
 
 def calibrate(args, et):
@@ -163,7 +263,7 @@ def calibrate(args, et):
         moved = 2 * nbytes
     ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
     gbs = moved / (ms * 1e-3) / 1e9
-    print(json.dumps({
+    print(json.dumps(with_timing({
         "metric": f"{args.workload} GB/s", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
@@ -173,6 +273,60 @@ def calibrate(args, et):
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": moved, "avg_launch_us": round(ms * 1e3, 3)},
+    })))
+
+
+def calibrate_read_sweep(args, et):
+    """Workload ``calibrate_read_sweep``: plain reads of 8 MiB ... 1 GiB by five different read kernels
+    (``et_hip_calibration_read_variant``), cold (the buffers of a size rotate through a 2.25 GiB pool),
+    each as a HIP-graph replay timed like every other workload; per kernel the launch times are fitted
+    to t = t0 + bytes / BW. What this answers: how long a read of the headline weight's 33 MB takes on
+    this device whatever kernel does it - the fixed cost t0 of a launch in a dependent chain plus the
+    transfer at the rate large reads sustain."""
+    import numpy as np
+    import torch
+
+    device = torch.device("cuda:0")
+    pool_bytes = 2304 << 20
+    pool = torch.randint(0, 255, (pool_bytes,), dtype=torch.uint8, device=device)
+    sink = torch.zeros(4 * 4096, dtype=torch.int32, device=device)
+    headline = 14336 * 2304
+    sizes = [8 << 20, 16 << 20, headline, 64 << 20, 128 << 20, 256 << 20, 512 << 20, 1024 << 20]
+    # (variant, workgroups): the LDS kernels hold a whole compute unit's LDS, one workgroup each
+    kernels = [("plain", 512), ("plain", 2048), ("deep", 512), ("deep", 1024), ("streaming", 1024), ("lds4", 256),
+               ("lds8", 256)]
+    table, fits = [], []
+    for variant, workgroups in kernels:
+        times = []
+        for size in sizes:
+            size -= size % 1024
+            copies = max(1, min(pool_bytes // size, -(-ROTATE_BYTES // size)))
+            views = [pool[i * size:(i + 1) * size] for i in range(copies)]
+            step = lambda i: et.calibration_read_variant(variant, views[i % copies], sink, workgroups)  # noqa: E731
+            steps = int(max(copies, min(args.steps, 4e-3 / (size / 4e12))))
+            ms, graphed, _ = time_steps(step, steps, min(args.warmup, 2 * copies), not args.no_graph)
+            times.append(ms * 1e-3)
+            table.append({"kernel": f"{variant} x{workgroups}", "bytes": size, "us": round(ms * 1e3, 3),
+                          "GBps": round(size / (ms * 1e-3) / 1e9, 1), "steps": steps, "copies": copies,
+                          "repetitions": LAST_TIMING.get("repetitions")})
+            print(json.dumps(table[-1]), file=sys.stderr, flush=True)
+        slope, t0 = np.polyfit(np.array(sizes, dtype=np.float64), np.array(times), 1)
+        fits.append({"kernel": f"{variant} x{workgroups}", "t0_us": round(t0 * 1e6, 3),
+                     "BW_GBps": round(1.0 / slope / 1e9, 1),
+                     "predicted_us_at_headline_bytes": round((t0 + headline * slope) * 1e6, 3),
+                     "measured_us_at_headline_bytes": round(times[2] * 1e6, 3)})
+    best = min(fits, key=lambda f: f["measured_us_at_headline_bytes"])
+    gbs = headline / (best["measured_us_at_headline_bytes"] * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "calibrate_read_sweep GB/s at the headline weight's size", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(best["measured_us_at_headline_bytes"] * 1e-3, 6), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "calibrate_read_sweep: plain reads of 8 MiB ... 1 GiB by five read kernels, cold, "
+                               "graph replay; fit t = t0 + bytes / BW per kernel",
+                   "best_kernel_at_headline_bytes": best["kernel"], "fits": fits, "table": table},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }))
 
 
@@ -198,7 +352,7 @@ def calibrate_mfma(args, et):
     operations = et.MFMA_OPERATIONS[kind] * 4 * iterations * 4 * workgroups
     tops = operations / (ms * 1e-3) / 1e12
     peak = INT8_PEAK_TOPS if kind.startswith("i8") else F16_PEAK_TFLOPS
-    print(json.dumps({
+    print(json.dumps(with_timing({
         "metric": f"{args.workload} TOP/s", "value": round(tops, 1), "unit": "TOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -208,7 +362,7 @@ def calibrate_mfma(args, et):
                    "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues"},
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(tops / peak, 4), "traffic": None},
-    }))
+    })))
 
 
 def make_kv_slabs(torch, kv_dtype, max_tokens, kv_heads, width, device):
@@ -310,7 +464,9 @@ def kv_decode(args, et):
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(("kv_attention_decode", context)) if args.kv_dtype == "f16" else None,
+                     "traffic": measured_traffic(("kv_attention_decode", context),
+                                                 et.kv_attention_kernel(states[0], query_heads, 1))
+                     if args.kv_dtype == "f16" else None,
                      "kernel": et.kv_attention_kernel(states[0], query_heads, 1),
                      "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
     }
@@ -330,7 +486,7 @@ def kv_decode(args, et):
             "sample": f"{calls} call(s) over {sample} of the {slots} slots, scaled by {slots // sample}; "
                       f"{elapsed:.1f} s of CPU work; scalar C restatement of the reference's f64 three-pass loop "
                       f"({per_step * 1e3:.0f} ms per step)"}
-    print(json.dumps(result))
+    print(json.dumps(with_timing(result)))
 
 
 DECODE_OPS = ("rms_norm_decode", "rotary_decode", "silu_mul_decode", "greedy_decode", "embedding_gather_decode")
@@ -452,7 +608,7 @@ def decode_op(args, et):
         result["cpu_baseline"] = {"value": round(algorithmic / (elapsed / calls) / 1e9, 4), "unit": "GB/s", "cores": 1,
                                   "kind": "port", "sample": f"{calls} full call(s) of the same workload, "
                                   f"{elapsed:.1f} s of CPU work ({elapsed / calls * 1e6:.0f} us per call)"}
-    print(json.dumps(result))
+    print(json.dumps(with_timing(result)))
 
 
 def quantized_embedding(args, et):
@@ -524,7 +680,7 @@ def quantized_embedding(args, et):
                                   "cores": 1, "kind": "port",
                                   "sample": f"{calls} call(s) on the first {cpu_tokens} ids, {elapsed:.1f} s of CPU "
                                             f"work ({per_token * 1e6:.1f} us per row); scalar C restatement"}
-    print(json.dumps(result))
+    print(json.dumps(with_timing(result)))
 
 
 def llama_decode(args, et):
@@ -918,6 +1074,8 @@ def main():
 
     if args.workload in ("calibrate_read", "calibrate_copy"):
         return calibrate(args, et)
+    if args.workload == "calibrate_read_sweep":
+        return calibrate_read_sweep(args, et)
     if args.workload.startswith("calibrate_mfma_"):
         return calibrate_mfma(args, et)
     if args.workload in DECODE_OPS:
@@ -1005,7 +1163,7 @@ def main():
     else:
         roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
-    roofline["traffic"] = MEASURED_TRAFFIC.get((args.workload, vectors, mode_name))
+    roofline["traffic"] = measured_traffic((args.workload, vectors, mode_name), req.kernel)
     roofline["kernel"] = req.kernel
     roofline["algorithmic_bytes_per_launch"] = algorithmic_bytes
     roofline["avg_launch_us"] = round(ms_per_step * 1e3, 3)
@@ -1037,7 +1195,7 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, vectors, mode_name, weight_host, x_host,
                                               args.cpu_seconds, algorithmic_bytes)
-    print(json.dumps(result))
+    print(json.dumps(with_timing(result)))
 
 
 if __name__ == "__main__":

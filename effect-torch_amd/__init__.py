@@ -18,6 +18,8 @@ from .quantized import (  # noqa: F401
     calibration_copy,
     calibration_mfma,
     calibration_read,
+    calibration_read_variant,
+    READ_VARIANTS,
     dequantize_rows,
     embedding_into,
     embedding_requirements,

@@ -1,4 +1,4 @@
-"""ctypes binding of ``lib/libet_hip.so`` (the C ABI declared in ``include/et_hip.h``).
+"""ctypes binding of ``lib/libet_hip.so`` (the C ABI declared in ``include/et_hip.h`` and ``include/et_hip_calibrate.h``).
 
 The library is loaded from inside the package directory only. There is no CPU
 fallback: if the shared object is missing this module raises on import of
@@ -183,6 +183,7 @@ SIGNATURES = {
     "et_hip_gguf_upload_tensor": (ctypes.c_int, [_vp, _u64, _vp, _u64, _vp, _vp]),
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
+    "et_hip_calibration_read_variant": (ctypes.c_int, [_i32, _vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),
     "et_hip_calibration_mfma": (ctypes.c_int, [_i32, ctypes.c_uint32, ctypes.c_uint32, _vp, _vp]),
     "et_hip_last_error": (ctypes.c_char_p, []),

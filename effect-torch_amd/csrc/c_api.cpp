@@ -10,6 +10,7 @@
 
 #include "et_codecs.h"
 #include "et_hip.h"
+#include "et_hip_calibrate.h"
 #include "kernels.h"
 #include "decode_host.h"
 #include "gguf.h"
@@ -744,6 +745,25 @@ int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uin
             et::calibration_read(src, bytes, sink, workgroups, static_cast<hipStream_t>(stream));
         if (status != hipSuccess) {
             *error = std::string("calibration_read: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
+int et_hip_calibration_read_variant(int32_t variant, const void* src, uint64_t bytes, uint32_t* sink,
+                                    uint32_t workgroups, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (src == nullptr || sink == nullptr || workgroups == 0 || workgroups > 65536 || (bytes >> 36) != 0 ||
+            reinterpret_cast<uintptr_t>(src) % 16 != 0 || variant < ET_READ_PLAIN || variant > ET_READ_LDS_8) {
+            *error = "calibration_read_variant: variant 0..4, source 16-byte aligned, sink non-NULL, "
+                     "1 <= workgroups <= 65536";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status =
+            et::calibration_read_variant(variant, src, bytes, sink, workgroups, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("calibration_read_variant: HIP error: ") + hipGetErrorString(status);
             return ET_ERR_EXECUTION;
         }
         return ET_OK;

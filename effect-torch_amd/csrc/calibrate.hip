@@ -44,6 +44,72 @@ __global__ __launch_bounds__(256) void read_kernel(const uint4* __restrict__ src
     if ((threadIdx.x & 63u) == 0) sink[blockIdx.x * 4u + (threadIdx.x >> 6)] = acc;
 }
 
+// The same read with U loads in flight per lane (and non-temporal loads when STREAMING): if the
+// device can deliver more than read_kernel reaches, a deeper queue per wave shows it.
+template <int U, bool STREAMING>
+__global__ __launch_bounds__(256) void read_deep_kernel(const uint4* __restrict__ src, uint32_t quads,
+                                                        uint32_t* __restrict__ sink) {
+    const uint32_t per_wg = (quads + gridDim.x - 1) / gridDim.x;
+    const uint32_t begin = blockIdx.x * per_wg;
+    const uint32_t end = min(begin + per_wg, quads);
+    uint32_t acc = 0;
+    uint32_t i = begin + threadIdx.x;
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+    const auto fetch = [&](uint32_t at) {
+        if constexpr (STREAMING) {
+            const v4u raw = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(src + at));
+            return make_uint4(raw.x, raw.y, raw.z, raw.w);
+        } else {
+            return src[at];
+        }
+    };
+    for (; i + (U - 1) * 256u < end; i += U * 256u) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = fetch(i + u * 256u);
+#pragma unroll
+        for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < end; i += 256u) {
+        const uint4 v = fetch(i);
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) acc ^= __shfl_xor(acc, offset);
+    if ((threadIdx.x & 63u) == 0) sink[blockIdx.x * 4u + (threadIdx.x >> 6)] = acc;
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
+
+// A read that uses no registers and no arithmetic: every wave only issues 1 KiB global-to-LDS
+// copies into its own ring of DEPTH slots and, once the ring is full, waits for the oldest copy
+// before it issues the next one - DEPTH KiB in flight per wave for the whole launch. One workgroup
+// per compute unit (WAVES * DEPTH = 128 KiB of LDS); workgroup w takes the w-th contiguous range.
+template <int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES) void read_lds_kernel(const uint8_t* __restrict__ src, uint32_t kib,
+                                                              uint32_t* __restrict__ sink) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t ring[];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t per_wg = (kib + gridDim.x - 1) / gridDim.x;
+    const uint32_t begin = blockIdx.x * per_wg;
+    const uint32_t end = min(begin + per_wg, kib);
+    uint8_t* mine = ring + wave * DEPTH * 1024u;
+    // jobs of this wave: begin + wave, begin + wave + WAVES, ...
+    uint32_t job = begin + wave, slot = 0;
+    for (; job < end; job += WAVES) {
+        if (slot >= static_cast<uint32_t>(DEPTH)) __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));  // the slot's last copy has landed
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src + static_cast<uint64_t>(job) * 1024u + lane * 16u),
+                                         reinterpret_cast<uint4*>(mine + (slot % DEPTH) * 1024u), 16, 0, 0);
+        slot += 1;
+    }
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    __syncthreads();
+    // one word of what arrived leaves, so that the copies have an observer
+    if (threadIdx.x < 4) sink[(blockIdx.x * 4u + threadIdx.x) % 1024u] = reinterpret_cast<const uint32_t*>(ring)[threadIdx.x * 256u];
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src,
                                                    uint4* __restrict__ dst, uint64_t quads) {
     const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256ull;
@@ -196,6 +262,43 @@ hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uin
     if (bytes < 16) return hipSuccess;
     hipLaunchKernelGGL(read_kernel, dim3(workgroups), dim3(256), 0, stream,
                        static_cast<const uint4*>(src), static_cast<uint32_t>(bytes / 16), sink);
+    return hipGetLastError();
+}
+
+hipError_t calibration_read_variant(int variant, const void* src, uint64_t bytes, uint32_t* sink,
+                                    uint32_t workgroups, hipStream_t stream) {
+    if (bytes < 1024) return hipSuccess;
+    const uint4* quads = static_cast<const uint4*>(src);
+    const uint32_t count = static_cast<uint32_t>(bytes / 16);
+    constexpr uint32_t kRingBytes = 128u * 1024u;
+    switch (variant) {
+        case kReadPlain: return calibration_read(src, bytes, sink, workgroups, stream);
+        case kReadDeep:
+            hipLaunchKernelGGL((read_deep_kernel<16, false>), dim3(workgroups), dim3(256), 0, stream, quads, count, sink);
+            break;
+        case kReadStreaming:
+            hipLaunchKernelGGL((read_deep_kernel<16, true>), dim3(workgroups), dim3(256), 0, stream, quads, count, sink);
+            break;
+        case kReadLds4: {
+            const auto kernel = read_lds_kernel<4, 32>;
+            if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRingBytes))
+                return status;
+            hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(256), kRingBytes, stream,
+                               static_cast<const uint8_t*>(src), static_cast<uint32_t>(bytes / 1024), sink);
+            break;
+        }
+        case kReadLds8: {
+            const auto kernel = read_lds_kernel<8, 16>;
+            if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRingBytes))
+                return status;
+            hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kRingBytes, stream,
+                               static_cast<const uint8_t*>(src), static_cast<uint32_t>(bytes / 1024), sink);
+            break;
+        }
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

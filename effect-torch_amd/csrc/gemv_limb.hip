@@ -25,7 +25,9 @@
 // meet in LDS. A workgroup walks a contiguous range of rows.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
+#include <cstdlib>
 
 #include "et_codecs.h"
 #include "gemv_common.h"
@@ -142,6 +144,8 @@ __device__ __forceinline__ float limb_value(const XLimbs& x, int d0, int d1, int
 // ---------------------------------------------------------------------------
 
 struct Q4KLimb {
+    static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 144u;
+    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -223,6 +227,8 @@ struct Q4KLimb {
 // value in qh[32] between the scales and the nibbles - bit g of qh[i] belongs to element i of
 // sub-block g. 176 bytes per block, every field 16-byte aligned.
 struct Q5KLimb {
+    static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 176u;
+    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -316,6 +322,8 @@ struct __attribute__((packed, aligned(4))) Dwords17 {
 
 // Q4_0: two 18-byte blocks = 36 bytes = 9 dwords (dword aligned when columns % 64 == 0).
 struct Q40Limb {
+    static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 18u;
+    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -374,6 +382,8 @@ struct Q40Limb {
 
 // Q8_0: two 34-byte blocks = 68 bytes = 17 dwords (dword aligned when columns % 64 == 0).
 struct Q80Limb {
+    static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 34u;
+    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -472,6 +482,8 @@ __device__ __forceinline__ void load_run_activations(const StageMemory& stage, u
 // scale, out of exactly 48 bytes of quants - three 16-byte loads, nothing read twice. Its 64 columns
 // are not consecutive, so it gathers its activation limbs run by run (load_activations).
 struct Q6KLimb {
+    static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 210u;
+    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
     struct Lane {
         uint32_t offset;  // byte offset of the lane's block within a row
         uint32_t half, j;
@@ -581,6 +593,8 @@ typedef struct __attribute__((packed, aligned(2))) { uint32_t v[3]; } Dwords3_a2
 // 16j + i is d * (scales[8*half + 2g + j] & 15) * ((qs[32*half + 16j + i] >> 2g) & 3) - dmin *
 // (scales[..] >> 4). A lane takes (half, j): runs g = 0..3, sixteen bytes of quants.
 struct Q2KLimb {
+    static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 84u;
+    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -654,6 +668,8 @@ struct Q2KLimb {
 // 32g + 16j + i is d * (scale[8*half + 2g + j] - 32) * (((qs[32*half + 16j + i] >> 2g) & 3) -
 // (hmask[16j + i] bit (4*half + g) ? 0 : 4)). A lane takes (half, j): runs g = 0..3.
 struct Q3KLimb {
+    static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 110u;
+    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -901,6 +917,240 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same GEMV with the weights brought in by global-to-LDS copies (one slice: columns <= 4096).
+//
+// What bounds gemv_limb_kernel is how many bytes a compute unit keeps in flight: a wave requests
+// the next row only after it has folded the one before, because a wave that issues a load into a
+// full memory queue stalls with all the arithmetic behind it. Here the two jobs are split between
+// waves. The workgroup's whole share of W - a contiguous range of rows, at most 158 KiB - is
+// requested at once by four LOADER waves as 1 KiB global_load_lds copies straight into LDS (no
+// registers; a loader that stalls on a full queue holds nothing up), and eight CONSUMER waves
+// prepare the activations meanwhile and then fold the rows out of LDS in the order they arrive
+// (row i of the share belongs to consumer i % 8). A consumer issues no global load after its
+// activation loads and no store before every copy has landed.
+//
+// Hand-over without barriers (s_barrier would tie the loaders to the consumers' prologue): loader
+// l publishes in LDS how many of its copies have landed (loads return in order per wave; one
+// counted s_waitcnt per copy), and a consumer polls the four counts until they cover its row.
+// The consumers meet each other through two LDS counters (`staged`, `folded`).
+// LDS: [weights: whole KiB][...][StageMemory x M][control]. With three vectors the stages overlap
+// the end of a full-size share: the copies that land there wait until every consumer has read
+// its limbs (`staged` == 2 * consumers).
+// ---------------------------------------------------------------------------
+// ET_HIP_GEMV_LDS_COPIES=0 in the environment keeps every shape on gemv_limb_kernel (for A/B timing).
+bool gemv_limb_dma_enabled() {
+    static const bool enabled = [] {
+        const char* value = std::getenv("ET_HIP_GEMV_LDS_COPIES");
+        return value == nullptr || value[0] != '0';
+    }();
+    return enabled;
+}
+
+constexpr int kDmaConsumers = 8;
+constexpr int kDmaLoaders = 4;
+constexpr int kDmaJobs = 40;  // copies per loader at most: vmcnt counts to 63
+constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaLoaders);
+constexpr uint32_t kDmaLdsBytes = 160u * 1024u;
+constexpr uint32_t kDmaMaxRows = 128;  // rows of a workgroup's share
+struct DmaControl {
+    uint32_t done[kDmaLoaders];  // copies of loader l that have landed
+    uint32_t staged;             // consumer arrivals: +1 after writing the stage, +1 after reading the limbs
+    uint32_t folded;             // consumers that have left all their results
+    uint32_t pad[2];
+    float result[kGemvLimbMaxVectors][kDmaMaxRows];
+};
+constexpr uint32_t kDmaControlAt = kDmaLdsBytes - 2048u;
+static_assert(sizeof(DmaControl) <= 2048, "control block");
+constexpr uint32_t kDmaMaxShareBytes = kDmaControlAt;  // whole KiB below the control block
+static_assert(kDmaMaxShareBytes / 1024u <= kDmaLoaders * kDmaJobs, "every KiB has a copy slot");
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
+
+// Hand-over words in LDS are accessed through their LDS addresses with instructions the compiler
+// does not look into. LDS serves a wave's requests in order, so "data, then counter" needs no
+// fence; an acquire / release at workgroup scope - or any LDS access the compiler can see next to
+// global-to-LDS copies, whose destinations it cannot tell from other LDS addresses - would make it
+// wait for every outstanding copy (vmcnt 0), exactly what a loader with forty copies in flight
+// must not do. These accesses touch the control block only, where no copy lands.
+__device__ __forceinline__ uint32_t lds_address(const void* pointer) {
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(pointer));  // low half of the flat address
+}
+__device__ __forceinline__ void lds_store_unseen(uint32_t address, uint32_t value) {
+    asm volatile("ds_write_b32 %0, %1" : : "v"(address), "v"(value) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_count(uint32_t address) {
+    uint32_t value;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(value) : "v"(address) : "memory");
+    return __builtin_amdgcn_readfirstlane(value);
+}
+__device__ __forceinline__ void lds_arrive(uint32_t address, bool one_lane) {
+    // this wave's LDS writes are complete (and the compiler keeps them above this line)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (one_lane) asm volatile("ds_add_u32 %0, %1" : : "v"(address), "v"(1u) : "memory");
+}
+__device__ __forceinline__ void lds_await(uint32_t address, uint32_t count) {
+    while (lds_count(address) < count) __builtin_amdgcn_s_sleep(1);
+}
+
+// The loader's copies sit in the LAST slots of its list of kDmaJobs (the first `skip` are empty), so
+// that "copy of slot I has landed" is the compile-time count vmcnt <= kDmaJobs - 1 - I.
+template <int I>
+__device__ __forceinline__ void dma_publish(uint32_t skip, uint32_t done_address) {
+    if constexpr (I < kDmaJobs) {
+        if (static_cast<uint32_t>(I) >= skip) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(kDmaJobs - 1 - I));
+            lds_store_unseen(done_address, static_cast<uint32_t>(I) - skip + 1u);
+        }
+        dma_publish<I + 1>(skip, done_address);
+    }
+}
+
+template <class T, int M>
+__global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
+    const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
+    const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
+    uint32_t rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr uint32_t kStageAt = kDmaControlAt - M * static_cast<uint32_t>(sizeof(StageMemory));
+    constexpr int NI = kSliceQuads / (64 * kDmaConsumers);  // float4s per consumer thread and vector
+    DmaControl* control = reinterpret_cast<DmaControl*>(lds + kDmaControlAt);
+    StageMemory* stage = reinterpret_cast<StageMemory*>(lds + kStageAt);
+
+    const uint32_t lane_id = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wg_row0 = blockIdx.x * rows_per_wg;
+    if (wg_row0 >= rows) return;
+    const uint32_t wg_rows = min(rows_per_wg, rows - wg_row0);
+    const uint32_t row_bytes = static_cast<uint32_t>(T::row_bytes(columns));
+    const uint32_t wg_bytes = wg_rows * row_bytes;
+    const uint32_t jobs = (wg_bytes + 1023u) >> 10;
+    const bool consumer = wave < static_cast<uint32_t>(kDmaConsumers);
+
+    // Activation loads go first: they must not queue behind the copies.
+    float4 xv[M][NI];
+    if (consumer) {
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                const uint32_t quad = threadIdx.x + i * 64u * kDmaConsumers;
+                xv[m][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (quad < (columns >> 2)) xv[m][i] = reinterpret_cast<const float4*>(x + m * x_row_stride)[quad];
+            }
+    }
+    if (threadIdx.x < 8) reinterpret_cast<uint32_t*>(control)[threadIdx.x] = 0u;
+    __syncthreads();  // the only barrier: the counters are zero, the activation loads are on their way
+
+    if (!consumer) {
+        // ---- loaders ------------------------------------------------------------------------
+        const uint32_t loader = wave - kDmaConsumers;
+        const uint32_t mine = jobs > loader ? (jobs - loader + kDmaLoaders - 1u) / kDmaLoaders : 0u;
+        const uint32_t skip = kDmaJobs - mine;
+        const uint8_t* source = weight + static_cast<uint64_t>(wg_row0) * row_bytes;
+        bool stage_free = false;
+        for (uint32_t i = 0; i < mine; i++) {
+            const uint32_t job = i * kDmaLoaders + loader;
+            if ((job + 1u) * 1024u > kStageAt && !stage_free) {
+                // this copy lands where the activation stages are: every consumer must have read its limbs
+                lds_await(lds_address(&control->staged), 2u * kDmaConsumers);
+                stage_free = true;
+            }
+            // lanes past the end of the share copy its last 16 bytes again, into bytes nobody reads
+            const uint32_t at = min(job * 1024u + lane_id * 16u, wg_bytes - 16u);
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + at),
+                                             reinterpret_cast<uint4*>(lds + job * 1024u), 16, 0, 0);
+        }
+        dma_publish<0>(skip, lds_address(&control->done[loader]));
+        return;
+    }
+
+    // ---- consumers ------------------------------------------------------------------------------
+    const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
+    const bool active = chunk < columns / kChunk;
+    const typename T::Lane lane = T::lane_setup(active ? chunk : 0u);
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int i = 0; i < NI; i++) stage_quad(stage[m], xv[m][i], threadIdx.x + i * 64u * kDmaConsumers);
+    lds_arrive(lds_address(&control->staged), lane_id == 0);
+    lds_await(lds_address(&control->staged), kDmaConsumers);
+    XLimbs xr[M];
+#pragma unroll
+    for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
+    lds_arrive(lds_address(&control->staged), lane_id == 0);  // the limbs are in registers
+
+    for (uint32_t local = wave; local < wg_rows; local += kDmaConsumers) {
+        // copies 0 .. last must have landed; copy j is number j / 4 of loader j % 4
+        const uint32_t last = ((local + 1u) * row_bytes - 1u) >> 10;
+        for (;;) {
+            bool ready = true;
+#pragma unroll
+            for (uint32_t l = 0; l < static_cast<uint32_t>(kDmaLoaders); l++) {
+                const uint32_t needed = last >= l ? (last - l) / kDmaLoaders + 1u : 0u;
+                ready = ready && lds_count(lds_address(&control->done[l])) >= needed;
+            }
+            if (ready) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        typename T::Data data;
+        T::load(lds + local * row_bytes, lane, data);
+        float value[M];
+        T::template fold<M>(data, lane, xr, value);
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float total = wave_sum(active ? value[m] : 0.f);
+            if (lane_id == 0) control->result[m][local] = total;
+        }
+    }
+    // Every copy has landed by now (the last row needed the last one): stores cannot stall a fold.
+    lds_arrive(lds_address(&control->folded), lane_id == 0);
+    if (wave != 0) return;
+    lds_await(lds_address(&control->folded), kDmaConsumers);
+    for (uint32_t local = lane_id; local < wg_rows; local += 64u) {
+        const uint32_t row = wg_row0 + local;
+        const float b = bias != nullptr ? bias[row] : 0.f;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float total = control->result[m][local];
+            y[static_cast<uint64_t>(m) * rows + row] = bias != nullptr ? total + b : total;
+        }
+    }
+}
+
+// Whether gemv_limb_dma_kernel takes this shape: one slice of columns, a share per compute unit that
+// fits LDS, enough rows per share to occupy the consumers.
+template <class T>
+bool dma_takes(uint32_t rows, uint32_t columns, uint32_t* rows_per_wg) {
+    if (columns > kSliceColumns) return false;
+    const uint32_t share = (rows + 255u) / 256u;
+    const uint64_t bytes = static_cast<uint64_t>(share) * (static_cast<uint64_t>(columns) / T::kBlockColumns) * T::kBlockBytes;
+    if (share < static_cast<uint32_t>(kDmaConsumers) || share > kDmaMaxRows || bytes > kDmaMaxShareBytes) return false;
+    *rows_per_wg = share;
+    return true;
+}
+
+template <class T, int M>
+hipError_t launch_dma(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
+                      float* y, uint32_t rows, uint32_t columns, uint32_t rows_per_wg, hipStream_t stream) {
+    static std::atomic<bool> allowed[64];
+    int device = 0;
+    if (hipError_t status = hipGetDevice(&device)) return status;
+    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+    const auto kernel = gemv_limb_dma_kernel<T, M>;
+    if (!allowed[device].load(std::memory_order_acquire)) {
+        if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLdsBytes))
+            return status;
+        allowed[device].store(true, std::memory_order_release);
+    }
+    const uint32_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDmaThreads), kDmaLdsBytes, stream, weight, x, x_row_stride, bias, y,
+                       rows, columns, rows_per_wg);
+    return hipGetLastError();
+}
+
 template <class T, int M, int R, int WAVES, int NK, bool LOOP>
 hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias,
                   float* y, uint32_t rows, uint32_t columns, uint32_t rows_per_wg, hipStream_t stream) {
@@ -954,6 +1204,11 @@ hipError_t launch_slices(const uint8_t* weight, const float* x, uint64_t x_row_s
                          const float* bias, float* y, uint32_t rows, uint32_t columns,
                          hipStream_t stream) {
     const uint32_t slices = (columns + kSliceColumns - 1) / kSliceColumns;
+    if constexpr (T::kLdsCopies && M <= 2) {  // three vectors need more registers than twelve waves leave
+        uint32_t rows_per_wg = 0;
+        if (gemv_limb_dma_enabled() && dma_takes<T>(rows, columns, &rows_per_wg))
+            return launch_dma<T, M>(weight, x, x_row_stride, bias, y, rows, columns, rows_per_wg, stream);
+    }
     if (slices <= 1) {
         return launch_rows<T, M, 8, 1>(weight, x, x_row_stride, bias, y, rows, columns, stream);
     }

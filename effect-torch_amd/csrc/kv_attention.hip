@@ -69,7 +69,8 @@ struct KvArgs {
 
 struct Span {
     uint32_t cursor, advance, needed, start;
-    uint32_t code, value;  // the first check of kv_prepare that fails, 0 = none
+    uint32_t code;   // the first check of kv_prepare that fails, 0 = none
+    uint64_t value;  // what that check reports; cursor + advance needs 33 bits
     bool ok;
 };
 
@@ -78,24 +79,28 @@ __device__ Span slot_span(const KvArgs& a, uint32_t slot) {
     Span s;
     s.cursor = a.cursors[slot];
     s.advance = a.advances[slot];
-    s.needed = s.cursor + s.advance;
-    s.start = a.context_window != 0 && s.needed > a.context_window ? s.needed - a.context_window : 0;
+    // The reference adds in usize and cannot wrap; a cursor near 2^32 (an idle slot's -1) must fail
+    // a check here, before any table access, instead of wrapping to a small context.
+    const uint64_t needed = static_cast<uint64_t>(s.cursor) + s.advance;
+    const uint64_t start = a.context_window != 0 && needed > a.context_window ? needed - a.context_window : 0;
     s.code = 0;
     s.value = 0;
     if (s.advance == 0 || s.advance > a.tokens) {
         s.code = kKvBadAdvance;
         s.value = s.advance;
-    } else if (s.needed - s.start > a.max_tokens) {
+    } else if (needed - start > a.max_tokens) {
         s.code = kKvOverCapacity;
-        s.value = s.needed - s.start;
-    } else if ((static_cast<uint64_t>(s.needed) + a.block_size - 1) / a.block_size > a.table_stride) {
+        s.value = needed - start;
+    } else if ((needed + a.block_size - 1) / a.block_size > a.table_stride) {
         s.code = kKvShortTable;
-        s.value = s.needed;
-    } else if (s.needed > a.max_context) {
+        s.value = needed;
+    } else if (needed > a.max_context) {  // max_context is 32 bits wide: passing means no wrap below
         s.code = kKvOverDeclared;
-        s.value = s.needed;
+        s.value = needed;
     }
     s.ok = s.code == 0;
+    s.needed = s.ok ? static_cast<uint32_t>(needed) : 0;
+    s.start = s.ok ? static_cast<uint32_t>(start) : 0;
     return s;
 }
 
@@ -146,10 +151,11 @@ __global__ void kv_zero_kernel(float* out, uint64_t count, unsigned long long* s
     if (i < slots) status[i] = 0;
 }
 
-// The status word of a slot: 0, or code << 32 | value. Written by one wave per slot, which also
+// The status word of a slot: 0, or code << 56 | value. Written by one wave per slot, which also
 // checks that the rows of the new positions lie inside the pool.
 __device__ void write_slot_status(const KvArgs& a, uint32_t slot, const Span& s, int lane) {
-    uint32_t code = s.code, value = s.value;
+    uint32_t code = s.code;
+    uint64_t value = s.value;
     if (s.ok) {
         uint32_t worst = 0;
         for (uint32_t token = lane; token < s.advance; token += 64) {
@@ -165,7 +171,7 @@ __device__ void write_slot_status(const KvArgs& a, uint32_t slot, const Span& s,
             value = worst;
         }
     }
-    if (lane == 0) a.status[slot] = (static_cast<unsigned long long>(code) << 32) | value;
+    if (lane == 0) a.status[slot] = (static_cast<unsigned long long>(code) << 56) | value;
 }
 
 // Positions a query attends to (napi/mod.rs:3481-3483).

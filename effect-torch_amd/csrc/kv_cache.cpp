@@ -197,7 +197,7 @@ int status_check(const et_kv_layer& layer, uint64_t tokens, const void* status_h
         std::memcpy(&word, static_cast<const char*>(status_host) + 8 * slot, sizeof word);
     if (word == 0) return ET_OK;
     slot -= 1;
-    const uint64_t code = word >> 32, value = word & 0xffffffffull;
+    const uint64_t code = word >> 56, value = word & 0x00ffffffffffffffull;
     switch (code) {
         case kKvBadAdvance:  // napi/mod.rs:3590-3594
             return fail(error, ET_ERR_EXECUTION,

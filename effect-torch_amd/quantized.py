@@ -458,6 +458,17 @@ def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, str
                                            sink.data_ptr(), workgroups, _stream_handle(stream)))
 
 
+READ_VARIANTS = {"plain": 0, "deep": 1, "streaming": 2, "lds4": 3, "lds8": 4}
+
+
+def calibration_read_variant(variant: str, src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
+    """The streaming read by one of several kernels (measurement aid, ``et_hip_calibration_read_variant``)."""
+    assert sink.numel() >= max(4 * workgroups, 1024) and sink.element_size() == 4
+    _check(N.lib().et_hip_calibration_read_variant(READ_VARIANTS[variant], src.data_ptr(),
+                                                   src.numel() * src.element_size(), sink.data_ptr(), workgroups,
+                                                   _stream_handle(stream)))
+
+
 def calibration_copy(src: torch.Tensor, dst: torch.Tensor, stream=None) -> None:
     """Plain copy ``dst <- src`` (measurement aid, ``et_hip_calibration_copy``)."""
     _check(N.lib().et_hip_calibration_copy(src.data_ptr(), dst.data_ptr(),

@@ -1,0 +1,57 @@
+/* Measurement aids of libet_hip.so: plain reads, a plain copy and matrix-core loops.
+ *
+ * These entry points are exported by the same library as the operator boundary (et_hip.h) but are
+ * not part of it: they mirror nothing in the reference and nothing on the operator path calls
+ * them. The benchmark uses them to put the rates this device sustains next to the published peaks
+ * and to calibrate hardware counters against a known number of bytes.
+ */
+#ifndef ET_HIP_CALIBRATE_H
+#define ET_HIP_CALIBRATE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A plain streaming read (`workgroups` workgroups of 256 lanes, each a
+ * contiguous range, 16-byte loads; `sink` receives four words per workgroup; at
+ * most 2^36 bytes) and a
+ * plain 16-byte copy, both of `bytes` rounded down to 16. They measure the
+ * bandwidth this device delivers to a kernel of a given footprint and calibrate
+ * hardware counters against a known number of bytes. They have no counterpart
+ * in the reference and are not part of the operator path. */
+int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
+                            void* stream);
+
+/* The same read by other kernels, to tell what the device delivers from what one read kernel
+ * reaches. `sink` holds at least 4 * workgroups words (at least 1024 for the LDS variants).
+ *   ET_READ_PLAIN     et_hip_calibration_read: four 16-byte loads in flight per lane, then the next four
+ *   ET_READ_DEEP      sixteen 16-byte loads in flight per lane
+ *   ET_READ_STREAMING ET_READ_DEEP with non-temporal loads
+ *   ET_READ_LDS_4 / ET_READ_LDS_8   one workgroup of 4 / 8 waves per `workgroups` entry that only issue
+ *                     1 KiB global-to-LDS copies (no registers, no arithmetic), each wave keeping
+ *                     32 / 16 KiB of copies in flight in a ring of LDS slots. */
+enum { ET_READ_PLAIN = 0, ET_READ_DEEP = 1, ET_READ_STREAMING = 2, ET_READ_LDS_4 = 3, ET_READ_LDS_8 = 4 };
+int et_hip_calibration_read_variant(int32_t variant, const void* src, uint64_t bytes, uint32_t* sink,
+                                    uint32_t workgroups, void* stream);
+int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* stream);
+
+/* Loops of matrix-core instructions that touch no memory: `workgroups` workgroups of four waves,
+ * every wave `iterations` rounds of four independent instructions of one kind, all operands ones;
+ * `sink` receives one float per thread (256 * workgroups), the sum of what the thread accumulated.
+ * ET_MFMA_I8: v_mfma_i32_32x32x32_i8 (65 536 operations each); ET_MFMA_I8_SCALED: the same
+ * instruction followed by the f32 epilogue of a contraction whose operands both carry a scale per 32
+ * columns (a tile of scale products from v_mfma_f32_32x32x2f32, one convert and one multiply-add per
+ * element); ET_MFMA_F16: v_mfma_f32_32x32x16_f16 (32 768 operations); ET_MFMA_F16_16X16:
+ * v_mfma_f32_16x16x32_f16 (16 384); ET_MFMA_I8_SCALED_BF16: ET_MFMA_I8_SCALED with the scale products from
+ * v_mfma_f32_32x32x16_bf16 (scales split into exact bfloat16 pieces). They measure what the matrix cores of this device sustain, the
+ * ceiling the batch kernels are compared with next to the published peak. No counterpart in the
+ * reference, not part of the operator path. */
+enum { ET_MFMA_I8 = 0, ET_MFMA_I8_SCALED = 1, ET_MFMA_F16 = 2, ET_MFMA_F16_16X16 = 3, ET_MFMA_I8_SCALED_BF16 = 4 };
+int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgroups, float* sink, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ET_HIP_CALIBRATE_H */

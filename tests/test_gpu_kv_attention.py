@@ -262,6 +262,25 @@ def test_device_side_checks_report_the_reference_errors(et, device):
         run_gpu(et, device, case, 0.1)
 
 
+@pytest.mark.parametrize("width", [128, 20])
+def test_a_cursor_at_the_top_of_32_bits_fails_a_check_instead_of_wrapping(et, device, width):
+    # cursor + advance is a usize sum in the reference (napi/mod.rs:3595) and cannot wrap; an idle
+    # slot's -1 inside the active batch must be reported, and no block-table entry may be read for it
+    rng = np.random.default_rng(5)
+    base = dict(slots=2, query_heads=4, kv_heads=2, width=width, block_size=16, contexts=[10, 20], tokens=1,
+                dtype=np.float16)
+    case = make_case(rng, advances=[1, 1], **base)
+    case["cursors"][1] = 0xFFFFFFFF
+    with pytest.raises(et.QuantizedError, match="live context 4294967296 exceeds pool capacity"):
+        run_gpu(et, device, case, 0.1, max_context=64)
+    with pytest.raises(et.QuantizedError, match="block table of slot 1 does not cover 4294967296 tokens"):
+        run_gpu(et, device, case, 0.1, max_context=64, context_window=8)
+    case["cursors"][1] = 0xFFFFFFF0
+    case["advances"][1] = 1
+    with pytest.raises(et.QuantizedError, match="live context 4294967281 exceeds pool capacity"):
+        run_gpu(et, device, case, 0.1, max_context=64)
+
+
 @pytest.mark.parametrize("dtype", [np.float16, "u8"])
 def test_decode_batch_at_full_size(et, device, dtype):
     # 32 slots x 32 query heads over 8 kv heads of width 128, contexts around 2048, block size 16

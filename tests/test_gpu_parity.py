@@ -356,6 +356,56 @@ def test_linear_full_size_q4k_batched_row_ranges(et, device, vectors):
     close(y12, got.astype(np.float64) + y2, 2e-3)
 
 
+@pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q5_K, oracle.Q8_0, oracle.Q4_0])
+@pytest.mark.parametrize("vectors,rows,columns", [(1, 2048, 4096), (2, 2100, 4096), (1, 4099, 1024), (2, 5003, 256),
+                                                  (3, 3000, 2048), (1, 30000, 512), (1, 1793, 4096)])
+def test_gemv_with_weights_copied_through_lds(et, device, codec, vectors, rows, columns):
+    # one or two vectors, one slice of columns, eight or more rows per compute unit: the loader waves
+    # copy the workgroup's share of W into LDS and the consumer waves fold it as it lands. Ragged last
+    # shares, shares that end inside a 1 KiB copy, narrow rows, bias; three vectors stay on the
+    # register-streaming kernel and must agree just the same.
+    rng = np.random.default_rng(codec * 17 + vectors + rows + columns)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    bias = rng.standard_normal(rows).astype(np.float32) if rows % 2 else None
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias)
+    again = run_linear(et, device, codec, rows, columns, x, weight, bias)
+    assert np.array_equal(got, again)  # arrival order of the copies does not reach the sums
+    close(got, oracle.linear_into(codec, rows, columns, x, weight, bias))
+    exact = x.astype(np.float64) @ oracle.decode_rows(codec, weight, columns).astype(np.float64).T
+    if bias is not None:
+        exact = exact + bias.astype(np.float64)
+    close(got, exact, oracle_noise=0)
+
+
+@pytest.mark.parametrize("vectors", [16, 64])
+def test_linear_full_size_q4k_batched_random_rows(et, device, vectors):
+    # the batched Q4_K 14336 x 4096 contraction on 1024 rows drawn at random from the whole matrix
+    cfg = synth.CONFIGS["q4_k_gemv_14336x4096"]
+    rng = np.random.default_rng(cfg["seed"] + 1000 + vectors)
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(vectors, cfg["columns"], rng)
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight)
+    picks = np.sort(rng.choice(cfg["rows"], 1024, replace=False))
+    want = oracle.linear_into(cfg["codec"], len(picks), cfg["columns"], x, np.ascontiguousarray(weight[picks]))
+    close(got[:, picks], want)
+
+
+def test_output_head_at_decode_batch(et, device):
+    # Q4_K 128256 x 4096 with 32 vectors (the output projection of a batched decode step) on row ranges
+    # at the start, in the middle and over the last two row tiles of the matrix
+    rows, columns, vectors = 128256, 4096, 32
+    rng = np.random.default_rng(128256)
+    base = synth.random_weight(oracle.Q4_K, 8192, columns, rng)
+    weight = np.concatenate([np.roll(base, r, axis=0) for r in range(-(-rows // 8192))])[:rows]
+    x = synth.random_activations(vectors, columns, rng)
+    got = run_linear(et, device, oracle.Q4_K, rows, columns, x, weight)
+    assert got.shape == (vectors, rows)
+    for begin, end in ((0, 160), (70000, 70130), (rows - 256, rows)):
+        want = oracle.linear_into(oracle.Q4_K, end - begin, columns, x, np.ascontiguousarray(weight[begin:end]))
+        close(got[:, begin:end], want)
+
+
 # --------------------------------------------------------------------------- int8-activation path
 
 def int8_close_to_f32_reference(got, ref, tol=2e-2):
@@ -413,6 +463,31 @@ def test_int8_full_size_prefill_row_ranges(et, device):
         want = oracle.linear_q8_rows(cfg["codec"], cfg["rows"], cfg["columns"], q, scale, total, weight,
                                      None, begin, begin + 16)
         close(got[:, begin:begin + 16], want[:, begin:begin + 16])
+
+
+def test_int8_full_size_prefill_against_the_f32_reference(et, device, capsys):
+    # config 3 (Q8_0 4096 x 14336, 512 vectors, int8 activations) against the f32-ACTIVATION reference
+    # on row ranges. Asserted: the per-vector bar (relative L2 <= 2e-2, elements within 2e-2 of the
+    # larger of |ref| and the row's peak). Reported, not asserted: the literal elementwise bar
+    # |a - b| <= 2e-2 * max(|b|, 1) - int8 rounding noise is proportional to |w|.|x| whatever the
+    # output's own size, so outputs that land near zero can miss it.
+    cfg = synth.CONFIGS["q8_0_gemm_i8_512x14336x4096"]
+    rng = np.random.default_rng(cfg["seed"])
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(512, cfg["columns"], rng, cfg["x_scale"])
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight, None, et.ActivationMode.INT8)
+    outside, worst, count = 0, 0.0, 0
+    for begin in (0, 1000, 2048, cfg["rows"] - 64):
+        ref = oracle.linear_into(cfg["codec"], 64, cfg["columns"], x, np.ascontiguousarray(weight[begin:begin + 64]))
+        mine = got[:, begin:begin + 64]
+        int8_close_to_f32_reference(mine, ref)
+        ratio = np.abs(mine.astype(np.float64) - ref) / (2e-2 * np.maximum(np.abs(ref), 1.0))
+        outside += int((ratio > 1.0).sum())
+        worst = max(worst, float(ratio.max()))
+        count += ratio.size
+    with capsys.disabled():
+        print(f"\n  literal bar |a-b| <= 2e-2*max(|b|,1): {outside} of {count} outputs outside "
+              f"({100.0 * outside / count:.3f} %), worst ratio {worst:.2f}")
 
 
 def test_gguf_file_to_contraction(et, device, tmp_path):
