@@ -247,7 +247,7 @@ def test_kv_attention_launch_shapes_and_status_wording(et):
         layer = decode.struct()
         words = [0] * 32
         words[slot] = word
-        words[-1] = (3 << 32) | 5  # a later slot's failure is not the one reported
+        words[-1] = (3 << 56) | 5  # a later slot's failure is not the one reported
         buf = ctypes.create_string_buffer(struct.pack("<32Q", *words), 256)
         status = _native.lib().et_hip_kv_attention_status_check(ctypes.byref(layer), 7, buf)
         return status, _native.last_error()
@@ -255,10 +255,12 @@ def test_kv_attention_launch_shapes_and_status_wording(et):
     layer = decode.struct()
     clean = ctypes.create_string_buffer(256)
     assert _native.lib().et_hip_kv_attention_status_check(ctypes.byref(layer), 7, clean) == 0
-    assert message((1 << 32) | 9, slot=3) == (2, "kv attention: advance 9 out of range for chunk length 7")
-    assert message((1 << 32) | 0) == (2, "kv attention: advance 0 out of range for chunk length 7")
-    assert message((2 << 32) | 70000) == (2, "kv attention: live context 70000 exceeds pool capacity 65536")
-    assert message((3 << 32) | 41, slot=30) == (2, "kv attention: block table of slot 30 does not cover 41 tokens")
+    assert message((1 << 56) | 9, slot=3) == (2, "kv attention: advance 9 out of range for chunk length 7")
+    assert message((1 << 56) | 0) == (2, "kv attention: advance 0 out of range for chunk length 7")
+    assert message((2 << 56) | 70000) == (2, "kv attention: live context 70000 exceeds pool capacity 65536")
+    # cursor + advance is a 33-bit sum: the value field is 56 bits wide
+    assert message((2 << 56) | (1 << 32)) == (2, "kv attention: live context 4294967296 exceeds pool capacity 65536")
+    assert message((3 << 56) | 41, slot=30) == (2, "kv attention: block table of slot 30 does not cover 41 tokens")
 
 
 def test_decode_operator_validation(et):
