@@ -170,6 +170,7 @@ def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
     }
 
 
+MIN_GRAPH_STEPS = 400     # a graph of fewer kernels pays its launch (about 15 us) per step: see time_steps
 MIN_REPETITIONS = 5       # timed replays of the K steps; the median is reported
 TIMED_WINDOW_MS = 20.0    # short replays are repeated until about this much device time is covered
 MAX_REPETITIONS = 400
@@ -181,7 +182,11 @@ def time_steps(step, steps, warmup, use_graph):
     steps unless disabled), repeated: every repetition is bracketed by its own pair of HIP events on
     that stream, the repetitions run back to back, and the MEDIAN over them is reported. A K-step
     replay shorter than the timed window is repeated more often (at least MIN_REPETITIONS times), so
-    that a short run is not one sample taken while the device clocks still ramp.
+    that a short run is not one sample taken while the device clocks still ramp. A graph of few
+    kernels would charge its own launch to them (about 15 us per replay: 0.75 us per step of a
+    20-step graph, none of it kernel time), so the K steps are captured `cycles` times over in one
+    graph until it holds MIN_GRAPH_STEPS of them; a repetition then times cycles * K steps and the
+    time per step is the replay time over that count.
     Returns (ms per step, graph used, wall seconds); LAST_TIMING holds repetitions / min / max."""
     import torch
 
@@ -190,17 +195,19 @@ def time_steps(step, steps, warmup, use_graph):
         step(i)
     torch.cuda.synchronize()
     graph = None
+    cycles = max(1, -(-MIN_GRAPH_STEPS // steps)) if use_graph else 1
     if use_graph:
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                for i in range(steps):
+                for i in range(steps * cycles):
                     step(i)
             graph.replay()  # one untimed replay
             torch.cuda.synchronize()
         except Exception as exc:  # noqa: BLE001 - report and fall back to plain enqueues
             print(f"HIP graph capture failed ({exc}); timing plain enqueues", file=sys.stderr)
             graph = None
+            cycles = 1
             torch.cuda.synchronize()
 
     def run_once():
@@ -228,11 +235,13 @@ def time_steps(step, steps, warmup, use_graph):
     wall = time.perf_counter() - wall0
     median = samples[len(samples) // 2] if len(samples) % 2 else 0.5 * (samples[len(samples) // 2 - 1] +
                                                                          samples[len(samples) // 2])
+    timed_steps = steps * cycles
     LAST_TIMING.clear()
-    LAST_TIMING.update({"repetitions": repetitions, "ms_per_step_min": round(samples[0] / steps, 6),
-                        "ms_per_step_max": round(samples[-1] / steps, 6),
-                        "timing": f"median of {repetitions} timed replays of the {steps} steps, one HIP event pair each"})
-    return median / steps, graph is not None, wall
+    LAST_TIMING.update({"repetitions": repetitions, "ms_per_step_min": round(samples[0] / timed_steps, 6),
+                        "ms_per_step_max": round(samples[-1] / timed_steps, 6),
+                        "timing": f"median of {repetitions} timed replays, one HIP event pair each, of a graph that holds "
+                                  f"the {steps} steps {cycles} time(s) over ({timed_steps} launches per replay)"})
+    return median / timed_steps, graph is not None, wall
 
 
 def with_timing(result):

@@ -37,6 +37,7 @@ from .kv_cache import (  # noqa: F401
     kv_attention_status_check,
     kv_attention_workspace,
     kv_attention_workspace_bytes,
+    kv_commit,
 )
 from .decode_ops import (  # noqa: F401
     RotaryLayout,
@@ -51,6 +52,7 @@ from .decode_ops import (  # noqa: F401
     rotary_pair_into,
     silu_mul_into,
 )
+from .decode_step import LlamaDecoder, LlamaShape, algorithmic_bytes_per_step  # noqa: F401
 from .gguf import (  # noqa: F401
     GgufFile,
     GgufMetadataValue,

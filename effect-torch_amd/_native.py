@@ -43,6 +43,7 @@ class EtPrepareSource(ctypes.Structure):
         ("x_row_stride", ctypes.c_uint64),
         ("second", ctypes.c_void_p),
         ("eps", ctypes.c_double),
+        ("second_dtype", ctypes.c_int32),
     ]
 
 
@@ -136,7 +137,7 @@ SIGNATURES = {
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_linear_enqueue_prepared_group_then_rotary": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp,
                                                                         _u64, ctypes.POINTER(EtRotaryAfter), _vp, _vp]),
-    "et_hip_linear_enqueue_prepared_then_norm": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp,
+    "et_hip_linear_enqueue_prepared_then_norm": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp, _i32,
                                                                 ctypes.c_double, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
     "et_hip_embedding_plan_destroy": (None, [_vp]),
@@ -152,6 +153,7 @@ SIGNATURES = {
                                                          _vp, _u64, _vp, _vp]),
     "et_hip_kv_attention_status_check": (ctypes.c_int, [_KV, _u64, _vp]),
     "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
+    "et_hip_kv_commit": (ctypes.c_int, [_KV, _vp]),
     "et_hip_rms_norm_into": (ctypes.c_int, [_T, _T, ctypes.c_double, _T, _vp]),
     "et_hip_rotary_into": (ctypes.c_int, [_T, _vp, _u64, ctypes.c_double, ctypes.c_double, _i32, _T, _vp]),
     "et_hip_rotary_pair_into": (ctypes.c_int, [_T, _T, _vp, _u64, ctypes.c_double, ctypes.c_double, _i32, _T, _T, _vp]),

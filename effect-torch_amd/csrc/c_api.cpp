@@ -272,8 +272,9 @@ int et_hip_linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const
 int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
                                              const uint8_t* weight, const float* bias, const float* residual,
                                              float* y, void* workspace, uint64_t workspace_bytes,
-                                             const et_linear_plan* next, const float* norm_weight, double eps,
-                                             void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                             const et_linear_plan* next, const void* norm_weight,
+                                             int32_t norm_weight_dtype, double eps, void* next_prepared,
+                                             uint64_t next_prepared_bytes, void* stream,
                                              const volatile int32_t* cancel) {
     return guarded([&](std::string* error) -> int {
         if (plan == nullptr || next == nullptr) {
@@ -281,7 +282,8 @@ int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const v
             return ET_ERR_INVALID;
         }
         return et::quantized::linear_enqueue_prepared_then_norm(*plan, prepared, weight, bias, residual, y, workspace,
-                                                                workspace_bytes, *next, norm_weight, eps, next_prepared,
+                                                                workspace_bytes, *next, norm_weight, norm_weight_dtype, eps,
+                                                                next_prepared,
                                                                 next_prepared_bytes, stream, cancel, error);
     });
 }
@@ -448,6 +450,27 @@ int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens, 
             return ET_ERR_INVALID;
         }
         return et::kv::status_check(*layer, tokens, status_host, error);
+    });
+}
+
+int et_hip_kv_commit(const et_kv_layer* layer, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (layer == nullptr || layer->cursors == nullptr || layer->advances == nullptr) {
+            *error = "kv commit: layer, cursors or advances is NULL";
+            return ET_ERR_INVALID;
+        }
+        if (layer->active_batch > layer->slots) {
+            *error = "kv commit: active batch " + std::to_string(layer->active_batch) + " exceeds " +
+                     std::to_string(layer->slots) + " slots";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status = et::commit_advances(const_cast<uint32_t*>(layer->cursors), layer->advances,
+                                                      layer->active_batch, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) {
+            *error = std::string("kv commit: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
     });
 }
 

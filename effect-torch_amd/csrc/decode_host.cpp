@@ -41,7 +41,9 @@ int rms_norm_into(const TensorView& x, const TensorView* weight, double eps, con
     const uint64_t columns = x.shape.back(), elements = numel(x);
     if (columns == 0 || elements == 0)
         return fail(error, ET_ERR_UNSUPPORTED, "rms_norm: zero-sized dimensions are unsupported");
-    if (weight != nullptr && (weight->dtype != x.dtype || weight->shape != std::vector<uint64_t>{columns}))
+    // composed.rs:700-705 wants the weight in the input's type; a half-float weight is widened on use
+    if (weight != nullptr && ((weight->dtype != x.dtype && weight->dtype != ET_DTYPE_F16) ||
+                              weight->shape != std::vector<uint64_t>{columns}))
         return fail(error, ET_ERR_UNSUPPORTED, "rms_norm: weight must match the last dimension and dtype");
     if (destination.dtype != x.dtype || destination.shape != x.shape)
         return fail(error, ET_ERR_EXECUTION, "rms_norm output: destination does not match the input shape");
@@ -51,8 +53,12 @@ int rms_norm_into(const TensorView& x, const TensorView* weight, double eps, con
         return fail(error, ET_ERR_UNSUPPORTED, "rms_norm: geometry exceeds the launch limits");
     if (x.data == nullptr || destination.data == nullptr || (weight != nullptr && weight->data == nullptr))
         return fail(error, ET_ERR_INVALID, "rms_norm: NULL device pointer");
-    return launched(rms_norm(f32_data(x), weight ? f32_data(*weight) : nullptr, eps, f32_out(destination),
-                             elements / columns, columns, static_cast<hipStream_t>(stream)),
+    const bool half = weight != nullptr && weight->dtype == ET_DTYPE_F16;
+    const void* w = weight == nullptr ? nullptr
+                    : half            ? static_cast<const void*>(static_cast<const uint16_t*>(weight->data) + weight->offset)
+                                      : static_cast<const void*>(f32_data(*weight));
+    return launched(rms_norm(f32_data(x), w, half ? 1 : 0, eps, f32_out(destination), elements / columns, columns,
+                             static_cast<hipStream_t>(stream)),
                     "rms_norm", error);
 }
 
@@ -210,7 +216,8 @@ int gather_rows_into(const TensorView& table, const TensorView& indexes, const T
     if (indexes.dtype != ET_DTYPE_U32 && indexes.dtype != ET_DTYPE_I64)
         return fail(error, ET_ERR_UNSUPPORTED, "index_select: indexes must be u32 or i64");
     const uint64_t count = numel(indexes), width = table.shape[1];
-    if (destination.dtype != table.dtype || destination.shape.size() != 2)
+    const bool widen = destination.dtype == ET_DTYPE_F32 && (table.dtype == ET_DTYPE_F16 || table.dtype == ET_DTYPE_BF16);
+    if ((destination.dtype != table.dtype && !widen) || destination.shape.size() != 2)
         return fail(error, ET_ERR_EXECUTION, "index_select destination rank mismatch: expected 2, got " +
                                                  std::to_string(destination.shape.size()));
     if (destination.shape[0] != count)
@@ -226,9 +233,14 @@ int gather_rows_into(const TensorView& table, const TensorView& indexes, const T
     if (table.data == nullptr || indexes.data == nullptr || destination.data == nullptr || status == nullptr)
         return fail(error, ET_ERR_INVALID, "index_select: NULL device pointer");
     const char* source = static_cast<const char*>(table.data) + table.offset * element;
-    char* target = const_cast<char*>(static_cast<const char*>(destination.data)) + destination.offset * element;
+    char* target = const_cast<char*>(static_cast<const char*>(destination.data)) + destination.offset * (widen ? 4 : element);
     const bool wide = indexes.dtype == ET_DTYPE_I64;
     const char* ids = static_cast<const char*>(indexes.data) + indexes.offset * (wide ? 8 : 4);
+    if (widen)
+        return launched(gather_rows_widen(source, table.dtype == ET_DTYPE_BF16 ? 1 : 0, table.shape[0], width, ids,
+                                          wide ? 1 : 0, count, reinterpret_cast<float*>(target), status,
+                                          static_cast<hipStream_t>(stream)),
+                        "index_select", error);
     return launched(gather_rows(source, table.shape[0], width * element, ids, wide ? 1 : 0, count, target, status,
                                 static_cast<hipStream_t>(stream)),
                     "index_select", error);

@@ -47,6 +47,29 @@ __device__ __forceinline__ double rms_row_scale(const float* __restrict__ in, ui
     return 1.0 / sqrt(mean_square + eps);
 }
 
+// The weight of an RMS norm: f32, or f16 widened on use (exact), or none (ones). The reference casts
+// a half-float parameter to the activations' type in front of the operator; reading the halves here
+// gives the same values without the cast's launch.
+struct NormWeight {
+    const void* data;  // [columns], or null
+    int32_t half;      // 0: float, 1: IEEE binary16
+};
+__device__ __forceinline__ float norm_weight_one(const NormWeight& w, uint32_t i) {
+    if (w.data == nullptr) return 1.f;
+    if (w.half) return static_cast<float>(static_cast<const _Float16*>(w.data)[i]);
+    return static_cast<const float*>(w.data)[i];
+}
+// elements 4 i .. 4 i + 3 (the array is 16-byte aligned for floats, 8-byte aligned for halves)
+__device__ __forceinline__ float4 norm_weight_four(const NormWeight& w, uint32_t i) {
+    if (w.data == nullptr) return make_float4(1.f, 1.f, 1.f, 1.f);
+    if (w.half) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        const h4 v = static_cast<const h4*>(w.data)[i];
+        return make_float4(static_cast<float>(v.x), static_cast<float>(v.y), static_cast<float>(v.z), static_cast<float>(v.w));
+    }
+    return static_cast<const float4*>(w.data)[i];
+}
+
 // Second pass: x * scale * weight in f64, rounded once.
 __device__ __forceinline__ float rms_one(float value, double scale, float w) {
     return static_cast<float>(static_cast<double>(value) * scale * static_cast<double>(w));

@@ -26,7 +26,7 @@ constexpr uint32_t kArgmaxChunk = 4096;  // logits per workgroup of the first st
 // One workgroup of 256 per row. VEC: the row is read as float4 (columns % 4 == 0, 16-byte aligned
 // rows); the first four vectors of a thread stay in registers for the second pass.
 template <bool VEC>
-__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const NormWeight weight,
                                                        double eps, float* __restrict__ out, uint32_t columns) {
     __shared__ double partial[4];
     const float* in = x + static_cast<uint64_t>(blockIdx.x) * columns;
@@ -35,18 +35,14 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
         float4 held[kRmsHeld];
         const double scale = rms_row_scale(in, columns, eps, held, partial);
         const uint32_t vectors = columns / 4;
-        const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
 #pragma unroll
         for (int j = 0; j < kRmsHeld; j++) {
             const uint32_t i = threadIdx.x + 256 * j;
-            if (i < vectors)
-                reinterpret_cast<float4*>(row)[i] =
-                    rms_four(held[j], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones);
+            if (i < vectors) reinterpret_cast<float4*>(row)[i] = rms_four(held[j], scale, norm_weight_four(weight, i));
         }
         for (uint32_t i = threadIdx.x + 256 * kRmsHeld; i < vectors; i += 256)
             reinterpret_cast<float4*>(row)[i] =
-                rms_four(reinterpret_cast<const float4*>(in)[i], scale,
-                         weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones);
+                rms_four(reinterpret_cast<const float4*>(in)[i], scale, norm_weight_four(weight, i));
     } else {
         double sum = 0.0;
         for (uint32_t i = threadIdx.x; i < columns; i += 256) sum += static_cast<double>(in[i]) * static_cast<double>(in[i]);
@@ -55,7 +51,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
         __syncthreads();
         const double mean_square = ((partial[0] + partial[1]) + (partial[2] + partial[3])) / static_cast<double>(columns);
         const double scale = 1.0 / sqrt(mean_square + eps);
-        for (uint32_t i = threadIdx.x; i < columns; i += 256) row[i] = rms_one(in[i], scale, weight != nullptr ? weight[i] : 1.f);
+        for (uint32_t i = threadIdx.x; i < columns; i += 256) row[i] = rms_one(in[i], scale, norm_weight_one(weight, i));
     }
 }
 
@@ -221,16 +217,82 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const Word* __restrict
     for (uint64_t i = threadIdx.x; i < row_words; i += 256) target[i] = source[i];
 }
 
+// The lookup of a half-float table into f32 rows: index_select followed by the cast the reference's
+// graph puts behind it, in one launch (the widening is exact). HALF: IEEE binary16, else bfloat16.
+template <bool HALF>
+__global__ __launch_bounds__(256) void gather_rows_widen_kernel(const uint16_t* __restrict__ table, uint64_t table_rows,
+                                                                uint64_t width, const void* __restrict__ indexes,
+                                                                int index_is_i64, float* __restrict__ out,
+                                                                unsigned long long* __restrict__ status) {
+    const uint64_t p = blockIdx.x;
+    const long long id = index_is_i64 ? static_cast<const long long*>(indexes)[p]
+                                      : static_cast<long long>(static_cast<const uint32_t*>(indexes)[p]);
+    const bool inside = id >= 0 && static_cast<uint64_t>(id) < table_rows;
+    if (threadIdx.x == 0) status[p] = inside ? 0ull : (1ull << 63) | (static_cast<unsigned long long>(id) & ~(1ull << 63));
+    if (!inside) return;
+    const uint16_t* source = table + static_cast<uint64_t>(id) * width;
+    float* target = out + p * width;
+    const auto widen = [](uint16_t bits) {
+        if constexpr (HALF) {
+            union {
+                uint16_t u;
+                _Float16 h;
+            } cvt;
+            cvt.u = bits;
+            return static_cast<float>(cvt.h);
+        } else {
+            return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+        }
+    };
+    if (width % 4 == 0 && reinterpret_cast<uintptr_t>(source) % 8 == 0 && reinterpret_cast<uintptr_t>(target) % 16 == 0) {
+        for (uint64_t i = threadIdx.x; i < width / 4; i += 256) {
+            const uint2 raw = reinterpret_cast<const uint2*>(source)[i];
+            reinterpret_cast<float4*>(target)[i] =
+                make_float4(widen(static_cast<uint16_t>(raw.x)), widen(static_cast<uint16_t>(raw.x >> 16)),
+                            widen(static_cast<uint16_t>(raw.y)), widen(static_cast<uint16_t>(raw.y >> 16)));
+        }
+    } else {
+        for (uint64_t i = threadIdx.x; i < width; i += 256) target[i] = widen(source[i]);
+    }
+}
+
+// kv_prepare's commit (crates/runtime-cpu/src/napi/mod.rs:4511-4517): cursor += advance for the active slots.
+__global__ __launch_bounds__(64) void commit_advances_kernel(uint32_t* __restrict__ cursors,
+                                                             const uint32_t* __restrict__ advances, uint32_t slots) {
+    const uint32_t slot = blockIdx.x * 64u + threadIdx.x;
+    if (slot < slots) cursors[slot] += advances[slot];
+}
+
 }  // namespace
 
-hipError_t rms_norm(const float* x, const float* weight, double eps, float* out, uint64_t rows, uint64_t columns,
-                    hipStream_t stream) {
-    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (columns % 4 == 0 && aligned(x) && aligned(out) && (weight == nullptr || aligned(weight)))
-        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps,
+hipError_t commit_advances(uint32_t* cursors, const uint32_t* advances, uint64_t slots, hipStream_t stream) {
+    if (slots == 0) return hipSuccess;
+    hipLaunchKernelGGL(commit_advances_kernel, dim3(static_cast<uint32_t>((slots + 63) / 64)), dim3(64), 0, stream, cursors,
+                       advances, static_cast<uint32_t>(slots));
+    return hipGetLastError();
+}
+
+hipError_t gather_rows_widen(const void* table, int table_is_bf16, uint64_t table_rows, uint64_t width, const void* indexes,
+                             int index_is_i64, uint64_t count, float* out, void* status, hipStream_t stream) {
+    auto* words = static_cast<unsigned long long*>(status);
+    if (table_is_bf16)
+        hipLaunchKernelGGL(gather_rows_widen_kernel<false>, dim3(static_cast<uint32_t>(count)), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(table), table_rows, width, indexes, index_is_i64, out, words);
+    else
+        hipLaunchKernelGGL(gather_rows_widen_kernel<true>, dim3(static_cast<uint32_t>(count)), dim3(256), 0, stream,
+                           static_cast<const uint16_t*>(table), table_rows, width, indexes, index_is_i64, out, words);
+    return hipGetLastError();
+}
+
+hipError_t rms_norm(const float* x, const void* weight, int weight_is_half, double eps, float* out, uint64_t rows,
+                    uint64_t columns, hipStream_t stream) {
+    const auto aligned = [](const void* p, uintptr_t to) { return reinterpret_cast<uintptr_t>(p) % to == 0; };
+    const NormWeight w = {weight, weight_is_half ? 1 : 0};
+    if (columns % 4 == 0 && aligned(x, 16) && aligned(out, 16) && aligned(weight, weight_is_half ? 8 : 16))
+        hipLaunchKernelGGL(rms_norm_kernel<true>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, w, eps,
                            out, static_cast<uint32_t>(columns));
     else
-        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, weight, eps,
+        hipLaunchKernelGGL(rms_norm_kernel<false>, dim3(static_cast<uint32_t>(rows)), dim3(256), 0, stream, x, w, eps,
                            out, static_cast<uint32_t>(columns));
     return hipGetLastError();
 }

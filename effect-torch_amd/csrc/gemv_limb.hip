@@ -923,20 +923,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
 // What bounds gemv_limb_kernel is how many bytes a compute unit keeps in flight: a wave requests
 // the next row only after it has folded the one before, because a wave that issues a load into a
 // full memory queue stalls with all the arithmetic behind it. Here the two jobs are split between
-// waves. The workgroup's whole share of W - a contiguous range of rows, at most 158 KiB - is
-// requested at once by four LOADER waves as 1 KiB global_load_lds copies straight into LDS (no
-// registers; a loader that stalls on a full queue holds nothing up), and eight CONSUMER waves
-// prepare the activations meanwhile and then fold the rows out of LDS in the order they arrive
-// (row i of the share belongs to consumer i % 8). A consumer issues no global load after its
-// activation loads and no store before every copy has landed.
+// waves. The workgroup's share of W - a contiguous range of rows, at most 158 KiB - is cut into
+// eight contiguous ranges, one per CONSUMER wave; consumer w's range is copied into LDS, as it lies
+// in memory, by LOADER wave w with 1 KiB global_load_lds copies (no registers; a loader that stalls
+// on a full queue holds nothing up), while the consumers prepare the activations and then fold
+// their rows out of LDS as they land. A consumer issues no global load after its activation loads.
 //
-// Hand-over without barriers (s_barrier would tie the loaders to the consumers' prologue): loader
-// l publishes in LDS how many of its copies have landed (loads return in order per wave; one
-// counted s_waitcnt per copy), and a consumer polls the four counts until they cover its row.
-// The consumers meet each other through two LDS counters (`staged`, `folded`).
-// LDS: [weights: whole KiB][...][StageMemory x M][control]. With three vectors the stages overlap
-// the end of a full-size share: the copies that land there wait until every consumer has read
-// its limbs (`staged` == 2 * consumers).
+// Hand-over without barriers (s_barrier would tie the loaders to the consumers' prologue): a
+// loader keeps DEPTH copies in flight; before it issues the next one it waits for the oldest
+// (loads return in order per wave: one counted s_waitcnt) and publishes in LDS how many of its
+// copies have landed; its consumer polls that one word until it covers the next row.
+// The last row of a range is folded by its loader, which knows first when its last copy has landed.
+// The consumers meet each other through one LDS counter (`staged`).
+// LDS: [the ranges, whole KiB each][...][StageMemory x M][control]; shapes whose ranges would reach
+// into the stages stay on gemv_limb_kernel.
 // ---------------------------------------------------------------------------
 // ET_HIP_GEMV_LDS_COPIES=0 in the environment keeps every shape on gemv_limb_kernel (for A/B timing).
 bool gemv_limb_dma_enabled() {
@@ -947,23 +947,22 @@ bool gemv_limb_dma_enabled() {
     return enabled;
 }
 
-constexpr int kDmaConsumers = 8;
-constexpr int kDmaLoaders = 4;
-constexpr int kDmaJobs = 40;  // copies per loader at most: vmcnt counts to 63
-constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaLoaders);
+constexpr int kDmaPairs = 8;  // ranges of a share: one loader and one consumer wave each (a workgroup has at most
+                              // sixteen waves)
+constexpr int kDmaConsumers = kDmaPairs;
+constexpr int kDmaLoaderRows = 1;  // rows at the end of a range that its loader folds (two and three measured slower:
+                                   // a loader that folds is late with the word its consumer waits for)
+constexpr int kDmaDepth = 4;  // copies a loader keeps in flight: more only lengthen the queue, and a loader says that a
+                              // copy has landed only when it may issue the copy DEPTH places later
+constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaPairs);
 constexpr uint32_t kDmaLdsBytes = 160u * 1024u;
-constexpr uint32_t kDmaMaxRows = 128;  // rows of a workgroup's share
 struct DmaControl {
-    uint32_t done[kDmaLoaders];  // copies of loader l that have landed
-    uint32_t staged;             // consumer arrivals: +1 after writing the stage, +1 after reading the limbs
-    uint32_t folded;             // consumers that have left all their results
-    uint32_t pad[2];
-    float result[kGemvLimbMaxVectors][kDmaMaxRows];
+    uint32_t landed[kDmaPairs];  // copies of loader w that have landed
+    uint32_t staged;             // consumers that have written their part of the stages
+    uint32_t pad[7];
 };
-constexpr uint32_t kDmaControlAt = kDmaLdsBytes - 2048u;
-static_assert(sizeof(DmaControl) <= 2048, "control block");
-constexpr uint32_t kDmaMaxShareBytes = kDmaControlAt;  // whole KiB below the control block
-static_assert(kDmaMaxShareBytes / 1024u <= kDmaLoaders * kDmaJobs, "every KiB has a copy slot");
+constexpr uint32_t kDmaControlAt = kDmaLdsBytes - 1024u;
+static_assert(sizeof(DmaControl) == 64, "sixteen words, zeroed by sixteen lanes");
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
 constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
@@ -972,8 +971,8 @@ constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 
 // does not look into. LDS serves a wave's requests in order, so "data, then counter" needs no
 // fence; an acquire / release at workgroup scope - or any LDS access the compiler can see next to
 // global-to-LDS copies, whose destinations it cannot tell from other LDS addresses - would make it
-// wait for every outstanding copy (vmcnt 0), exactly what a loader with forty copies in flight
-// must not do. These accesses touch the control block only, where no copy lands.
+// wait for every outstanding copy (vmcnt 0), exactly what a loader with copies in flight must not
+// do. These accesses touch the control block only, where no copy lands.
 __device__ __forceinline__ uint32_t lds_address(const void* pointer) {
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(pointer));  // low half of the flat address
 }
@@ -994,20 +993,51 @@ __device__ __forceinline__ void lds_await(uint32_t address, uint32_t count) {
     while (lds_count(address) < count) __builtin_amdgcn_s_sleep(1);
 }
 
-// The loader's copies sit in the LAST slots of its list of kDmaJobs (the first `skip` are empty), so
-// that "copy of slot I has landed" is the compile-time count vmcnt <= kDmaJobs - 1 - I.
-template <int I>
-__device__ __forceinline__ void dma_publish(uint32_t skip, uint32_t done_address) {
-    if constexpr (I < kDmaJobs) {
-        if (static_cast<uint32_t>(I) >= skip) {
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(kDmaJobs - 1 - I));
-            lds_store_unseen(done_address, static_cast<uint32_t>(I) - skip + 1u);
+// load_limbs for a wave with copies in flight: the same reads, unseen by the compiler.
+__device__ __forceinline__ void load_limbs_unseen(const StageMemory& stage, uint32_t lane, bool active, XLimbs& out) {
+    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v4u v;
+            asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_address(&stage.limbs[k][limb_slot(4u * lane + j) * 4u])) : "memory");
+            out.limb[k][4 * j + 0] = static_cast<int>(v.x);
+            out.limb[k][4 * j + 1] = static_cast<int>(v.y);
+            out.limb[k][4 * j + 2] = static_cast<int>(v.z);
+            out.limb[k][4 * j + 3] = static_cast<int>(v.w);
         }
-        dma_publish<I + 1>(skip, done_address);
+    }
+    uint32_t unit, sum0, sum1;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(unit) : "v"(lds_address(&stage.unit[lane])) : "memory");
+    asm volatile("ds_read_b32 %0, %1" : "=v"(sum0) : "v"(lds_address(&stage.sum[0][lane])) : "memory");
+    asm volatile("ds_read_b32 %0, %1" : "=v"(sum1) : "v"(lds_address(&stage.sum[1][lane])) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // the values are used only from here on: every register above is written by now
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) out.limb[k][j] = active ? out.limb[k][j] : 0;
+    out.s = active ? __uint_as_float(unit) : 0.f;
+    out.sum[0] = active ? __uint_as_float(sum0) : 0.f;
+    out.sum[1] = active ? __uint_as_float(sum1) : 0.f;
+}
+
+// The last copies of a loader: `outstanding` <= DEPTH of them are in flight, in the last slots of a
+// list of DEPTH, so that "the copy of slot I has landed" is the compile-time count vmcnt <= DEPTH - 1 - I.
+template <int DEPTH, int I, class F>
+__device__ __forceinline__ void dma_drain(uint32_t outstanding, uint32_t landed_address, uint32_t& landed, const F& after) {
+    if constexpr (I < DEPTH) {
+        if (static_cast<uint32_t>(I) >= DEPTH - outstanding) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1 - I));
+            lds_store_unseen(landed_address, ++landed);
+            after(landed);
+        }
+        dma_drain<DEPTH, I + 1>(outstanding, landed_address, landed, after);
     }
 }
 
-template <class T, int M>
+template <class T, int M, int DEPTH>
 __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
@@ -1024,13 +1054,36 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     if (wg_row0 >= rows) return;
     const uint32_t wg_rows = min(rows_per_wg, rows - wg_row0);
     const uint32_t row_bytes = static_cast<uint32_t>(T::row_bytes(columns));
-    const uint32_t wg_bytes = wg_rows * row_bytes;
-    const uint32_t jobs = (wg_bytes + 1023u) >> 10;
     const bool consumer = wave < static_cast<uint32_t>(kDmaConsumers);
+    // the range this wave works on: rows [first, first + count) of the share, `range_kib` KiB of LDS each
+    const uint32_t pair = consumer ? wave : wave - kDmaConsumers;
+    const uint32_t per_pair = (rows_per_wg + kDmaPairs - 1u) / kDmaPairs;
+    const uint32_t first = min(pair * per_pair, wg_rows);
+    const uint32_t count = min(per_pair, wg_rows - first);
+    const uint32_t range_kib = (per_pair * row_bytes + 1023u) >> 10;
+    uint8_t* range = lds + pair * (range_kib << 10);
 
-    // Activation loads go first: they must not queue behind the copies.
+    const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
+    const bool active = chunk < columns / kChunk;
+    const typename T::Lane lane = T::lane_setup(active ? chunk : 0u);
+    XLimbs xr[M];
+    // Folds a row of the range that is in registers and stores the result. The loaders keep few copies
+    // in flight, so a store finds room in the memory queue.
+    const auto fold_row = [&](uint32_t r, const typename T::Data& data) {
+        float value[M];
+        T::template fold<M>(data, lane, xr, value);
+        const uint32_t row = wg_row0 + first + r;
+        const float b = bias != nullptr ? bias[row] : 0.f;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float total = wave_sum(active ? value[m] : 0.f);
+            if (lane_id == 0) y[static_cast<uint64_t>(m) * rows + row] = bias != nullptr ? total + b : total;
+        }
+    };
+
     float4 xv[M][NI];
     if (consumer) {
+        // Activation loads go first in the consumers: nothing of theirs may queue behind a copy.
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
@@ -1039,94 +1092,93 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
                 xv[m][i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (quad < (columns >> 2)) xv[m][i] = reinterpret_cast<const float4*>(x + m * x_row_stride)[quad];
             }
-    }
-    if (threadIdx.x < 8) reinterpret_cast<uint32_t*>(control)[threadIdx.x] = 0u;
-    __syncthreads();  // the only barrier: the counters are zero, the activation loads are on their way
-
-    if (!consumer) {
+        if (threadIdx.x < 16) reinterpret_cast<uint32_t*>(control)[threadIdx.x] = 0u;
+        __syncthreads();  // the only barrier: the counters are zero before anybody counts
+    } else {
         // ---- loaders ------------------------------------------------------------------------
-        const uint32_t loader = wave - kDmaConsumers;
-        const uint32_t mine = jobs > loader ? (jobs - loader + kDmaLoaders - 1u) / kDmaLoaders : 0u;
-        const uint32_t skip = kDmaJobs - mine;
-        const uint8_t* source = weight + static_cast<uint64_t>(wg_row0) * row_bytes;
-        bool stage_free = false;
-        for (uint32_t i = 0; i < mine; i++) {
-            const uint32_t job = i * kDmaLoaders + loader;
-            if ((job + 1u) * 1024u > kStageAt && !stage_free) {
-                // this copy lands where the activation stages are: every consumer must have read its limbs
-                lds_await(lds_address(&control->staged), 2u * kDmaConsumers);
-                stage_free = true;
-            }
-            // lanes past the end of the share copy its last 16 bytes again, into bytes nobody reads
-            const uint32_t at = min(job * 1024u + lane_id * 16u, wg_bytes - 16u);
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + at),
-                                             reinterpret_cast<uint4*>(lds + job * 1024u), 16, 0, 0);
+        const uint32_t bytes = count * row_bytes;
+        const uint32_t copies = (bytes + 1023u) >> 10;
+        const uint8_t* source = weight + (static_cast<uint64_t>(wg_row0) + first) * row_bytes;
+        const uint32_t landed_address = lds_address(&control->landed[pair]);
+        const auto copy = [&](uint32_t i) {
+            const uint32_t at = i * 1024u + lane_id * 16u;
+            if (at < bytes)  // the last copy of a range stops where the range ends
+                // streamed once: non-temporal (aux bit 1), the caches keep nothing of it
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + at),
+                                                 reinterpret_cast<uint4*>(range + i * 1024u), 16, 0, 2);
+        };
+        // The first copies wait for the barrier, i.e. until the consumers have issued their activation
+        // loads: issued ahead of it they delay those loads, and with them every fold, by half a microsecond.
+        __syncthreads();
+        const uint32_t head = min(copies, static_cast<uint32_t>(DEPTH));
+        for (uint32_t i = 0; i < head; i++) copy(i);
+        // The loader folds the last row of its range itself (below), next to the consumer folding the
+        // row before: one fold after the last byte instead of two. Its
+        // limbs come out of the stages as soon as the consumers have written them, while its first
+        // copies are on their way (measured: later in the stream this costs a quarter microsecond).
+        lds_await(lds_address(&control->staged), kDmaConsumers);
+#pragma unroll
+        for (int m = 0; m < M; m++) load_limbs_unseen(stage[m], lane_id, active, xr[m]);
+        uint32_t landed = 0;
+        for (uint32_t i = head; i < copies; i++) {
+            // the oldest copy in flight has landed: say so, then take its place in the queue
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));
+            lds_store_unseen(landed_address, ++landed);
+            copy(i);
         }
-        dma_publish<0>(skip, lds_address(&control->done[loader]));
+        // With every copy issued the loader is free: it folds the last kDmaLoaderRows rows of the range
+        // itself, each the moment its last copy has landed.
+        const uint32_t own = min(count, static_cast<uint32_t>(kDmaLoaderRows));
+        uint32_t next_own = count - own;
+        const auto fold_landed = [&](uint32_t have) {
+            while (next_own < count && have >= (((next_own + 1u) * row_bytes + 1023u) >> 10)) {
+                typename T::Data data;
+                T::load(range + next_own * row_bytes, lane, data);
+                fold_row(next_own, data);
+                next_own += 1u;
+            }
+        };
+        dma_drain<DEPTH, 0>(head, landed_address, landed, fold_landed);
         return;
     }
 
     // ---- consumers ------------------------------------------------------------------------------
-    const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
-    const bool active = chunk < columns / kChunk;
-    const typename T::Lane lane = T::lane_setup(active ? chunk : 0u);
 #pragma unroll
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int i = 0; i < NI; i++) stage_quad(stage[m], xv[m][i], threadIdx.x + i * 64u * kDmaConsumers);
     lds_arrive(lds_address(&control->staged), lane_id == 0);
     lds_await(lds_address(&control->staged), kDmaConsumers);
-    XLimbs xr[M];
 #pragma unroll
     for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
-    lds_arrive(lds_address(&control->staged), lane_id == 0);  // the limbs are in registers
 
-    for (uint32_t local = wave; local < wg_rows; local += kDmaConsumers) {
-        // copies 0 .. last must have landed; copy j is number j / 4 of loader j % 4
-        const uint32_t last = ((local + 1u) * row_bytes - 1u) >> 10;
-        for (;;) {
-            bool ready = true;
-#pragma unroll
-            for (uint32_t l = 0; l < static_cast<uint32_t>(kDmaLoaders); l++) {
-                const uint32_t needed = last >= l ? (last - l) / kDmaLoaders + 1u : 0u;
-                ready = ready && lds_count(lds_address(&control->done[l])) >= needed;
-            }
-            if (ready) break;
-            __builtin_amdgcn_s_sleep(1);
-        }
+    const uint32_t landed_address = lds_address(&control->landed[pair]);
+    // Row r needs the copies that hold bytes [0, (r + 1) * row_bytes) of the range. (Reading row r + 1
+    // out of LDS ahead of the fold of row r, when it has landed by then, measured slower: the consumers
+    // are bound by their arithmetic, two of them and two loaders to a SIMD, not by LDS latency.)
+    const uint32_t mine = count - min(count, static_cast<uint32_t>(kDmaLoaderRows));  // the last rows are the loader's
+    for (uint32_t r = 0; r < mine; r++) {
+        lds_await(landed_address, ((r + 1u) * row_bytes + 1023u) >> 10);
         typename T::Data data;
-        T::load(lds + local * row_bytes, lane, data);
-        float value[M];
-        T::template fold<M>(data, lane, xr, value);
-#pragma unroll
-        for (int m = 0; m < M; m++) {
-            const float total = wave_sum(active ? value[m] : 0.f);
-            if (lane_id == 0) control->result[m][local] = total;
-        }
-    }
-    // Every copy has landed by now (the last row needed the last one): stores cannot stall a fold.
-    lds_arrive(lds_address(&control->folded), lane_id == 0);
-    if (wave != 0) return;
-    lds_await(lds_address(&control->folded), kDmaConsumers);
-    for (uint32_t local = lane_id; local < wg_rows; local += 64u) {
-        const uint32_t row = wg_row0 + local;
-        const float b = bias != nullptr ? bias[row] : 0.f;
-#pragma unroll
-        for (int m = 0; m < M; m++) {
-            const float total = control->result[m][local];
-            y[static_cast<uint64_t>(m) * rows + row] = bias != nullptr ? total + b : total;
-        }
+        T::load(range + r * row_bytes, lane, data);
+        fold_row(r, data);
     }
 }
 
 // Whether gemv_limb_dma_kernel takes this shape: one slice of columns, a share per compute unit that
-// fits LDS, enough rows per share to occupy the consumers.
-template <class T>
+// fits LDS below the activation stages, enough rows per share to occupy the consumers.
+template <class T, int M>
 bool dma_takes(uint32_t rows, uint32_t columns, uint32_t* rows_per_wg) {
     if (columns > kSliceColumns) return false;
     const uint32_t share = (rows + 255u) / 256u;
-    const uint64_t bytes = static_cast<uint64_t>(share) * (static_cast<uint64_t>(columns) / T::kBlockColumns) * T::kBlockBytes;
-    if (share < static_cast<uint32_t>(kDmaConsumers) || share > kDmaMaxRows || bytes > kDmaMaxShareBytes) return false;
+    // With fewer than four rows to a range gemv_limb_kernel, which has all of them in flight from its
+    // first instructions, is the faster one (Q8_0 4096 x 4096, two rows to a range: 5.1 against 5.5 us).
+    if (share < 4u * kDmaPairs) return false;
+    const uint64_t row_bytes = (static_cast<uint64_t>(columns) / T::kBlockColumns) * T::kBlockBytes;
+    const uint64_t per_pair = (share + kDmaPairs - 1u) / kDmaPairs;
+    const uint64_t range_bytes = ((per_pair * row_bytes + 1023u) / 1024u) * 1024u;  // as laid out in LDS
+    const uint64_t stage_at = kDmaControlAt - M * sizeof(StageMemory);
+    if (range_bytes * kDmaPairs > stage_at) return false;
     *rows_per_wg = share;
     return true;
 }
@@ -1138,7 +1190,7 @@ hipError_t launch_dma(const uint8_t* weight, const float* x, uint64_t x_row_stri
     int device = 0;
     if (hipError_t status = hipGetDevice(&device)) return status;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    const auto kernel = gemv_limb_dma_kernel<T, M>;
+    const auto kernel = gemv_limb_dma_kernel<T, M, kDmaDepth>;
     if (!allowed[device].load(std::memory_order_acquire)) {
         if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLdsBytes))
@@ -1204,9 +1256,9 @@ hipError_t launch_slices(const uint8_t* weight, const float* x, uint64_t x_row_s
                          const float* bias, float* y, uint32_t rows, uint32_t columns,
                          hipStream_t stream) {
     const uint32_t slices = (columns + kSliceColumns - 1) / kSliceColumns;
-    if constexpr (T::kLdsCopies && M <= 2) {  // three vectors need more registers than twelve waves leave
+    if constexpr (T::kLdsCopies && M == 1) {  // more vectors need more registers than sixteen waves leave
         uint32_t rows_per_wg = 0;
-        if (gemv_limb_dma_enabled() && dma_takes<T>(rows, columns, &rows_per_wg))
+        if (gemv_limb_dma_enabled() && dma_takes<T, M>(rows, columns, &rows_per_wg))
             return launch_dma<T, M>(weight, x, x_row_stride, bias, y, rows, columns, rows_per_wg, stream);
     }
     if (slices <= 1) {
@@ -1245,6 +1297,19 @@ uint32_t gemv_limb_max_vectors(int32_t codec) {
     // Q2_K, Q3_K and Q6_K keep 62 and more registers of activation state per vector (48 limb words,
     // 12 dot offsets, 2 units, run sums): three vectors do not fit next to the rows in flight.
     return codec == kQ6_K || codec == kQ3_K || codec == kQ2_K ? 2u : kGemvLimbMaxVectors;
+}
+
+bool gemv_limb_copies_through_lds(int32_t codec, uint64_t rows, uint64_t columns, uint32_t vectors) {
+    if (vectors != 1 || rows > 0xffffffffull || columns > kSliceColumns || !gemv_limb_dma_enabled()) return false;
+    const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
+    uint32_t rows_per_wg = 0;
+    switch (codec) {
+        case kQ4_K: return dma_takes<Q4KLimb, 1>(n, k, &rows_per_wg);
+        case kQ5_K: return dma_takes<Q5KLimb, 1>(n, k, &rows_per_wg);
+        case kQ4_0: return dma_takes<Q40Limb, 1>(n, k, &rows_per_wg);
+        case kQ8_0: return dma_takes<Q80Limb, 1>(n, k, &rows_per_wg);
+        default: return false;
+    }
 }
 
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors) {

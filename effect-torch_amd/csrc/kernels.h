@@ -38,6 +38,8 @@ hipError_t gather_f32(const float* src, const IndexLayout& layout, uint64_t coun
 constexpr uint32_t kGemvLimbMaxVectors = 3;
 uint32_t gemv_limb_max_vectors(int32_t codec);  // per launch: 3, or 2 for Q6_K
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors);
+// whether that launch runs as gemv_limb_dma_kernel (weights copied through LDS by loader waves)
+bool gemv_limb_copies_through_lds(int32_t codec, uint64_t rows, uint64_t columns, uint32_t vectors);
 hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
                      hipStream_t stream);
@@ -82,15 +84,16 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
 // followed by quantize_tiles, one launch less. columns % 256 == 0, 16-byte aligned rows.
 hipError_t quantize_tiles_silu_mul(const float* gate, const float* up, uint64_t row_stride, uint64_t vectors,
                                    uint64_t columns, uint8_t* tiles, hipStream_t stream);
-hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const float* weight, double eps,
-                                   uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream);
+// weight: [columns] floats, or half floats (weight_is_half; widened on use), or null.
+hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const void* weight, int weight_is_half,
+                                   double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream);
 // The same with x = y computed in the same launch from the unsummed K shares of a contraction:
 // y[m, n] = shares in share order (+ bias[n]) (+ residual[m, n], which may be y itself), written to
 // y [vectors, columns] - the bytes reduce_group_kernel writes - and then normed and quantised.
 hipError_t quantize_tiles_rms_norm_of_shares(const float* shares, uint32_t share_count, uint64_t launch_rows,
-                                             const float* bias, const float* residual, float* y, const float* weight,
-                                             double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles,
-                                             hipStream_t stream);
+                                             const float* bias, const float* residual, float* y, const void* weight,
+                                             int weight_is_half, double eps, uint64_t vectors, uint64_t columns,
+                                             uint8_t* tiles, hipStream_t stream);
 
 // ---- gemm_i8.hip: matrix-core contraction over quantised activation tiles ---------
 bool gemm_i8_supported(int32_t codec, uint64_t columns);
@@ -212,9 +215,14 @@ KvLaunchShape kv_attention_shape(const KvAttention& p);
 hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t stream);
 
 // ---- decode_ops.hip: the small operators next to the contraction in a decode step ----
-// Dense f32 rows; weight may be null. rows, columns < 2^32.
-hipError_t rms_norm(const float* x, const float* weight, double eps, float* out, uint64_t rows, uint64_t columns,
-                    hipStream_t stream);
+// Dense f32 rows; weight: [columns] floats, or half floats (weight_is_half), or null. rows, columns < 2^32.
+hipError_t rms_norm(const float* x, const void* weight, int weight_is_half, double eps, float* out, uint64_t rows,
+                    uint64_t columns, hipStream_t stream);
+// cursors[slot] += advances[slot] for slot < slots: the commit of a decode step.
+hipError_t commit_advances(uint32_t* cursors, const uint32_t* advances, uint64_t slots, hipStream_t stream);
+// gather_rows for a table of half floats (or bfloat16) into f32 rows.
+hipError_t gather_rows_widen(const void* table, int table_is_bf16, uint64_t table_rows, uint64_t width, const void* indexes,
+                             int index_is_i64, uint64_t count, float* out, void* status, hipStream_t stream);
 // x, out: [rows, steps, head_dim]; offsets: 1 or `batch` device words; rows % batch == 0.
 hipError_t rotary(const float* x, const uint32_t* offsets, uint32_t offsets_len, double theta, double sign,
                   int interleaved, float* out, uint64_t batch, uint64_t rows, uint64_t steps, uint64_t head_dim,

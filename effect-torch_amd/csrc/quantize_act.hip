@@ -169,7 +169,7 @@ struct ShareSource {
 template <bool SHARES>
 __global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const float* x, uint64_t x_row_stride,
                                                                          const ShareSource source,
-                                                                         const float* __restrict__ weight, double eps,
+                                                                         const NormWeight weight, double eps,
                                                                          uint32_t vectors, uint32_t columns,
                                                                          uint8_t* __restrict__ tiles) {
     __shared__ double squares[kRmsThreads];
@@ -225,14 +225,11 @@ __global__ __launch_bounds__(kRmsThreads) void quantize_halves_rms_kernel(const 
     const double scale = 1.0 / sqrt(mean_square + eps);
     const uint32_t vector_tiles = (vectors + 31u) >> 5, stages = columns >> 8;
     const uint32_t wave = threadIdx.x >> 6, quad = threadIdx.x & 63u;
-    const float4 ones = make_float4(1.f, 1.f, 1.f, 1.f);
     if (wave < stages)
-        quantize_halves_store(rms_four(held, scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[threadIdx.x] : ones),
-                              v, wave, quad, vector_tiles, tiles);
+        quantize_halves_store(rms_four(held, scale, norm_weight_four(weight, threadIdx.x)), v, wave, quad, vector_tiles, tiles);
     for (uint32_t stage = wave + kRmsThreads / 64u; stage < stages; stage += kRmsThreads / 64u) {
         const uint32_t i = 64u * stage + quad;
-        quantize_halves_store(rms_four(in[i], scale, weight != nullptr ? reinterpret_cast<const float4*>(weight)[i] : ones),
-                              v, stage, quad, vector_tiles, tiles);
+        quantize_halves_store(rms_four(in[i], scale, norm_weight_four(weight, i)), v, stage, quad, vector_tiles, tiles);
     }
 }
 
@@ -297,26 +294,27 @@ hipError_t quantize_tiles_silu_mul(const float* gate, const float* up, uint64_t 
     return hipGetLastError();
 }
 
-hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const float* weight, double eps,
-                                   uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream) {
+hipError_t quantize_tiles_rms_norm(const float* x, uint64_t x_row_stride, const void* weight, int weight_is_half,
+                                   double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles, hipStream_t stream) {
     if (columns % 256 != 0 || vectors > 0x7fffffffull) return hipErrorInvalidValue;
     if (vectors == 0 || columns == 0) return hipSuccess;
     hipLaunchKernelGGL(quantize_halves_rms_kernel<false>, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream,
-                       x, x_row_stride, ShareSource{}, weight, eps, static_cast<uint32_t>(vectors),
+                       x, x_row_stride, ShareSource{}, NormWeight{weight, weight_is_half ? 1 : 0}, eps, static_cast<uint32_t>(vectors),
                        static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
 }
 
 hipError_t quantize_tiles_rms_norm_of_shares(const float* shares, uint32_t share_count, uint64_t launch_rows,
-                                             const float* bias, const float* residual, float* y, const float* weight,
-                                             double eps, uint64_t vectors, uint64_t columns, uint8_t* tiles,
-                                             hipStream_t stream) {
+                                             const float* bias, const float* residual, float* y, const void* weight,
+                                             int weight_is_half, double eps, uint64_t vectors, uint64_t columns,
+                                             uint8_t* tiles, hipStream_t stream) {
     if (columns % 256 != 0 || vectors > 0x7fffffffull || share_count == 0 || launch_rows < columns || launch_rows % 4 != 0)
         return hipErrorInvalidValue;
     if (vectors == 0 || columns == 0) return hipSuccess;
     const ShareSource source = {shares, share_count, launch_rows, launch_rows * vectors, bias, residual, y};
     hipLaunchKernelGGL(quantize_halves_rms_kernel<true>, dim3(static_cast<uint32_t>(vectors)), dim3(kRmsThreads), 0, stream,
-                       y, columns, source, weight, eps, static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
+                       y, columns, source, NormWeight{weight, weight_is_half ? 1 : 0}, eps, static_cast<uint32_t>(vectors),
+                       static_cast<uint32_t>(columns), tiles);
     return hipGetLastError();
 }
 

@@ -251,7 +251,11 @@ bool TensorView::is_contiguous() const {
 const char* kernel_name(const et_linear_plan& plan) {
     switch (plan.kernel) {
         case LinearKernel::kNone: return "none";
-        case LinearKernel::kGemvLimb: return "gemv_limb";
+        case LinearKernel::kGemvLimb:
+            return gemv_limb_copies_through_lds(plan.codec, plan.rows, plan.columns,
+                                                static_cast<uint32_t>(plan.vectors_per_launch))
+                       ? "gemv_limb_dma"
+                       : "gemv_limb";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
         case LinearKernel::kGemmI8:
             return plan.k_splits > 1 ? "quantize_act+gemm_i8+reduce" : "quantize_act+gemm_i8";
@@ -379,18 +383,23 @@ int linear_prepare_input_from(const et_linear_plan& plan, const et_prepare_sourc
                                                  " bytes is smaller than the " + std::to_string(prepared_input_bytes(plan)) +
                                                  " required");
     const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool half_weight = source.kind == ET_PREPARE_RMS_NORM && source.second_dtype == ET_DTYPE_F16;
+    if (source.second_dtype != ET_DTYPE_F32 && !half_weight)
+        return fail(error, ET_ERR_UNSUPPORTED,
+                    "quantized_linear: the second operand must be f32 (an rms norm weight may be f16)");
+    const bool second_aligned = half_weight ? reinterpret_cast<uintptr_t>(source.second) % 8 == 0 : aligned(source.second);
     if (source.x == nullptr || !aligned(source.x) || source.x_row_stride % 4 != 0 || source.x_row_stride < plan.columns ||
-        !aligned(prepared) || !aligned(source.second) || (source.kind == ET_PREPARE_SILU_MUL && source.second == nullptr))
+        !aligned(prepared) || !second_aligned || (source.kind == ET_PREPARE_SILU_MUL && source.second == nullptr))
         return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
     hipError_t status;
     if (source.kind == ET_PREPARE_RMS_NORM) {
         if (!(source.eps == source.eps))
             return fail(error, ET_ERR_INVALID, "quantized_linear: rms norm epsilon is not a number");
-        status = quantize_tiles_rms_norm(source.x, source.x_row_stride, source.second, source.eps, plan.vectors,
-                                         plan.columns, static_cast<uint8_t*>(prepared), as_stream(stream));
+        status = quantize_tiles_rms_norm(source.x, source.x_row_stride, source.second, half_weight ? 1 : 0, source.eps,
+                                         plan.vectors, plan.columns, static_cast<uint8_t*>(prepared), as_stream(stream));
     } else {
-        status = quantize_tiles_silu_mul(source.x, source.second, source.x_row_stride, plan.vectors, plan.columns,
-                                         static_cast<uint8_t*>(prepared), as_stream(stream));
+        status = quantize_tiles_silu_mul(source.x, static_cast<const float*>(source.second), source.x_row_stride,
+                                         plan.vectors, plan.columns, static_cast<uint8_t*>(prepared), as_stream(stream));
     }
     if (status != hipSuccess) return hip_failure(error, "quantized_linear", status);
     return ET_OK;
@@ -546,9 +555,10 @@ int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, co
 
 int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* prepared, const uint8_t* weight,
                                       const float* bias, const float* residual, float* y, void* workspace,
-                                      uint64_t workspace_bytes, const et_linear_plan& next, const float* norm_weight,
-                                      double eps, void* next_prepared, uint64_t next_prepared_bytes, void* stream,
-                                      const volatile int32_t* cancel, std::string* error) {
+                                      uint64_t workspace_bytes, const et_linear_plan& next, const void* norm_weight,
+                                      int32_t norm_weight_dtype, double eps, void* next_prepared,
+                                      uint64_t next_prepared_bytes, void* stream, const volatile int32_t* cancel,
+                                      std::string* error) {
     if (next.columns != plan.rows || next.vectors != plan.vectors)
         return fail(error, ET_ERR_INVALID,
                     "quantized_linear: the next contraction must take this one's result: " + std::to_string(plan.vectors) +
@@ -558,8 +568,12 @@ int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* pr
         return fail(error, ET_ERR_UNSUPPORTED,
                     "quantized_linear: this plan's prepared input cannot be computed from an operator on the fly");
     if (!(eps == eps)) return fail(error, ET_ERR_INVALID, "quantized_linear: rms norm epsilon is not a number");
+    if (norm_weight_dtype != ET_DTYPE_F32 && norm_weight_dtype != ET_DTYPE_F16)
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: an rms norm weight must be f32 or f16");
+    const bool half_weight = norm_weight_dtype == ET_DTYPE_F16;
     const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-    if (y == nullptr || !aligned(y) || !aligned(residual) || !aligned(bias) || !aligned(norm_weight) || !aligned(next_prepared))
+    if (y == nullptr || !aligned(y) || !aligned(residual) || !aligned(bias) ||
+        reinterpret_cast<uintptr_t>(norm_weight) % (half_weight ? 8 : 16) != 0 || !aligned(next_prepared))
         return fail(error, ET_ERR_INVALID, "quantized_linear: activations and prepared input must be 16-byte aligned rows");
     if (next_prepared == nullptr || next_prepared_bytes < prepared_input_bytes(next))
         return fail(error, ET_ERR_EXECUTION, "quantized_linear: prepared-input buffer of " + std::to_string(next_prepared_bytes) +
@@ -577,6 +591,7 @@ int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* pr
         source.x = y;
         source.x_row_stride = plan.rows;
         source.second = norm_weight;
+        source.second_dtype = norm_weight_dtype;
         source.eps = eps;
         return linear_prepare_input_from(next, source, next_prepared, next_prepared_bytes, stream, error);
     }
@@ -595,7 +610,7 @@ int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* pr
     if (hipError_t status = contract_tiles(plan, weight, static_cast<const uint8_t*>(prepared), out, as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);
     if (hipError_t status = quantize_tiles_rms_norm_of_shares(partials, layout.count, layout.launch_rows, bias, residual, y,
-                                                              norm_weight, eps, plan.vectors, plan.rows,
+                                                              norm_weight, half_weight ? 1 : 0, eps, plan.vectors, plan.rows,
                                                               static_cast<uint8_t*>(next_prepared), as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);
     return ET_OK;

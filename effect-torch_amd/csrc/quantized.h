@@ -122,7 +122,8 @@ int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, co
 // et_hip_linear_enqueue_prepared_then_norm in et_hip.h).
 int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* prepared, const uint8_t* weight,
                                       const float* bias, const float* residual, float* y, void* workspace,
-                                      uint64_t workspace_bytes, const et_linear_plan& next, const float* norm_weight,
+                                      uint64_t workspace_bytes, const et_linear_plan& next, const void* norm_weight,
+                                      int32_t norm_weight_dtype,
                                       double eps, void* next_prepared, uint64_t next_prepared_bytes, void* stream,
                                       const volatile int32_t* cancel, std::string* error);
 

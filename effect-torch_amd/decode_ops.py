@@ -71,11 +71,15 @@ def greedy_workspace_bytes(rows: int, vocabulary: int) -> int:
 
 
 def greedy_tokens(logits: torch.Tensor, *, workspace: Optional[torch.Tensor] = None, stream=None,
-                  synchronize: bool = True):
-    """Greedy token per row of ``[.., vocabulary]`` logits as an int32 tensor. With ``synchronize`` a
-    logit that is not finite raises the reference's error here; otherwise ``(tokens, status)``."""
+                  synchronize: bool = True, tokens: Optional[torch.Tensor] = None):
+    """Greedy token per row of ``[.., vocabulary]`` logits as an int32 tensor (``tokens``, when given:
+    a contiguous int32 tensor of one element per row that receives them). With ``synchronize`` a logit
+    that is not finite raises the reference's error here; otherwise ``(tokens, status)``."""
     rows = logits.numel() // logits.shape[-1] if logits.dim() and logits.shape[-1] else 0
-    tokens = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)
+    if tokens is None:
+        tokens = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)
+    elif tokens.dtype != torch.int32 or tokens.numel() != rows or not tokens.is_contiguous():
+        raise QuantizedError(N.ERR_INVALID, "sample: tokens must be a contiguous int32 tensor of one element per row")
     status = torch.empty(4 * max(rows, 1), dtype=torch.uint8, device=logits.device)
     if workspace is None:
         need = greedy_workspace_bytes(rows, logits.shape[-1]) if rows else 0

@@ -81,6 +81,13 @@ def kv_attention_kernel(layer: KvLayer, query_heads: int, tokens: int) -> str:
     return N.lib().et_hip_kv_attention_kernel(ctypes.byref(layer.struct()), query_heads, tokens).decode()
 
 
+def kv_commit(layer: "KvLayer", *, stream=None) -> None:
+    """``cursor += advance`` for the layer's active slots, on the device (``et_hip_kv_commit``): the commit
+    of a decode step (crates/runtime-cpu/src/napi/mod.rs:4511-4517). Layers sharing one cursor tensor are
+    committed by one call."""
+    _check(N.lib().et_hip_kv_commit(ctypes.byref(layer.struct()), _stream_handle(stream)))
+
+
 def kv_attention_status_check(layer: KvLayer, tokens: int, status: torch.Tensor) -> None:
     host = status.cpu().numpy().tobytes()  # synchronises with the producing stream
     buf = ctypes.create_string_buffer(host, len(host))

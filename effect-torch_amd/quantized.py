@@ -314,10 +314,41 @@ class RawLinear:
         _check(N.lib().et_hip_linear_plan_create(int(codec), rows, columns, vectors, int(has_bias),
                                                  int(activation_mode), ctypes.byref(out)))
         self.requirements = QuantizedRequirements(out.value, GgmlQuant(codec), rows, columns)
+        self.rows, self.columns, self.vectors = rows, columns, vectors
+
+    # The C entry points below take raw device pointers and cannot see how large the buffers behind
+    # them are; a kernel that reads past one faults the GPU. These checks are what the holder of the
+    # tensors can do for them: every operand must hold at least what the plan will touch.
+    def _holds(self, what: str, tensor: Optional[torch.Tensor], nbytes: int) -> None:
+        if tensor is None:
+            return
+        have = tensor.numel() * tensor.element_size()
+        if not tensor.is_contiguous() and what != "x":
+            raise QuantizedError(N.ERR_INVALID, f"quantized_linear: {what} must be contiguous")
+        if have < nbytes:
+            raise QuantizedError(N.ERR_INVALID, f"quantized_linear: {what} holds {have} bytes, the plan "
+                                                f"[{self.vectors} x {self.columns}] -> [{self.vectors} x {self.rows}] "
+                                                f"touches {nbytes}")
+
+    def _check_weight(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
+        self._holds("weight", weight, self.rows * (self.requirements.codec.encoded_row_bytes(self.columns) or 0))
+        self._holds("bias", bias, 4 * self.rows)
+
+    def _check_input(self, x: torch.Tensor) -> None:
+        if x.dim() != 2 or x.shape[1] < self.columns or x.shape[0] < self.vectors or x.stride(1) != 1:
+            raise QuantizedError(N.ERR_INVALID, f"quantized_linear: activations of shape {tuple(x.shape)} for a plan of "
+                                                f"{self.vectors} vectors x {self.columns} columns")
+
+    def _check_output(self, y: torch.Tensor, residual: Optional[torch.Tensor] = None) -> None:
+        self._holds("y", y, 4 * self.vectors * self.rows)
+        self._holds("residual", residual, 4 * self.vectors * self.rows)
 
     def enqueue(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                 y: torch.Tensor, workspace: Optional[torch.Tensor] = None, stream=None,
                 cancelled: Optional[CancellationFlag] = None) -> None:
+        self._check_input(x)
+        self._check_weight(weight, bias)
+        self._check_output(y)
         ws_ptr = workspace.data_ptr() if workspace is not None else None
         ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
         _check(N.lib().et_hip_linear_enqueue(self.requirements._handle, x.data_ptr(), x.stride(0),
@@ -333,6 +364,7 @@ class RawLinear:
         return int(N.lib().et_hip_linear_plan_prepared_input_bytes(self.requirements._handle))
 
     def prepare_input(self, x: torch.Tensor, prepared: torch.Tensor, stream=None) -> None:
+        self._check_input(x)
         _check(N.lib().et_hip_linear_prepare_input(self.requirements._handle, x.data_ptr(), x.stride(0),
                                                    prepared.data_ptr(), prepared.numel() * prepared.element_size(),
                                                    _stream_handle(stream)))
@@ -344,8 +376,12 @@ class RawLinear:
 
     def _prepare_from(self, kind: int, x: torch.Tensor, second: Optional[torch.Tensor], eps: float,
                       prepared: torch.Tensor, stream) -> None:
+        self._check_input(x)
+        if second is not None:
+            self._holds("second operand", second, second.element_size() * self.columns *
+                        (self.vectors if kind == N.PREPARE_SILU_MUL else 1))
         source = N.EtPrepareSource(kind, x.data_ptr(), x.stride(0), second.data_ptr() if second is not None else None,
-                                   float(eps))
+                                   float(eps), _weight_dtype(second))
         _check(N.lib().et_hip_linear_prepare_input_from(self.requirements._handle, ctypes.byref(source),
                                                         prepared.data_ptr(), prepared.numel() * prepared.element_size(),
                                                         _stream_handle(stream)))
@@ -368,6 +404,9 @@ class RawLinear:
                          cancelled: Optional[CancellationFlag] = None) -> None:
         """``y = W x (+ bias) (+ residual)`` from activations prepared once by any plan of the same
         columns, vectors and activation mode; ``residual`` may be ``y``."""
+        self._holds("prepared input", prepared, self.prepared_input_bytes)
+        self._check_weight(weight, bias)
+        self._check_output(y, residual)
         ws_ptr = workspace.data_ptr() if workspace is not None else None
         ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
         _check(N.lib().et_hip_linear_enqueue_prepared(
@@ -383,15 +422,30 @@ class RawLinear:
         """:meth:`enqueue_prepared`, then ``next_prepared`` = the prepared input of
         ``rms_norm(y) * norm_weight`` for ``following`` (``et_hip_linear_enqueue_prepared_then_norm``):
         the same bytes as the two calls, one launch less where this plan shares K over workgroups."""
+        self._holds("prepared input", prepared, self.prepared_input_bytes)
+        self._check_weight(weight, bias)
+        self._check_output(y, residual)
+        if norm_weight is not None:
+            self._holds("norm weight", norm_weight, norm_weight.element_size() * self.rows)
         ws_ptr = workspace.data_ptr() if workspace is not None else None
         ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
         _check(N.lib().et_hip_linear_enqueue_prepared_then_norm(
             self.requirements._handle, prepared.data_ptr(), weight.data_ptr(),
             bias.data_ptr() if bias is not None else None, residual.data_ptr() if residual is not None else None,
             y.data_ptr(), ws_ptr, ws_bytes, following.requirements._handle,
-            norm_weight.data_ptr() if norm_weight is not None else None, float(eps), next_prepared.data_ptr(),
+            norm_weight.data_ptr() if norm_weight is not None else None, _weight_dtype(norm_weight), float(eps),
+            next_prepared.data_ptr(),
             next_prepared.numel() * next_prepared.element_size(), _stream_handle(stream),
             cancelled.ptr if cancelled is not None else None))
+
+
+def _weight_dtype(weight: Optional[torch.Tensor]) -> int:
+    """``et_dtype`` of a second operand: f32, or f16 for an rms norm weight held as half floats."""
+    if weight is None or weight.dtype == torch.float32:
+        return N.DTYPE_F32
+    if weight.dtype == torch.float16:
+        return N.DTYPE_F16
+    raise QuantizedError(N.ERR_UNSUPPORTED, f"quantized_linear: second operand of dtype {weight.dtype}")
 
 
 class LinearGroup:
@@ -411,6 +465,7 @@ class LinearGroup:
                          residuals: Optional[Sequence[Optional[torch.Tensor]]] = None, stream=None,
                          cancelled: Optional[CancellationFlag] = None) -> None:
         count = len(self.plans)
+        self._check_members(prepared, weights, ys, biases, residuals)
         pointers = lambda tensors: (ctypes.c_void_p * count)(  # noqa: E731
             *[t.data_ptr() if t is not None else None for t in tensors])
         _check(N.lib().et_hip_linear_enqueue_prepared_group(
@@ -420,6 +475,16 @@ class LinearGroup:
             workspace.data_ptr() if workspace is not None else None,
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
+
+    def _check_members(self, prepared, weights, ys, biases, residuals) -> None:
+        """Every member's operands hold what its plan touches (see RawLinear._holds)."""
+        count = len(self.plans)
+        if len(weights) != count or len(ys) != count:
+            raise QuantizedError(N.ERR_INVALID, f"quantized_linear: a group of {count} plans takes {count} weights and results")
+        self.plans[0]._holds("prepared input", prepared, self.plans[0].prepared_input_bytes)
+        for index, plan in enumerate(self.plans):
+            plan._check_weight(weights[index], biases[index] if biases is not None else None)
+            plan._check_output(ys[index], residuals[index] if residuals is not None else None)
 
     def enqueue_prepared_then_rotary(self, prepared: torch.Tensor, weights: Sequence[torch.Tensor],
                                      ys: Sequence[torch.Tensor], workspace: Optional[torch.Tensor],
@@ -436,10 +501,13 @@ class LinearGroup:
 def _group_then_rotary(group: "LinearGroup", prepared, weights, ys, workspace, rotate, offsets, theta, sign, layout,
                        head_dim, biases, residuals, stream, cancelled) -> None:
     count = len(group.plans)
+    group._check_members(prepared, weights, ys, biases, residuals)
     pointers = lambda tensors: (ctypes.c_void_p * count)(  # noqa: E731
         *[t.data_ptr() if t is not None else None for t in tensors])
     if offsets.dtype not in (torch.uint32, torch.int32) or not offsets.is_contiguous():
         raise ValueError("rotary offsets must be a contiguous u32 device tensor")
+    if offsets.numel() not in (1, group.plans[0].vectors):
+        raise QuantizedError(N.ERR_INVALID, f"rotary embedding: {offsets.numel()} offsets for batch {group.plans[0].vectors}")
     after = N.EtRotaryAfter(sum(1 << i for i in rotate), offsets.data_ptr(), offsets.numel(), float(theta), float(sign),
                             int(layout), int(head_dim))
     _check(N.lib().et_hip_linear_enqueue_prepared_group_then_rotary(

@@ -188,8 +188,10 @@ typedef struct et_prepare_source {
     int32_t kind;           /* et_prepare_kind */
     const float* x;         /* [vectors, columns] f32, rows x_row_stride elements apart, 16-byte aligned */
     uint64_t x_row_stride;
-    const float* second;    /* see the kinds above */
+    const void* second;     /* see the kinds above; f32 [..] */
     double eps;             /* ET_PREPARE_RMS_NORM */
+    int32_t second_dtype;   /* ET_DTYPE_F32 (0), or ET_DTYPE_F16 for an rms norm weight held as half floats: it is
+                               widened on use, the cast the reference's graph puts in front of the operator */
 } et_prepare_source;
 int et_hip_linear_plan_fused_prepare(const et_linear_plan* plan);
 int et_hip_linear_prepare_input_from(const et_linear_plan* plan, const et_prepare_source* source,
@@ -220,13 +222,14 @@ int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepa
  * et_hip_linear_enqueue_prepared followed by et_hip_linear_prepare_input_from(ET_PREPARE_RMS_NORM).
  * Where this plan shares K over workgroups, the launch that would only sum the shares sums them,
  * writes y, norms and quantises: one launch less. Other plans run the two steps one after the
- * other. norm_weight: [rows] f32 or NULL. No counterpart in the reference, whose executor runs one
- * operator at a time. */
+ * other. norm_weight: [rows] f32 or f16 (norm_weight_dtype: ET_DTYPE_F32 / ET_DTYPE_F16; halves are
+ * widened on use) or NULL. No counterpart in the reference, whose executor runs one operator at a time. */
 int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
                                              const uint8_t* weight, const float* bias, const float* residual,
                                              float* y, void* workspace, uint64_t workspace_bytes,
-                                             const et_linear_plan* next, const float* norm_weight, double eps,
-                                             void* next_prepared, uint64_t next_prepared_bytes, void* stream,
+                                             const et_linear_plan* next, const void* norm_weight,
+                                             int32_t norm_weight_dtype, double eps, void* next_prepared,
+                                             uint64_t next_prepared_bytes, void* stream,
                                              const volatile int32_t* cancel);
 
 /* ---- quantized_embedding (= bit-exact dequantisation of selected rows) ---- */
@@ -341,6 +344,13 @@ int et_hip_kv_attention_prepared_into(const et_kv_layer* layer, const et_tensor*
 int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
                                      const void* status_host);
 /* Name of the kernel variant these sizes select, for profiles and diagnostics. */
+/* The commit of a step (crates/runtime-cpu/src/napi/mod.rs:4511-4517): cursor += advance for the
+ * layer's active slots, on the device, after the step's last attention call - so that a decode loop
+ * replays one captured graph per step without a host round trip. Writes layer->cursors (the caller's
+ * array, as everything the struct points to). Layers that share their cursor array are committed by
+ * one call. */
+int et_hip_kv_commit(const et_kv_layer* layer, void* stream);
+
 const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_heads,
                                        uint64_t tokens);
 
@@ -352,7 +362,10 @@ const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_
 
 /* = rms_norm_forward_into (crates/runtime-cpu/src/composed.rs:1491-1533) for
  * f32: out = x * (1 / sqrt(mean(x^2) + eps)) * weight over the last dimension,
- * in f64, rounded once. weight: NULL or [columns]. */
+ * in f64, rounded once. weight: NULL or [columns], f32 - or f16, widened on use: the
+ * reference wants the weight in the activations' type (composed.rs:700-705) and a model
+ * whose norms are stored as half floats casts them in front of the operator; here the
+ * operator reads the halves itself (the widening is exact, the result the same). */
 int et_hip_rms_norm_into(const et_tensor* x, const et_tensor* weight, double eps,
                          const et_tensor* destination, void* stream);
 
@@ -418,7 +431,9 @@ int et_hip_greedy_status_check(uint64_t rows, const void* status_host);
 
 /* = index_select_into along dimension 0 (crates/runtime-cpu/src/indexing.rs:396-430)
  * of a [rows, width] table of any element type: destination[p, :] =
- * table[indexes[p], :] (the dense embedding lookup; f16 tables stay f16).
+ * table[indexes[p], :] (the dense embedding lookup; f16 tables stay f16). An f32
+ * destination for an f16 / bf16 table receives the rows widened (exact): the lookup and
+ * the cast a model with a half-float table puts behind it, in one launch.
  * indexes: u32 or i64, any shape, contiguous; destination [count, width].
  * `status`: device, 8 bytes per index, written by the call; an index outside
  * the table leaves its row alone and et_hip_gather_rows_status_check returns

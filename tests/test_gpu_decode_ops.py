@@ -159,3 +159,49 @@ def test_add(et, device):
         assert np.array_equal(out.cpu().numpy(), oracle.add(a, b))
         et.add_into(ad, bd, ad)  # in place, as the residual stream is updated
         assert np.array_equal(ad.cpu().numpy(), oracle.add(a, b))
+
+
+@pytest.mark.parametrize("shape", [(32, 4096), (3, 1000), (2, 33)])
+def test_rms_norm_with_a_half_float_weight_is_the_widened_weight(et, device, shape):
+    # a weight stored as half floats is widened on use: the bits of the same call with the f32 copy
+    rng = np.random.default_rng(7 + shape[-1])
+    x = torch.from_numpy((rng.standard_normal(shape) * 3).astype(np.float32)).to(device)
+    half = torch.from_numpy((1.0 + 0.2 * rng.standard_normal(shape[-1])).astype(np.float16)).to(device)
+    wide, narrow = torch.empty_like(x), torch.empty_like(x)
+    et.rms_norm_into(x, half.float(), 1e-5, wide)
+    et.rms_norm_into(x, half, 1e-5, narrow)
+    assert torch.equal(wide, narrow)
+    want = oracle.rms_norm(x.cpu().numpy(), half.float().cpu().numpy(), 1e-5)
+    assert ulps(narrow.cpu().numpy(), want).max() <= 1.0
+    with pytest.raises(et.QuantizedError, match="weight must match the last dimension and dtype"):
+        et.rms_norm_into(x, half.to(torch.bfloat16), 1e-5, narrow)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("width", [4096, 100, 7])
+def test_gather_rows_widens_half_float_tables(et, device, dtype, width):
+    rng = np.random.default_rng(width)
+    table = torch.from_numpy(rng.standard_normal((300, width)).astype(np.float32)).to(device).to(dtype)
+    ids = torch.from_numpy(rng.integers(0, 300, 40).astype(np.int64)).to(device)
+    out = torch.full((40, width), float("nan"), device=device)
+    et.gather_rows_into(table, ids, out)
+    assert torch.equal(out, table[ids].float())  # index_select, then the exact cast
+    bad = ids.clone()
+    bad[3] = 300
+    with pytest.raises(et.QuantizedError, match="index_select: index 300 is out of bounds for extent 300"):
+        et.gather_rows_into(table, bad, out)
+    with pytest.raises(et.QuantizedError, match="index_select"):
+        et.gather_rows_into(table, ids, torch.empty((40, width), dtype=torch.float64, device=device))
+
+
+def test_kv_commit_advances_the_active_cursors(et, device):
+    # cursor += advance for the active slots (crates/runtime-cpu/src/napi/mod.rs:4511-4517)
+    slab = torch.zeros((64, 2, 128), dtype=torch.float16, device=device)
+    table = torch.arange(12, dtype=torch.int32, device=device).reshape(3, 4) % 4
+    cursors = torch.tensor([5, 0, 17], dtype=torch.int32, device=device)
+    advances = torch.tensor([1, 3, 2], dtype=torch.int32, device=device)
+    layer = et.KvLayer(slab, slab.clone(), 16, table, cursors, advances, 32, active_batch=2)
+    et.kv_commit(layer)
+    et.kv_commit(layer)
+    torch.cuda.synchronize()
+    assert cursors.tolist() == [7, 6, 17]  # the slot beyond the active batch stays

@@ -640,6 +640,11 @@ def test_prepared_input_of_an_operator_on_the_fly(et, device):
             plan.prepare_input(normed, plain)
             plan.prepare_input_rms_norm(x, w, 1e-5, fused)
             assert torch.equal(plain, fused)
+            if w is not None:  # a weight held as half floats is widened on use: the bytes of its f32 copy
+                half = w.to(torch.float16)
+                plan.prepare_input_rms_norm(x, half.float(), 1e-5, plain)
+                plan.prepare_input_rms_norm(x, half, 1e-5, fused)
+                assert torch.equal(plain, fused)
         gate, up = x * 2.0, to_dev(synth.random_activations(vectors, columns, rng), device)
         product = torch.empty_like(gate)
         et.silu_mul_into(gate, up, product)
@@ -739,7 +744,7 @@ def test_contraction_then_norm_prepared_input_in_the_reduction_launch(et, device
         prepared = torch.empty(plan.prepared_input_bytes, dtype=torch.uint8, device=device)
         plan.prepare_input(x, prepared)
         workspace = torch.empty(max(plan.requirements.workspace_bytes, 16), dtype=torch.uint8, device=device)
-        for w in (norm_weight, None):
+        for w in (norm_weight, None, norm_weight.to(torch.float16)):  # the last: half floats, widened on use
             # in place, as a residual stream is updated
             y_two, y_one = stream_in.clone(), stream_in.clone()
             next_two, next_one = (torch.zeros(following.prepared_input_bytes, dtype=torch.uint8, device=device)

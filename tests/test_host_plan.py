@@ -289,3 +289,27 @@ def test_decode_operator_validation(et):
         et.gather_rows_into(table, torch.zeros(3, dtype=torch.int64), torch.zeros(2, 4, dtype=torch.float16), stream=0)
     with pytest.raises(et.QuantizedError, match="index_select: indexes must be u32 or i64"):
         et.gather_rows_into(table, torch.zeros(3, dtype=torch.float32), torch.zeros(3, 4, dtype=torch.float16), stream=0)
+
+
+def test_raw_pointer_wrappers_refuse_operands_smaller_than_the_plan(et):
+    # The C entry points take raw device pointers; a buffer smaller than what the plan touches would make a
+    # kernel read or write past it. The host mirror checks sizes first and raises before anything is enqueued.
+    import torch
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, 14336, 4096, 32)
+    x = torch.zeros(32, 4096)
+    y = torch.zeros(32, 14336)
+    full = torch.zeros((14336, 2304), dtype=torch.uint8)
+    with pytest.raises(et.QuantizedError, match="weight holds 18874368 bytes, the plan .* touches 33030144"):
+        plan.enqueue(x, full[:8192], None, y)
+    with pytest.raises(et.QuantizedError, match="y holds"):
+        plan.enqueue(x, full, None, y[:, :4096].contiguous())
+    with pytest.raises(et.QuantizedError, match="activations of shape"):
+        plan.enqueue(x[:16], full, None, y)
+    prepared = torch.zeros(max(plan.prepared_input_bytes, 16), dtype=torch.uint8)
+    with pytest.raises(et.QuantizedError, match="prepared input holds"):
+        plan.enqueue_prepared(prepared[:100], full, None, y)
+    with pytest.raises(et.QuantizedError, match="residual holds"):
+        plan.enqueue_prepared(prepared, full, None, y, residual=torch.zeros(8))
+    group = et.LinearGroup([plan, plan])
+    with pytest.raises(et.QuantizedError, match="weight holds"):
+        group.enqueue_prepared(prepared, [full, full[:100]], [y, y])
