@@ -108,8 +108,9 @@ class pinned_to_one_core:
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=2000)
-    p.add_argument("--warmup", type=int, default=200)
+    p.add_argument("--steps", type=int, default=None, help="timed steps (default 2000; llama3_8b_batched_decode: 128)")
+    p.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 200; "
+                   "llama3_8b_batched_decode: 2)")
     p.add_argument("--workload", default="q4_k_gemv_14336x4096",
                    help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,f16,f16_16x16}, "
                         "kv_attention_decode")
@@ -128,7 +129,13 @@ def parse_args():
     p.add_argument("--no-graph", action="store_true", help="enqueue the steps one by one instead of replaying a HIP graph")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
-    return p.parse_args()
+    args = p.parse_args()
+    decode = args.workload == "llama3_8b_batched_decode"
+    if args.steps is None:
+        args.steps = 128 if decode else 2000
+    if args.warmup is None:
+        args.warmup = 2 if decode else 200
+    return args
 
 
 def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
@@ -693,14 +700,18 @@ def quantized_embedding(args, et):
 
 
 def llama_decode(args, et):
-    """Workload ``llama3_8b_batched_decode`` (the end-to-end batched-decode configuration): one decode step of a Llama-3-8B-shaped
-    model for 32 slots at context 2048, every operator through the C ABI - per layer RMS norm, the
-    q / k / v / o and gate / up / down contractions on Q4_K weights (M = 32, f32 activations), rotary
-    on q and k at the slots' cursors, paged key/value-cache attention over f16 slabs, SiLU * up and the
-    two residual sums; then the final norm, the Q4_K output projection to 128256 logits, greedy
-    selection and the lookup of the chosen tokens' embeddings for the next step. Weights are
-    synthetic (one random matrix per shape, rolled by layer into 32 distinct buffers); the step is
-    captured once into a HIP graph and replayed."""
+    """Workload ``llama3_8b_batched_decode`` (the end-to-end batched-decode configuration): greedy decode of
+    ``--steps`` tokens (default 128) for 32 sequences of a Llama-3-8B-shaped model from a prefilled context
+    of ``--context`` positions (default 2048), every operator through the C ABI (effect_torch_amd.LlamaDecoder):
+    per step the lookup of the sequences' tokens in the half-float embedding table, per layer RMS norm (half-
+    float weights), the q / k / v / o and gate / up / down contractions on Q4_K weights (M = 32, f32
+    activations), rotary on q and k at the sequences' cursors, paged key/value-cache attention over half-float
+    slabs in blocks of 16, SiLU * up and the two residual sums; then the final norm, the Q4_K output projection
+    to 128256 logits, greedy selection INTO the token buffer the next step reads, and the cursors' advance on
+    the device. One step is captured as one HIP graph; the timed region replays it ``--steps`` times - every
+    replay is another step, the context grows by one position per step - and the repetitions start from the
+    same state. Weights are synthetic (one random matrix per shape, rolled by layer into distinct buffers), the
+    prefilled cache is random."""
     import numpy as np
     import torch
     import oracle
@@ -708,167 +719,60 @@ def llama_decode(args, et):
 
     device = torch.device("cuda:0")
     torch.manual_seed(0x11A3A)
-    hidden, heads, kv_heads, width, ffn, vocab = 4096, 32, 8, 128, 14336, 128256
+    steps, warmup = args.steps, min(args.warmup, 8)
+    shape = et.LlamaShape(layers=args.layers)
+    hidden, heads, kv_heads, width, ffn, vocab = shape.hidden, shape.heads, shape.kv_heads, shape.head_dim, shape.ffn, shape.vocab
     layers, slots, context, block = args.layers, 32, args.context, 16
+    max_context = context + max(steps, warmup)
     mode = et.ActivationMode.INT8 if args.mode == "int8" else et.ActivationMode.F32
-    Q4K = et.GgmlQuant.Q4_K
     rng = np.random.default_rng(0x11A3A)
 
-    shapes = {"wq": (hidden, hidden), "wk": (kv_heads * width, hidden), "wv": (kv_heads * width, hidden),
-              "wo": (hidden, hidden), "gate": (ffn, hidden), "up": (ffn, hidden), "down": (hidden, ffn),
-              "head": (vocab, hidden)}
+    shapes = shape.linear_shapes()
     host = {name: synth.random_weight(synth.Q4_K, rows, columns, rng) for name, (rows, columns) in shapes.items()}
     base = {name: torch.from_numpy(w).to(device) for name, w in host.items()}
     weights = [{name: (base[name] if layer == 0 else torch.roll(base[name], layer, 0).contiguous())
                 for name in shapes if name != "head"} for layer in range(layers)]
-    norms_host = [rng.standard_normal((2, hidden)).astype(np.float32) for _ in range(layers)]
+    # random-init norms around 1/16 keep the residual stream of these (far from trained) weights inside the
+    # half floats of the slabs over 32 layers; half floats, widened on use
+    norms_host = [((1.0 + 0.1 * rng.standard_normal((2, hidden))) / 16.0).astype(np.float16) for _ in range(layers)]
     norms = [torch.from_numpy(n).to(device) for n in norms_host]
-    final_norm = torch.randn(hidden, device=device)
-    plans = {name: et.RawLinear(Q4K, rows, columns, slots, False, mode) for name, (rows, columns) in shapes.items()}
-    linear_ws = torch.empty(max(max(p.requirements.workspace_bytes for p in plans.values()), 16), dtype=torch.uint8,
-                            device=device)
-    # q / k / v and gate / up read the same activations: they are quantised once per distinct input, and
-    # the residual sums ride in the epilogues of the o and down contractions (--unfused: one operator per
-    # launch, as the reference's executor runs them; the results have the same bits either way).
-    fused = not args.unfused
-    shared_hidden = torch.empty(max(plans["wq"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
-    shared_ffn = torch.empty(max(plans["down"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
-    shared_attended = torch.empty(max(plans["wo"].prepared_input_bytes, 16), dtype=torch.uint8, device=device)
+    final_norm = torch.from_numpy(((1.0 + 0.1 * rng.standard_normal(hidden)) / 16.0).astype(np.float16)).to(device)
+    embedding_base = rng.standard_normal((8192, hidden)).astype(np.float16)  # row t of the table = base[t % 8192]
+    embedding = torch.from_numpy(embedding_base).to(device).repeat(-(-vocab // 8192), 1)[:vocab].contiguous()
 
-    blocks_per_slot = -(-context // block)
+    blocks_per_slot = -(-max_context // block)
     total_blocks = slots * blocks_per_slot
     table_host = rng.permutation(total_blocks).reshape(slots, blocks_per_slot).astype(np.int32)
-    cursors_host = np.full(slots, context - 1, dtype=np.int32)
-    advances_host = np.ones(slots, dtype=np.int32)
-    table, cursors, advances = (torch.from_numpy(a).to(device) for a in (table_host, cursors_host, advances_host))
+    cursors_host = np.full(slots, context, dtype=np.int32)   # `context` positions are cached; the step adds one
+    tokens_host = rng.integers(0, vocab, slots).astype(np.int32)
+    table, cursors, tokens = (torch.from_numpy(a).to(device) for a in (table_host, cursors_host, tokens_host))
+    advances = torch.ones(slots, dtype=torch.int32, device=device)
     kv = []
     for _ in range(layers):
         k_slab, v_slab, k_scales, v_scales, kv_row_bytes = make_kv_slabs(torch, args.kv_dtype, total_blocks * block,
                                                                          kv_heads, width, device)
-        kv.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, context, k_scales=k_scales,
+        kv.append(et.KvLayer(k_slab, v_slab, block, table, cursors, advances, max_context, k_scales=k_scales,
                              v_scales=v_scales))
-    kv_ws = et.kv_attention_workspace(kv[0], heads, 1)
-    greedy_ws = torch.empty(et.greedy_workspace_bytes(slots, vocab), dtype=torch.uint8, device=device)
-    embedding = torch.randn(vocab, hidden, device=device)
-    tokens = torch.from_numpy(rng.integers(0, vocab, slots).astype(np.int32)).to(device)
-    scale = 1.0 / float(np.sqrt(width))
+    decoder = et.LlamaDecoder(shape, et.GgmlQuant.Q4_K, slots, weights, base["head"], norms, final_norm, embedding, kv,
+                              tokens, mode=mode, fused=not args.unfused)
+    start_cursors, start_tokens = cursors.clone(), tokens.clone()
 
-    f32 = lambda *shape: torch.empty(shape, device=device)  # noqa: E731
-    x, h, q, k, v = f32(slots, hidden), f32(slots, hidden), f32(slots, hidden), f32(slots, kv_heads * width), \
-        f32(slots, kv_heads * width)
-    attended, projected, gate, up, down = f32(slots, hidden), f32(slots, hidden), f32(slots, ffn), f32(slots, ffn), \
-        f32(slots, hidden)
-    logits = f32(slots, vocab)
-    chosen = torch.empty(slots, dtype=torch.int32, device=device)
-    keep = []
+    def restart():
+        """The state every repetition starts from. (The rows the steps append lie behind the prefilled
+        context and are written before they are read, so the slabs need no restoring.)"""
+        cursors.copy_(start_cursors)
+        tokens.copy_(start_tokens)
 
-    # the norms and SiLU * up are applied while their results are quantised, where the plans can;
-    # q / k / v, and gate / up, then run as one launch each
-    on_the_fly = fused and all(plans[name].fused_prepare for name in ("wq", "gate", "down", "head"))
-    if on_the_fly:
-        qkv_group = et.LinearGroup([plans["wq"], plans["wk"], plans["wv"]])
-        ffn_group = et.LinearGroup([plans["gate"], plans["up"]])
-        group_ws = torch.empty(max(qkv_group.workspace_bytes, ffn_group.workspace_bytes, 16), dtype=torch.uint8,
-                               device=device)
-
-    # (following plan, its norm weight) after a layer's down projection: the next layer's attention
-    # norm, or the final norm in front of the output head
-    after_down = lambda index: (plans["wq"], norms[index + 1][0]) if index + 1 < layers else (plans["head"], final_norm)  # noqa: E731
-
-    def layer_step(index, prepared_by_previous=False):
-        w, kvl = weights[index], kv[index]
-        if on_the_fly:
-            # the layer before has left this norm's prepared input behind (enqueue_prepared_then_norm)
-            if not prepared_by_previous:
-                plans["wq"].prepare_input_rms_norm(x, norms[index][0], 1e-5, shared_hidden)
-        else:
-            et.rms_norm_into(x, norms[index][0], 1e-5, h)
-        if fused:
-            if on_the_fly:
-                # q and k rotated at the slots' cursors in the launch that sums the group's K shares
-                qkv_group.enqueue_prepared_then_rotary(shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v], group_ws,
-                                                       (0, 1), cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, width)
-            else:
-                plans["wq"].prepare_input(h, shared_hidden)
-                plans["wq"].enqueue_prepared(shared_hidden, w["wq"], None, q, linear_ws)
-                plans["wk"].enqueue_prepared(shared_hidden, w["wk"], None, k, linear_ws)
-                plans["wv"].enqueue_prepared(shared_hidden, w["wv"], None, v, linear_ws)
-        else:
-            plans["wq"].enqueue(h, w["wq"], None, q, linear_ws)
-            plans["wk"].enqueue(h, w["wk"], None, k, linear_ws)
-            plans["wv"].enqueue(h, w["wv"], None, v, linear_ws)
-        q4, k4, v4 = q.view(slots, heads, 1, width), k.view(slots, kv_heads, 1, width), v.view(slots, kv_heads, 1, width)
-        if on_the_fly:
-            pass  # rotated above
-        elif fused:
-            et.rotary_pair_into(q4, k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4, k4)
-        else:
-            et.rotary_into(q4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, q4)
-            et.rotary_into(k4, cursors, 500000.0, 1.0, et.RotaryLayout.HALF_SPLIT, k4)
-        if on_the_fly:
-            # the attention kernel quantises its result for Wo in its epilogue
-            keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
-                                             workspace=kv_ws, synchronize=False, prepared_for=plans["wo"],
-                                             prepared=shared_attended))
-        else:
-            keep.append(et.kv_attention_into(kvl, q4, k4, v4, scale, None, attended.view(slots, heads, 1, width),
-                                             workspace=kv_ws, synchronize=False))
-        if on_the_fly:
-            # x += attended Wo, then the ffn norm inside the quantiser, in the launch that sums Wo's K shares
-            plans["wo"].enqueue_prepared_then_norm(shared_attended, w["wo"], None, x, linear_ws, plans["gate"],
-                                                   norms[index][1], 1e-5, shared_hidden, residual=x)
-        elif fused:
-            plans["wo"].prepare_input(attended, shared_hidden)
-            plans["wo"].enqueue_prepared(shared_hidden, w["wo"], None, x, linear_ws, residual=x)
-        else:
-            plans["wo"].enqueue(attended, w["wo"], None, projected, linear_ws)
-            et.add_into(x, projected, x)
-        if not on_the_fly:
-            et.rms_norm_into(x, norms[index][1], 1e-5, h)
-        if fused:
-            if on_the_fly:
-                ffn_group.enqueue_prepared(shared_hidden, [w["gate"], w["up"]], [gate, up], group_ws)
-            else:
-                plans["gate"].prepare_input(h, shared_hidden)
-                plans["gate"].enqueue_prepared(shared_hidden, w["gate"], None, gate, linear_ws)
-                plans["up"].enqueue_prepared(shared_hidden, w["up"], None, up, linear_ws)
-        else:
-            plans["gate"].enqueue(h, w["gate"], None, gate, linear_ws)
-            plans["up"].enqueue(h, w["up"], None, up, linear_ws)
-        if on_the_fly:
-            plans["down"].prepare_input_silu_mul(gate, up, shared_ffn)
-        else:
-            et.silu_mul_into(gate, up, gate)
-        if on_the_fly:
-            following, norm_weight = after_down(index)
-            plans["down"].enqueue_prepared_then_norm(shared_ffn, w["down"], None, x, linear_ws, following, norm_weight,
-                                                     1e-5, shared_hidden, residual=x)
-        elif fused:
-            plans["down"].prepare_input(gate, shared_ffn)
-            plans["down"].enqueue_prepared(shared_ffn, w["down"], None, x, linear_ws, residual=x)
-        else:
-            plans["down"].enqueue(gate, w["down"], None, down, linear_ws)
-            et.add_into(x, down, x)
-
-    def step():
-        keep.clear()
-        keep.append(et.gather_rows_into(embedding, tokens.view(torch.uint32), x, synchronize=False))
-        for index in range(layers):
-            layer_step(index, prepared_by_previous=on_the_fly and index > 0)
-        if on_the_fly:
-            plans["head"].enqueue_prepared(shared_hidden, base["head"], None, logits, linear_ws)
-        else:
-            et.rms_norm_into(x, final_norm, 1e-5, h)
-            plans["head"].enqueue(h, base["head"], None, logits, linear_ws)
-        keep.append(et.greedy_tokens(logits, workspace=greedy_ws, synchronize=False)[1])
-
-    # Parity gate: layer 0 for two slots against the CPU oracle chained the same way.
-    et.gather_rows_into(embedding, tokens.view(torch.uint32), x)
-    x0 = x.cpu().numpy()[:2].copy()
-    layer_step(0)
+    # Parity gate: the embedding rows exactly, then layer 0 for two slots against the CPU oracle chained the same way.
+    decoder.embed()
     torch.cuda.synchronize()
-    et.kv_attention_status_check(kv[0], 1, keep[-1])
-    got = x.cpu().numpy()[:2]
+    x0 = decoder.x.cpu().numpy()[:2].copy()
+    assert np.array_equal(x0.view(np.uint32), embedding_base[tokens_host[:2] % 8192].astype(np.float32).view(np.uint32)), \
+        "parity gate failed: embedding rows differ"
+    decoder.layer_step(0)
+    torch.cuda.synchronize()
+    et.kv_attention_status_check(kv[0], 1, decoder.status[-1])
+    got = decoder.x.cpu().numpy()[:2]
     lin = lambda name, act: oracle.linear_rows(synth.Q4_K, shapes[name][0], shapes[name][1], act, host[name], None, 0,  # noqa: E731
                                                shapes[name][0])
     if args.mode == "int8":
@@ -876,85 +780,111 @@ def llama_decode(args, et):
             qa, sa, ta = oracle.quantize_q8(np.ascontiguousarray(act))
             return oracle.linear_q8_rows(synth.Q4_K, shapes[name][0], shapes[name][1], qa, sa, ta, host[name], None, 0,
                                          shapes[name][0])
-    hh = oracle.rms_norm(x0, norms_host[0][0], 1e-5)
+    norm0 = norms_host[0].astype(np.float32)
+    scale = 1.0 / float(np.sqrt(width))
+    hh = oracle.rms_norm(x0, norm0[0], 1e-5)
     q_ref = oracle.rotary(lin("wq", hh).reshape(2, heads, 1, width), cursors_host[:2], 500000.0)
     k_ref = oracle.rotary(lin("wk", hh).reshape(2, kv_heads, 1, width), cursors_host[:2], 500000.0)
     v_ref = lin("wv", hh).reshape(2, kv_heads, 1, width)
     # the slabs already hold the rows this very step appended; the oracle writes the same values again
     slabs_host = kv_slabs_to_host(np, torch, kv[0])
-    att = oracle.kv_attention(slabs_host[0], slabs_host[1], block,
-                              table_host[:2].view(np.uint32), cursors_host[:2].view(np.uint32),
-                              advances_host[:2].view(np.uint32), q_ref, k_ref, v_ref, scale, k_scales=slabs_host[2],
-                              v_scales=slabs_host[3])
+    ones = np.ones(2, np.uint32)
+    att = oracle.kv_attention(slabs_host[0], slabs_host[1], block, table_host[:2].view(np.uint32),
+                              cursors_host[:2].view(np.uint32), ones, q_ref, k_ref, v_ref, scale,
+                              k_scales=slabs_host[2], v_scales=slabs_host[3])
     x1 = oracle.add(x0, lin("wo", att.reshape(2, hidden)))
-    hh = oracle.rms_norm(x1, norms_host[0][1], 1e-5)
+    hh = oracle.rms_norm(x1, norm0[1], 1e-5)
     want = oracle.add(x1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
     relative = float(np.linalg.norm(got - want) / np.linalg.norm(want))
     assert relative <= (2e-2 if args.mode == "int8" else 1e-3), f"parity gate failed: relative L2 error {relative:.3g}"
 
-    for _ in range(max(args.warmup, 1)):
-        step()
+    restart()
+    for _ in range(max(warmup, 1)):
+        decoder.step()
     torch.cuda.synchronize()
+    et.greedy_status_check(decoder.status[-1])
+    restart()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        step()
-    graph.replay()
-    torch.cuda.synchronize()
+        decoder.step()
     stream = torch.cuda.current_stream()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    repetitions = max(MIN_REPETITIONS, 1)
+    samples, finals = [], []
     wall0 = time.perf_counter()
-    start.record(stream)
-    for _ in range(args.steps):
-        graph.replay()
-    stop.record(stream)
-    torch.cuda.synchronize()
+    for _ in range(repetitions + 1):  # the first repetition is not counted
+        restart()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(steps):
+            graph.replay()
+        stop.record(stream)
+        torch.cuda.synchronize()
+        samples.append(start.elapsed_time(stop))
+        finals.append((tokens.cpu().numpy().copy(), cursors.cpu().numpy().copy()))
     wall = time.perf_counter() - wall0
-    ms = start.elapsed_time(stop) / args.steps
-    et.greedy_status_check(keep[-1])
+    samples = sorted(samples[1:])
+    et.greedy_status_check(decoder.status[-1])
+    # every repetition is the same decode: the same last tokens, every cursor at context + steps
+    for final_tokens, final_cursors in finals:
+        assert np.array_equal(final_cursors, cursors_host + steps), "the cursors did not advance one position per step"
+        assert np.array_equal(final_tokens, finals[0][0]), "repetitions of the same decode chose different tokens"
+    ms_total = samples[len(samples) // 2]
+    ms = ms_total / steps
     seconds = ms * 1e-3
-    weight_bytes = layers * sum(host[n].size for n in shapes if n != "head") + host["head"].size
-    kv_bytes = layers * 2 * slots * context * kv_heads * kv_row_bytes
-    algorithmic = weight_bytes + kv_bytes + slots * vocab * 4 * 2
+    mean_context = context + (steps - 1) / 2.0 + 1.0  # positions a step attends to, averaged over the steps
+    parts = et.algorithmic_bytes_per_step(shape, et.GgmlQuant.Q4_K, slots, layers, 1, kv_row_bytes)
+    weight_bytes, logits_bytes = parts["weights"], parts["logits"]
+    kv_bytes = int(parts["kv"] * mean_context)
+    algorithmic = weight_bytes + kv_bytes + logits_bytes
     gbs = algorithmic / seconds / 1e9
+    fused = not args.unfused
     result = {
         "metric": "batched decode tok/s", "value": round(slots / seconds, 1), "unit": "tok/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "int8" if args.mode == "int8" else "f32", "data": "synthetic",
-        "config": {"workload": f"llama3_8b_batched_decode: {layers} layers, hidden {hidden}, {heads}/{kv_heads} heads x {width}, "
-                               f"ffn {ffn}, vocab {vocab}; Q4_K weights, {args.kv_dtype} kv slabs in blocks of {block}; {slots} slots at "
-                               f"context {context}; {'int8' if args.mode == 'int8' else 'f32'} activations",
-                   "launch": "one HIP graph of the whole step, replayed K times",
+        "repetitions": repetitions, "ms_per_step_min": round(samples[0] / steps, 4), "ms_per_step_max": round(samples[-1] / steps, 4),
+        "config": {"workload": f"llama3_8b_batched_decode: {steps} greedy steps, context {context}->{context + steps - 1} cached "
+                               f"positions per sequence, {slots} sequences; {layers} layers, hidden {hidden}, {heads}/{kv_heads} "
+                               f"heads x {width}, ffn {ffn}, vocab {vocab}; Q4_K weights, f16 embedding table and norm "
+                               f"weights, {args.kv_dtype} kv slabs in blocks of {block}; "
+                               f"{'int8' if args.mode == 'int8' else 'f32'} activations",
+                   "launch": f"one HIP graph of a whole step, replayed {steps} times per repetition; the chosen tokens and the "
+                             "advanced cursors stay on the device between steps",
+                   "timing": f"median of {repetitions} repetitions of the whole {steps}-step decode, one HIP event pair each, "
+                             "after one uncounted repetition",
                    "operators": "one quantisation per distinct input, residual sums in the contraction epilogues"
                                 if fused else "one launch sequence per operator",
-                   "weight_bytes": weight_bytes, "kv_bytes_read": kv_bytes, "layer0_relative_l2_error": relative,
-                   "host_wall_ms": round(wall * 1e3, 3)},
+                   "weight_bytes": weight_bytes, "kv_bytes_read_per_step_mean": kv_bytes,
+                   "layer0_relative_l2_error": relative, "host_wall_ms": round(wall * 1e3, 3)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 1)},
     }
     if not args.no_cpu:
         # one layer for one slot and 2048 rows of the output projection on one core, scaled to the step
-        t0 = time.perf_counter()
-        one = x0[:1]
-        hh = oracle.rms_norm(one, norms_host[0][0], 1e-5)
-        q1 = oracle.rotary(lin("wq", hh).reshape(1, heads, 1, width), cursors_host[:1], 500000.0)
-        k1 = oracle.rotary(lin("wk", hh).reshape(1, kv_heads, 1, width), cursors_host[:1], 500000.0)
-        v1 = lin("wv", hh).reshape(1, kv_heads, 1, width)
-        a1 = oracle.kv_attention(slabs_host[0], slabs_host[1], block,
-                                 table_host[:1].view(np.uint32), cursors_host[:1].view(np.uint32),
-                                 advances_host[:1].view(np.uint32), q1, k1, v1, scale, k_scales=slabs_host[2],
-                                 v_scales=slabs_host[3])
-        y1 = oracle.add(one, lin("wo", a1.reshape(1, hidden)))
-        hh = oracle.rms_norm(y1, norms_host[0][1], 1e-5)
-        oracle.add(y1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
-        t1 = time.perf_counter()
-        oracle.linear_rows(synth.Q4_K, vocab, hidden, hh, host["head"], None, 0, 2048)
-        t2 = time.perf_counter()
+        with pinned_to_one_core() as pin:
+            t0 = time.perf_counter()
+            one = x0[:1]
+            hh = oracle.rms_norm(one, norm0[0], 1e-5)
+            q1 = oracle.rotary(lin("wq", hh).reshape(1, heads, 1, width), cursors_host[:1], 500000.0)
+            k1 = oracle.rotary(lin("wk", hh).reshape(1, kv_heads, 1, width), cursors_host[:1], 500000.0)
+            v1 = lin("wv", hh).reshape(1, kv_heads, 1, width)
+            a1 = oracle.kv_attention(slabs_host[0], slabs_host[1], block,
+                                     table_host[:1].view(np.uint32), cursors_host[:1].view(np.uint32),
+                                     ones[:1], q1, k1, v1, scale, k_scales=slabs_host[2], v_scales=slabs_host[3])
+            y1 = oracle.add(one, lin("wo", a1.reshape(1, hidden)))
+            hh = oracle.rms_norm(y1, norm0[1], 1e-5)
+            oracle.add(y1, lin("down", oracle.silu_mul(lin("gate", hh), lin("up", hh))))
+            t1 = time.perf_counter()
+            oracle.linear_rows(synth.Q4_K, vocab, hidden, hh, host["head"], None, 0, 2048)
+            t2 = time.perf_counter()
+            pinned = pin.describe()
         per_token = (t1 - t0) * layers + (t2 - t1) * vocab / 2048
         result["cpu_baseline"] = {"value": round(1.0 / per_token, 4), "unit": "tok/s", "cores": 1, "kind": "port",
-                                  "sample": f"one layer for one slot ({t1 - t0:.2f} s incl. copying the slabs) x {layers} "
+                                  "sample": f"one layer for one slot at context {context} ({t1 - t0:.2f} s) x {layers} "
                                             f"layers + 2048 of {vocab} output rows ({t2 - t1:.2f} s) scaled; scalar C "
-                                            f"restatement of the reference's loops ({per_token:.1f} s per token)"}
+                                            f"restatement of the reference's loops ({per_token:.1f} s per token); {pinned}"}
     print(json.dumps(result))
 
 
