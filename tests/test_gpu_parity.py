@@ -807,12 +807,15 @@ def test_group_launch_then_rotary_in_the_reduction_launch(et, device):
     pair.enqueue_prepared_then_rotary(prepared, big_weights, one, None, (0,), cursors, 10000.0, -1.0,
                                       et.RotaryLayout.HALF_SPLIT, head_dim)
     assert torch.equal(two[0], one[0]) and torch.equal(two[1], one[1])
+    three = [torch.empty((vectors, plan.rows), device=device) for plan in group.plans]
     with pytest.raises(et.QuantizedError, match="not whole heads"):
-        group.enqueue_prepared_then_rotary(prepared, weights, one, workspace, (0,), cursors, 500000.0, 1.0,
+        group.enqueue_prepared_then_rotary(prepared, weights, three, workspace, (0,), cursors, 500000.0, 1.0,
                                            et.RotaryLayout.HALF_SPLIT, 96)
     with pytest.raises(et.QuantizedError, match="offsets for batch"):
-        group.enqueue_prepared_then_rotary(prepared, weights, one, workspace, (0,), cursors[:5].contiguous(), 500000.0, 1.0,
+        group.enqueue_prepared_then_rotary(prepared, weights, three, workspace, (0,), cursors[:5].contiguous(), 500000.0, 1.0,
                                            et.RotaryLayout.HALF_SPLIT, head_dim)
+    with pytest.raises(et.QuantizedError, match="a group of 3 plans takes 3 weights and results"):
+        group.enqueue_prepared(prepared, weights, one, workspace)
 
 
 # --------------------------------------------------------------------------- measurement aids
