@@ -14,6 +14,7 @@ from .quantized import (  # noqa: F401
     QuantizedRequirements,
     LinearGroup,
     RawLinear,
+    STATIC_WORKSPACE_BYTES,
     MFMA_OPERATIONS,
     calibration_copy,
     calibration_mfma,

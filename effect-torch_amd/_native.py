@@ -133,6 +133,7 @@ SIGNATURES = {
     "et_hip_linear_group_workspace_bytes": (ctypes.c_int, [_vp, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint64)]),
     "et_hip_linear_enqueue_prepared_group": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _u64,
                                                             _vp, _vp]),
+    "et_hip_linear_enqueue_static_workspace": (ctypes.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _vp]),
     "et_hip_linear_prepare_input_from": (ctypes.c_int, [_vp, ctypes.POINTER(EtPrepareSource), _vp, _u64, _vp]),
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_linear_enqueue_prepared_group_then_rotary": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp,

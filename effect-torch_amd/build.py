@@ -37,6 +37,7 @@ SOURCES = {
     # matrix-core results straight into VGPRs, as in the batch kernels (no accumulation-register moves)
     "calibrate.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "quantized.cpp": [],
+    "static_workspace.cpp": [],
     "kv_cache.cpp": [],
     "decode_host.cpp": [],
     "gguf.cpp": [],

@@ -189,6 +189,19 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
     });
 }
 
+int et_hip_linear_enqueue_static_workspace(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
+                                           const uint8_t* weight, const float* bias, float* y, void* stream,
+                                           const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (plan == nullptr) {
+            *error = "quantized_linear: plan is NULL";
+            return ET_ERR_INVALID;
+        }
+        return et::quantized::linear_enqueue_static_workspace(*plan, x, x_row_stride, weight, bias, y, stream, cancel,
+                                                              error);
+    });
+}
+
 uint64_t et_hip_linear_plan_prepared_input_bytes(const et_linear_plan* plan) {
     return plan ? et::quantized::prepared_input_bytes(*plan) : 0;
 }

@@ -101,6 +101,11 @@ int linear_prepare_input_from(const et_linear_plan& plan, const et_prepare_sourc
                               uint64_t prepared_bytes, void* stream, std::string* error);
 // Several plans of the same columns and vectors against one prepared input in one launch (see
 // et_hip_linear_enqueue_prepared_group in et_hip.h).
+// linear_enqueue with the workspace in a device array of the library's own (static_workspace.cpp): for
+// callers that cannot allocate. Plans that need more than ET_HIP_STATIC_WORKSPACE_BYTES are refused.
+int linear_enqueue_static_workspace(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
+                                    const uint8_t* weight, const float* bias, float* y, void* stream,
+                                    const volatile int32_t* cancel, std::string* error);
 int linear_group_workspace_bytes(const et_linear_plan* const* plans, uint32_t count, uint64_t* bytes, std::string* error);
 int linear_enqueue_prepared_group(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
                                   const uint8_t* const* weights, const float* const* biases,

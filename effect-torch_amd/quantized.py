@@ -304,6 +304,9 @@ def quantize_activations(x: torch.Tensor, stream=None):
     return q, scale[:, :vectors], total[:, :vectors]
 
 
+STATIC_WORKSPACE_BYTES = 16 << 20  # ET_HIP_STATIC_WORKSPACE_BYTES of include/et_hip.h
+
+
 class RawLinear:
     """Raw-pointer plan/enqueue pair (``et_hip_linear_plan_create`` / ``et_hip_linear_enqueue``)
     for dense ``[vectors, columns]`` inputs; what a timing loop or a graph capture uses."""
@@ -357,6 +360,19 @@ class RawLinear:
                                              y.data_ptr(), ws_ptr, ws_bytes, _stream_handle(stream),
                                              cancelled.ptr if cancelled is not None else None))
 
+
+    def enqueue_static_workspace(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                                 y: torch.Tensor, stream=None, cancelled: Optional[CancellationFlag] = None) -> None:
+        """:meth:`enqueue` with the library's own static device workspace (``et_hip_linear_enqueue_static_workspace``):
+        no allocation anywhere; plans that need more than ``STATIC_WORKSPACE_BYTES`` are refused; calls that
+        overlap in time on one GPU race on the array."""
+        self._check_input(x)
+        self._check_weight(weight, bias)
+        self._check_output(y)
+        _check(N.lib().et_hip_linear_enqueue_static_workspace(
+            self.requirements._handle, x.data_ptr(), x.stride(0), weight.data_ptr(),
+            bias.data_ptr() if bias is not None else None, y.data_ptr(), _stream_handle(stream),
+            cancelled.ptr if cancelled is not None else None))
 
     @property
     def prepared_input_bytes(self) -> int:

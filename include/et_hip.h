@@ -162,6 +162,21 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
                           const uint8_t* weight, const float* bias, float* y, void* workspace,
                           uint64_t workspace_bytes, void* stream, const volatile int32_t* cancel);
 
+/* et_hip_linear_enqueue without a workspace argument: the scratch memory the kernels need
+ * (activation tiles, K-share partials, the dense copy of strided rows) is a device array inside the
+ * library, ET_HIP_STATIC_WORKSPACE_BYTES per GPU, held from its first use on that GPU until the
+ * process ends. It has no counterpart in the reference; it exists for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The call allocates nothing and frees nothing. A plan whose et_hip_linear_plan_workspace_bytes
+ * exceeds the array is refused (ET_ERR_UNSUPPORTED, "... the static workspace holds ..."): such
+ * callers bring their own workspace to et_hip_linear_enqueue. Every call on a GPU uses the same
+ * array: calls that overlap in time on one GPU race on it - serialise them (one stream, or events).
+ * Results are those of et_hip_linear_enqueue, bit for bit. */
+#define ET_HIP_STATIC_WORKSPACE_BYTES (16u << 20)
+int et_hip_linear_enqueue_static_workspace(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
+                                           const uint8_t* weight, const float* bias, float* y, void* stream,
+                                           const volatile int32_t* cancel);
+
 /* Contractions that share their activations (q / k / v, gate / up of a decode step) can share the
  * quantised form the matrix-core kernels consume: prepare it once, then enqueue every plan of the
  * same columns, vectors and activation mode from it. `residual` (dense [vectors, rows], may be y
