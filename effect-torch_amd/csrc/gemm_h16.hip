@@ -748,9 +748,11 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     }
     if (g.tile_rows == 128)
         return launch_group<kQ4_K, 4, 2, 2>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
-    // 64-row tiles: three stages of activation lead and one of weights measured ahead of two and three
-    // (14336 x 4096 with 32 vectors 23.2 -> 22.1 us, 4096 x 14336 24.5 -> 23.8, the decode step -0.5 %)
-    return launch_group<kQ4_K, 2, 3, 1>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+    // 64-row tiles: two stages of activation lead and three of weights. Timestamps taken inside the kernel
+    // show the operands of a stage in LDS well before its barrier with either split of the ring; what the
+    // stage waits for is its slowest consumer. (14336 x 4096 with 32 vectors, contraction alone: 20.6 us
+    // against 21.7 with three and one; 4096 x 14336 22.5 against 23.6; more loader waves changed nothing.)
+    return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
