@@ -145,7 +145,8 @@ __device__ __forceinline__ float limb_value(const XLimbs& x, int d0, int d1, int
 
 struct Q4KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 144u;
-    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
+    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -228,7 +229,8 @@ struct Q4KLimb {
 // sub-block g. 176 bytes per block, every field 16-byte aligned.
 struct Q5KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 176u;
-    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
+    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -323,7 +325,8 @@ struct __attribute__((packed, aligned(4))) Dwords17 {
 // Q4_0: two 18-byte blocks = 36 bytes = 9 dwords (dword aligned when columns % 64 == 0).
 struct Q40Limb {
     static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 18u;
-    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
+    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -383,7 +386,8 @@ struct Q40Limb {
 // Q8_0: two 34-byte blocks = 68 bytes = 17 dwords (dword aligned when columns % 64 == 0).
 struct Q80Limb {
     static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 34u;
-    static constexpr bool kLdsCopies = true;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
+    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -483,7 +487,8 @@ __device__ __forceinline__ void load_run_activations(const StageMemory& stage, u
 // are not consecutive, so it gathers its activation limbs run by run (load_activations).
 struct Q6KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 210u;
-    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = false;    // gemv_limb_kernel only: a share of 14336 rows (56 x 3360 bytes) does not fit LDS
+    static constexpr bool kLoaderFolds = false;
     struct Lane {
         uint32_t offset;  // byte offset of the lane's block within a row
         uint32_t half, j;
@@ -594,7 +599,8 @@ typedef struct __attribute__((packed, aligned(2))) { uint32_t v[3]; } Dwords3_a2
 // (scales[..] >> 4). A lane takes (half, j): runs g = 0..3, sixteen bytes of quants.
 struct Q2KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 84u;
-    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
+    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec; LDS serves the lanes' loads at any alignment
+    static constexpr bool kLoaderFolds = false;  // the loaders only copy: the run-wise activation gather is the consumers'
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -669,7 +675,10 @@ struct Q2KLimb {
 // (hmask[16j + i] bit (4*half + g) ? 0 : 4)). A lane takes (half, j): runs g = 0..3.
 struct Q3KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 110u;
-    static constexpr bool kLdsCopies = false;  // every load of a lane is aligned to its size: LDS can serve it
+    // gemv_limb_kernel only. LDS serves the lanes' 2-byte-aligned 16-byte reads, but slowly: through
+    // gemv_limb_dma_kernel 14336 x 4096 measured 10.5 us against 9.6.
+    static constexpr bool kLdsCopies = false;
+    static constexpr bool kLoaderFolds = false;
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -954,6 +963,10 @@ constexpr int kDmaLoaderRows = 1;  // rows at the end of a range that its loader
                                    // a loader that folds is late with the word its consumer waits for)
 constexpr int kDmaDepth = 4;  // copies a loader keeps in flight: more only lengthen the queue, and a loader says that a
                               // copy has landed only when it may issue the copy DEPTH places later
+constexpr int kDmaHead = kDmaDepth;  // copies a loader issues before it does anything else, at most eight
+                                     // (wait_copies_in_flight). Six and eight measured slower (Q4_K 14336 x 4096:
+                                     // 7.9 and 8.2 against 7.7 us): a longer queue only delays everybody's first rows.
+constexpr uint32_t kDmaLateEighths = 2;  // share of a range that a loader which only copies folds at the end
 constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaPairs);
 constexpr uint32_t kDmaLdsBytes = 160u * 1024u;
 struct DmaControl {
@@ -1023,17 +1036,19 @@ __device__ __forceinline__ void load_limbs_unseen(const StageMemory& stage, uint
     out.sum[1] = active ? __uint_as_float(sum1) : 0.f;
 }
 
-// The last copies of a loader: `outstanding` <= DEPTH of them are in flight, in the last slots of a
-// list of DEPTH, so that "the copy of slot I has landed" is the compile-time count vmcnt <= DEPTH - 1 - I.
-template <int DEPTH, int I, class F>
-__device__ __forceinline__ void dma_drain(uint32_t outstanding, uint32_t landed_address, uint32_t& landed, const F& after) {
-    if constexpr (I < DEPTH) {
-        if (static_cast<uint32_t>(I) >= DEPTH - outstanding) {
-            __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1 - I));
-            lds_store_unseen(landed_address, ++landed);
-            after(landed);
-        }
-        dma_drain<DEPTH, I + 1>(outstanding, landed_address, landed, after);
+// Waits until at most `left` (wave-uniform, below kDmaHead) of this wave's copies are in flight: the
+// count of s_waitcnt is an immediate, so one instruction per value.
+__device__ __forceinline__ void wait_copies_in_flight(uint32_t left) {
+    switch (left) {
+        case 0: __builtin_amdgcn_s_waitcnt(vmcnt_only(0)); break;
+        case 1: __builtin_amdgcn_s_waitcnt(vmcnt_only(1)); break;
+        case 2: __builtin_amdgcn_s_waitcnt(vmcnt_only(2)); break;
+        case 3: __builtin_amdgcn_s_waitcnt(vmcnt_only(3)); break;
+        case 4: __builtin_amdgcn_s_waitcnt(vmcnt_only(4)); break;
+        case 5: __builtin_amdgcn_s_waitcnt(vmcnt_only(5)); break;
+        case 6: __builtin_amdgcn_s_waitcnt(vmcnt_only(6)); break;
+        case 7: __builtin_amdgcn_s_waitcnt(vmcnt_only(7)); break;
+        default: break;
     }
 }
 
@@ -1045,6 +1060,11 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr uint32_t kStageAt = kDmaControlAt - M * static_cast<uint32_t>(sizeof(StageMemory));
     constexpr int NI = kSliceQuads / (64 * kDmaConsumers);  // float4s per consumer thread and vector
+    static_assert(DEPTH <= kDmaHead && kDmaHead <= 8, "the steady loop starts with DEPTH copies in flight; wait_copies_in_flight counts to seven");
+    constexpr int kLoaderRows = T::kLoaderFolds ? kDmaLoaderRows : 0;  // rows at the end of a range that its loader folds
+    // Codecs whose fold is long against their bytes (the 2- and 3-bit ones): a loader has issued its few copies
+    // early and would idle; once they have all landed it folds the last kDmaLateEighths / 8 of the range.
+    constexpr bool kLate = !T::kLoaderFolds;
     DmaControl* control = reinterpret_cast<DmaControl*>(lds + kDmaControlAt);
     StageMemory* stage = reinterpret_cast<StageMemory*>(lds + kStageAt);
 
@@ -1062,6 +1082,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     const uint32_t count = min(per_pair, wg_rows - first);
     const uint32_t range_kib = (per_pair * row_bytes + 1023u) >> 10;
     uint8_t* range = lds + pair * (range_kib << 10);
+    const uint32_t late = kLate ? count * kDmaLateEighths / 8u : 0u;  // rows the loader folds after its last copy
 
     const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
     const bool active = chunk < columns / kChunk;
@@ -1110,35 +1131,62 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
         // The first copies wait for the barrier, i.e. until the consumers have issued their activation
         // loads: issued ahead of it they delay those loads, and with them every fold, by half a microsecond.
         __syncthreads();
-        const uint32_t head = min(copies, static_cast<uint32_t>(DEPTH));
+        const uint32_t head = min(copies, static_cast<uint32_t>(kDmaHead));
         for (uint32_t i = 0; i < head; i++) copy(i);
         // The loader folds the last row of its range itself (below), next to the consumer folding the
         // row before: one fold after the last byte instead of two. Its
         // limbs come out of the stages as soon as the consumers have written them, while its first
         // copies are on their way (measured: later in the stream this costs a quarter microsecond).
-        lds_await(lds_address(&control->staged), kDmaConsumers);
+        if constexpr (kLoaderRows > 0) {
+            lds_await(lds_address(&control->staged), kDmaConsumers);
 #pragma unroll
-        for (int m = 0; m < M; m++) load_limbs_unseen(stage[m], lane_id, active, xr[m]);
-        uint32_t landed = 0;
-        for (uint32_t i = head; i < copies; i++) {
+            for (int m = 0; m < M; m++) load_limbs_unseen(stage[m], lane_id, active, xr[m]);
+        }
+        uint32_t landed = 0, in_flight = head;
+        if (in_flight > static_cast<uint32_t>(DEPTH)) {  // down to the steady depth
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH));
+            landed = in_flight - DEPTH;
+            in_flight = DEPTH;
+            lds_store_unseen(landed_address, landed);
+        }
+        for (uint32_t i = head; i < copies; i++) {  // only with DEPTH copies in flight (head = kDmaHead < copies)
             // the oldest copy in flight has landed: say so, then take its place in the queue
             __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));
             lds_store_unseen(landed_address, ++landed);
             copy(i);
         }
-        // With every copy issued the loader is free: it folds the last kDmaLoaderRows rows of the range
+        // With every copy issued the loader is free: it folds the last kLoaderRows rows of the range
         // itself, each the moment its last copy has landed.
-        const uint32_t own = min(count, static_cast<uint32_t>(kDmaLoaderRows));
+        const uint32_t own = min(count, static_cast<uint32_t>(kLoaderRows));
         uint32_t next_own = count - own;
         const auto fold_landed = [&](uint32_t have) {
-            while (next_own < count && have >= (((next_own + 1u) * row_bytes + 1023u) >> 10)) {
-                typename T::Data data;
-                T::load(range + next_own * row_bytes, lane, data);
-                fold_row(next_own, data);
-                next_own += 1u;
+            if constexpr (kLoaderRows > 0) {
+                while (next_own < count && have >= (((next_own + 1u) * row_bytes + 1023u) >> 10)) {
+                    typename T::Data data;
+                    T::load(range + next_own * row_bytes, lane, data);
+                    fold_row(next_own, data);
+                    next_own += 1u;
+                }
             }
         };
-        dma_drain<DEPTH, 0>(head, landed_address, landed, fold_landed);
+        for (uint32_t left = in_flight; left > 0u; left--) {
+            wait_copies_in_flight(left - 1u);
+            lds_store_unseen(landed_address, ++landed);
+            fold_landed(landed);
+        }
+        if constexpr (kLate) {
+            // nothing of this wave is in flight any more: ordinary LDS reads from here on
+            if (late != 0u) {
+                lds_await(lds_address(&control->staged), kDmaConsumers);
+#pragma unroll
+                for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
+                for (uint32_t r = count - late; r < count; r++) {
+                    typename T::Data data;
+                    T::load(range + r * row_bytes, lane, data);
+                    fold_row(r, data);
+                }
+            }
+        }
         return;
     }
 
@@ -1156,7 +1204,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     // Row r needs the copies that hold bytes [0, (r + 1) * row_bytes) of the range. (Reading row r + 1
     // out of LDS ahead of the fold of row r, when it has landed by then, measured slower: the consumers
     // are bound by their arithmetic, two of them and two loaders to a SIMD, not by LDS latency.)
-    const uint32_t mine = count - min(count, static_cast<uint32_t>(kDmaLoaderRows));  // the last rows are the loader's
+    const uint32_t mine = count - (kLate ? late : min(count, static_cast<uint32_t>(kLoaderRows)));  // the last rows are the loader's
     for (uint32_t r = 0; r < mine; r++) {
         lds_await(landed_address, ((r + 1u) * row_bytes + 1023u) >> 10);
         typename T::Data data;
@@ -1308,6 +1356,7 @@ bool gemv_limb_copies_through_lds(int32_t codec, uint64_t rows, uint64_t columns
         case kQ5_K: return dma_takes<Q5KLimb, 1>(n, k, &rows_per_wg);
         case kQ4_0: return dma_takes<Q40Limb, 1>(n, k, &rows_per_wg);
         case kQ8_0: return dma_takes<Q80Limb, 1>(n, k, &rows_per_wg);
+        case kQ2_K: return dma_takes<Q2KLimb, 1>(n, k, &rows_per_wg);
         default: return false;
     }
 }
