@@ -278,11 +278,15 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
     for (int t = 0; t < MT; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+    // With one limb the integer sums start at the bits of 1.5 * 2^23 instead of zero: a block's sum
+    // (|c| <= 32 * 128 * 127 < 2^22) added to those bits IS the float 12582912 + c, so the epilogue turns
+    // it into c with one subtraction - exact, and half the issue time of an int-to-float convert.
+    constexpr int kFloatBias = 0x4B400000;
     v16i zero_i;
     v16f zero_f;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-        zero_i[r] = 0;
+        zero_i[r] = LIMBS == 1 ? kFloatBias : 0;
         zero_f[r] = 0.f;
     }
 
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         // The NB * MT (block, tile) steps of the stage as a software pipeline. Each step reads its
         // A operands (and the activation scales) from LDS one step ahead, issues its MFMAs, and
         // runs the f32 epilogue of an earlier step while they execute: with one limb the previous
-        // step's (its results are double-buffered), with three limbs its own (three results of
+        // step's (its integer sums are double-buffered), with three limbs its own (three results of
         // sixteen registers each leave no room for a second set).
         constexpr int kSteps = NB * MT;
         const auto read_step = [&](int step, v4i (&a)[LIMBS], float& x_scale, uint2& x_pieces) {
@@ -397,7 +401,7 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 if constexpr (LIMBS == 1) {
-                    acc[t][r] = fmaf(static_cast<float>(c[0][r]), sd[r], acc[t][r]);
+                    acc[t][r] = fmaf(__int_as_float(c[0][r]) - 12582912.0f, sd[r], acc[t][r]);
                 } else {
                     // |c0 + 256 c1| < 2^28 is exact in int32; the top limb joins in f32
                     const float low = static_cast<float>(c[0][r] + (c[1][r] << 8));
@@ -410,35 +414,62 @@ __global__ __launch_bounds__(kThreads) void gemm_i8_kernel(
         float x_scale_next = 0.f;
         uint2 x_pieces_next = make_uint2(0u, 0u);
         read_step(0, a_next, x_scale_next, x_pieces_next);
-        v16f sd_previous;
-        v16i c_previous[LIMBS];
-#pragma unroll
-        for (int step = 0; step < kSteps; step++) {
-            const int bb = step / MT;
-            // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1
-            // product in the MFMA result layout.
-            v16f sd;
+        // Scale products s[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1 product in
+        // the MFMA result layout.
+        const auto scale_products = [&](int bb, float x_scale, const uint2& x_pieces) -> v16f {
             if constexpr (kPieces)
-                sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_scale_pieces(x_pieces_next).values, w_pieces[bb].values,
-                                                             zero_f, 0, 0, 0);
+                return __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_scale_pieces(x_pieces).values, w_pieces[bb].values,
+                                                               zero_f, 0, 0, 0);
             else
-                sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale_next : 0.f, w_scale[bb], zero_f, 0, 0, 0);
-            v16i c[LIMBS];
+                return __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? x_scale : 0.f, w_scale[bb], zero_f, 0, 0, 0);
+        };
+        if constexpr (LIMBS == 1) {
+            // Every matrix instruction is followed by half of an epilogue, sixteen VALU instructions that
+            // do not depend on it, so the matrix pipe and the VALU run side by side within the wave:
+            //   scale products of step s   | the integer sums of step s become floats (in place)
+            //   integer MFMA of step s + 1 | acc += sums * scale products of step s
+            // The integer sums alternate between two register sets; the scale products need one.
+            v16i c_now = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[0], bw[0], zero_i, 0, 0, 0);
+            float x_scale = x_scale_next;
+            uint2 x_pieces = x_pieces_next;
+            if (1 < kSteps) read_step(1, a_next, x_scale_next, x_pieces_next);
 #pragma unroll
-            for (int l = 0; l < LIMBS; l++)
-                c[l] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[l], bw[bb], zero_i, 0, 0, 0);
-            if (step + 1 < kSteps) read_step(step + 1, a_next, x_scale_next, x_pieces_next);
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (LIMBS == 1) {
-                if (step > 0) epilogue(step - 1, sd_previous, c_previous);
-                sd_previous = sd;
-                c_previous[0] = c[0];
-            } else {
-                epilogue(step, sd, c);
+            for (int step = 0; step < kSteps; step++) {
+                const int t = step % MT;
+                // the matrix instruction first in each half (scheduling barriers: the compiler would put it last)
+                __builtin_amdgcn_sched_barrier(0);
+                const v16f sd = scale_products(step / MT, x_scale, x_pieces);
+                __builtin_amdgcn_sched_barrier(0);
+                float sums[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) sums[r] = __int_as_float(c_now[r]) - 12582912.0f;
+                __builtin_amdgcn_sched_barrier(0);
+                if (step + 1 < kSteps) {
+                    c_now = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[0], bw[(step + 1) / MT], zero_i, 0, 0, 0);
+                    x_scale = x_scale_next;
+                    x_pieces = x_pieces_next;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (step + 2 < kSteps) read_step(step + 2, a_next, x_scale_next, x_pieces_next);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[t][r] = fmaf(sums[r], sd[r], acc[t][r]);
             }
             __builtin_amdgcn_sched_barrier(0);
+        } else {
+#pragma unroll
+            for (int step = 0; step < kSteps; step++) {
+                const int bb = step / MT;
+                const v16f sd = scale_products(bb, x_scale_next, x_pieces_next);
+                v16i c[LIMBS];
+#pragma unroll
+                for (int l = 0; l < LIMBS; l++)
+                    c[l] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a_next[l], bw[bb], zero_i, 0, 0, 0);
+                if (step + 1 < kSteps) read_step(step + 1, a_next, x_scale_next, x_pieces_next);
+                __builtin_amdgcn_sched_barrier(0);
+                epilogue(step, sd, c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if constexpr (LIMBS == 1) epilogue(kSteps - 1, sd_previous, c_previous);
     }
 
     // ---- combine the K shares, add bias, store ----------------------------------
