@@ -41,11 +41,13 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # When either differs from what runs now, `roofline.traffic` is null until the profile is re-taken.
 MEASURED_TRAFFIC = {
     ("q4_k_gemv_14336x4096", 1, "f32"): {
-        "bytes": 33338900, "kernel": "gemv_limb", "source": "gemv_limb.hip",
-        "sha256": "", "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
+        "bytes": 33316300, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
+        "sha256": "c97830386ce6b1bbaa1f8903e935411df72db510501e31dcf2e961dfcea3d1d8",
+        "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("kv_attention_decode", 2048): {
-        "bytes": 270009600, "kernel": "kv_attend", "source": "kv_attention.hip",
-        "sha256": "", "profile": "profiles/kv_attend_decode_32slots_ctx2048_f16.md"},
+        "bytes": 270084300, "kernel": "kv_attend", "source": "kv_attention.hip",
+        "sha256": "ab443b662f85428cacde8b1f6661a293f79c242c4d6576d7dd6b73d1c87f1ef9",
+        "profile": "profiles/kv_attend_decode_32slots_ctx2048_f16.md"},
 }
 
 
@@ -112,7 +114,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 200; "
                    "llama3_8b_batched_decode: 2)")
     p.add_argument("--workload", default="q4_k_gemv_14336x4096",
-                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,f16,f16_16x16}, "
+                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,i8_biased,i8_biased_matrix_only,i8_biased_valu_only,f16,f16_16x16}, "
                         "kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
@@ -350,7 +352,9 @@ def calibrate_mfma(args, et):
     """Loops of one matrix-core instruction that touch no memory (``calibrate_mfma_i8``, ``_i8_scaled``,
     ``_i8_scaled_bf16``, ``_f16``, ``_f16_16x16``): what the matrix cores of this device sustain, next to the published peak.
     ``_i8_scaled`` adds the f32 epilogue of a contraction whose operands both carry a scale per 32
-    columns: the ceiling of that arithmetic whatever feeds it."""
+    columns: the ceiling of that arithmetic whatever feeds it. ``_i8_biased`` is the step of the int8
+    batch kernel as it runs now; ``_i8_biased_matrix_only`` / ``_i8_biased_valu_only`` are its matrix and
+    its VALU instructions alone (rates quoted as if each were the whole step)."""
     import torch
 
     kind = args.workload[len("calibrate_mfma_"):]
@@ -362,8 +366,13 @@ def calibrate_mfma(args, et):
     step = lambda i: et.calibration_mfma(kind, iterations, sink)  # noqa: E731
     ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
     torch.cuda.synchronize()
-    expected = {"i8": 32.0, "i8_scaled": 16.0, "i8_scaled_bf16": 16.0, "f16": 16.0, "f16_16x16": 32.0}[kind] * iterations * \
-        (16 if kind == "f16_16x16" else 64)
+    if kind == "i8_biased_valu_only":  # the sums stay at their starting bits: every element adds 0
+        expected = 0.0
+    elif kind == "i8_biased_matrix_only":  # only the last step's results are summed: 16 elements of 32 * 0.5
+        expected = 256.0
+    else:
+        expected = {"i8": 32.0, "i8_scaled": 16.0, "i8_scaled_bf16": 16.0, "i8_biased": 16.0, "f16": 16.0,
+                    "f16_16x16": 32.0}[kind] * iterations * (16 if kind == "f16_16x16" else 64)
     assert torch.all(sink == expected), (float(sink[0]), expected)
     operations = et.MFMA_OPERATIONS[kind] * 4 * iterations * 4 * workgroups
     tops = operations / (ms * 1e-3) / 1e12
@@ -487,21 +496,23 @@ def kv_decode(args, et):
                      "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
     }
     if not args.no_cpu:
-        calls, t0 = 0, time.perf_counter()
         sample = 4
-        while time.perf_counter() - t0 < args.cpu_seconds or calls == 0:
-            oracle.kv_attention(k_ref, v_ref, block, table_host[:sample].view(np.uint32),
-                                cursors_host[:sample].view(np.uint32), advances_host[:sample].view(np.uint32),
-                                q_host[:sample], k_host[:sample], v_host[:sample], scale, k_scales=ks_ref,
-                                v_scales=vs_ref)
-            calls += 1
-        elapsed = time.perf_counter() - t0
+        with pinned_to_one_core() as pin:
+            calls, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < args.cpu_seconds or calls == 0:
+                oracle.kv_attention(k_ref, v_ref, block, table_host[:sample].view(np.uint32),
+                                    cursors_host[:sample].view(np.uint32), advances_host[:sample].view(np.uint32),
+                                    q_host[:sample], k_host[:sample], v_host[:sample], scale, k_scales=ks_ref,
+                                    v_scales=vs_ref)
+                calls += 1
+            elapsed = time.perf_counter() - t0
+            where = pin.describe()
         per_step = elapsed / calls * (slots / sample)
         result["cpu_baseline"] = {
             "value": round(algorithmic / per_step / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{calls} call(s) over {sample} of the {slots} slots, scaled by {slots // sample}; "
                       f"{elapsed:.1f} s of CPU work; scalar C restatement of the reference's f64 three-pass loop "
-                      f"({per_step * 1e3:.0f} ms per step)"}
+                      f"({per_step * 1e3:.0f} ms per step); {where}"}
     print(json.dumps(with_timing(result)))
 
 
@@ -616,14 +627,16 @@ def decode_op(args, et):
                      "algorithmic_bytes_per_launch": algorithmic, "avg_launch_us": round(ms * 1e3, 3)},
     }
     if not args.no_cpu:
-        calls, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < min(args.cpu_seconds, 3.0) or calls == 0:
-            cpu()
-            calls += 1
-        elapsed = time.perf_counter() - t0
+        with pinned_to_one_core() as pin:
+            calls, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < min(args.cpu_seconds, 3.0) or calls == 0:
+                cpu()
+                calls += 1
+            elapsed = time.perf_counter() - t0
+            where = pin.describe()
         result["cpu_baseline"] = {"value": round(algorithmic / (elapsed / calls) / 1e9, 4), "unit": "GB/s", "cores": 1,
                                   "kind": "port", "sample": f"{calls} full call(s) of the same workload, "
-                                  f"{elapsed:.1f} s of CPU work ({elapsed / calls * 1e6:.0f} us per call)"}
+                                  f"{elapsed:.1f} s of CPU work ({elapsed / calls * 1e6:.0f} us per call); {where}"}
     print(json.dumps(with_timing(result)))
 
 
@@ -686,16 +699,18 @@ def quantized_embedding(args, et):
     }
     if not args.no_cpu:
         cpu_tokens = min(tokens, 512)
-        calls, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < min(args.cpu_seconds, 5.0) or calls == 0:
-            oracle.embedding_into(int(codec), rows, columns, ids_host[0][:cpu_tokens], table_host)
-            calls += 1
-        elapsed = time.perf_counter() - t0
+        with pinned_to_one_core() as pin:
+            calls, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < min(args.cpu_seconds, 5.0) or calls == 0:
+                oracle.embedding_into(int(codec), rows, columns, ids_host[0][:cpu_tokens], table_host)
+                calls += 1
+            elapsed = time.perf_counter() - t0
+            where = pin.describe()
         per_token = elapsed / calls / cpu_tokens
         result["cpu_baseline"] = {"value": round((8 + row_bytes + 4 * columns) / per_token / 1e9, 4), "unit": "GB/s",
                                   "cores": 1, "kind": "port",
                                   "sample": f"{calls} call(s) on the first {cpu_tokens} ids, {elapsed:.1f} s of CPU "
-                                            f"work ({per_token * 1e6:.1f} us per row); scalar C restatement"}
+                                            f"work ({per_token * 1e6:.1f} us per row); scalar C restatement; {where}"}
     print(json.dumps(with_timing(result)))
 
 

@@ -826,8 +826,8 @@ int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* st
 int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgroups, float* sink, void* stream) {
     return guarded([&](std::string* error) -> int {
         if (sink == nullptr || workgroups == 0 || workgroups > 65536 || iterations == 0 || iterations > (1u << 20) ||
-            kind < ET_MFMA_I8 || kind > ET_MFMA_I8_SCALED_BF16) {
-            *error = "calibration_mfma: kind 0..4, 1 <= iterations <= 2^20, 1 <= workgroups <= 65536, sink non-NULL";
+            kind < ET_MFMA_I8 || kind > ET_MFMA_I8_BIASED_VALU_ONLY) {
+            *error = "calibration_mfma: kind 0..7, 1 <= iterations <= 2^20, 1 <= workgroups <= 65536, sink non-NULL";
             return ET_ERR_INVALID;
         }
         const hipError_t status = et::calibration_mfma(kind, iterations, workgroups, sink, static_cast<hipStream_t>(stream));

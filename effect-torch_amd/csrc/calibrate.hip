@@ -132,6 +132,8 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 //   kMfmaF16       v_mfma_f32_32x32x16_f16, accumulating: 16 * iterations
 //   kMfmaF16Small  v_mfma_f32_16x16x32_f16, accumulating: 32 * iterations
 //   kMfmaI8ScaledBf16  kMfmaI8Scaled with the scale products from a bfloat16 instruction (see below)
+//   kMfmaI8Biased (and ...MatrixOnly, ...ValuOnly)  the step of the int8 batch kernel as it runs now (see below);
+//                  element = 32 * 0.5 * iterations (0.5 * iterations per element for ...MatrixOnly's last step only)
 template <int KIND>
 __global__ __launch_bounds__(256) void mfma_kernel(float* __restrict__ sink, uint32_t iterations) {
     float total = 0.f;
@@ -214,6 +216,72 @@ __global__ __launch_bounds__(256) void mfma_kernel(float* __restrict__ sink, uin
         for (int k = 0; k < 4; k++)
 #pragma unroll
             for (int r = 0; r < 16; r++) total += acc[k][r];
+    } else if constexpr (KIND == kMfmaI8Biased || KIND == kMfmaI8BiasedMatrixOnly || KIND == kMfmaI8BiasedValuOnly) {
+        // The step of gemm_i8.hip's one-limb loop as it is now: the integer sums start at the bits of
+        // 1.5 * 2^23 (their bits are then the float 12582912 + sum: one subtraction instead of a convert),
+        // the scale products come from v_mfma_f32_32x32x16_bf16 with ready-made operand pieces, and each
+        // matrix instruction is followed by sixteen VALU instructions that do not depend on it:
+        //   scale products | 16 subtractions;  integer MFMA of the next step | 16 multiply-adds.
+        // kMfmaI8BiasedMatrixOnly leaves the VALU instructions out, kMfmaI8BiasedValuOnly the matrix ones
+        // (same registers, fed by empty asm statements): together they show how much of the two the
+        // device runs side by side.
+        const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+        v16i bias;
+#pragma unroll
+        for (int r = 0; r < 16; r++) bias[r] = 0x4B400000;
+        v16f zero_f = {};
+        float acc[4][16] = {};
+        const bool first_half = threadIdx.x % 64 < 32;
+        union {
+            uint4 words;
+            v8bf values;
+        } row_operand, vector_operand;
+        // 0.5 and 1.0 in bfloat16: K slot 0 of the first lane half carries the product, the rest zeros
+        row_operand.words = make_uint4(first_half ? 0x3f00u : 0u, 0u, 0u, 0u);
+        uint32_t vector_piece = 0x3f80u;
+        v4i a = ones;
+        v16i c_now = bias;
+        v16f sd = zero_f;
+        if constexpr (KIND != kMfmaI8BiasedValuOnly) c_now = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ones, bias, 0, 0, 0);
+        for (uint32_t it = 0; it < iterations; it++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                asm volatile("" : "+v"(vector_piece));
+                vector_operand.words = make_uint4(vector_piece, 0u, 0u, 0u);
+                asm volatile("" : "+v"(a));
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (KIND != kMfmaI8BiasedValuOnly)
+                    sd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vector_operand.values, row_operand.values, zero_f, 0, 0, 0);
+                else
+                    asm volatile("" : "+v"(sd));
+                if constexpr (KIND == kMfmaI8BiasedMatrixOnly) asm volatile("" : : "v"(sd));  // a use: the instruction stays
+                __builtin_amdgcn_sched_barrier(0);
+                float sums[16];
+                if constexpr (KIND != kMfmaI8BiasedMatrixOnly) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sums[r] = __int_as_float(c_now[r]) - 12582912.0f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (KIND != kMfmaI8BiasedValuOnly)
+                    c_now = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, ones, bias, 0, 0, 0);
+                else
+                    asm volatile("" : "+v"(c_now));
+                if constexpr (KIND == kMfmaI8BiasedMatrixOnly) asm volatile("" : : "v"(c_now));
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (KIND != kMfmaI8BiasedMatrixOnly) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[k][r] = fmaf(sums[r], sd[r], acc[k][r]);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += acc[k][r];
+        if constexpr (KIND == kMfmaI8BiasedMatrixOnly) {  // keep the last results alive
+#pragma unroll
+            for (int r = 0; r < 16; r++) total += (__int_as_float(c_now[r]) - 12582912.0f) * sd[r];
+        }
     } else if constexpr (KIND == kMfmaF16) {
         v8h ones;
 #pragma unroll
@@ -252,6 +320,9 @@ hipError_t calibration_mfma(int kind, uint32_t iterations, uint32_t workgroups, 
         case kMfmaF16: hipLaunchKernelGGL(mfma_kernel<kMfmaF16>, grid, block, 0, stream, sink, iterations); break;
         case kMfmaF16Small: hipLaunchKernelGGL(mfma_kernel<kMfmaF16Small>, grid, block, 0, stream, sink, iterations); break;
         case kMfmaI8ScaledBf16: hipLaunchKernelGGL(mfma_kernel<kMfmaI8ScaledBf16>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaI8Biased: hipLaunchKernelGGL(mfma_kernel<kMfmaI8Biased>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaI8BiasedMatrixOnly: hipLaunchKernelGGL(mfma_kernel<kMfmaI8BiasedMatrixOnly>, grid, block, 0, stream, sink, iterations); break;
+        case kMfmaI8BiasedValuOnly: hipLaunchKernelGGL(mfma_kernel<kMfmaI8BiasedValuOnly>, grid, block, 0, stream, sink, iterations); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -253,7 +253,8 @@ hipError_t calibration_read_variant(int variant, const void* src, uint64_t bytes
 hipError_t calibration_copy(const void* src, void* dst, uint64_t bytes, hipStream_t stream);
 // Loops of matrix-core instructions without memory traffic: four waves per workgroup, four
 // independent instructions per wave and round; sink gets one float per thread (256 * workgroups).
-enum : int { kMfmaI8 = 0, kMfmaI8Scaled = 1, kMfmaF16 = 2, kMfmaF16Small = 3, kMfmaI8ScaledBf16 = 4 };
+enum : int { kMfmaI8 = 0, kMfmaI8Scaled = 1, kMfmaF16 = 2, kMfmaF16Small = 3, kMfmaI8ScaledBf16 = 4,
+              kMfmaI8Biased = 5, kMfmaI8BiasedMatrixOnly = 6, kMfmaI8BiasedValuOnly = 7 };
 hipError_t calibration_mfma(int kind, uint32_t iterations, uint32_t workgroups, float* sink, hipStream_t stream);
 
 }  // namespace et

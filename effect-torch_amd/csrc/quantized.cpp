@@ -4,6 +4,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstring>
+#include <initializer_list>
 #include <limits>
 #include <sstream>
 
@@ -108,31 +109,37 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     if (plan->rows > 0xffffffffull || plan->columns > 0xffffffffull || plan->vectors > 0xffffffffull)
         return fail(error, ET_ERR_UNSUPPORTED,
                     "quantized_linear: rows, columns and vectors must each fit 32 bits");
+    // The workspace, part after part, each at a multiple of 256 bytes. Every size is a checked product
+    // (rows, columns and vectors each fit 32 bits, their products times a byte count need not fit 64):
+    // one that overflows leaves `fits` false and the plan is refused below.
     uint64_t cursor = 0;
+    bool fits = true;
+    const auto take = [&](std::initializer_list<uint64_t> factors) -> uint64_t {  // offset of a part of prod(factors) bytes
+        const uint64_t offset = cursor;
+        uint64_t bytes = 0;
+        if (!fits || !checked_product(std::vector<uint64_t>(factors), &bytes) || bytes > kMax - 255 - cursor) {
+            fits = false;
+            return 0;
+        }
+        cursor = align_up(cursor + bytes, 256);
+        return offset;
+    };
     // Space to densify a strided or misaligned f32 input.
-    plan->gather_offset = 0;
-    plan->gather_bytes = plan->vectors * plan->columns * 4u;
-    cursor = align_up(plan->gather_bytes, 256);
-    plan->bias_offset = cursor;  // dense copy of a strided bias
-    cursor = align_up(cursor + plan->rows * 4u, 256);
+    plan->gather_offset = take({plan->vectors, plan->columns, 4});
+    plan->gather_bytes = fits ? plan->vectors * plan->columns * 4u : 0;
+    plan->bias_offset = take({plan->rows, 4});  // dense copy of a strided bias
     const auto plan_matrix_core = [&](LinearKernel kernel, int limbs) {
         plan->kernel = kernel;
-        plan->q_offset = cursor;  // activation tiles, see tile_blob_bytes()
-        cursor = align_up(cursor + tile_workspace_bytes(limbs, plan->vectors, plan->columns), 256);
+        // activation tiles, see tile_blob_bytes(): one blob per 256-column stage and 32-vector tile
+        plan->q_offset = take({(plan->columns + 255) / 256, (plan->vectors + 31) / 32, tile_blob_bytes(limbs)});
         if (limbs == 2) {  // gemm_h16 chooses its own tile height and keeps partial results by whole tiles
-            plan->k_splits = gemm_h16_group_geometry(plan->codec, &plan->rows, 1, plan->columns, plan->vectors).k_splits;
-            if (plan->k_splits > 1) {
-                plan->partial_offset = cursor;
-                cursor = align_up(cursor + gemm_h16_group_partial_bytes(plan->codec, &plan->rows, 1, plan->columns,
-                                                                        plan->vectors), 256);
-            }
+            const GemmGroupGeometry g = gemm_h16_group_geometry(plan->codec, &plan->rows, 1, plan->columns, plan->vectors);
+            plan->k_splits = g.k_splits;
+            if (plan->k_splits > 1) plan->partial_offset = take({g.k_splits, plan->vectors, g.row_tiles, g.tile_rows, 4});
             return;
         }
         plan->k_splits = gemm_i8_k_splits(plan->codec, limbs, plan->rows, plan->columns, plan->vectors);
-        if (plan->k_splits > 1) {
-            plan->partial_offset = cursor;
-            cursor = align_up(cursor + plan->k_splits * plan->vectors * plan->rows * 4u, 256);
-        }
+        if (plan->k_splits > 1) plan->partial_offset = take({plan->k_splits, plan->vectors, plan->rows, 4});
     };
     if (plan->activation_mode == ET_ACT_INT8) {
         if (!gemm_i8_supported(plan->codec, plan->columns))
@@ -158,6 +165,7 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         return fail(error, ET_ERR_INVALID, "quantized_linear: unknown activation mode " +
                                                std::to_string(plan->activation_mode));
     }
+    if (!fits) return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: workspace byte size overflow");
     plan->workspace_bytes = cursor;
     return ET_OK;
 }
@@ -609,6 +617,7 @@ int linear_enqueue_prepared_then_norm(const et_linear_plan& plan, const void* pr
     out.leave_shares = true;
     if (hipError_t status = contract_tiles(plan, weight, static_cast<const uint8_t*>(prepared), out, as_stream(stream)))
         return hip_failure(error, "quantized_linear", status);
+    if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
     if (hipError_t status = quantize_tiles_rms_norm_of_shares(partials, layout.count, layout.launch_rows, bias, residual, y,
                                                               norm_weight, half_weight ? 1 : 0, eps, plan.vectors, plan.rows,
                                                               static_cast<uint8_t*>(next_prepared), as_stream(stream)))
@@ -628,6 +637,9 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         return fail(error, ET_ERR_INVALID, "quantized_linear: NULL operand");
     hipStream_t s = as_stream(stream);
     auto* scratch = static_cast<uint8_t*>(workspace);
+    // every part of the workspace starts at a multiple of 256 bytes and is read in 16-byte pieces
+    if (scratch != nullptr && reinterpret_cast<uintptr_t>(scratch) % 16 != 0)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: the workspace must be 16-byte aligned");
 
     // The kernels read activations with 16-byte loads.
     const bool aligned = (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (x_row_stride % 4 == 0) &&
@@ -661,6 +673,8 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         if (hipError_t status =
                 quantize_tiles(x, x_row_stride, plan.vectors, plan.columns, limbs_of(plan), tiles, s))
             return hip_failure(error, "quantized_linear", status);
+        // between the launches of one call, as the reference polls between rows (quantized.rs:451,459)
+        if (cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
         float* partials = plan.k_splits > 1 ? reinterpret_cast<float*>(scratch + plan.partial_offset) : nullptr;
         if (hipError_t status = contract_tiles(plan, weight, tiles, GemmOutput{bias, nullptr, y, partials}, s))
             return hip_failure(error, "quantized_linear", status);
@@ -668,6 +682,7 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
     }
 
     for (uint64_t v0 = 0; v0 < plan.vectors; v0 += plan.vectors_per_launch) {
+        if (v0 != 0 && cancelled(cancel)) return fail(error, ET_ERR_CANCELLED, "operation aborted");
         const uint32_t count = static_cast<uint32_t>(
             plan.vectors - v0 < plan.vectors_per_launch ? plan.vectors - v0 : plan.vectors_per_launch);
         const float* xv = x + v0 * x_row_stride;
@@ -782,6 +797,8 @@ int embedding_requirements(const TensorView& indexes, const TensorView& weight, 
     uint64_t row_bytes = 0;
     if (int status = validate_weight("quantized_embedding", weight, codec, rows, columns, &row_bytes, error))
         return status;
+    if (columns > 0xffff0000ull)  // the kernel counts columns, in chunks of 1024, in 32 bits
+        return fail(error, ET_ERR_UNSUPPORTED, "quantized_embedding: columns must fit 32 bits");
     plan->codec = codec;
     plan->rows = rows;
     plan->columns = columns;

@@ -559,8 +559,10 @@ def calibration_copy(src: torch.Tensor, dst: torch.Tensor, stream=None) -> None:
                                            src.numel() * src.element_size(), _stream_handle(stream)))
 
 
-MFMA_KINDS = {"i8": 0, "i8_scaled": 1, "f16": 2, "f16_16x16": 3, "i8_scaled_bf16": 4}
-MFMA_OPERATIONS = {"i8": 65536, "i8_scaled": 65536, "f16": 32768, "f16_16x16": 16384, "i8_scaled_bf16": 65536}
+MFMA_KINDS = {"i8": 0, "i8_scaled": 1, "f16": 2, "f16_16x16": 3, "i8_scaled_bf16": 4, "i8_biased": 5,
+              "i8_biased_matrix_only": 6, "i8_biased_valu_only": 7}
+MFMA_OPERATIONS = {"i8": 65536, "i8_scaled": 65536, "f16": 32768, "f16_16x16": 16384, "i8_scaled_bf16": 65536,
+                   "i8_biased": 65536, "i8_biased_matrix_only": 65536, "i8_biased_valu_only": 65536}
 
 
 def calibration_mfma(kind: str, iterations: int, sink: torch.Tensor, stream=None) -> None:

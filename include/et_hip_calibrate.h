@@ -45,10 +45,14 @@ int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* st
  * columns (a tile of scale products from v_mfma_f32_32x32x2f32, one convert and one multiply-add per
  * element); ET_MFMA_F16: v_mfma_f32_32x32x16_f16 (32 768 operations); ET_MFMA_F16_16X16:
  * v_mfma_f32_16x16x32_f16 (16 384); ET_MFMA_I8_SCALED_BF16: ET_MFMA_I8_SCALED with the scale products from
- * v_mfma_f32_32x32x16_bf16 (scales split into exact bfloat16 pieces). They measure what the matrix cores of this device sustain, the
+ * v_mfma_f32_32x32x16_bf16 (scales split into exact bfloat16 pieces); ET_MFMA_I8_BIASED: the step of the
+ * int8 batch kernel as it runs now (integer sums that start at the bits of 1.5 * 2^23, one subtraction and
+ * one multiply-add per element, each matrix instruction followed by half of them), ..._MATRIX_ONLY and
+ * ..._VALU_ONLY its matrix and its VALU instructions alone. They measure what the matrix cores of this device sustain, the
  * ceiling the batch kernels are compared with next to the published peak. No counterpart in the
  * reference, not part of the operator path. */
-enum { ET_MFMA_I8 = 0, ET_MFMA_I8_SCALED = 1, ET_MFMA_F16 = 2, ET_MFMA_F16_16X16 = 3, ET_MFMA_I8_SCALED_BF16 = 4 };
+enum { ET_MFMA_I8 = 0, ET_MFMA_I8_SCALED = 1, ET_MFMA_F16 = 2, ET_MFMA_F16_16X16 = 3, ET_MFMA_I8_SCALED_BF16 = 4,
+       ET_MFMA_I8_BIASED = 5, ET_MFMA_I8_BIASED_MATRIX_ONLY = 6, ET_MFMA_I8_BIASED_VALU_ONLY = 7 };
 int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgroups, float* sink, void* stream);
 
 #ifdef __cplusplus

@@ -125,6 +125,17 @@ def test_linear_plan_rejects_malformed_geometry(et):
         et.linear_requirements(x, _w(1, 210), None, et.GgmlQuant.Q6_K, (1, 256), et.ActivationMode.INT8)
 
 
+def test_workspace_sizes_are_checked_products(et):
+    # rows, columns and vectors each fit 32 bits; vectors * columns * 4 does not fit 64: refused, not wrapped
+    with pytest.raises(et.QuantizedError, match="workspace byte size overflow"):
+        et.RawLinear(et.GgmlQuant.Q4_K, 1, 2**32 - 256, 2**32 - 1)
+    with pytest.raises(et.QuantizedError, match="workspace byte size overflow"):
+        et.RawLinear(et.GgmlQuant.Q8_0, 64, 2**32 - 256, 2**32 - 1, False, et.ActivationMode.INT8)
+    # the largest sizes that do fit plan as before
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, 14336, 4096, 512)
+    assert plan.requirements.workspace_bytes >= 512 * 4096 * 4
+
+
 def test_embedding_plan(et):
     Q5 = et.GgmlQuant.Q5_K
     plan = et.embedding_requirements(torch.zeros((2, 3), dtype=torch.int64), _w(3, 176), Q5, (3, 256))
