@@ -125,6 +125,95 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
 }
 
 
+// quantize_kernel<LIMBS, true> for large inputs: a workgroup makes ONE blob - a 256-column stage of a
+// 32-vector tile - in LDS and writes it out linearly. The kernel above stores every dword where it
+// belongs in memory, sixteen bytes at a time in lines 512 bytes apart (measured on 512 x 14336: 29.4 MB
+// written for 11.0 MB of blobs); here a wave reads one vector's stage as 1 KiB of consecutive floats and
+// the blob leaves as consecutive 16-byte stores. Same arithmetic, same bytes.
+// LDS rows of the operand planes have a pitch of 528 bytes (512 + 16): a wave writes one vector's
+// dwords into all sixteen chunks at once, and with 512 they would share four banks.
+template <int LIMBS>
+__global__ __launch_bounds__(256) void quantize_blob_kernel(const float* __restrict__ x, uint64_t x_row_stride,
+                                                            uint32_t vectors, uint32_t columns,
+                                                            uint8_t* __restrict__ tiles) {
+    constexpr float kRange = LIMBS == 1 ? 127.f : 8323072.f;
+    constexpr uint32_t kBlob = tile_blob_bytes(LIMBS);
+    constexpr uint32_t kPitch = 528u, kPlane = 16u * kPitch, kTablesAt = LIMBS * kPlane;
+    constexpr uint32_t kTableBytes = kBlob - LIMBS * 8192u;
+    __shared__ __attribute__((aligned(16))) uint8_t blob[kTablesAt + kTableBytes];
+    const uint32_t vector_tiles = (vectors + 31u) >> 5;
+    const uint32_t stage = blockIdx.x / vector_tiles, tile = blockIdx.x - stage * vector_tiles;
+    const uint32_t quad_in_stage = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t quad = stage * 64u + quad_in_stage;  // of the row
+    // the tables' padding (behind the pieces) leaves as zeros
+    for (uint32_t at = 2048u + 2048u + threadIdx.x * 4u; at < kTableBytes; at += 1024u)
+        *reinterpret_cast<uint32_t*>(blob + kTablesAt + at) = 0u;
+    float4 in[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {  // a wave takes vectors wave, wave + 4, ...: all loads go out first
+        const uint32_t m = 4u * k + wave, v = tile * 32u + m;
+        in[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (v < vectors && 4u * quad < columns) in[k] = *reinterpret_cast<const float4*>(x + v * x_row_stride + 4u * quad);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const uint32_t m = 4u * k + wave;
+        float amax = fmaxf(fmaxf(fabsf(in[k].x), fabsf(in[k].y)), fmaxf(fabsf(in[k].z), fabsf(in[k].w)));
+        amax = fmaxf(amax, dpp_f32<0xB1>(amax));
+        amax = fmaxf(amax, dpp_f32<0x4E>(amax));
+        amax = fmaxf(amax, dpp_f32<0x141>(amax));
+        const float inv = amax > 0.f ? kRange / amax : 0.f;
+        int qi[4];
+        const float values[4] = {in[k].x, in[k].y, in[k].z, in[k].w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float r = rintf(values[i] * inv);
+            r = fminf(fmaxf(r, -kRange), kRange);
+            qi[i] = static_cast<int>(r);
+        }
+        int total_q = (qi[0] + qi[1]) + (qi[2] + qi[3]);
+        total_q += dpp_i32<0xB1>(total_q);
+        total_q += dpp_i32<0x4E>(total_q);
+        total_q += dpp_i32<0x141>(total_q);
+        const uint32_t chunk = quad_in_stage >> 2, dword = quad_in_stage & 3u;
+        uint8_t* slot = blob + chunk * kPitch + m * 16u + dword * 4u;
+        if constexpr (LIMBS == 1) {
+            *reinterpret_cast<uint32_t*>(slot) = (static_cast<uint32_t>(qi[0]) & 0xffu) | ((static_cast<uint32_t>(qi[1]) & 0xffu) << 8) |
+                                                 ((static_cast<uint32_t>(qi[2]) & 0xffu) << 16) |
+                                                 ((static_cast<uint32_t>(qi[3]) & 0xffu) << 24);
+        } else {
+            uint32_t u[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) u[i] = static_cast<uint32_t>(qi[i] + 0x808080);
+#pragma unroll
+            for (int limb = 0; limb < LIMBS; limb++)
+                *reinterpret_cast<uint32_t*>(slot + limb * kPlane) =
+                    (((u[0] >> (8 * limb)) & 0xffu) | (((u[1] >> (8 * limb)) & 0xffu) << 8) |
+                     (((u[2] >> (8 * limb)) & 0xffu) << 16) | (((u[3] >> (8 * limb)) & 0xffu) << 24)) ^ 0x80808080u;
+        }
+        if ((quad_in_stage & 7u) == 0) {
+            const float unit = amax / kRange;
+            float* tables = reinterpret_cast<float*>(blob + kTablesAt);
+            const uint32_t block = quad_in_stage >> 3;
+            tables[block * 32u + m] = unit;
+            tables[256u + block * 32u + m] = unit * static_cast<float>(total_q);
+            const uint32_t s0 = __float_as_uint(unit) & 0xffff0000u;
+            const float rest = unit - __uint_as_float(s0);
+            const uint32_t s1 = __float_as_uint(rest) & 0xffff0000u;
+            const uint32_t s2 = __float_as_uint(rest - __uint_as_float(s1));
+            reinterpret_cast<uint2*>(tables + 512u)[block * 32u + m] = make_uint2((s0 >> 16) | s1, s2 >> 16);
+        }
+    }
+    __syncthreads();
+    uint8_t* out = tiles + static_cast<uint64_t>(blockIdx.x) * kBlob;
+    for (uint32_t at = threadIdx.x * 16u; at < kBlob; at += 4096u) {
+        // the planes without their pitch padding, then the tables as they are
+        const uint32_t from = at < LIMBS * 8192u ? (at / 8192u) * kPlane + ((at % 8192u) / 512u) * kPitch + at % 512u
+                                                 : kTablesAt + (at - LIMBS * 8192u);
+        *reinterpret_cast<uint4*>(out + at) = *reinterpret_cast<const uint4*>(blob + from);
+    }
+}
+
 // SILU_MUL: the activations are silu(x) * second, element by element (the input of a gated
 // feed-forward's down projection), computed on the fly with silu_mul_kernel's arithmetic.
 template <bool SILU_MUL>
@@ -270,6 +359,18 @@ hipError_t quantize_tiles(const float* x, uint64_t x_row_stride, uint64_t vector
         return hipGetLastError();
     }
     if (limbs != 1 && limbs != 3) return hipErrorInvalidValue;
+    // Enough blobs to occupy the device: a workgroup per blob, assembled in LDS and written once.
+    const uint64_t blobs = ((columns + 255) / 256) * ((vectors + 31) / 32);
+    if (blobs >= 512 && blobs <= 0x7fffffffull) {
+        const dim3 blob_grid(static_cast<uint32_t>(blobs)), blob_block(256);
+        if (limbs == 1)
+            hipLaunchKernelGGL(quantize_blob_kernel<1>, blob_grid, blob_block, 0, stream, x, x_row_stride,
+                               static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
+        else
+            hipLaunchKernelGGL(quantize_blob_kernel<3>, blob_grid, blob_block, 0, stream, x, x_row_stride,
+                               static_cast<uint32_t>(vectors), static_cast<uint32_t>(columns), tiles);
+        return hipGetLastError();
+    }
     const Geometry g = geometry_for(total);
     const dim3 grid(g.blocks), block(g.threads);
     if (limbs == 1)

@@ -625,6 +625,38 @@ def test_shared_prepared_input_and_residual_epilogue(et, device, mode):
         small.prepare_input(x[:2], prepared)
 
 
+@pytest.mark.parametrize("mode,blob_bytes,limbs", [("INT8", 12288, 1), ("F32", 28672, 3)])
+def test_large_inputs_prepare_blob_by_blob_with_the_same_bytes(et, device, mode, blob_bytes, limbs):
+    # Inputs of 512 and more blobs (256-column stages x 32-vector tiles) are quantised by a kernel that
+    # assembles each blob in LDS; smaller ones by the kernel that stores every dword where it belongs.
+    # The same rows prepared 32 at a time (few blobs per call) must give the same bytes, blob by blob -
+    # what lies behind the last valid vector of a ragged tile is not compared.
+    rng = np.random.default_rng(4242 + limbs)
+    columns, vectors = 14336, 500  # 56 stages x 16 tiles = 896 blobs; the last tile holds 20 vectors
+    act = et.ActivationMode[mode]
+    x = to_dev(synth.random_activations(vectors, columns, rng), device)
+    x[3, 512:768] = 0.0  # a stage of zeros: unit 0
+    big = et.RawLinear(et.GgmlQuant.Q8_0, 64, columns, vectors, False, act)
+    stages, tiles = columns // 256, -(-vectors // 32)
+    assert big.prepared_input_bytes == stages * tiles * blob_bytes
+    prepared = torch.zeros(big.prepared_input_bytes, dtype=torch.uint8, device=device)
+    big.prepare_input(x, prepared)
+    whole = prepared.cpu().numpy().reshape(stages, tiles, blob_bytes)
+    for tile in range(tiles):
+        count = min(32, vectors - 32 * tile)
+        small = et.RawLinear(et.GgmlQuant.Q8_0, 64, columns, count, False, act)
+        part = torch.zeros(small.prepared_input_bytes, dtype=torch.uint8, device=device)
+        small.prepare_input(x[32 * tile:32 * tile + count], part)
+        want = part.cpu().numpy().reshape(stages, blob_bytes)
+        got = whole[:, tile]
+        planes = lambda a: a[:, :limbs * 8192].reshape(stages, limbs, 16, 32, 16)[:, :, :, :count]  # noqa: E731
+        assert np.array_equal(planes(got), planes(want)), tile
+        tables = lambda a: a[:, limbs * 8192:limbs * 8192 + 2048].reshape(stages, 2, 8, 32, 4)[:, :, :, :count]  # noqa: E731
+        assert np.array_equal(tables(got), tables(want)), tile
+        pieces = lambda a: a[:, limbs * 8192 + 2048:limbs * 8192 + 4096].reshape(stages, 8, 32, 8)[:, :, :count]  # noqa: E731
+        assert np.array_equal(pieces(got), pieces(want)), tile
+
+
 def test_prepared_input_of_an_operator_on_the_fly(et, device):
     # rms_norm(x) * w and silu(gate) * up applied while the activations are quantised: the prepared
     # bytes, and so every contraction from them, are those of the operator followed by prepare_input
