@@ -180,6 +180,8 @@ def cpu_baseline(cfg, vectors, mode, weight, x, seconds, algorithmic_bytes):
 
 
 MIN_GRAPH_STEPS = 400     # a graph of fewer kernels pays its launch (about 15 us) per step: see time_steps
+MAX_GRAPH_STEPS = 2000    # ... and one of up to this many when the steps are short (a replay of about 15 ms)
+GRAPH_WINDOW_MS = 15.0
 MIN_REPETITIONS = 5       # timed replays of the K steps; the median is reported
 TIMED_WINDOW_MS = 20.0    # short replays are repeated until about this much device time is covered
 MAX_REPETITIONS = 400
@@ -194,17 +196,25 @@ def time_steps(step, steps, warmup, use_graph):
     that a short run is not one sample taken while the device clocks still ramp. A graph of few
     kernels would charge its own launch to them (about 15 us per replay: 0.75 us per step of a
     20-step graph, none of it kernel time), so the K steps are captured `cycles` times over in one
-    graph until it holds MIN_GRAPH_STEPS of them; a repetition then times cycles * K steps and the
-    time per step is the replay time over that count.
+    graph until it holds MIN_GRAPH_STEPS of them - more, up to MAX_GRAPH_STEPS, while a replay stays
+    under about GRAPH_WINDOW_MS (judged by the warm-up steps' own time): a run with K = 20 then times
+    the same kind of replay as one with K = 2000; a repetition times cycles * K steps and the time per
+    step is the replay time over that count.
     Returns (ms per step, graph used, wall seconds); LAST_TIMING holds repetitions / min / max."""
     import torch
 
     stream = torch.cuda.current_stream()
+    warm = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    warm[0].record(stream)
     for i in range(warmup):
         step(i)
+    warm[1].record(stream)
     torch.cuda.synchronize()
     graph = None
-    cycles = max(1, -(-MIN_GRAPH_STEPS // steps)) if use_graph else 1
+    # an upper estimate of a step (plain enqueues carry their launch time): how many fit the window
+    estimate_ms = warm[0].elapsed_time(warm[1]) / warmup if warmup > 0 else GRAPH_WINDOW_MS
+    wanted = int(min(MAX_GRAPH_STEPS, max(MIN_GRAPH_STEPS, GRAPH_WINDOW_MS / max(estimate_ms, 1e-4))))
+    cycles = max(1, -(-wanted // steps)) if use_graph else 1
     if use_graph:
         try:
             graph = torch.cuda.CUDAGraph()
