@@ -430,7 +430,6 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const uint4 header = *reinterpret_cast<const uint4*>(row_in_slot);
         const float d_block = half_bits_to_float(header.x & 0xffffu);
         const float dmin_block = half_bits_to_float(header.x >> 16);
-        const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
         uint4 fifth = make_uint4(0u, 0u, 0u, 0u);  // Q5_K: qh of this lane half's sixteen columns
         if constexpr (CODEC == kQ5_K) fifth = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 16u * half);
 
@@ -494,10 +493,19 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 }
             }
         }
-        // unit[m] * d[n] for the sixteen vectors this lane accumulates: a rank-1 product in the
-        // result layout (only the k = 0 half of the lanes carries a value).
-        const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
-                                                             zero, 0, 0, 0);
+        // unit[m] * d[n] for the sixteen vectors this lane accumulates, m = 8 * (r / 4) + 4 * half + r % 4:
+        // four 16-byte LDS reads that every lane of a half shares, sixteen multiplications. (The same
+        // products as a rank-1 v_mfma_f32_32x32x2f32 in the result layout cost 64 cycles of the matrix
+        // pipe, and matrix and VALU instructions do not run side by side on this device.)
+        float sd[16];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float4 units = *reinterpret_cast<const float4*>(slot + kUnitAt + (8u * j + 4u * half) * 4u);
+            sd[4 * j + 0] = units.x * d_block;
+            sd[4 * j + 1] = units.y * d_block;
+            sd[4 * j + 2] = units.z * d_block;
+            sd[4 * j + 3] = units.w * d_block;
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
     }
