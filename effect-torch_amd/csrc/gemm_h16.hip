@@ -7,7 +7,9 @@
 //
 // Activations are 24-bit fixed point per vector and stage, X = rint(x * (2^23 - 1) / max|x|), split
 // into two balanced 12-bit halves X = 4096 * hi + lo with |lo|, |hi| <= 2048: integers a half float
-// holds exactly. On the weight side the 6-bit sub-block scale is folded into the operand:
+// holds exactly. The tiles hold hi and lo / 4096 (exact as well: a power of two), so that both halves
+// of a sub-block add up in ONE accumulator, hi * w + (lo / 4096) * w = X * w / 4096, and the factor
+// 4096 rides on the row scale: one multiply-add per element and stage in the epilogue. On the weight side the 6-bit sub-block scale is folded into the operand:
 // sc_g * nib <= 63 * 15 = 945 (Q5_K: 63 * 31 = 1953), exact in a half float as well. Every product (< 2^21) is exact in
 // the f32 the matrix core accumulates in, so v_mfma_f32_32x32x16_f16 sums whole super-blocks with
 // f32 accumulation error only, and the f32 scales unit[m] * d[n] are applied once per stage instead
@@ -49,6 +51,7 @@ constexpr int kThreads = 64 * (kConsumers + kLoaders);
 // workgroup copies per weight row; two groups (64 rows) make twice as many workgroups.
 constexpr uint32_t kSmallRows = 64;  // rows of a workgroup with RG = 2: the unit of the K-share rule
 
+constexpr float kPlaneRatio = 4096.0f;          // what the accumulators lack: the tiles hold hi and lo / 4096
 constexpr uint32_t kBlob = tile_blob_bytes(2);  // in memory and in LDS
 constexpr uint32_t kUnitAt = 32768u;            // unit[m]
 constexpr uint32_t kSumsAt = 32768u + 128u;     // xsum[g][m]
@@ -301,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + Codec<CODEC>::in_tail(108u)));
             const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
             const uint4 hm = *reinterpret_cast<const uint4*>(row_in_slot + 16u * half);  // hmask of these columns
-            v16f p_lo = zero, p_hi = zero;
+            v16f p = zero;
 #pragma unroll
             for (int bb = 0; bb < NB; bb++) {
                 const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
@@ -323,15 +326,15 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
                 const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
                           hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
-                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
-                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
-                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
             }
-            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
+            for (int r = 0; r < 16; r++) acc[r] = fmaf(p[r], sd[r], acc[r]);
             continue;
         }
         if constexpr (CODEC == kQ2_K) {
@@ -341,7 +344,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             const uint32_t dd = *reinterpret_cast<const uint32_t*>(row_in_slot + Codec<CODEC>::in_tail(80u));
             const float d_block = half_bits_to_float(dd & 0xffffu), dmin_block = half_bits_to_float(dd >> 16);
             const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
-            v16f p_lo = zero, p_hi = zero, m_lo = zero, m_hi = zero;
+            v16f p = zero, m = zero;  // products, and the sums of the activations times the minima
 #pragma unroll
             for (int bb = 0; bb < NB; bb++) {
                 const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
@@ -358,23 +361,23 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
                 const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
                           hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
-                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
-                m_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bm, m_lo, 0, 0, 0);
-                m_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bm, m_hi, 0, 0, 0);
-                p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
-                p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
-                m_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bm, m_lo, 0, 0, 0);
-                m_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bm, m_hi, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bm, m, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bm, m, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bm, m, 0, 0, 0);
+                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bm, m, 0, 0, 0);
             }
-            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
-            const v16f sm = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? dmin_block : 0.f,
+            const v16f sm = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * dmin_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
-                acc_min[r] = fmaf(fmaf(4096.0f, m_hi[r], m_lo[r]), sm[r], acc_min[r]);
+                acc[r] = fmaf(p[r], sd[r], acc[r]);
+                acc_min[r] = fmaf(m[r], sm[r], acc_min[r]);
             }
             continue;
         }
@@ -385,7 +388,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             // four accumulators, (X_lo, X_hi) x (s_lo, s_hi), joined once per stage.
             const float d_block = half_bits_to_float(*reinterpret_cast<const uint16_t*>(row_in_slot + Codec<CODEC>::in_tail(208u)));
             const float unit = *reinterpret_cast<const float*>(slot + kUnitAt + in_half * 4u);
-            v16f p_ll = zero, p_lh = zero, p_hl = zero, p_hh = zero;  // activation half, scale part
+            v16f p_l = zero, p_h = zero;  // by scale part; both activation halves go into one sum
 #pragma unroll
             for (int bb = 0; bb < NB; bb++) {
                 const uint32_t b = b_base + bb, n = b >> 2, t = b & 3u;
@@ -408,27 +411,24 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
                 const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
                           hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p_ll = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bl0, p_ll, 0, 0, 0);
-                p_lh = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bh0, p_lh, 0, 0, 0);
-                p_hl = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bl0, p_hl, 0, 0, 0);
-                p_hh = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bh0, p_hh, 0, 0, 0);
-                p_ll = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bl1, p_ll, 0, 0, 0);
-                p_lh = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bh1, p_lh, 0, 0, 0);
-                p_hl = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bl1, p_hl, 0, 0, 0);
-                p_hh = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bh1, p_hh, 0, 0, 0);
+                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bl0, p_l, 0, 0, 0);
+                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bh0, p_h, 0, 0, 0);
+                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bl0, p_l, 0, 0, 0);
+                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bh0, p_h, 0, 0, 0);
+                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bl1, p_l, 0, 0, 0);
+                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bh1, p_h, 0, 0, 0);
+                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bl1, p_l, 0, 0, 0);
+                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bh1, p_h, 0, 0, 0);
             }
-            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? d_block : 0.f,
+            const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float high = fmaf(16.0f, p_hh[r], p_hl[r]), low = fmaf(16.0f, p_lh[r], p_ll[r]);
-                acc[r] = fmaf(fmaf(4096.0f, high, low), sd[r], acc[r]);
-            }
+            for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(16.0f, p_h[r], p_l[r]), sd[r], acc[r]);
             continue;
         }
 
         const uint4 header = *reinterpret_cast<const uint4*>(row_in_slot);
-        const float d_block = half_bits_to_float(header.x & 0xffffu);
+        const float d_scaled = kPlaneRatio * half_bits_to_float(header.x & 0xffffu);
         const float dmin_block = half_bits_to_float(header.x >> 16);
         uint4 fifth = make_uint4(0u, 0u, 0u, 0u);  // Q5_K: qh of this lane half's sixteen columns
         if constexpr (CODEC == kQ5_K) fifth = *reinterpret_cast<const uint4*>(row_in_slot + 16u + 16u * half);
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             b0 = nibbles_times(w0, w1, sc2);
             b1 = nibbles_times(w2, w3, sc2);
         };
-        v16f p_lo = zero, p_hi = zero;
+        v16f p = zero;
         v8h b0, b1;
         prepare(0, b0, b1);
 #pragma unroll
@@ -477,10 +477,10 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
             const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
                       hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-            p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p_lo, 0, 0, 0);
-            p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p_hi, 0, 0, 0);
-            p_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p_lo, 0, 0, 0);
-            p_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p_hi, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
             if (bb + 1 < NB) {
                 v8h n0, n1;
                 prepare(bb + 1, n0, n1);
@@ -501,13 +501,13 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const float4 units = *reinterpret_cast<const float4*>(slot + kUnitAt + (8u * j + 4u * half) * 4u);
-            sd[4 * j + 0] = units.x * d_block;
-            sd[4 * j + 1] = units.y * d_block;
-            sd[4 * j + 2] = units.z * d_block;
-            sd[4 * j + 3] = units.w * d_block;
+            sd[4 * j + 0] = units.x * d_scaled;
+            sd[4 * j + 1] = units.y * d_scaled;
+            sd[4 * j + 2] = units.z * d_scaled;
+            sd[4 * j + 3] = units.w * d_scaled;
         }
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(4096.0f, p_hi[r], p_lo[r]), sd[r], acc[r]);
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(p[r], sd[r], acc[r]);
     }
 
     // ---- combine the sub-block shares, add bias, store ----

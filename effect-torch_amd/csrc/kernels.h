@@ -69,7 +69,7 @@ hipError_t quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 // limbs = 3: 24-bit fixed point in three balanced signed bytes, scale = max|x| / (127 * 65536).
 // limbs = 2 is the layout of gemm_h16: 24-bit fixed point per vector and 256-column stage in two
 // balanced 12-bit halves, each a half float:
-//   half l (0 low, 1 high), 8-column part c (0..31), vector m: 8 half floats at  l*16384 + c*512 + m*16
+//   half l (0: low / 4096, 1: high), 8-column part c (0..31), vector m: 8 half floats at  l*16384 + c*512 + m*16
 //   unit[m] f32 (max|x| / (2^23 - 1)) at  32768 + m*4
 //   xsum[sub-block g (0..7)][m] f32 at  32768 + 128 + g*128 + m*4
 // and padding up to 34 KiB.

@@ -20,8 +20,9 @@ __device__ __forceinline__ int dpp_i32(int v) {
 }
 
 // Activations for gemm_h16: per vector and 256-column stage, X = clamp(rint(x * (2^23 - 1) / amax))
-// as two balanced 12-bit halves, X = 4096 * hi + lo with lo in [-2048, 2047], both written as half
-// floats (exact); unit = amax / (2^23 - 1); xsum[g] = unit * (integer sum of X over sub-block g).
+// as two balanced 12-bit halves, X = 4096 * hi + lo with lo in [-2048, 2047], written as the half floats
+// hi and lo / 4096 (both exact: integers below 2^11 and a power of two), so that the two products of a
+// weight with them add up to X * w / 4096 in one accumulator; unit = amax / (2^23 - 1); xsum[g] = unit * (integer sum of X over sub-block g).
 // One wave per (vector, stage): lane `quad` holds columns 4 quad .. 4 quad + 3 of the stage. Blob
 // layout: see tile_blob_bytes() in kernels.h.
 __device__ __forceinline__ void quantize_halves_store(const float4& in, uint32_t v, uint32_t stage, uint32_t quad,
@@ -54,7 +55,7 @@ __device__ __forceinline__ void quantize_halves_store(const float4& in, uint32_t
         const int q = static_cast<int>(r);
         const int lo = ((q + 2048) & 4095) - 2048;
         total += q;
-        low.h[i] = static_cast<_Float16>(lo);
+        low.h[i] = static_cast<_Float16>(static_cast<float>(lo) * (1.0f / 4096.0f));
         high.h[i] = static_cast<_Float16>((q - lo) >> 12);  // exact: q - lo is a multiple of 4096
     }
     total += dpp_i32<0xB1>(total);   // the eight lanes of a 32-column sub-block
