@@ -49,7 +49,7 @@ constexpr int kThreads = 64 * (kConsumers + kLoaders);
 // RG = 32-row groups per workgroup (2 or 4): the eight consumers are RG groups of 8 / RG waves that
 // split the eight sub-blocks of a stage, RG each. Four groups (128 rows) halve the activation bytes a
 // workgroup copies per weight row; two groups (64 rows) make twice as many workgroups.
-constexpr uint32_t kSmallRows = 64;  // rows of a workgroup with RG = 2: the unit of the K-share rule
+// NARROW = at most sixteen vectors: see Operands.
 
 constexpr float kPlaneRatio = 4096.0f;          // what the accumulators lack: the tiles hold hi and lo / 4096
 constexpr uint32_t kBlob = tile_blob_bytes(2);  // in memory and in LDS
@@ -178,7 +178,46 @@ __device__ __forceinline__ v8h bytes_minus_times(uint32_t first, uint32_t second
     return u.all;
 }
 
-template <int CODEC, int RG, int AX, int AW>
+// The activation operands of sub-block b for one lane (matrix row i = in_half, K group = half), two per
+// 16-column chunk in the order they are contracted: low and high plane of vector i - or, NARROW (at most
+// sixteen vectors), one: rows 0-15 of the matrix are the high plane of vectors 0-15 and rows 16-31 their
+// low plane, so one instruction contracts both planes and the two halves of the result are added once
+// per stage.
+template <bool NARROW>
+struct Operands {
+    static constexpr int kPlanes = NARROW ? 1 : 2;
+    v8h x[2 * kPlanes];
+    __device__ __forceinline__ void load(const uint8_t* slot, uint32_t b, uint32_t half, uint32_t in_half) {
+        if constexpr (NARROW) {
+            const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + (in_half & 15u) * 16u +
+                                   (in_half < 16u ? 16384u : 0u);
+            x[0] = *reinterpret_cast<const v8h*>(chunk);
+            x[1] = *reinterpret_cast<const v8h*>(chunk + 512u);
+        } else {
+            const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
+            x[0] = *reinterpret_cast<const v8h*>(chunk);
+            x[1] = *reinterpret_cast<const v8h*>(chunk + 16384u);
+            x[2] = *reinterpret_cast<const v8h*>(chunk + 512u);
+            x[3] = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
+        }
+    }
+    // p += x * (b0 for the first chunk, b1 for the second)
+    __device__ __forceinline__ v16f contract(v8h b0, v8h b1, v16f p) const {
+#pragma unroll
+        for (int i = 0; i < kPlanes; i++) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[i], b0, p, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kPlanes; i++) p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[kPlanes + i], b1, p, 0, 0, 0);
+        return p;
+    }
+};
+// What a stage adds for accumulator r of a lane: the product sum itself, or both planes' halves of it.
+template <bool NARROW>
+__device__ __forceinline__ float stage_sum(const v16f& p, int r) {
+    if constexpr (NARROW) return p[r] + p[r + 8];
+    return p[r];
+}
+
+template <int CODEC, int RG, int AX, int AW, bool NARROW>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
     uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
@@ -282,14 +321,16 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const uint32_t wave_k = wave / kRowGroups;  // share of the stage's sub-blocks
     const uint32_t n0 = row0 + wave_n * 32u;
     const uint32_t m0 = tile * 32u;
-    float acc[16];
+    constexpr int R = NARROW ? 8 : 16;  // vectors a lane accumulates: m = 8 (r / 4) + 4 half + r % 4
+    float acc[R];
     v16f acc_min, zero;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-        acc[r] = 0.f;
         acc_min[r] = 0.f;
         zero[r] = 0.f;
     }
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
 
     for (uint32_t stage = 0; stage < stages; stage++) {
         __builtin_amdgcn_s_barrier();
@@ -322,19 +363,14 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const _Float16 sc_h = static_cast<_Float16>(static_cast<float>(sc));
                 const v2h sc2 = {sc_h, sc_h};
                 const v8h b0 = bytes_minus_times<4>(w0, w1, sc2), b1 = bytes_minus_times<4>(w2, w3, sc2);
-                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
-                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
-                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
-                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
+                Operands<NARROW> x;
+                x.load(slot, b, half, in_half);
+                p = x.contract(b0, b1, p);
             }
             const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[r] = fmaf(p[r], sd[r], acc[r]);
+            for (int r = 0; r < R; r++) acc[r] = fmaf(stage_sum<NARROW>(p, r), sd[r], acc[r]);
             continue;
         }
         if constexpr (CODEC == kQ2_K) {
@@ -357,27 +393,19 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const v2h sc2 = {sc_h, sc_h};
                 const v8h b0 = nibbles_times(w0, w1, sc2), b1 = nibbles_times(w2, w3, sc2);
                 const v8h bm = {mn_h, mn_h, mn_h, mn_h, mn_h, mn_h, mn_h, mn_h};
-                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
-                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
-                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
-                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
-                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bm, m, 0, 0, 0);
-                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bm, m, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
-                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bm, m, 0, 0, 0);
-                m = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bm, m, 0, 0, 0);
+                Operands<NARROW> x;
+                x.load(slot, b, half, in_half);
+                p = x.contract(b0, b1, p);
+                m = x.contract(bm, bm, m);
             }
             const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
             const v16f sm = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * dmin_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[r] = fmaf(p[r], sd[r], acc[r]);
-                acc_min[r] = fmaf(m[r], sm[r], acc_min[r]);
+            for (int r = 0; r < R; r++) {
+                acc[r] = fmaf(stage_sum<NARROW>(p, r), sd[r], acc[r]);
+                acc_min[r] = fmaf(stage_sum<NARROW>(m, r), sm[r], acc_min[r]);
             }
             continue;
         }
@@ -407,23 +435,16 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const v2h lo2 = {s_lo, s_lo}, hi2 = {s_hi, s_hi};
                 const v8h bl0 = nibbles_times<32>(w0, w1, lo2), bl1 = nibbles_times<32>(w2, w3, lo2);
                 const v8h bh0 = nibbles_times<32>(w0, w1, hi2), bh1 = nibbles_times<32>(w2, w3, hi2);
-                const uint8_t* chunk = slot + ((2u * b + half) * 2u) * 512u + in_half * 16u;
-                const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
-                const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
-                          hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bl0, p_l, 0, 0, 0);
-                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, bh0, p_h, 0, 0, 0);
-                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bl0, p_l, 0, 0, 0);
-                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, bh0, p_h, 0, 0, 0);
-                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bl1, p_l, 0, 0, 0);
-                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, bh1, p_h, 0, 0, 0);
-                p_l = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bl1, p_l, 0, 0, 0);
-                p_h = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, bh1, p_h, 0, 0, 0);
+                Operands<NARROW> x;
+                x.load(slot, b, half, in_half);
+                p_l = x.contract(bl0, bl1, p_l);
+                p_h = x.contract(bh0, bh1, p_h);
             }
             const v16f sd = __builtin_amdgcn_mfma_f32_32x32x2f32(half == 0 ? unit : 0.f, half == 0 ? kPlaneRatio * d_block : 0.f,
                                                                  zero, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[r] = fmaf(fmaf(16.0f, p_h[r], p_l[r]), sd[r], acc[r]);
+            for (int r = 0; r < R; r++)
+                acc[r] = fmaf(fmaf(16.0f, stage_sum<NARROW>(p_h, r), stage_sum<NARROW>(p_l, r)), sd[r], acc[r]);
             continue;
         }
 
@@ -473,23 +494,19 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         prepare(0, b0, b1);
 #pragma unroll
         for (int bb = 0; bb < NB; bb++) {
-            const uint8_t* chunk = slot + ((2u * (b_base + bb) + half) * 2u) * 512u + in_half * 16u;
-            const v8h lo0 = *reinterpret_cast<const v8h*>(chunk), lo1 = *reinterpret_cast<const v8h*>(chunk + 512u);
-            const v8h hi0 = *reinterpret_cast<const v8h*>(chunk + 16384u),
-                      hi1 = *reinterpret_cast<const v8h*>(chunk + 16384u + 512u);
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo0, b0, p, 0, 0, 0);
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi0, b0, p, 0, 0, 0);
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo1, b1, p, 0, 0, 0);
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi1, b1, p, 0, 0, 0);
+            Operands<NARROW> x;
+            x.load(slot, b_base + bb, half, in_half);
+            p = x.contract(b0, b1, p);
             if (bb + 1 < NB) {
                 v8h n0, n1;
                 prepare(bb + 1, n0, n1);
                 b0 = n0;
                 b1 = n1;
+                constexpr int kMatrix = 2 * Operands<NARROW>::kPlanes;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x002, 12, 0);  // twelve VALU
+                for (int i = 0; i < kMatrix; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 48 / kMatrix, 0);  // its share of the VALU work
                 }
             }
         }
@@ -497,9 +514,9 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         // four 16-byte LDS reads that every lane of a half shares, sixteen multiplications. (The same
         // products as a rank-1 v_mfma_f32_32x32x2f32 in the result layout cost 64 cycles of the matrix
         // pipe, and matrix and VALU instructions do not run side by side on this device.)
-        float sd[16];
+        float sd[R];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < R / 4; j++) {
             const float4 units = *reinterpret_cast<const float4*>(slot + kUnitAt + (8u * j + 4u * half) * 4u);
             sd[4 * j + 0] = units.x * d_scaled;
             sd[4 * j + 1] = units.y * d_scaled;
@@ -507,7 +524,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             sd[4 * j + 3] = units.w * d_scaled;
         }
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = fmaf(p[r], sd[r], acc[r]);
+        for (int r = 0; r < R; r++) acc[r] = fmaf(stage_sum<NARROW>(p, r), sd[r], acc[r]);
     }
 
     // ---- combine the sub-block shares, add bias, store ----
@@ -515,7 +532,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     float* exchange = reinterpret_cast<float*>(lds);  // [wave_k - 1][wave_n][16][64 lanes]
     if (wave_k > 0) {
 #pragma unroll
-        for (int r = 0; r < 16; r++)
+        for (int r = 0; r < R; r++)
             exchange[(((wave_k - 1u) * kRowGroups + wave_n) * 16 + r) * 64 + lane] = acc[r] - acc_min[r];
     }
     __syncthreads();
@@ -528,7 +545,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const uint32_t launch_row = row_tile * kRows + wave_n * 32u + in_half;  // among the rows of all members
     const uint64_t launch_rows = static_cast<uint64_t>(group.row_tiles) * kRows;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
+    for (int r = 0; r < R; r++) {
         float value = acc[r] - acc_min[r];
 #pragma unroll
         for (int k = 1; k < kSplit; k++) value += exchange[(((k - 1) * kRowGroups + wave_n) * 16 + r) * 64 + lane];
@@ -672,13 +689,29 @@ uint64_t gemm_h16_group_partial_bytes(int32_t codec, const uint64_t* rows, uint3
 }
 
 namespace {
-template <int CODEC, int RG, int AX, int AW>
-hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+// The launch that follows a contraction with K shares, unless the caller's next launch sums them itself.
+hipError_t sum_shares(const Group& group, const float* partials, uint32_t vectors, uint32_t k_splits, uint32_t tile_rows,
+                      hipStream_t stream, bool leave_shares, const GemmRotary* rotary) {
+    if (k_splits <= 1 || leave_shares) return hipSuccess;
+    if (rotary != nullptr) {
+        const uint64_t pairs = static_cast<uint64_t>(group.row_tiles) * tile_rows / 2 * vectors;
+        hipLaunchKernelGGL(reduce_group_rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0,
+                           stream, group, partials, vectors, k_splits, tile_rows, *rotary);
+    } else {
+        const uint64_t items = static_cast<uint64_t>(group.row_tiles) * tile_rows * vectors / 4;
+        hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
+                           group, partials, vectors, k_splits, tile_rows);
+    }
+    return hipGetLastError();
+}
+
+template <int CODEC, int RG, int AX, int AW, bool NARROW>
+hipError_t launch_tiles(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
                         uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares,
                         const GemmRotary* rotary) {
     using S = Shape<CODEC, RG, AX, AW>;
     static_assert(S::kLdsBytes <= 160 * 1024, "LDS of a gfx950 CU: 160 KiB, all of it dynamic here");
-    const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW>;
+    const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW, NARROW>;
     Group group = {};
     group.count = count;
     uint64_t row_tiles = 0;
@@ -706,16 +739,19 @@ hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(grid)), dim3(kThreads), S::kLdsBytes, stream, group, tiles,
                        vector_tiles, columns, vectors, k_splits, partials);
     if (hipError_t status = hipGetLastError()) return status;
-    if (k_splits > 1 && !leave_shares && rotary != nullptr) {
-        const uint64_t pairs = row_tiles * S::kRows / 2 * vectors;
-        hipLaunchKernelGGL(reduce_group_rotary_kernel, dim3(static_cast<uint32_t>((pairs + 255) / 256)), dim3(256), 0,
-                           stream, group, partials, vectors, k_splits, S::kRows, *rotary);
-    } else if (k_splits > 1 && !leave_shares) {
-        const uint64_t items = row_tiles * S::kRows * vectors / 4;
-        hipLaunchKernelGGL(reduce_group_kernel, dim3(static_cast<uint32_t>((items + 255) / 256)), dim3(256), 0, stream,
-                           group, partials, vectors, k_splits, S::kRows);
-    }
-    return hipGetLastError();
+    return sum_shares(group, partials, vectors, k_splits, S::kRows, stream, leave_shares, rotary);
+}
+
+// At most sixteen vectors: both planes of a vector ride in one matrix instruction (Operands<true>).
+template <int CODEC, int RG, int AX, int AW>
+hipError_t launch_group(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
+                        uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares,
+                        const GemmRotary* rotary) {
+    if (vectors <= 16u)
+        return launch_tiles<CODEC, RG, AX, AW, true>(members, count, tiles, partials, columns, vectors, k_splits, stream,
+                                                     leave_shares, rotary);
+    return launch_tiles<CODEC, RG, AX, AW, false>(members, count, tiles, partials, columns, vectors, k_splits, stream,
+                                                  leave_shares, rotary);
 }
 }  // namespace
 

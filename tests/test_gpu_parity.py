@@ -281,6 +281,61 @@ def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vecto
         close(got[:, :check_rows], want)
 
 
+@pytest.mark.parametrize("codec,vectors,rows,columns", [(oracle.Q4_K, 7, 100, 8192), (oracle.Q4_K, 16, 1000, 4096),
+                                                        (oracle.Q4_K, 17, 33, 9216), (oracle.Q5_K, 16, 520, 8448),
+                                                        (oracle.Q5_K, 12, 64, 14336), (oracle.Q6_K, 9, 300, 4096),
+                                                        (oracle.Q3_K, 16, 130, 2048), (oracle.Q2_K, 8, 14336, 4096),
+                                                        (oracle.Q4_K, 13, 28672, 4096)])
+def test_linear_up_to_sixteen_vectors_contract_both_planes_in_one_instruction(et, device, codec, vectors, rows, columns):
+    # batches of 7 ... 16 vectors: rows 0-15 of the matrix instruction's activation operand are the
+    # high plane of the vectors and rows 16-31 their low plane, added once per stage - every K-quant,
+    # 64- and 128-row tiles, with and without K shares, rows that end inside a tile (17 vectors: the
+    # ordinary tile beside them)
+    rng = np.random.default_rng(7 * rows + columns + vectors)
+    weight = synth.random_weight(codec, rows, columns, rng)
+    x = synth.random_activations(vectors, columns, rng)
+    bias = rng.standard_normal(rows).astype(np.float32)
+    plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
+                                  torch.zeros(rows), et.GgmlQuant(codec), (rows, columns), et.ActivationMode.F32)
+    assert plan.kernel.startswith("quantize_halves+gemm_h16")
+    got = run_linear(et, device, codec, rows, columns, x, weight, bias, et.ActivationMode.F32)
+    again = run_linear(et, device, codec, rows, columns, x, weight, bias, et.ActivationMode.F32)
+    assert np.array_equal(got, again)
+    begin = max(0, rows - 200)  # the last rows (a ragged tile where there is one) against the oracle
+    want = oracle.linear_rows(codec, rows, columns, x, weight, bias, begin, rows)[:, begin:]
+    close(got[:, begin:], want)
+    start = rows - min(rows, 40)  # and against exact arithmetic
+    exact = x.astype(np.float64) @ oracle.decode_rows(codec, weight[start:], columns).astype(np.float64).T + bias[start:]
+    close(got[:, start:], exact, oracle_noise=0)
+
+
+def test_group_launch_of_fewer_than_seventeen_vectors(et, device):
+    # two matrices behind one prepared input of 12 vectors (the narrow tile) with 8192 columns: tiles of
+    # both members in one launch, the first member ending inside a tile; bias and residual ride on the
+    # launch that sums the K shares
+    rng = np.random.default_rng(4242)
+    columns, vectors, sizes = 8192, 12, (100, 64)
+    x_host = synth.random_activations(vectors, columns, rng)
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors, rows == 64) for rows in sizes]
+    group = et.LinearGroup(plans)
+    assert group.workspace_bytes > 0  # K shares
+    prepared = torch.empty(plans[0].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[0].prepare_input(to_dev(x_host, device), prepared)
+    host_weights = [synth.random_weight(oracle.Q4_K, rows, columns, rng) for rows in sizes]
+    weights = [to_dev(w, device) for w in host_weights]
+    bias_host = rng.standard_normal(64).astype(np.float32)
+    residual_host = rng.standard_normal((vectors, 100)).astype(np.float32)
+    workspace = torch.empty(group.workspace_bytes, dtype=torch.uint8, device=device)
+    ys = [torch.full((vectors, rows), float("nan"), device=device) for rows in sizes]
+    group.enqueue_prepared(prepared, weights, ys, workspace, biases=[None, to_dev(bias_host, device)],
+                           residuals=[to_dev(residual_host, device), None])
+    for index, rows in enumerate(sizes):
+        want = oracle.linear_rows(oracle.Q4_K, rows, columns, x_host, host_weights[index],
+                                  bias_host if index == 1 else None)
+        got = ys[index].cpu().numpy()
+        close(got - residual_host if index == 0 else got, want)
+
+
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q8_0, oracle.Q4_0, oracle.Q6_K])
 def test_linear_unit_vectors_select_decoded_weights(et, device, codec):
     rng = np.random.default_rng(800 + codec)
