@@ -35,6 +35,7 @@ from .kv_cache import (  # noqa: F401
     KvLayer,
     kv_attention_into,
     kv_attention_kernel,
+    kv_attention_projected_into,
     kv_attention_status_check,
     kv_attention_workspace,
     kv_attention_workspace_bytes,

@@ -64,6 +64,37 @@ class EtRotaryAfter(ctypes.Structure):
     ]
 
 
+class EtGroupShares(ctypes.Structure):
+    """``et_group_shares`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("shares", ctypes.c_void_p),
+        ("count", ctypes.c_uint32),
+        ("vectors", ctypes.c_uint64),
+        ("launch_rows", ctypes.c_uint64),
+        ("first_row", ctypes.c_uint64 * 4),
+    ]
+
+
+class EtKvProjected(ctypes.Structure):
+    """``et_kv_projected`` of include/et_hip.h."""
+
+    _fields_ = [
+        ("shares", EtGroupShares),
+        ("q_member", ctypes.c_uint32),
+        ("k_member", ctypes.c_uint32),
+        ("v_member", ctypes.c_uint32),
+        ("q_bias", ctypes.c_void_p),
+        ("k_bias", ctypes.c_void_p),
+        ("v_bias", ctypes.c_void_p),
+        ("offsets", ctypes.c_void_p),
+        ("offsets_len", ctypes.c_uint64),
+        ("theta", ctypes.c_double),
+        ("sign", ctypes.c_double),
+        ("layout", ctypes.c_int32),
+    ]
+
+
 class EtKvLayer(ctypes.Structure):
     """``et_kv_layer`` of include/et_hip.h."""
 
@@ -138,6 +169,9 @@ SIGNATURES = {
     "et_hip_linear_enqueue_prepared": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_linear_enqueue_prepared_group_then_rotary": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp,
                                                                         _u64, ctypes.POINTER(EtRotaryAfter), _vp, _vp]),
+    "et_hip_linear_group_shares_layout": (ctypes.c_int, [_vp, ctypes.c_uint32, ctypes.POINTER(EtGroupShares)]),
+    "et_hip_linear_enqueue_prepared_group_shares": (ctypes.c_int, [_vp, ctypes.c_uint32, _vp, _vp, _vp, _u64,
+                                                                   ctypes.POINTER(EtGroupShares), _vp, _vp]),
     "et_hip_linear_enqueue_prepared_then_norm": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _vp, _vp, _i32,
                                                                 ctypes.c_double, _vp, _u64, _vp, _vp]),
     "et_hip_embedding_requirements": (ctypes.c_int, [_T, _T, _i32, _u64, _u64, _PP]),
@@ -152,6 +186,8 @@ SIGNATURES = {
     "et_hip_kv_attention_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp, _vp]),
     "et_hip_kv_attention_prepared_into": (ctypes.c_int, [_KV, _T, _T, _T, ctypes.c_double, _u64, _T, _vp, _u64, _vp, _vp,
                                                          _vp, _u64, _vp, _vp]),
+    "et_hip_kv_attention_projected_into": (ctypes.c_int, [_KV, ctypes.POINTER(EtKvProjected), ctypes.c_double, _u64, _T, _vp,
+                                                          _u64, _vp, _vp, _vp, _u64, _vp, _vp]),
     "et_hip_kv_attention_status_check": (ctypes.c_int, [_KV, _u64, _vp]),
     "et_hip_kv_attention_kernel": (ctypes.c_char_p, [_KV, _u64, _u64]),
     "et_hip_kv_commit": (ctypes.c_int, [_KV, _vp]),

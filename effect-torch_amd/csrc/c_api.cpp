@@ -282,6 +282,23 @@ int et_hip_linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const
     });
 }
 
+int et_hip_linear_group_shares_layout(const et_linear_plan* const* plans, uint32_t count, et_group_shares* layout) {
+    return guarded([&](std::string* error) -> int {
+        return et::quantized::linear_enqueue_prepared_group_shares(plans, count, nullptr, nullptr, nullptr, 0, layout,
+                                                                   false, nullptr, nullptr, error);
+    });
+}
+
+int et_hip_linear_enqueue_prepared_group_shares(const et_linear_plan* const* plans, uint32_t count,
+                                                const void* prepared, const uint8_t* const* weights,
+                                                void* workspace, uint64_t workspace_bytes, et_group_shares* layout,
+                                                void* stream, const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        return et::quantized::linear_enqueue_prepared_group_shares(plans, count, prepared, weights, workspace,
+                                                                   workspace_bytes, layout, true, stream, cancel, error);
+    });
+}
+
 int et_hip_linear_enqueue_prepared_then_norm(const et_linear_plan* plan, const void* prepared,
                                              const uint8_t* weight, const float* bias, const float* residual,
                                              float* y, void* workspace, uint64_t workspace_bytes,
@@ -453,6 +470,26 @@ int et_hip_kv_attention_prepared_into(const et_kv_layer* layer, const et_tensor*
         }
         return et::kv::attention_into(*layer, qv, kv, vv, scale, window, dst, workspace, workspace_bytes, status,
                                       stream, cancel, error, consumer, prepared, prepared_bytes);
+    });
+}
+
+int et_hip_kv_attention_projected_into(const et_kv_layer* layer, const et_kv_projected* projected, double scale,
+                                       uint64_t window, const et_tensor* destination, void* workspace,
+                                       uint64_t workspace_bytes, void* status, const et_linear_plan* consumer,
+                                       void* prepared, uint64_t prepared_bytes, void* stream,
+                                       const volatile int32_t* cancel) {
+    return guarded([&](std::string* error) -> int {
+        if (layer == nullptr || projected == nullptr) {
+            *error = "kv attention: layer or projection is NULL";
+            return ET_ERR_INVALID;
+        }
+        TensorView dst;
+        if (!TensorView::from_c(destination, &dst, error)) {
+            *error = "kv attention: " + *error;
+            return ET_ERR_INVALID;
+        }
+        return et::kv::attention_projected_into(*layer, *projected, scale, window, dst, workspace, workspace_bytes,
+                                                status, stream, cancel, error, consumer, prepared, prepared_bytes);
     });
 }
 

@@ -179,6 +179,22 @@ enum : uint32_t {
     kKvOverDeclared = 4,  // value = cursor + advance, above the caller's max_context
     kKvBlockOutside = 5,  // value = physical row
 };
+// q, k and v of a decode step as the unsummed K shares of the group launch that projected them
+// (gemm_h16_group with leave_shares): share s of vector m, launch row n at
+// shares[(s * vectors + m) * launch_rows + n]; the projections start at launch rows q_row, k_row, v_row.
+struct KvProjected {
+    const float* shares;  // null: q, k, v arrive as tensors
+    uint32_t count, vectors;
+    uint64_t launch_rows;
+    uint32_t q_row, k_row, v_row;
+    const float* q_bias;  // [query_heads * width], or null
+    const float* k_bias;  // [kv_heads * width], or null
+    const float* v_bias;
+    const uint32_t* offsets;  // rotary positions of q and k: 1 or `vectors` device words
+    uint32_t offsets_len;
+    int32_t interleaved;
+    double theta, sign;
+};
 struct KvAttention {
     void* k_slab;
     void* v_slab;
@@ -202,6 +218,10 @@ struct KvAttention {
     // gemm_h16's tiles (quantize_tiles with two halves) - by the attention kernel itself where one
     // workgroup holds whole 256-column stages of a row, by a quantiser launch otherwise.
     uint8_t* prepared = nullptr;
+    // Optional (tokens == 1, a shape the streaming kernel takes): q, k, v above are unused; every workgroup
+    // sums the shares of the rows it needs, adds the biases and rotates q and k - the bytes of
+    // reduce_group_rotary_kernel - before it attends (kv_attention returns hipErrorInvalidValue for other shapes).
+    KvProjected projected = {};
 };
 struct KvLaunchShape {
     bool streaming;

@@ -26,6 +26,7 @@
 #include <cmath>
 #include <type_traits>
 
+#include "decode_math.h"
 #include "et_hip.h"
 #include "kernels.h"
 #include "quantize_halves.h"
@@ -65,6 +66,7 @@ struct KvArgs {
     float scale_log2;  // scale * log2(e)
     uint8_t* prepared;       // see KvAttention::prepared; null = none, or a quantiser launch follows
     uint32_t vector_tiles;   // of the prepared activations: ceil(batch / 32)
+    KvProjected projected;   // see KvAttention::projected; shares == null: q, k, v above
 };
 
 struct Span {
@@ -484,6 +486,42 @@ __device__ __forceinline__ void merge_splits(const KvArgs& a, uint64_t query, ui
 // served from the same K / V registers. WAVES = 8 when the launch has enough rows of queries to give
 // every compute unit a workgroup without splitting the context (no partial records, no merge
 // launch), else 4.
+// q of the workgroup's G heads, then k and v of its kv head, for one slot, from the K shares of the
+// projection: the sums in share order, the bias, the rotary pairs of q and k - what
+// reduce_group_rotary_kernel (gemm_h16.hip) stores. out: [(G + 2)][width] floats in LDS.
+template <int G>
+__device__ void project_rows(const KvArgs& a, uint32_t slot, uint32_t head0, uint32_t kv_head, float* out,
+                             uint32_t threads) {
+    const KvProjected& s = a.projected;
+    const uint32_t width = a.width, half = width / 2;
+    const uint64_t share_stride = s.launch_rows * s.vectors;
+    const auto summed = [&](uint32_t first_row, const float* bias, uint32_t row) {
+        const float* first = s.shares + static_cast<uint64_t>(slot) * s.launch_rows + first_row + row;
+        float total = first[0];
+        for (uint32_t k = 1; k < s.count; k++) total += first[k * share_stride];
+        return bias != nullptr ? total + bias[row] : total;
+    };
+    const uint32_t offset = s.offsets_len == 1 ? s.offsets[0] : s.offsets[slot];
+    const uint32_t rotated = (G + 1) * half;  // the pairs of the G query heads, then of the key head
+    for (uint32_t item = threadIdx.x; item < rotated + width; item += threads) {
+        if (item < rotated) {
+            const uint32_t h = item / half, index = item - h * half;
+            const uint32_t head = h < G ? head0 + h : kv_head;
+            const uint32_t first_row = h < G ? s.q_row : s.k_row;
+            const float* bias = h < G ? s.q_bias : s.k_bias;
+            const uint32_t lo = s.interleaved ? 2u * index : index, hi = s.interleaved ? lo + 1u : lo + half;
+            float value_lo = summed(first_row, bias, head * width + lo);
+            float value_hi = summed(first_row, bias, head * width + hi);
+            rotate_pair(value_lo, value_hi, offset, 0u, index, width, s.theta, s.sign, value_lo, value_hi);
+            out[h * width + lo] = value_lo;
+            out[h * width + hi] = value_hi;
+        } else {
+            const uint32_t d = item - rotated;
+            out[(G + 1) * width + d] = summed(s.v_row, s.v_bias, kv_head * width + d);
+        }
+    }
+}
+
 template <typename T, int LPT, int G, int U, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
     constexpr int kWaves = WAVES;
@@ -496,6 +534,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
     __shared__ float merge_m[GROUPS][G];
     __shared__ float merge_l[GROUPS][G];
     __shared__ float merge_acc[GROUPS][G][LPT * DPL + 4];
+    __shared__ __attribute__((aligned(16))) float projected[(G + 2) * LPT * DPL];  // q of the G heads, k, v: only with a.projected.shares
 
     uint32_t index = blockIdx.x;
     const uint32_t split = index % a.splits;
@@ -536,15 +575,22 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
             rows_of_block[i] = row >= a.max_tokens ? kNoBlock : static_cast<uint32_t>(row);
         }
     }
+    const bool from_shares = a.projected.shares != nullptr;  // one token per slot
+    if (from_shares) project_rows<G>(a, slot, head0, kv_head, projected, kThreads);
     __syncthreads();
 
     float q[G][DPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        const float* source = a.q + ((static_cast<uint64_t>(slot) * a.query_heads + head0 + g) * a.tokens + token) *
-                                        a.width + sub * DPL;
+        if (from_shares) {
 #pragma unroll
-        for (int d = 0; d < DPL; d++) q[g][d] = source[d] * a.scale_log2;
+            for (int d = 0; d < DPL; d++) q[g][d] = projected[g * (LPT * DPL) + sub * DPL + d] * a.scale_log2;
+        } else {
+            const float* source = a.q + ((static_cast<uint64_t>(slot) * a.query_heads + head0 + g) * a.tokens + token) *
+                                            a.width + sub * DPL;
+#pragma unroll
+            for (int d = 0; d < DPL; d++) q[g][d] = source[d] * a.scale_log2;
+        }
     }
     // Softmax state: per query head in every lane (rows of 8 lanes), or spread over the 16 lanes of a
     // row, lane r holding head r / (16 / G) (see attend_step_scatter).
@@ -612,8 +658,8 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
         const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + kv_head) * a.tokens + arrival) *
                                     a.width + sub * DPL;
         Piece<T> kp[1], vp[1];
-        kp[0].template from_input<LPT>(a.k + source);
-        vp[0].template from_input<LPT>(a.v + source);
+        kp[0].template from_input<LPT>(from_shares ? projected + G * (LPT * DPL) + sub * DPL : a.k + source);
+        vp[0].template from_input<LPT>(from_shares ? projected + (G + 1) * (LPT * DPL) + sub * DPL : a.v + source);
         if (live[0] && arrival == token && chunk == 0) {
             const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
             const uint32_t row = base + within_block(a, position);
@@ -966,6 +1012,8 @@ hipError_t kv_attention(const KvAttention& p, void* workspace, hipStream_t strea
                              (static_cast<uint64_t>(streaming_group(p)) * p.width) % 256 == 0;
     a.prepared = fused_tiles ? p.prepared : nullptr;
     a.vector_tiles = (p.batch + 31u) / 32u;
+    a.projected = p.projected;
+    if (p.projected.shares != nullptr && !(shape.streaming && p.tokens == 1)) return hipErrorInvalidValue;
     const auto finish = [&](hipError_t error) -> hipError_t {
         if (error != hipSuccess || p.prepared == nullptr || fused_tiles || p.batch == 0) return error;
         const uint64_t columns = static_cast<uint64_t>(p.query_heads) * p.width;

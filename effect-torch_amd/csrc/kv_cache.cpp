@@ -93,7 +93,8 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
                    const quantized::TensorView& v, double scale, uint64_t window,
                    const quantized::TensorView& destination, void* workspace, uint64_t workspace_bytes,
                    void* status, void* stream, const volatile int32_t* cancel, std::string* error,
-                   const et_linear_plan* consumer, void* prepared, uint64_t prepared_bytes) {
+                   const et_linear_plan* consumer, void* prepared, uint64_t prepared_bytes,
+                   const et_kv_projected* projected) {
     // napi/mod.rs:3331-3344
     const size_t rank = q.shape.size();
     if (rank < 4 || q.dtype != ET_DTYPE_F32 || k.dtype != ET_DTYPE_F32 || v.dtype != ET_DTYPE_F32 ||
@@ -130,8 +131,8 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
     if (batch == 0) return ET_OK;
     if (status == nullptr) return fail(error, ET_ERR_INVALID, "kv attention: status block is NULL");
     if (layer.k_slab == nullptr || layer.v_slab == nullptr || layer.block_table == nullptr ||
-        layer.cursors == nullptr || layer.advances == nullptr || q.data == nullptr || k.data == nullptr ||
-        v.data == nullptr || destination.data == nullptr)
+        layer.cursors == nullptr || layer.advances == nullptr || destination.data == nullptr ||
+        (projected == nullptr && (q.data == nullptr || k.data == nullptr || v.data == nullptr)))
         return fail(error, ET_ERR_INVALID, "kv attention: NULL device pointer");
     if (layer.slab_dtype == ET_DTYPE_U8 &&
         (layer.k_scales == nullptr || layer.v_scales == nullptr || reinterpret_cast<uintptr_t>(layer.k_scales) % 4 != 0 ||
@@ -145,9 +146,38 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
     p.cursors = layer.cursors;
     p.advances = layer.advances;
     p.window = static_cast<uint32_t>(window);
-    p.q = static_cast<const float*>(q.data) + q.offset;
-    p.k = static_cast<const float*>(k.data) + k.offset;
-    p.v = static_cast<const float*>(v.data) + v.offset;
+    if (projected == nullptr) {
+        p.q = static_cast<const float*>(q.data) + q.offset;
+        p.k = static_cast<const float*>(k.data) + k.offset;
+        p.v = static_cast<const float*>(v.data) + v.offset;
+    } else {
+        // the projections as the group launch left them: shares of rows [q | k | v], each from its own first row
+        const et_group_shares& s = projected->shares;
+        const uint64_t q_rows = query_heads * width, kv_rows = kv_heads * width;
+        if (tokens != 1) return fail(error, ET_ERR_UNSUPPORTED, "kv attention: projections as K shares take one token per slot");
+        if (s.shares == nullptr || reinterpret_cast<uintptr_t>(s.shares) % 4 != 0 || s.count == 0 || s.count > kLimit ||
+            s.vectors != batch || s.launch_rows > kLimit || projected->q_member >= ET_HIP_LINEAR_GROUP_MOST ||
+            projected->k_member >= ET_HIP_LINEAR_GROUP_MOST || projected->v_member >= ET_HIP_LINEAR_GROUP_MOST)
+            return fail(error, ET_ERR_INVALID, "kv attention: the K shares do not describe [" + std::to_string(batch) +
+                                                   "] projected vectors");
+        const uint64_t q_row = s.first_row[projected->q_member], k_row = s.first_row[projected->k_member],
+                       v_row = s.first_row[projected->v_member];
+        if (q_row + q_rows > s.launch_rows || k_row + kv_rows > s.launch_rows || v_row + kv_rows > s.launch_rows)
+            return fail(error, ET_ERR_INVALID, "kv attention: the projections do not fit the rows of the shares");
+        if (projected->layout != ET_ROTARY_HALF_SPLIT && projected->layout != ET_ROTARY_INTERLEAVED_PAIRS)
+            return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(projected->layout));
+        if (width % 2 != 0)
+            return fail(error, ET_ERR_UNSUPPORTED, "rotary: expected a float rank >= 2 tensor with even head dimension");
+        if (projected->offsets_len != 1 && projected->offsets_len != batch)
+            return fail(error, ET_ERR_UNSUPPORTED, "rotary embedding: " + std::to_string(projected->offsets_len) +
+                                                       " offsets for batch " + std::to_string(batch));
+        if (projected->offsets == nullptr) return fail(error, ET_ERR_INVALID, "rotary: NULL device pointer");
+        p.projected = KvProjected{s.shares, s.count, static_cast<uint32_t>(batch), s.launch_rows,
+                                  static_cast<uint32_t>(q_row), static_cast<uint32_t>(k_row), static_cast<uint32_t>(v_row),
+                                  projected->q_bias, projected->k_bias, projected->v_bias, projected->offsets,
+                                  static_cast<uint32_t>(projected->offsets_len),
+                                  projected->layout == ET_ROTARY_INTERLEAVED_PAIRS ? 1 : 0, projected->theta, projected->sign};
+    }
     p.out = const_cast<float*>(static_cast<const float*>(destination.data)) + destination.offset;
     p.scale = scale;
     p.status = status;
@@ -170,6 +200,8 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
         p.prepared = static_cast<uint8_t*>(prepared);
     }
     const KvLaunchShape shape = kv_attention_shape(p);
+    if (projected != nullptr && !shape.streaming)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: this geometry's kernel takes q, k and v as tensors");
     if (shape.streaming) {
         // the streaming kernel moves 16 bytes per lane
         const auto misaligned = [](const void* pointer) { return reinterpret_cast<uintptr_t>(pointer) % 16 != 0; };
@@ -187,6 +219,28 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
     if (launched != hipSuccess)
         return fail(error, ET_ERR_EXECUTION, std::string("kv attention: HIP error: ") + hipGetErrorString(launched));
     return ET_OK;
+}
+
+int attention_projected_into(const et_kv_layer& layer, const et_kv_projected& projected, double scale, uint64_t window,
+                             const quantized::TensorView& destination, void* workspace, uint64_t workspace_bytes,
+                             void* status, void* stream, const volatile int32_t* cancel, std::string* error,
+                             const et_linear_plan* consumer, void* prepared, uint64_t prepared_bytes) {
+    // q is the destination's shape; k and v that of the layer's heads, one token each
+    const size_t rank = destination.shape.size();
+    if (rank < 4 || destination.dtype != ET_DTYPE_F32)
+        return fail(error, ET_ERR_UNSUPPORTED, "kv attention: expected matching rank-4-or-higher f32 tensors");
+    quantized::TensorView q = destination, k = destination;
+    q.data = nullptr;
+    k.data = nullptr;
+    k.offset = 0;
+    k.shape[rank - 3] = layer.kv_heads;
+    uint64_t stride = 1;
+    for (size_t d = rank; d-- > 0;) {  // contiguous
+        k.strides[d] = stride;
+        stride *= k.shape[d];
+    }
+    return attention_into(layer, q, k, k, scale, window, destination, workspace, workspace_bytes, status, stream, cancel,
+                          error, consumer, prepared, prepared_bytes, &projected);
 }
 
 int status_check(const et_kv_layer& layer, uint64_t tokens, const void* status_host, std::string* error) {

@@ -537,6 +537,48 @@ int linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans
     return ET_OK;
 }
 
+int linear_enqueue_prepared_group_shares(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                         const uint8_t* const* weights, void* workspace, uint64_t workspace_bytes,
+                                         et_group_shares* layout, bool launch, void* stream,
+                                         const volatile int32_t* cancel, std::string* error) {
+    if (int rc = check_group(plans, count, error)) return rc;
+    if (layout == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: NULL layout");
+    static_assert(ET_HIP_LINEAR_GROUP_MOST == kGemmGroupMost, "the header's bound is the kernel's");
+    uint64_t rows[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) rows[i] = plans[i]->rows;
+    const uint64_t vectors = plans[0]->vectors;
+    const GemmGroupGeometry g = gemm_h16_group_geometry(plans[0]->codec, rows, count, plans[0]->columns, vectors);
+    *layout = et_group_shares{};
+    layout->count = g.k_splits;
+    layout->vectors = vectors;
+    layout->launch_rows = g.row_tiles * g.tile_rows;
+    uint64_t first = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        layout->first_row[i] = first;
+        first += (rows[i] + g.tile_rows - 1) / g.tile_rows * g.tile_rows;
+    }
+    if (!launch) return ET_OK;
+    if (g.k_splits <= 1) return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: this group does not share K over workgroups");
+    if (weights == nullptr || prepared == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+    GemmMember members[kGemmGroupMost];
+    for (uint32_t i = 0; i < count; i++) {
+        if (weights[i] == nullptr) return fail(error, ET_ERR_INVALID, "quantized_linear: NULL device pointer");
+        members[i] = GemmMember{weights[i], nullptr, nullptr, nullptr, plans[i]->rows};
+    }
+    if (cancel != nullptr && *cancel != 0) return fail(error, ET_ERR_CANCELLED, "operation aborted");
+    const uint64_t need = group_partial_bytes(plans, count);
+    if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(error, ET_ERR_EXECUTION, "quantized_linear: workspace of " + std::to_string(workspace_bytes) +
+                                                 " bytes is smaller than the " + std::to_string(need) + " the group needs");
+    layout->shares = static_cast<const float*>(workspace);
+    if (vectors == 0) return ET_OK;
+    if (hipError_t status = gemm_h16_group(plans[0]->codec, members, count, static_cast<const uint8_t*>(prepared),
+                                           static_cast<float*>(workspace), plans[0]->columns, vectors, as_stream(stream),
+                                           true))
+        return hip_failure(error, "quantized_linear", status);
+    return ET_OK;
+}
+
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                             const volatile int32_t* cancel, std::string* error) {

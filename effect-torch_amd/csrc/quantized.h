@@ -120,6 +120,12 @@ int linear_enqueue_prepared_group_then_rotary(const et_linear_plan* const* plans
                                               const float* const* residuals, float* const* ys, void* workspace,
                                               uint64_t workspace_bytes, const et_rotary_after& rotary, void* stream,
                                               const volatile int32_t* cancel, std::string* error);
+// The group's launch without the one that sums its K shares (see et_hip_linear_enqueue_prepared_group_shares
+// in et_hip.h); prepared == nullptr: the layout only.
+int linear_enqueue_prepared_group_shares(const et_linear_plan* const* plans, uint32_t count, const void* prepared,
+                                         const uint8_t* const* weights, void* workspace, uint64_t workspace_bytes,
+                                         et_group_shares* layout, bool launch, void* stream,
+                                         const volatile int32_t* cancel, std::string* error);
 int linear_enqueue_prepared(const et_linear_plan& plan, const void* prepared, const uint8_t* weight, const float* bias,
                             const float* residual, float* y, void* workspace, uint64_t workspace_bytes, void* stream,
                             const volatile int32_t* cancel, std::string* error);

@@ -23,7 +23,8 @@ import torch
 
 from .decode_ops import (RotaryLayout, add_into, gather_rows_into, greedy_tokens, greedy_workspace_bytes,
                          rms_norm_into, rotary_into, rotary_pair_into, silu_mul_into)
-from .kv_cache import KvLayer, kv_attention_into, kv_attention_workspace, kv_commit
+from .kv_cache import (KvLayer, kv_attention_into, kv_attention_kernel, kv_attention_projected_into,
+                       kv_attention_workspace, kv_commit)
 from .quantized import ActivationMode, GgmlQuant, LinearGroup, RawLinear
 
 LINEARS = ("wq", "wk", "wv", "wo", "gate", "up", "down")
@@ -89,6 +90,9 @@ class LlamaDecoder:
             self.ffn_group = LinearGroup([plans["gate"], plans["up"]])
             self.group_ws = u8(max(self.qkv_group.workspace_bytes, self.ffn_group.workspace_bytes))
         self.kv_ws = kv_attention_workspace(kv[0], shape.heads, 1)
+        # q / k / v can stay the K shares of their group launch when the attention kernel is the one that sums them
+        self.project_in_attention = (self.on_the_fly and self.qkv_group.shares_layout().count > 1 and
+                                     kv_attention_kernel(kv[0], shape.heads, 1).split("+")[0] == "kv_attend")
         self.greedy_ws = u8(greedy_workspace_bytes(slots, shape.vocab))
         kv_width = shape.kv_heads * shape.head_dim
         self.x, self.h = f32(slots, shape.hidden), f32(slots, shape.hidden)
@@ -123,13 +127,24 @@ class LlamaDecoder:
         if self.on_the_fly:
             if not prepared_by_previous:
                 plans["wq"].prepare_input_rms_norm(x, self.norms[index][0], eps, self.shared_hidden)
-            # q and k rotated at the slots' cursors in the launch that sums the group's K shares
-            self.qkv_group.enqueue_prepared_then_rotary(self.shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v],
-                                                        self.group_ws, (0, 1), self.cursors, theta, 1.0, half_split, width)
-            # the attention kernel quantises its result for Wo in its epilogue
-            self.status.append(kv_attention_into(kvl, q4, k4, v4, self.scale, None, attended4, workspace=self.kv_ws,
-                                                 synchronize=False, prepared_for=plans["wo"],
-                                                 prepared=self.shared_attended))
+            if self.project_in_attention:
+                # the attention kernel sums the group's K shares, rotates q and k at the slots' cursors,
+                # appends, attends and quantises its result for Wo
+                shares = self.qkv_group.enqueue_prepared_shares(self.shared_hidden, [w["wq"], w["wk"], w["wv"]],
+                                                                self.group_ws)
+                self.status.append(kv_attention_projected_into(
+                    kvl, shares, (0, 1, 2), (None, None, None), self.cursors, theta, 1.0, half_split, self.scale, None,
+                    attended4, workspace=self.kv_ws, synchronize=False, prepared_for=plans["wo"],
+                    prepared=self.shared_attended))
+            else:
+                # q and k rotated at the slots' cursors in the launch that sums the group's K shares
+                self.qkv_group.enqueue_prepared_then_rotary(self.shared_hidden, [w["wq"], w["wk"], w["wv"]], [q, k, v],
+                                                            self.group_ws, (0, 1), self.cursors, theta, 1.0, half_split,
+                                                            width)
+                # the attention kernel quantises its result for Wo in its epilogue
+                self.status.append(kv_attention_into(kvl, q4, k4, v4, self.scale, None, attended4, workspace=self.kv_ws,
+                                                     synchronize=False, prepared_for=plans["wo"],
+                                                     prepared=self.shared_attended))
             # x += attended Wo, then the ffn norm inside the quantiser, in the launch that sums Wo's K shares
             plans["wo"].enqueue_prepared_then_norm(self.shared_attended, w["wo"], None, x, self.linear_ws, plans["gate"],
                                                    self.norms[index][1], eps, self.shared_hidden, residual=x)

@@ -9,7 +9,7 @@ host in the reference.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -132,4 +132,41 @@ def kv_attention_into(layer: KvLayer, q: torch.Tensor, k: torch.Tensor, v: torch
     if not synchronize:
         return status
     kv_attention_status_check(layer, tokens, status)
+    return None
+
+
+def kv_attention_projected_into(layer: KvLayer, shares, members: Sequence[int],
+                                biases: Sequence[Optional[torch.Tensor]], offsets: torch.Tensor, theta: float,
+                                sign: float, layout: int, scale: float, window: Optional[int],
+                                destination: torch.Tensor, *, workspace: Optional[torch.Tensor] = None,
+                                cancelled: Optional[CancellationFlag] = None, stream=None, synchronize: bool = True,
+                                prepared_for=None, prepared: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """:func:`kv_attention_into` for one token per slot whose q, k and v are still the unsummed K
+    shares of their projections (``shares``: what ``LinearGroup.enqueue_prepared_shares`` returned;
+    ``members``: which plans of that group are q, k and v; ``biases``: theirs, or None): the attention
+    launch sums the rows it needs, adds the biases and rotates q and k at ``offsets`` before it attends
+    (``et_hip_kv_attention_projected_into``). ``destination``: ``[.., query_heads, 1, head_dim]``."""
+    struct = layer.struct()
+    heads = destination.shape[-3] if destination.dim() >= 3 else 0
+    if offsets.dtype not in (torch.uint32, torch.int32) or not offsets.is_contiguous():
+        raise ValueError("rotary offsets must be a contiguous u32 device tensor")
+    if workspace is None:
+        need = int(N.lib().et_hip_kv_attention_workspace_bytes(ctypes.byref(struct), heads, 1)) if heads else 0
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=destination.device)
+    status = torch.empty(8 * max(layer.cursors.numel(), 1), dtype=torch.uint8, device=destination.device)
+    pointer = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+    projected = N.EtKvProjected(shares, int(members[0]), int(members[1]), int(members[2]), pointer(biases[0]),
+                                pointer(biases[1]), pointer(biases[2]), offsets.data_ptr(), offsets.numel(),
+                                float(theta), float(sign), int(layout))
+    desc = _desc(destination)
+    _check(N.lib().et_hip_kv_attention_projected_into(
+        ctypes.byref(struct), ctypes.byref(projected), float(scale), int(window or 0), _ref(desc),
+        workspace.data_ptr(), workspace.numel(), status.data_ptr(),
+        prepared_for.requirements._handle if prepared_for is not None else None,
+        prepared.data_ptr() if prepared is not None else None,
+        prepared.numel() * prepared.element_size() if prepared is not None else 0, _stream_handle(stream),
+        cancelled.ptr if cancelled is not None else None))
+    if not synchronize:
+        return status
+    kv_attention_status_check(layer, 1, status)
     return None

@@ -492,6 +492,30 @@ class LinearGroup:
             workspace.numel() * workspace.element_size() if workspace is not None else 0,
             _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
 
+    def shares_layout(self) -> "N.EtGroupShares":
+        """Where :meth:`enqueue_prepared_shares` leaves the K shares (``count`` <= 1: this group does not
+        share K over workgroups; ``et_hip_linear_group_shares_layout``)."""
+        layout = N.EtGroupShares()
+        _check(N.lib().et_hip_linear_group_shares_layout(self._handles, len(self.plans), ctypes.byref(layout)))
+        return layout
+
+    def enqueue_prepared_shares(self, prepared: torch.Tensor, weights: Sequence[torch.Tensor], workspace: torch.Tensor,
+                                stream=None, cancelled: Optional[CancellationFlag] = None) -> "N.EtGroupShares":
+        """The group's launch without the one that sums its K shares: ``workspace`` keeps them for the
+        launch that takes the results (``et_hip_linear_enqueue_prepared_group_shares``)."""
+        count = len(self.plans)
+        if len(weights) != count:
+            raise QuantizedError(N.ERR_INVALID, f"quantized_linear: a group of {count} plans takes {count} weights")
+        self.plans[0]._holds("prepared input", prepared, self.plans[0].prepared_input_bytes)
+        for index, plan in enumerate(self.plans):
+            plan._check_weight(weights[index])
+        layout = N.EtGroupShares()
+        _check(N.lib().et_hip_linear_enqueue_prepared_group_shares(
+            self._handles, count, prepared.data_ptr(), (ctypes.c_void_p * count)(*[w.data_ptr() for w in weights]),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), ctypes.byref(layout),
+            _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
+        return layout
+
     def _check_members(self, prepared, weights, ys, biases, residuals) -> None:
         """Every member's operands hold what its plan touches (see RawLinear._holds)."""
         count = len(self.plans)

@@ -225,6 +225,30 @@ int et_hip_linear_enqueue_prepared_group(const et_linear_plan* const* plans, uin
                                          const float* const* residuals, float* const* ys, void* workspace,
                                          uint64_t workspace_bytes, void* stream,
                                          const volatile int32_t* cancel);
+
+/* et_hip_linear_enqueue_prepared_group for a group that shares K over workgroups, WITHOUT the launch
+ * that sums the shares: `workspace` keeps them, `layout` says where, and the launch that takes the
+ * results (et_hip_kv_attention_projected_into for the q / k / v projections of a decode step) sums
+ * the rows it needs itself, in share order - one launch less. Biases and residuals are the summing
+ * launch's business. ET_ERR_UNSUPPORTED for a group that does not share K
+ * (et_hip_linear_group_shares_layout: count <= 1). No counterpart in the reference. */
+#define ET_HIP_LINEAR_GROUP_MOST 4
+typedef struct et_group_shares {
+    const float* shares;   /* share s of vector m, launch row n: shares[(s * vectors + m) * launch_rows + n] */
+    uint32_t count;        /* K shares; <= 1: the group does not share K */
+    uint64_t vectors;
+    uint64_t launch_rows;  /* the members' rows, each member rounded up to whole tiles */
+    uint64_t first_row[ET_HIP_LINEAR_GROUP_MOST];  /* launch row of row 0 of plans[i] */
+} et_group_shares;
+/* The layout alone (shares = NULL): what the plans decide, for a caller that chooses its path. */
+int et_hip_linear_group_shares_layout(const et_linear_plan* const* plans, uint32_t count,
+                                      et_group_shares* layout);
+int et_hip_linear_enqueue_prepared_group_shares(const et_linear_plan* const* plans, uint32_t count,
+                                                const void* prepared, const uint8_t* const* weights,
+                                                void* workspace, uint64_t workspace_bytes,
+                                                et_group_shares* layout, void* stream,
+                                                const volatile int32_t* cancel);
+
 int et_hip_linear_enqueue_prepared(const et_linear_plan* plan, const void* prepared,
                                    const uint8_t* weight, const float* bias, const float* residual,
                                    float* y, void* workspace, uint64_t workspace_bytes, void* stream,
@@ -352,6 +376,33 @@ int et_hip_kv_attention_prepared_into(const et_kv_layer* layer, const et_tensor*
                                       uint64_t workspace_bytes, void* status, const et_linear_plan* consumer,
                                       void* prepared, uint64_t prepared_bytes, void* stream,
                                       const volatile int32_t* cancel);
+/* et_hip_kv_attention_prepared_into for a decode step whose q, k and v are still the unsummed K
+ * shares of their projections (et_hip_linear_enqueue_prepared_group_shares): every workgroup of the
+ * attention kernel first sums the shares of the rows it needs in share order, adds the biases and
+ * rotates q and k at `offsets` (rotary_forward_into's arithmetic, composed.rs:2683-2729) - the bytes
+ * et_hip_linear_enqueue_prepared_group_then_rotary leaves in q, k and v - then appends and attends
+ * as et_hip_kv_attention_into does with those tensors. One token per slot; destination
+ * [.., query_heads, 1, head_dim]. `consumer` / `prepared` as in et_hip_kv_attention_prepared_into, or
+ * NULL / NULL / 0. ET_ERR_UNSUPPORTED for geometries the streaming attention kernel does not take
+ * (et_hip_kv_attention_kernel names another one): such callers sum and rotate first. No counterpart
+ * in the reference, whose executor runs one operator at a time. */
+typedef struct et_kv_projected {
+    et_group_shares shares;            /* vectors = slots */
+    uint32_t q_member, k_member, v_member;  /* which plans of the group are q, k and v */
+    const float* q_bias;               /* [query_heads * head_dim] device floats, or NULL */
+    const float* k_bias;               /* [kv_heads * head_dim], or NULL */
+    const float* v_bias;
+    const uint32_t* offsets;           /* rotary positions: DEVICE array of 1 or `slots` u32 (the cursors) */
+    uint64_t offsets_len;
+    double theta, sign;
+    int32_t layout;                    /* et_rotary_layout */
+} et_kv_projected;
+int et_hip_kv_attention_projected_into(const et_kv_layer* layer, const et_kv_projected* projected,
+                                       double scale, uint64_t window, const et_tensor* destination,
+                                       void* workspace, uint64_t workspace_bytes, void* status,
+                                       const et_linear_plan* consumer, void* prepared,
+                                       uint64_t prepared_bytes, void* stream,
+                                       const volatile int32_t* cancel);
 /* After the stream has completed and `status` has been copied to the host: 0, or
  * ET_ERR_EXECUTION with the reference's message for the first failing slot, e.g.
  * "kv attention: advance {a} out of range for chunk length {tokens}"

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import oracle
+from effect_torch_amd import synth
 
 pytestmark = pytest.mark.gpu
 
@@ -356,3 +357,87 @@ def test_prepared_input_of_the_next_contraction_from_the_attention_launch(et, de
         et.kv_attention_into(layer, q, dev(case["k"]), dev(case["v"]), scale, 0, torch.empty_like(q),
                              prepared_for=et.RawLinear(et.GgmlQuant.Q4_K, 64, heads * width, 4),
                              prepared=torch.zeros(1 << 20, dtype=torch.uint8, device=device))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, "u8"])
+@pytest.mark.parametrize("slots,kv_heads,group,width,contexts_top,with_bias", [
+    (32, 8, 4, 128, 150, False),   # a decode step's geometry: eight-wave workgroups, no context splits
+    (32, 8, 4, 128, 150, True),
+    (12, 2, 8, 64, 400, True),     # eight heads per workgroup, narrow tile of the contraction, context splits + merge
+    (7, 4, 1, 128, 90, False),     # one head per workgroup
+])
+def test_attention_sums_and_rotates_the_k_shares_of_the_projections(et, device, dtype, slots, kv_heads, group, width,
+                                                                    contexts_top, with_bias):
+    # q, k, v of a decode step left as the K shares of their group launch: the attention launch sums them,
+    # adds the biases, rotates q and k at the cursors, appends and attends - the bytes of the group launch
+    # that rotates in its reduction followed by the attention launch, for the result, the slabs, the scales
+    # and the prepared input of the next contraction
+    rng = np.random.default_rng(9300 + slots + group + int(with_bias))
+    heads, columns = group * kv_heads, 1024
+    contexts = rng.integers(0, contexts_top, slots)
+    case = make_case(rng, slots=slots, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=contexts, tokens=1, advances=[1] * slots, dtype=dtype)
+    scale = 1.0 / np.sqrt(width)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    sizes = (heads * width, kv_heads * width, kv_heads * width)
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, slots, with_bias) for rows in sizes]
+    group_launch = et.LinearGroup(plans)
+    assert group_launch.shares_layout().count > 1
+    weights = [dev(synth.random_weight(oracle.Q4_K, rows, columns, rng)) for rows in sizes]
+    biases = [dev(rng.standard_normal(rows).astype(np.float32)) if with_bias else None for rows in sizes]
+    x = dev(synth.random_activations(slots, columns, rng))
+    hidden = torch.empty(plans[0].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[0].prepare_input(x, hidden)
+    consumer = et.RawLinear(et.GgmlQuant.Q4_K, 64, heads * width, slots)
+    workspace = torch.empty(group_launch.workspace_bytes, dtype=torch.uint8, device=device)
+    for layout in (et.RotaryLayout.HALF_SPLIT, et.RotaryLayout.INTERLEAVED_PAIRS):
+        results = []
+        for in_attention in (False, True):
+            k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+            scales = [dev(case[name]) if case.get(name) is not None else None for name in ("k_scales", "v_scales")]
+            cursors = dev(case["cursors"].view(np.int32))
+            layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)), cursors,
+                               dev(case["advances"].view(np.int32)), case["max_context"], k_scales=scales[0],
+                               v_scales=scales[1])
+            assert et.kv_attention_kernel(layer, heads, 1).split("+")[0] == "kv_attend"
+            out = torch.full((slots, heads, 1, width), float("nan"), device=device)
+            prepared = torch.zeros(consumer.prepared_input_bytes, dtype=torch.uint8, device=device)
+            if in_attention:
+                shares = group_launch.enqueue_prepared_shares(hidden, weights, workspace)
+                et.kv_attention_projected_into(layer, shares, (0, 1, 2), biases, cursors, 500000.0, 1.0, layout, scale, 0,
+                                               out, prepared_for=consumer, prepared=prepared)
+            else:
+                ys = [torch.empty((slots, rows), device=device) for rows in sizes]
+                group_launch.enqueue_prepared_then_rotary(hidden, weights, ys, workspace, (0, 1), cursors, 500000.0, 1.0,
+                                                          layout, width, biases=biases if with_bias else None)
+                et.kv_attention_into(layer, ys[0].view(slots, heads, 1, width), ys[1].view(slots, kv_heads, 1, width),
+                                     ys[2].view(slots, kv_heads, 1, width), scale, 0, out, prepared_for=consumer,
+                                     prepared=prepared)
+            results.append([out, k_slab, v_slab, prepared] + [s for s in scales if s is not None])
+        assert torch.isfinite(results[0][0]).all()
+        for two, one in zip(*results):
+            assert torch.equal(two.view(torch.uint8), one.view(torch.uint8))
+
+
+def test_attention_from_k_shares_is_refused_where_the_kernel_takes_tensors(et, device):
+    # head width 20: the any-width kernel; the caller sums and rotates first
+    rng = np.random.default_rng(9400)
+    slots, kv_heads, group, width, columns = 4, 2, 2, 20, 1024
+    heads = group * kv_heads
+    case = make_case(rng, slots=slots, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=[3, 0, 40, 9], tokens=1, advances=[1] * slots, dtype=np.float32)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    sizes = (heads * width, kv_heads * width, kv_heads * width)
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, 8) for rows in sizes]
+    group_launch = et.LinearGroup(plans)
+    cursors = dev(case["cursors"].view(np.int32))
+    layer = et.KvLayer(dev(case["k_slab"]), dev(case["v_slab"]), 16, dev(case["table"].view(np.int32)), cursors,
+                       dev(case["advances"].view(np.int32)), case["max_context"])
+    assert et.kv_attention_kernel(layer, heads, 1).startswith("kv_attend_any")
+    shares = group_launch.shares_layout()
+    shares.shares = cursors.data_ptr()  # never read
+    shares.vectors = slots
+    out = torch.empty((slots, heads, 1, width), device=device)
+    with pytest.raises(et.QuantizedError, match="takes q, k and v as tensors"):
+        et.kv_attention_projected_into(layer, shares, (0, 1, 2), (None, None, None), cursors, 10000.0, 1.0,
+                                       et.RotaryLayout.HALF_SPLIT, 1.0, 0, out)
