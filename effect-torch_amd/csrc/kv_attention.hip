@@ -522,7 +522,8 @@ __device__ void project_rows(const KvArgs& a, uint32_t slot, uint32_t head0, uin
     }
 }
 
-template <typename T, int LPT, int G, int U, int WAVES>
+// PROJECTED: q, k, v arrive as the K shares of their projections (KvArgs::projected, one token per slot).
+template <typename T, int LPT, int G, int U, int WAVES, bool PROJECTED>
 __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
     constexpr int kWaves = WAVES;
     constexpr int kThreads = 64 * WAVES;
@@ -534,7 +535,7 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
     __shared__ float merge_m[GROUPS][G];
     __shared__ float merge_l[GROUPS][G];
     __shared__ float merge_acc[GROUPS][G][LPT * DPL + 4];
-    __shared__ __attribute__((aligned(16))) float projected[(G + 2) * LPT * DPL];  // q of the G heads, k, v: only with a.projected.shares
+    __shared__ __attribute__((aligned(16))) float projected[PROJECTED ? (G + 2) * LPT * DPL : 4];  // q of the G heads, k, v
 
     uint32_t index = blockIdx.x;
     const uint32_t split = index % a.splits;
@@ -575,14 +576,14 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
             rows_of_block[i] = row >= a.max_tokens ? kNoBlock : static_cast<uint32_t>(row);
         }
     }
-    const bool from_shares = a.projected.shares != nullptr;  // one token per slot
-    if (from_shares) project_rows<G>(a, slot, head0, kv_head, projected, kThreads);
+    constexpr bool from_shares = PROJECTED;
+    if constexpr (from_shares) project_rows<G>(a, slot, head0, kv_head, projected, kThreads);
     __syncthreads();
 
     float q[G][DPL];
 #pragma unroll
     for (int g = 0; g < G; g++) {
-        if (from_shares) {
+        if constexpr (from_shares) {
 #pragma unroll
             for (int d = 0; d < DPL; d++) q[g][d] = projected[g * (LPT * DPL) + sub * DPL + d] * a.scale_log2;
         } else {
@@ -658,8 +659,13 @@ __global__ __launch_bounds__(64 * WAVES) void kv_attend_kernel(const KvArgs a) {
         const uint64_t source = ((static_cast<uint64_t>(slot) * a.kv_heads + kv_head) * a.tokens + arrival) *
                                     a.width + sub * DPL;
         Piece<T> kp[1], vp[1];
-        kp[0].template from_input<LPT>(from_shares ? projected + G * (LPT * DPL) + sub * DPL : a.k + source);
-        vp[0].template from_input<LPT>(from_shares ? projected + (G + 1) * (LPT * DPL) + sub * DPL : a.v + source);
+        if constexpr (from_shares) {
+            kp[0].template from_input<LPT>(projected + G * (LPT * DPL) + sub * DPL);
+            vp[0].template from_input<LPT>(projected + (G + 1) * (LPT * DPL) + sub * DPL);
+        } else {
+            kp[0].template from_input<LPT>(a.k + source);
+            vp[0].template from_input<LPT>(a.v + source);
+        }
         if (live[0] && arrival == token && chunk == 0) {
             const uint32_t base = rows_of_block[min(block_of(a, position) - first_block, kKvTableEntries - 1u)];
             const uint32_t row = base + within_block(a, position);
@@ -888,10 +894,16 @@ __global__ void kv_merge_kernel(const KvArgs a) {
 template <typename T, int LPT, int G>
 hipError_t launch_streaming(const KvArgs& a, uint32_t workgroups, int waves, hipStream_t stream) {
     constexpr int U = G >= 8 ? 2 : 4;
-    if (waves == 8)
-        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8>), dim3(workgroups), dim3(512), 0, stream, a);
-    else
-        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4>), dim3(workgroups), dim3(256), 0, stream, a);
+    if (a.projected.shares != nullptr) {
+        if (waves == 8)
+            hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8, true>), dim3(workgroups), dim3(512), 0, stream, a);
+        else
+            hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4, true>), dim3(workgroups), dim3(256), 0, stream, a);
+    } else if (waves == 8) {
+        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 8, false>), dim3(workgroups), dim3(512), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((kv_attend_kernel<T, LPT, G, U, 4, false>), dim3(workgroups), dim3(256), 0, stream, a);
+    }
     return hipGetLastError();
 }
 
