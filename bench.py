@@ -45,8 +45,8 @@ MEASURED_TRAFFIC = {
         "sha256": "c97830386ce6b1bbaa1f8903e935411df72db510501e31dcf2e961dfcea3d1d8",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("kv_attention_decode", 2048): {
-        "bytes": 270084300, "kernel": "kv_attend", "source": "kv_attention.hip",
-        "sha256": "ab443b662f85428cacde8b1f6661a293f79c242c4d6576d7dd6b73d1c87f1ef9",
+        "bytes": 270024900, "kernel": "kv_attend", "source": "kv_attention.hip",
+        "sha256": "590105a686a613206e4bfe632266890d8f03aa1f6a00829b1aa81122a1f041fd",
         "profile": "profiles/kv_attend_decode_32slots_ctx2048_f16.md"},
 }
 
