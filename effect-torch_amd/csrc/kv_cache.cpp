@@ -162,7 +162,15 @@ int attention_into(const et_kv_layer& layer, const quantized::TensorView& q, con
                                                    "] projected vectors");
         const uint64_t q_row = s.first_row[projected->q_member], k_row = s.first_row[projected->k_member],
                        v_row = s.first_row[projected->v_member];
-        if (q_row + q_rows > s.launch_rows || k_row + kv_rows > s.launch_rows || v_row + kv_rows > s.launch_rows)
+        // a projection ends where the next member of the launch (or the launch) does
+        const auto room = [&](uint64_t first) {
+            uint64_t end = s.launch_rows;
+            for (uint64_t other : s.first_row)
+                if (other > first && other < end) end = other;
+            return first <= end ? end - first : 0;
+        };
+        if (q_rows > room(q_row) || kv_rows > room(k_row) || kv_rows > room(v_row) || k_row == v_row || q_row == k_row ||
+            q_row == v_row)
             return fail(error, ET_ERR_INVALID, "kv attention: the projections do not fit the rows of the shares");
         if (projected->layout != ET_ROTARY_HALF_SPLIT && projected->layout != ET_ROTARY_INTERLEAVED_PAIRS)
             return fail(error, ET_ERR_INVALID, "rotary: unknown layout " + std::to_string(projected->layout));

@@ -324,3 +324,51 @@ def test_raw_pointer_wrappers_refuse_operands_smaller_than_the_plan(et):
     group = et.LinearGroup([plan, plan])
     with pytest.raises(et.QuantizedError, match="weight holds"):
         group.enqueue_prepared(prepared, [full, full[:100]], [y, y])
+
+
+def test_projections_left_as_k_shares_layout_and_validation(et):
+    import torch
+    q4k = et.GgmlQuant.Q4_K
+    plans = [et.RawLinear(q4k, rows, 4096, 32) for rows in (4096, 1024, 1000)]
+    group = et.LinearGroup(plans)
+    layout = group.shares_layout()
+    # 64-row tiles, two K shares; the ragged last member is rounded up to whole tiles
+    assert (layout.count, layout.vectors, layout.launch_rows) == (2, 32, 4096 + 1024 + 1024)
+    assert list(layout.first_row)[:3] == [0, 4096, 5120]
+    assert group.workspace_bytes == layout.count * 32 * layout.launch_rows * 4
+    big = et.LinearGroup([et.RawLinear(q4k, 14336, 4096, 32) for _ in range(2)])
+    assert big.shares_layout().count == 1  # 128-row tiles fill the device: no shares to leave
+    prepared = torch.zeros(plans[0].prepared_input_bytes, dtype=torch.uint8)
+    heavy = torch.zeros(14336 * 2304, dtype=torch.uint8)
+    with pytest.raises(et.QuantizedError, match="this group does not share K over workgroups"):
+        big.enqueue_prepared_shares(prepared, [heavy, heavy], torch.zeros(16, dtype=torch.uint8), stream=0)
+    weights = [torch.zeros(rows * 2304, dtype=torch.uint8) for rows in (4096, 1024, 1000)]
+    with pytest.raises(et.QuantizedError, match="workspace of 16 bytes is smaller than the"):
+        group.enqueue_prepared_shares(prepared, weights, torch.zeros(16, dtype=torch.uint8), stream=0)
+
+    decode = _kv_layer(et, torch, slots=32, kv_heads=8, width=128, max_tokens=32 * 64, block_size=16,
+                       dtype=torch.float16, max_context=40)
+    cursors = torch.zeros(32, dtype=torch.int32)
+    out = torch.zeros(32, 32, 1, 128)
+    layout.shares = prepared.data_ptr()  # validation never reads it
+
+    def fails(message, layer=decode, shares=layout, offsets=cursors, rotary=et.RotaryLayout.HALF_SPLIT, destination=out):
+        with pytest.raises(et.QuantizedError, match=message):
+            et.kv_attention_projected_into(layer, shares, (0, 1, 2), (None, None, None), offsets, 500000.0, 1.0, rotary,
+                                           1.0, None, destination, stream=0)
+
+    fails("rotary embedding: 5 offsets for batch 32", offsets=cursors[:5].contiguous())
+    fails("rotary: unknown layout 7", rotary=7)
+    fails("projections as K shares take one token per slot", destination=torch.zeros(32, 32, 3, 128))
+    fails("expected matching rank-4-or-higher f32 tensors", destination=torch.zeros(32, 1, 128))
+    fewer = et.LinearGroup([et.RawLinear(q4k, rows, 4096, 32) for rows in (2048, 1024, 1024)]).shares_layout()
+    fewer.shares = prepared.data_ptr()
+    fails("the projections do not fit the rows of the shares", shares=fewer)
+    other = et.LinearGroup([et.RawLinear(q4k, rows, 4096, 16) for rows in (4096, 1024, 1024)]).shares_layout()
+    other.shares = prepared.data_ptr()
+    fails(r"the K shares do not describe \[32\] projected vectors", shares=other)
+    odd = _kv_layer(et, torch, slots=32, kv_heads=8, width=12, max_tokens=32 * 64, block_size=16, max_context=40)
+    narrow = et.LinearGroup([et.RawLinear(q4k, rows, 4096, 32) for rows in (32 * 12, 8 * 12, 8 * 12)]).shares_layout()
+    narrow.shares = prepared.data_ptr()
+    fails("this geometry's kernel takes q, k and v as tensors", layer=odd, shares=narrow,
+          destination=torch.zeros(32, 32, 1, 12))
