@@ -114,7 +114,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 200; "
                    "llama3_8b_batched_decode: 2)")
     p.add_argument("--workload", default="q4_k_gemv_14336x4096",
-                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,i8_biased,i8_biased_matrix_only,i8_biased_valu_only,f16,f16_16x16}, "
+                   help="one of effect_torch_amd.synth.CONFIGS, calibrate_read, calibrate_copy, calibrate_mfma_{i8,i8_scaled,i8_scaled_bf16,i8_biased,i8_biased_matrix_only,i8_biased_valu_only,f16,f16_16x16}, calibrate_contraction, "
                         "kv_attention_decode")
     p.add_argument("--vectors", type=int, default=None, help="activation vectors M (default: first of the workload)")
     p.add_argument("--mode", choices=["f32", "int8"], default=None)
@@ -356,6 +356,53 @@ def calibrate_read_sweep(args, et):
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
     }))
+
+
+def calibrate_contraction(args, et, synth):
+    """Workload ``calibrate_contraction``: the batched Q4_K contraction at 14336 x 4096 (``--vectors`` 32 by
+    default, or 7 ... 32) as the operator path launches it, then with its consumers' arithmetic left out,
+    with its copies left out, and with the weight or the activation copies alone left out - the same
+    waves, waits and barriers every time. Says what bounds the kernel: the path into LDS or the
+    instruction stream. ``value`` is the whole kernel's rate."""
+    import numpy as np
+    import torch
+
+    device = torch.device("cuda:0")
+    rows, columns = 14336, 4096
+    vectors = args.vectors or 32
+    rng = np.random.default_rng(11)
+    base = torch.from_numpy(synth.random_weight(synth.Q4_K, rows, columns, rng)).to(device)
+    copies = 1 if args.hot else -(-ROTATE_BYTES // base.numel())
+    weights = [base] + [torch.roll(base, i, 0).contiguous() for i in range(1, copies)]
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors)
+    x = torch.randn(vectors, columns, device=device)
+    prepared = torch.empty(plan.prepared_input_bytes, dtype=torch.uint8, device=device)
+    plan.prepare_input(x, prepared)
+    y = torch.empty(vectors, rows, device=device)
+    want = torch.empty_like(y)
+    plan.enqueue_prepared(prepared, weights[0], None, want, torch.empty(16, dtype=torch.uint8, device=device))
+    et.calibration_contraction("whole", plan, weights[0], prepared, y)
+    torch.cuda.synchronize()
+    assert torch.equal(y, want), "the probe's whole kernel is the operator path's"
+    table = {}
+    for probe in et.CONTRACTION_PROBES:
+        step = lambda i: et.calibration_contraction(probe, plan, weights[i % copies], prepared, y)  # noqa: E731
+        ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
+        table[probe] = round(ms * 1e3, 2)
+    moved = base.numel() + vectors * (columns + rows) * 4
+    gbs = moved / (table["whole"] * 1e-6) / 1e9
+    print(json.dumps(with_timing({
+        "metric": "calibrate_contraction GB/s of the whole kernel", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(table["whole"] * 1e-3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"calibrate_contraction: Q4_K {rows}x{columns}, {vectors} vectors, contraction kernel alone "
+                               f"({'hot' if args.hot else 'cold, %d weight buffers' % copies}); us per launch by probe",
+                   "us_per_launch": table,
+                   "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": moved, "avg_launch_us": table["whole"]},
+    })))
 
 
 def calibrate_mfma(args, et):
@@ -1042,6 +1089,8 @@ def main():
         return calibrate_read_sweep(args, et)
     if args.workload.startswith("calibrate_mfma_"):
         return calibrate_mfma(args, et)
+    if args.workload == "calibrate_contraction":
+        return calibrate_contraction(args, et, synth)
     if args.workload in DECODE_OPS:
         assert torch.cuda.is_available() and et.is_available(), "bench.py needs a gfx950 GPU"
         return decode_op(args, et)

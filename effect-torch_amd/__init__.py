@@ -16,6 +16,8 @@ from .quantized import (  # noqa: F401
     RawLinear,
     STATIC_WORKSPACE_BYTES,
     MFMA_OPERATIONS,
+    CONTRACTION_PROBES,
+    calibration_contraction,
     calibration_copy,
     calibration_mfma,
     calibration_read,

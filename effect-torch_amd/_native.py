@@ -224,6 +224,7 @@ SIGNATURES = {
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_read_variant": (ctypes.c_int, [_i32, _vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),
+    "et_hip_calibration_contraction": (ctypes.c_int, [_i32, _vp, _vp, _vp, _u64, _u64, _u64, _vp]),
     "et_hip_calibration_mfma": (ctypes.c_int, [_i32, ctypes.c_uint32, ctypes.c_uint32, _vp, _vp]),
     "et_hip_last_error": (ctypes.c_char_p, []),
 }

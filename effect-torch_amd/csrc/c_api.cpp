@@ -876,6 +876,29 @@ int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgrou
     });
 }
 
+int et_hip_calibration_contraction(int32_t probe, const void* weight, const void* prepared, float* y, uint64_t rows,
+                                   uint64_t columns, uint64_t vectors, void* stream) {
+    return guarded([&](std::string* error) -> int {
+        if (weight == nullptr || prepared == nullptr || y == nullptr || probe < ET_CONTRACTION_WHOLE ||
+            probe > ET_CONTRACTION_NO_ACTIVATION_COPIES || reinterpret_cast<uintptr_t>(prepared) % 16 != 0) {
+            *error = "calibration_contraction: probe 0..4, operands non-NULL, prepared input 16-byte aligned";
+            return ET_ERR_INVALID;
+        }
+        const hipError_t status =
+            et::gemm_h16_probe(probe, static_cast<const uint8_t*>(weight), static_cast<const uint8_t*>(prepared), y, rows,
+                               columns, vectors, static_cast<hipStream_t>(stream));
+        if (status == hipErrorInvalidValue) {
+            *error = "calibration_contraction: a Q4_K shape of 64-row tiles without K shares and at most 32 vectors";
+            return ET_ERR_UNSUPPORTED;
+        }
+        if (status != hipSuccess) {
+            *error = std::string("calibration_contraction: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        return ET_OK;
+    });
+}
+
 const char* et_hip_last_error(void) { return g_last_error.c_str(); }
 
 }  // extern "C"

@@ -27,6 +27,7 @@
 
 #include <atomic>
 #include <cstdint>
+#include <type_traits>
 
 #include "decode_math.h"
 #include "et_codecs.h"
@@ -217,7 +218,12 @@ __device__ __forceinline__ float stage_sum(const v16f& p, int r) {
     return p[r];
 }
 
-template <int CODEC, int RG, int AX, int AW, bool NARROW>
+// PROBE (measurement only, et_hip_calibration_contraction; results are then meaningless): the same
+// kernel with its consumers' arithmetic, or some of its copies, left out - every wave, barrier and
+// wait stays.
+enum : int { kProbeNone = 0, kProbeNoArithmetic = 1, kProbeNoCopies = 2, kProbeNoWeightCopies = 3, kProbeNoActivationCopies = 4 };
+
+template <int CODEC, int RG, int AX, int AW, bool NARROW, int PROBE = kProbeNone>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
     const Group group, const uint8_t* __restrict__ tiles, uint32_t vector_tiles, uint32_t columns,
     uint32_t vectors, uint32_t k_splits, float* __restrict__ partials) {
@@ -263,6 +269,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             for (int i = 0; i < S::kActivationRounds; i++) {
                 uint32_t job = i * kActivationLoaders + loader;
                 if (job >= static_cast<uint32_t>(kActivationJobs)) job -= kActivationJobs;
+                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoActivationCopies) continue;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(blob + job * 1024u + lane * 16u),
                                                  reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
             }
@@ -299,6 +306,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const uint32_t row = min(row0 + at / kRowBytes, rows - 1u);
                 const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * kStageBytes +
                                      Codec<CODEC>::source_of(at % kRowBytes);
+                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoWeightCopies) continue;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
             }
@@ -338,6 +346,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * kWeightBytes;
         const uint32_t b_base = wave_k * NB;
         const uint8_t* row_in_slot = region + (wave_n * 32u + in_half) * kRowBytes;  // this lane's weight row
+        if constexpr (PROBE == kProbeNoArithmetic) continue;
 
         if constexpr (CODEC == kQ3_K) {
             // value = d * (sc - 32) * (v - 4), v = two bits of qs | the hmask bit << 2, a 6-bit scale per 16
@@ -705,13 +714,13 @@ hipError_t sum_shares(const Group& group, const float* partials, uint32_t vector
     return hipGetLastError();
 }
 
-template <int CODEC, int RG, int AX, int AW, bool NARROW>
+template <int CODEC, int RG, int AX, int AW, bool NARROW, int PROBE = kProbeNone>
 hipError_t launch_tiles(const GemmMember* members, uint32_t count, const uint8_t* tiles, float* partials,
                         uint32_t columns, uint32_t vectors, uint32_t k_splits, hipStream_t stream, bool leave_shares,
                         const GemmRotary* rotary) {
     using S = Shape<CODEC, RG, AX, AW>;
     static_assert(S::kLdsBytes <= 160 * 1024, "LDS of a gfx950 CU: 160 KiB, all of it dynamic here");
-    const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW, NARROW>;
+    const auto kernel = gemm_h16_kernel<CODEC, RG, AX, AW, NARROW, PROBE>;
     Group group = {};
     group.count = count;
     uint64_t row_tiles = 0;
@@ -804,6 +813,32 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     // stage waits for is its slowest consumer. (14336 x 4096 with 32 vectors, contraction alone: 20.6 us
     // against 21.7 with three and one; 4096 x 14336 22.5 against 23.6; more loader waves changed nothing.)
     return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
+}
+
+hipError_t gemm_h16_probe(int probe, const uint8_t* weight, const uint8_t* tiles, float* y, uint64_t rows,
+                          uint64_t columns, uint64_t vectors, hipStream_t stream) {
+    if (!gemm_h16_supported(kQ4_K, columns) || rows == 0 || rows > 0xffffffffull || vectors == 0 || vectors > 32)
+        return hipErrorInvalidValue;
+    const GemmGroupGeometry g = gemm_h16_group_geometry(kQ4_K, &rows, 1, columns, vectors);
+    if (g.tile_rows != 64 || g.k_splits != 1) return hipErrorInvalidValue;  // the 64-row tiles, whole K each
+    const GemmMember one = {weight, nullptr, nullptr, y, rows};
+    const uint32_t k = static_cast<uint32_t>(columns), m = static_cast<uint32_t>(vectors);
+    const auto run = [&](auto narrow) -> hipError_t {
+        constexpr bool N = decltype(narrow)::value;
+        switch (probe) {
+            case kProbeNone: return launch_tiles<kQ4_K, 2, 2, 3, N>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeNoArithmetic:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoArithmetic>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeNoCopies:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoCopies>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeNoWeightCopies:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoWeightCopies>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeNoActivationCopies:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoActivationCopies>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            default: return hipErrorInvalidValue;
+        }
+    };
+    return vectors <= 16 ? run(std::true_type{}) : run(std::false_type{});
 }
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,

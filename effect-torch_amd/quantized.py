@@ -589,6 +589,21 @@ MFMA_OPERATIONS = {"i8": 65536, "i8_scaled": 65536, "f16": 32768, "f16_16x16": 1
                    "i8_biased": 65536, "i8_biased_matrix_only": 65536, "i8_biased_valu_only": 65536}
 
 
+CONTRACTION_PROBES = {"whole": 0, "no_arithmetic": 1, "no_copies": 2, "no_weight_copies": 3, "no_activation_copies": 4}
+
+
+def calibration_contraction(probe: str, plan: "RawLinear", weight: torch.Tensor, prepared: torch.Tensor, y: torch.Tensor,
+                            stream=None) -> None:
+    """The batched Q4_K contraction of ``plan`` as it is (``whole``) or with a part left out (measurement
+    aid, ``et_hip_calibration_contraction``; ``y`` is meaningful for ``whole`` only)."""
+    plan._holds("prepared input", prepared, plan.prepared_input_bytes)
+    plan._check_weight(weight)
+    plan._check_output(y)
+    _check(N.lib().et_hip_calibration_contraction(CONTRACTION_PROBES[probe], weight.data_ptr(), prepared.data_ptr(),
+                                                  y.data_ptr(), plan.rows, plan.columns, plan.vectors,
+                                                  _stream_handle(stream)))
+
+
 def calibration_mfma(kind: str, iterations: int, sink: torch.Tensor, stream=None) -> None:
     """Rounds of four independent matrix-core instructions per wave, no memory traffic (measurement
     aid, ``et_hip_calibration_mfma``); ``sink`` is f32 with 256 elements per workgroup."""

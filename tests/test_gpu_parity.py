@@ -921,3 +921,28 @@ def test_matrix_core_calibration_loops_sum_what_they_should(et, device, kind, pe
     assert torch.all(sink == per_round * rounds * elements), (float(sink[0]), per_round * rounds * elements)
     with pytest.raises(et.QuantizedError, match="calibration_mfma"):
         et.calibration_mfma(kind, 0, sink)
+
+
+@pytest.mark.parametrize("vectors", [12, 32])
+def test_contraction_probe_runs_the_operator_paths_kernel(et, device, vectors):
+    """The measurement aid that takes the batched Q4_K kernel apart launches, as `whole`, the kernel of
+    the operator path (the same bits); the partial kernels run to completion; other shapes are refused."""
+    rng = np.random.default_rng(515 + vectors)
+    rows, columns = 14336, 1024
+    weight = to_dev(synth.random_weight(oracle.Q4_K, rows, columns, rng), device)
+    x = to_dev(synth.random_activations(vectors, columns, rng), device)
+    plan = et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, vectors)
+    assert plan.requirements.kernel == "quantize_halves+gemm_h16"  # 64-row tiles, no K shares
+    prepared = torch.empty(plan.prepared_input_bytes, dtype=torch.uint8, device=device)
+    plan.prepare_input(x, prepared)
+    want = torch.empty((vectors, rows), device=device)
+    plan.enqueue_prepared(prepared, weight, None, want, torch.empty(16, dtype=torch.uint8, device=device))
+    got = torch.full_like(want, float("nan"))
+    et.calibration_contraction("whole", plan, weight, prepared, got)
+    assert torch.equal(got, want)
+    for probe in ("no_arithmetic", "no_copies", "no_weight_copies", "no_activation_copies"):
+        et.calibration_contraction(probe, plan, weight, prepared, got)
+    torch.cuda.synchronize()
+    shared = et.RawLinear(et.GgmlQuant.Q4_K, 4096, columns, vectors)  # K shared over workgroups
+    with pytest.raises(et.QuantizedError, match="64-row tiles without K shares"):
+        et.calibration_contraction("whole", shared, weight, prepared, got)
