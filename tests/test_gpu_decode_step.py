@@ -26,7 +26,11 @@ from test_gpu_parity import close
 
 pytestmark = pytest.mark.gpu
 
-FOLLOWED = [0, 9, 20, 31]
+def followed_slots(slots):
+    """The slots the oracle follows: the first, the last and two in between."""
+    return sorted({0, 9 % slots, 20 % slots, slots - 1})
+
+
 STEPS = 3
 
 
@@ -42,6 +46,7 @@ class Model:
         self.shape = shape = et.LlamaShape(layers=layers)
         self.shapes = shapes = shape.linear_shapes()
         self.slots, self.layers = slots, layers
+        self.followed = followed_slots(slots)
         Q4K = synth.Q4_K
         # every matrix at its full height; only the output projection is a block of 8192 rows tiled
         base = {name: synth.random_weight(Q4K, 8192 if name == "head" else rows, columns, rng)
@@ -87,14 +92,14 @@ class Model:
         return oracle.linear_into(synth.Q4_K, rows, columns, x, weight)
 
     def oracle_layer(self, layer, x, cursors):
-        s, n = self.shape, len(FOLLOWED)
+        s, n = self.shape, len(self.followed)
         norms = self.norms_host[layer].astype(np.float32)  # widened on use
         h = oracle.rms_norm(x, norms[0], s.eps)
         q = oracle.rotary(self.linear("wq", layer, h).reshape(n, s.heads, 1, s.head_dim), cursors, s.rope_theta)
         k = oracle.rotary(self.linear("wk", layer, h).reshape(n, s.kv_heads, 1, s.head_dim), cursors, s.rope_theta)
         v = self.linear("wv", layer, h).reshape(n, s.kv_heads, 1, s.head_dim)
         k_slab, v_slab = self.slabs_host[layer]
-        attended = oracle.kv_attention(k_slab, v_slab, self.block, self.table_host[FOLLOWED], cursors,
+        attended = oracle.kv_attention(k_slab, v_slab, self.block, self.table_host[self.followed], cursors,
                                        np.ones(n, np.uint32), q, k, v, 1.0 / np.sqrt(s.head_dim))
         x = oracle.add(x, self.linear("wo", layer, attended.reshape(n, s.hidden)))
         h = oracle.rms_norm(x, norms[1], s.eps)
@@ -102,45 +107,47 @@ class Model:
                                                                          self.linear("up", layer, h))))
 
 
-@pytest.mark.parametrize("fused", [True, False], ids=["fused", "one_operator_per_launch"])
-def test_decode_steps_follow_the_oracle_chain(et, device, fused):
-    layers, slots = 2, 32
+@pytest.mark.parametrize("fused,slots", [(True, 32), (False, 32), (True, 12)],
+                         ids=["fused", "one_operator_per_launch", "fused_12_slots"])
+def test_decode_steps_follow_the_oracle_chain(et, device, fused, slots):
+    # 12 slots: the contractions' narrow tile, attention workgroups of four waves with the context split
+    layers = 2
     model = Model(et, device, layers, slots, fused)
     dec, shape = model.decoder, model.shape
     if fused:
         assert dec.on_the_fly, "the Q4_K plans of these shapes take their inputs on the fly"
-    tokens_ref = model.tokens_host[FOLLOWED].copy()
-    cursors_ref = model.contexts[FOLLOWED].copy()
+    tokens_ref = model.tokens_host[model.followed].copy()
+    cursors_ref = model.contexts[model.followed].copy()
     for step in range(STEPS):
         dec.status.clear()
         dec.embed()
         torch.cuda.synchronize()
         et.gather_rows_status_check(shape.vocab, dec.status[-1])
-        assert np.array_equal(dec.tokens.cpu().numpy()[FOLLOWED], tokens_ref), f"step {step}: input tokens differ"
+        assert np.array_equal(dec.tokens.cpu().numpy()[model.followed], tokens_ref), f"step {step}: input tokens differ"
         x_ref = model.embedding_base[tokens_ref % 4096].astype(np.float32)
-        assert np.array_equal(dec.x.cpu().numpy()[FOLLOWED].view(np.uint32), x_ref.view(np.uint32))
+        assert np.array_equal(dec.x.cpu().numpy()[model.followed].view(np.uint32), x_ref.view(np.uint32))
         for layer in range(layers):
             dec.layer_step(layer, prepared_by_previous=dec.on_the_fly and layer > 0)
             torch.cuda.synchronize()
             et.kv_attention_status_check(dec.kv[layer], 1, dec.status[-1])
             x_ref = model.oracle_layer(layer, x_ref, cursors_ref)
-            close(dec.x.cpu().numpy()[FOLLOWED], x_ref)
+            close(dec.x.cpu().numpy()[model.followed], x_ref)
         dec.project()
         torch.cuda.synchronize()
         logits = dec.logits.cpu().numpy()
         logits_ref = model.linear("head", None, oracle.rms_norm(x_ref, model.final_norm_host.astype(np.float32), shape.eps))
-        close(logits[FOLLOWED], logits_ref)
+        close(logits[model.followed], logits_ref)
         dec.select_and_commit()
         torch.cuda.synchronize()
         et.greedy_status_check(dec.status[-1])
         chosen = dec.tokens.cpu().numpy()
         assert np.array_equal(chosen, np.argmax(logits, axis=1).astype(np.int32)), "greedy tokens are not the argmax"
         want = oracle.argmax_rows(logits_ref).astype(np.int32)
-        for i, slot in enumerate(FOLLOWED):
+        for i, slot in enumerate(model.followed):
             if chosen[slot] != want[i]:  # only a tie within the f32 bar may be decided differently
                 gap = logits_ref[i, want[i]] - logits_ref[i, chosen[slot]]
                 assert gap <= 1e-3 * max(abs(float(logits_ref[i, want[i]])), 1.0), (step, slot, chosen[slot], want[i], gap)
-        tokens_ref = chosen[FOLLOWED].copy()
+        tokens_ref = chosen[model.followed].copy()
         cursors_ref = cursors_ref + 1
         assert np.array_equal(dec.cursors.cpu().numpy().view(np.uint32), model.contexts + step + 1)
     # the rows the steps appended for the followed slots: the oracle's, within one half-float step
@@ -148,7 +155,7 @@ def test_decode_steps_follow_the_oracle_chain(et, device, fused):
         for which in range(2):
             slab = (dec.kv[layer].k_slab, dec.kv[layer].v_slab)[which].cpu().numpy()
             ref = model.slabs_host[layer][which]
-            for i, slot in enumerate(FOLLOWED):
+            for i, slot in enumerate(model.followed):
                 for position in range(int(model.contexts[slot]), int(model.contexts[slot]) + STEPS):
                     row = int(model.table_host[slot, position // model.block]) * model.block + position % model.block
                     # The two chains round f32 rows that agree within the f32 bar, and that bar follows the
