@@ -361,8 +361,8 @@ def calibrate_read_sweep(args, et):
 def calibrate_contraction(args, et, synth):
     """Workload ``calibrate_contraction``: the batched Q4_K contraction at 14336 x 4096 (``--vectors`` 32 by
     default, or 7 ... 32) as the operator path launches it, then with its consumers' arithmetic left out,
-    with its copies left out, and with the weight or the activation copies alone left out - the same
-    waves, waits and barriers every time. Says what bounds the kernel: the path into LDS or the
+    with its copies left out, with the weight or the activation copies alone left out, and with only
+    the weight or only the activation copies (no arithmetic) - the same waves, waits and barriers every time. Says what bounds the kernel: the path into LDS or the
     instruction stream. ``value`` is the whole kernel's rate."""
     import numpy as np
     import torch

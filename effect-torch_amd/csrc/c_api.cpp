@@ -880,8 +880,8 @@ int et_hip_calibration_contraction(int32_t probe, const void* weight, const void
                                    uint64_t columns, uint64_t vectors, void* stream) {
     return guarded([&](std::string* error) -> int {
         if (weight == nullptr || prepared == nullptr || y == nullptr || probe < ET_CONTRACTION_WHOLE ||
-            probe > ET_CONTRACTION_NO_ACTIVATION_COPIES || reinterpret_cast<uintptr_t>(prepared) % 16 != 0) {
-            *error = "calibration_contraction: probe 0..4, operands non-NULL, prepared input 16-byte aligned";
+            probe > ET_CONTRACTION_ACTIVATION_COPIES_ONLY || reinterpret_cast<uintptr_t>(prepared) % 16 != 0) {
+            *error = "calibration_contraction: probe 0..6, operands non-NULL, prepared input 16-byte aligned";
             return ET_ERR_INVALID;
         }
         const hipError_t status =

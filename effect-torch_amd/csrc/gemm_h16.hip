@@ -221,7 +221,8 @@ __device__ __forceinline__ float stage_sum(const v16f& p, int r) {
 // PROBE (measurement only, et_hip_calibration_contraction; results are then meaningless): the same
 // kernel with its consumers' arithmetic, or some of its copies, left out - every wave, barrier and
 // wait stays.
-enum : int { kProbeNone = 0, kProbeNoArithmetic = 1, kProbeNoCopies = 2, kProbeNoWeightCopies = 3, kProbeNoActivationCopies = 4 };
+enum : int { kProbeNone = 0, kProbeNoArithmetic = 1, kProbeNoCopies = 2, kProbeNoWeightCopies = 3, kProbeNoActivationCopies = 4,
+              kProbeWeightCopiesOnly = 5, kProbeActivationCopiesOnly = 6 };
 
 template <int CODEC, int RG, int AX, int AW, bool NARROW, int PROBE = kProbeNone>
 __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
             for (int i = 0; i < S::kActivationRounds; i++) {
                 uint32_t job = i * kActivationLoaders + loader;
                 if (job >= static_cast<uint32_t>(kActivationJobs)) job -= kActivationJobs;
-                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoActivationCopies) continue;
+                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoActivationCopies || PROBE == kProbeWeightCopiesOnly) continue;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(blob + job * 1024u + lane * 16u),
                                                  reinterpret_cast<uint4*>(slot + job * 1024u), 16, 0, 0);
             }
@@ -306,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
                 const uint32_t row = min(row0 + at / kRowBytes, rows - 1u);
                 const uint8_t* src = weight + row * row_bytes + static_cast<uint64_t>(first_stage + s) * kStageBytes +
                                      Codec<CODEC>::source_of(at % kRowBytes);
-                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoWeightCopies) continue;
+                if constexpr (PROBE == kProbeNoCopies || PROBE == kProbeNoWeightCopies || PROBE == kProbeActivationCopiesOnly) continue;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src),
                                                  reinterpret_cast<uint4*>(region + job * 1024u), 16, 0, 0);
             }
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void gemm_h16_kernel(
         const uint8_t* region = lds + S::kWeightRingAt + (stage % S::kWeightDepth) * kWeightBytes;
         const uint32_t b_base = wave_k * NB;
         const uint8_t* row_in_slot = region + (wave_n * 32u + in_half) * kRowBytes;  // this lane's weight row
-        if constexpr (PROBE == kProbeNoArithmetic) continue;
+        if constexpr (PROBE == kProbeNoArithmetic || PROBE == kProbeWeightCopiesOnly || PROBE == kProbeActivationCopiesOnly) continue;
 
         if constexpr (CODEC == kQ3_K) {
             // value = d * (sc - 32) * (v - 4), v = two bits of qs | the hmask bit << 2, a 6-bit scale per 16
@@ -835,6 +836,10 @@ hipError_t gemm_h16_probe(int probe, const uint8_t* weight, const uint8_t* tiles
                 return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoWeightCopies>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
             case kProbeNoActivationCopies:
                 return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeNoActivationCopies>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeWeightCopiesOnly:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeWeightCopiesOnly>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
+            case kProbeActivationCopiesOnly:
+                return launch_tiles<kQ4_K, 2, 2, 3, N, kProbeActivationCopiesOnly>(&one, 1, tiles, nullptr, k, m, 1, stream, false, nullptr);
             default: return hipErrorInvalidValue;
         }
     };

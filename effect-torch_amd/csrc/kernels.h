@@ -162,7 +162,8 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
                           bool leave_shares = false, const GemmRotary* rotary = nullptr);
 // Measurement only (et_hip_calibration_contraction): the Q4_K kernel of 64-row tiles without K shares
 // as it is (probe 0), without its consumers' arithmetic (1), without its copies (2), without the weight
-// (3) or the activation copies (4); at most 32 vectors. y receives meaningless values for probes > 0.
+// (3) or the activation copies (4), with the weight (5) or the activation copies (6) and nothing else; at
+// most 32 vectors. y receives meaningless values for probes > 0.
 hipError_t gemm_h16_probe(int probe, const uint8_t* weight, const uint8_t* tiles, float* y, uint64_t rows,
                           uint64_t columns, uint64_t vectors, hipStream_t stream);
 // Where a one-matrix launch with K shares leaves them: share k, vector m, row n at

@@ -589,7 +589,8 @@ MFMA_OPERATIONS = {"i8": 65536, "i8_scaled": 65536, "f16": 32768, "f16_16x16": 1
                    "i8_biased": 65536, "i8_biased_matrix_only": 65536, "i8_biased_valu_only": 65536}
 
 
-CONTRACTION_PROBES = {"whole": 0, "no_arithmetic": 1, "no_copies": 2, "no_weight_copies": 3, "no_activation_copies": 4}
+CONTRACTION_PROBES = {"whole": 0, "no_arithmetic": 1, "no_copies": 2, "no_weight_copies": 3, "no_activation_copies": 4,
+                      "weight_copies_only": 5, "activation_copies_only": 6}
 
 
 def calibration_contraction(probe: str, plan: "RawLinear", weight: torch.Tensor, prepared: torch.Tensor, y: torch.Tensor,

@@ -59,12 +59,13 @@ int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgrou
  * workgroups, e.g. 14336 x 4096) taken apart: the kernel as the operator path launches it
  * (ET_CONTRACTION_WHOLE), without its consumer waves' arithmetic (every copy, wait and barrier stays),
  * without its copies (arithmetic and barriers stay), without the weight or the activation copies
- * alone. `prepared` is what et_hip_linear_prepare_input left for a plan of these sizes; y
+ * alone, and with the weight or the activation copies and no arithmetic. `prepared` is what et_hip_linear_prepare_input left for a plan of these sizes; y
  * [vectors, rows] receives the result for ET_CONTRACTION_WHOLE and meaningless values otherwise.
  * The durations say which of the two - the path into LDS or the instruction stream - a change has
  * to shorten. No counterpart in the reference, not part of the operator path. */
 enum { ET_CONTRACTION_WHOLE = 0, ET_CONTRACTION_NO_ARITHMETIC = 1, ET_CONTRACTION_NO_COPIES = 2,
-       ET_CONTRACTION_NO_WEIGHT_COPIES = 3, ET_CONTRACTION_NO_ACTIVATION_COPIES = 4 };
+       ET_CONTRACTION_NO_WEIGHT_COPIES = 3, ET_CONTRACTION_NO_ACTIVATION_COPIES = 4,
+       ET_CONTRACTION_WEIGHT_COPIES_ONLY = 5, ET_CONTRACTION_ACTIVATION_COPIES_ONLY = 6 };
 int et_hip_calibration_contraction(int32_t probe, const void* weight, const void* prepared, float* y,
                                    uint64_t rows, uint64_t columns, uint64_t vectors, void* stream);
 

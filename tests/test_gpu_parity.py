@@ -940,7 +940,8 @@ def test_contraction_probe_runs_the_operator_paths_kernel(et, device, vectors):
     got = torch.full_like(want, float("nan"))
     et.calibration_contraction("whole", plan, weight, prepared, got)
     assert torch.equal(got, want)
-    for probe in ("no_arithmetic", "no_copies", "no_weight_copies", "no_activation_copies"):
+    for probe in ("no_arithmetic", "no_copies", "no_weight_copies", "no_activation_copies", "weight_copies_only",
+                  "activation_copies_only"):
         et.calibration_contraction(probe, plan, weight, prepared, got)
     torch.cuda.synchronize()
     shared = et.RawLinear(et.GgmlQuant.Q4_K, 4096, columns, vectors)  # K shared over workgroups
