@@ -359,7 +359,7 @@ def test_prepared_input_of_the_next_contraction_from_the_attention_launch(et, de
                              prepared=torch.zeros(1 << 20, dtype=torch.uint8, device=device))
 
 
-@pytest.mark.parametrize("dtype", [np.float16, np.float32, "u8"])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, "bf16", "u8"])
 @pytest.mark.parametrize("slots,kv_heads,group,width,contexts_top,with_bias", [
     (32, 8, 4, 128, 150, False),   # a decode step's geometry: eight-wave workgroups, no context splits
     (32, 8, 4, 128, 150, True),
@@ -393,7 +393,8 @@ def test_attention_sums_and_rotates_the_k_shares_of_the_projections(et, device, 
     for layout in (et.RotaryLayout.HALF_SPLIT, et.RotaryLayout.INTERLEAVED_PAIRS):
         results = []
         for in_attention in (False, True):
-            k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+            slab = lambda a: dev(a.view(np.int16)).view(torch.bfloat16) if dtype == "bf16" else dev(a)  # noqa: E731
+            k_slab, v_slab = slab(case["k_slab"]), slab(case["v_slab"])
             scales = [dev(case[name]) if case.get(name) is not None else None for name in ("k_scales", "v_scales")]
             cursors = dev(case["cursors"].view(np.int32))
             layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)), cursors,
@@ -441,3 +442,47 @@ def test_attention_from_k_shares_is_refused_where_the_kernel_takes_tensors(et, d
     with pytest.raises(et.QuantizedError, match="takes q, k and v as tensors"):
         et.kv_attention_projected_into(layer, shares, (0, 1, 2), (None, None, None), cursors, 10000.0, 1.0,
                                        et.RotaryLayout.HALF_SPLIT, 1.0, 0, out)
+
+
+@pytest.mark.parametrize("active_batch,context_window,window", [(5, 0, 0), (None, 60, 0), (None, 0, 33), (6, 80, 50)])
+def test_attention_from_k_shares_with_inactive_slots_and_sliding_windows(et, device, active_batch, context_window, window):
+    # the same bytes as the two launches it replaces, also where slots beyond the active batch get zeros and
+    # where the context's or the operator's window cuts the cached rows
+    rng = np.random.default_rng(9500 + (active_batch or 0) + context_window + window)
+    slots, kv_heads, group, width, columns = 8, 2, 4, 128, 1024
+    heads = group * kv_heads
+    case = make_case(rng, slots=slots, query_heads=heads, kv_heads=kv_heads, width=width, block_size=16,
+                     contexts=rng.integers(0, 150, slots), tokens=1, advances=[1] * slots, dtype=np.float16)
+    scale = 1.0 / np.sqrt(width)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    sizes = (heads * width, kv_heads * width, kv_heads * width)
+    plans = [et.RawLinear(et.GgmlQuant.Q4_K, rows, columns, slots) for rows in sizes]
+    group_launch = et.LinearGroup(plans)
+    weights = [dev(synth.random_weight(oracle.Q4_K, rows, columns, rng)) for rows in sizes]
+    hidden = torch.empty(plans[0].prepared_input_bytes, dtype=torch.uint8, device=device)
+    plans[0].prepare_input(dev(synth.random_activations(slots, columns, rng)), hidden)
+    workspace = torch.empty(group_launch.workspace_bytes, dtype=torch.uint8, device=device)
+    results = []
+    for in_attention in (False, True):
+        k_slab, v_slab = dev(case["k_slab"]), dev(case["v_slab"])
+        cursors = dev(case["cursors"].view(np.int32))
+        layer = et.KvLayer(k_slab, v_slab, case["block_size"], dev(case["table"].view(np.int32)), cursors,
+                           dev(case["advances"].view(np.int32)), case["max_context"], active_batch=active_batch,
+                           context_window=context_window)
+        out = torch.full((slots, heads, 1, width), float("nan"), device=device)
+        if in_attention:
+            shares = group_launch.enqueue_prepared_shares(hidden, weights, workspace)
+            et.kv_attention_projected_into(layer, shares, (0, 1, 2), (None, None, None), cursors, 10000.0, 1.0,
+                                           et.RotaryLayout.INTERLEAVED_PAIRS, scale, window, out)
+        else:
+            ys = [torch.empty((slots, rows), device=device) for rows in sizes]
+            group_launch.enqueue_prepared_then_rotary(hidden, weights, ys, workspace, (0, 1), cursors, 10000.0, 1.0,
+                                                      et.RotaryLayout.INTERLEAVED_PAIRS, width)
+            et.kv_attention_into(layer, ys[0].view(slots, heads, 1, width), ys[1].view(slots, kv_heads, 1, width),
+                                 ys[2].view(slots, kv_heads, 1, width), scale, window, out)
+        results.append([out, k_slab, v_slab])
+    assert torch.isfinite(results[0][0]).all()
+    if active_batch is not None:
+        assert torch.all(results[1][0][active_batch:] == 0)
+    for two, one in zip(*results):
+        assert torch.equal(two.view(torch.uint8), one.view(torch.uint8))
