@@ -130,6 +130,8 @@ def parse_args():
     p.add_argument("--hot", action="store_true", help="reuse one weight buffer (cache-resident; not the headline)")
     p.add_argument("--no-graph", action="store_true", help="enqueue the steps one by one instead of replaying a HIP graph")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-decode", action="store_true", help="headline workload: skip the batched-decode leg that fills "
+                                                            "the line's `decode` object")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
     args = p.parse_args()
     decode = args.workload == "llama3_8b_batched_decode"
@@ -771,7 +773,7 @@ def quantized_embedding(args, et):
     print(json.dumps(with_timing(result)))
 
 
-def llama_decode(args, et):
+def llama_decode(args, et, emit=True):
     """Workload ``llama3_8b_batched_decode`` (the end-to-end batched-decode configuration): greedy decode of
     ``--steps`` tokens (default 128) for 32 sequences of a Llama-3-8B-shaped model from a prefilled context
     of ``--context`` positions (default 2048), every operator through the C ABI (effect_torch_amd.LlamaDecoder):
@@ -957,7 +959,36 @@ def llama_decode(args, et):
                                   "sample": f"one layer for one slot at context {context} ({t1 - t0:.2f} s) x {layers} "
                                             f"layers + 2048 of {vocab} output rows ({t2 - t1:.2f} s) scaled; scalar C "
                                             f"restatement of the reference's loops ({per_token:.1f} s per token); {pinned}"}
-    print(json.dumps(result))
+    if emit:
+        print(json.dumps(result))
+    return result
+
+
+def decode_leg(args, et):
+    """The metric's second half next to the headline: the 128-step greedy batched decode of ``llama_decode`` run
+    in the same process (its own parity gate first, no CPU leg), reduced to the figures of one object."""
+    import gc
+    import torch
+    leg = argparse.Namespace(**vars(args))
+    leg.steps, leg.warmup, leg.mode, leg.no_cpu, leg.unfused = 128, 8, "f32", True, False
+    leg.layers, leg.context, leg.kv_dtype = 32, 2048, "f16"
+    t0 = time.perf_counter()
+    try:
+        full = llama_decode(leg, et, emit=False)
+    except Exception as error:  # the headline line is printed whatever happens here
+        return {"error": f"{type(error).__name__}: {error}"}
+    finally:
+        gc.collect()
+        torch.cuda.empty_cache()
+    roofline = full["roofline"]
+    return {"metric": full["metric"], "value": full["value"], "unit": full["unit"], "steps": full["steps"],
+            "ms_per_step": full["ms_per_step"], "ms_per_step_min": full["ms_per_step_min"],
+            "ms_per_step_max": full["ms_per_step_max"], "repetitions": full["repetitions"], "dtype": full["dtype"],
+            "algorithmic_bytes": roofline["algorithmic_bytes_per_launch"], "achieved_gbs": roofline["achieved"],
+            "frac": roofline["frac"], "workload": full["config"]["workload"], "launch": full["config"]["launch"],
+            "timing": full["config"]["timing"],
+            "layer0_relative_l2_error": full["config"]["layer0_relative_l2_error"],
+            "leg_wall_s": round(time.perf_counter() - t0, 1)}
 
 
 def gguf_upload(args, et):
@@ -1208,7 +1239,13 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, vectors, mode_name, weight_host, x_host,
                                               args.cpu_seconds, algorithmic_bytes)
-    print(json.dumps(with_timing(result)))
+    result = with_timing(result)
+    if args.workload == "q4_k_gemv_14336x4096" and vectors == 1 and mode_name == "f32" and not args.hot and not args.no_decode:
+        # "...; batched decode tok/s": the end-to-end configuration, measured after the headline with its buffers freed
+        del weights, base, ys, x, workspace
+        torch.cuda.empty_cache()
+        result["decode"] = decode_leg(args, et)
+    print(json.dumps(result))
 
 
 if __name__ == "__main__":
