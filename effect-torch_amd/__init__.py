@@ -27,11 +27,13 @@ from .quantized import (  # noqa: F401
     embedding_into,
     embedding_requirements,
     embedding_status_check,
+    handover_timeouts,
     is_available,
     linear_into,
     linear_requirements,
     quantize_activations,
     quantized_linear,
+    set_handover_spin_limit,
 )
 from .kv_cache import (  # noqa: F401
     KvLayer,

@@ -221,6 +221,8 @@ SIGNATURES = {
     "et_hip_gguf_read_tensor_into": (ctypes.c_int, [_vp, _u64, _vp, _u64, _vp]),
     "et_hip_gguf_upload_tensor": (ctypes.c_int, [_vp, _u64, _vp, _u64, _vp, _vp]),
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
+    "et_hip_handover_timeouts": (ctypes.c_int, [_vp]),
+    "et_hip_test_set_handover_spin_limit": (None, [ctypes.c_uint32]),
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_read_variant": (ctypes.c_int, [_i32, _vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),

@@ -28,6 +28,8 @@ COMMON = [
 SOURCES = {
     "dequant.hip": ["-ffp-contract=off"],
     "gemv_limb.hip": [],
+    "gemv_mma.hip": [],
+    "lds_handover.cpp": [],
     "gemv_generic.hip": [],
     "quantize_act.hip": ["-ffp-contract=off"],
     "gemm_i8.hip": [],

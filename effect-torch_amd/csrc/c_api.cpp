@@ -12,6 +12,7 @@
 #include "et_hip.h"
 #include "et_hip_calibrate.h"
 #include "kernels.h"
+#include "lds_handover.h"
 #include "decode_host.h"
 #include "gguf.h"
 #include "kv_cache.h"
@@ -900,5 +901,25 @@ int et_hip_calibration_contraction(int32_t probe, const void* weight, const void
 }
 
 const char* et_hip_last_error(void) { return g_last_error.c_str(); }
+
+int et_hip_handover_timeouts(uint64_t* count) {
+    return guarded([&](std::string* error) -> int {
+        if (count == nullptr) {
+            *error = "handover_timeouts: count is NULL";
+            return ET_ERR_INVALID;
+        }
+        uint32_t word = 0;
+        if (hipError_t status = et::handover_timeouts(&word)) {
+            *error = std::string("handover_timeouts: HIP error: ") + hipGetErrorString(status);
+            return ET_ERR_EXECUTION;
+        }
+        *count = word;
+        return ET_OK;
+    });
+}
+
+void et_hip_test_set_handover_spin_limit(uint32_t limit) {
+    et::handover_set_spin_limit(limit == ET_HANDOVER_DEFAULT_SPIN_LIMIT ? et::kHandoverSpinLimit : limit);
+}
 
 }  // extern "C"

@@ -32,6 +32,7 @@
 #include "et_codecs.h"
 #include "gemv_common.h"
 #include "kernels.h"
+#include "lds_handover.h"
 
 namespace et {
 namespace {
@@ -977,35 +978,6 @@ struct DmaControl {
 constexpr uint32_t kDmaControlAt = kDmaLdsBytes - 1024u;
 static_assert(sizeof(DmaControl) == 64, "sixteen words, zeroed by sixteen lanes");
 
-// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
-constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
-
-// Hand-over words in LDS are accessed through their LDS addresses with instructions the compiler
-// does not look into. LDS serves a wave's requests in order, so "data, then counter" needs no
-// fence; an acquire / release at workgroup scope - or any LDS access the compiler can see next to
-// global-to-LDS copies, whose destinations it cannot tell from other LDS addresses - would make it
-// wait for every outstanding copy (vmcnt 0), exactly what a loader with copies in flight must not
-// do. These accesses touch the control block only, where no copy lands.
-__device__ __forceinline__ uint32_t lds_address(const void* pointer) {
-    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(pointer));  // low half of the flat address
-}
-__device__ __forceinline__ void lds_store_unseen(uint32_t address, uint32_t value) {
-    asm volatile("ds_write_b32 %0, %1" : : "v"(address), "v"(value) : "memory");
-}
-__device__ __forceinline__ uint32_t lds_count(uint32_t address) {
-    uint32_t value;
-    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(value) : "v"(address) : "memory");
-    return __builtin_amdgcn_readfirstlane(value);
-}
-__device__ __forceinline__ void lds_arrive(uint32_t address, bool one_lane) {
-    // this wave's LDS writes are complete (and the compiler keeps them above this line)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (one_lane) asm volatile("ds_add_u32 %0, %1" : : "v"(address), "v"(1u) : "memory");
-}
-__device__ __forceinline__ void lds_await(uint32_t address, uint32_t count) {
-    while (lds_count(address) < count) __builtin_amdgcn_s_sleep(1);
-}
-
 // load_limbs for a wave with copies in flight: the same reads, unseen by the compiler.
 __device__ __forceinline__ void load_limbs_unseen(const StageMemory& stage, uint32_t lane, bool active, XLimbs& out) {
     typedef uint32_t v4u __attribute__((ext_vector_type(4)));
@@ -1036,28 +1008,13 @@ __device__ __forceinline__ void load_limbs_unseen(const StageMemory& stage, uint
     out.sum[1] = active ? __uint_as_float(sum1) : 0.f;
 }
 
-// Waits until at most `left` (wave-uniform, below kDmaHead) of this wave's copies are in flight: the
-// count of s_waitcnt is an immediate, so one instruction per value.
-__device__ __forceinline__ void wait_copies_in_flight(uint32_t left) {
-    switch (left) {
-        case 0: __builtin_amdgcn_s_waitcnt(vmcnt_only(0)); break;
-        case 1: __builtin_amdgcn_s_waitcnt(vmcnt_only(1)); break;
-        case 2: __builtin_amdgcn_s_waitcnt(vmcnt_only(2)); break;
-        case 3: __builtin_amdgcn_s_waitcnt(vmcnt_only(3)); break;
-        case 4: __builtin_amdgcn_s_waitcnt(vmcnt_only(4)); break;
-        case 5: __builtin_amdgcn_s_waitcnt(vmcnt_only(5)); break;
-        case 6: __builtin_amdgcn_s_waitcnt(vmcnt_only(6)); break;
-        case 7: __builtin_amdgcn_s_waitcnt(vmcnt_only(7)); break;
-        default: break;
-    }
-}
-
 template <class T, int M, int DEPTH>
 __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
-    uint32_t rows_per_wg) {
+    uint32_t rows_per_wg, uint32_t spin_limit, uint32_t* timeouts) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    Patience patience{spin_limit, timeouts};  // every wait on another wave is bounded (lds_handover.h)
     constexpr uint32_t kStageAt = kDmaControlAt - M * static_cast<uint32_t>(sizeof(StageMemory));
     constexpr int NI = kSliceQuads / (64 * kDmaConsumers);  // float4s per consumer thread and vector
     static_assert(DEPTH <= kDmaHead && kDmaHead <= 8, "the steady loop starts with DEPTH copies in flight; wait_copies_in_flight counts to seven");
@@ -1138,7 +1095,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
         // limbs come out of the stages as soon as the consumers have written them, while its first
         // copies are on their way (measured: later in the stream this costs a quarter microsecond).
         if constexpr (kLoaderRows > 0) {
-            lds_await(lds_address(&control->staged), kDmaConsumers);
+            lds_await(lds_address(&control->staged), kDmaConsumers, patience);
 #pragma unroll
             for (int m = 0; m < M; m++) load_limbs_unseen(stage[m], lane_id, active, xr[m]);
         }
@@ -1177,7 +1134,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
         if constexpr (kLate) {
             // nothing of this wave is in flight any more: ordinary LDS reads from here on
             if (late != 0u) {
-                lds_await(lds_address(&control->staged), kDmaConsumers);
+                lds_await(lds_address(&control->staged), kDmaConsumers, patience);
 #pragma unroll
                 for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
                 for (uint32_t r = count - late; r < count; r++) {
@@ -1196,7 +1153,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
 #pragma unroll
         for (int i = 0; i < NI; i++) stage_quad(stage[m], xv[m][i], threadIdx.x + i * 64u * kDmaConsumers);
     lds_arrive(lds_address(&control->staged), lane_id == 0);
-    lds_await(lds_address(&control->staged), kDmaConsumers);
+    lds_await(lds_address(&control->staged), kDmaConsumers, patience);
 #pragma unroll
     for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
 
@@ -1206,7 +1163,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     // are bound by their arithmetic, two of them and two loaders to a SIMD, not by LDS latency.)
     const uint32_t mine = count - (kLate ? late : min(count, static_cast<uint32_t>(kLoaderRows)));  // the last rows are the loader's
     for (uint32_t r = 0; r < mine; r++) {
-        lds_await(landed_address, ((r + 1u) * row_bytes + 1023u) >> 10);
+        lds_await(landed_address, ((r + 1u) * row_bytes + 1023u) >> 10, patience);
         typename T::Data data;
         T::load(range + r * row_bytes, lane, data);
         fold_row(r, data);
@@ -1245,9 +1202,11 @@ hipError_t launch_dma(const uint8_t* weight, const float* x, uint64_t x_row_stri
             return status;
         allowed[device].store(true, std::memory_order_release);
     }
+    HandoverState handover;
+    if (hipError_t status = handover_state(&handover)) return status;
     const uint32_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDmaThreads), kDmaLdsBytes, stream, weight, x, x_row_stride, bias, y,
-                       rows, columns, rows_per_wg);
+                       rows, columns, rows_per_wg, handover.limit, handover.timeouts);
     return hipGetLastError();
 }
 

@@ -127,10 +127,11 @@ struct Q4KMma {
                 for (int k = 0; k < 3; k++) acc[g][k] += __mul24(c0[k], s_lo) + __mul24(c1[k], s_hi);
             }
         }
-        const float m0 = __builtin_amdgcn_cvt_f32_ubyte0(mn[0]), m1 = __builtin_amdgcn_cvt_f32_ubyte1(mn[0]);
-        const float m2 = __builtin_amdgcn_cvt_f32_ubyte2(mn[0]), m3 = __builtin_amdgcn_cvt_f32_ubyte3(mn[0]);
-        const float m4 = __builtin_amdgcn_cvt_f32_ubyte0(mn[1]), m5 = __builtin_amdgcn_cvt_f32_ubyte1(mn[1]);
-        const float m6 = __builtin_amdgcn_cvt_f32_ubyte2(mn[1]), m7 = __builtin_amdgcn_cvt_f32_ubyte3(mn[1]);
+        // (the compiler turns these into v_cvt_f32_ubyte0..3)
+        const float m0 = static_cast<float>(mn[0] & 0xffu), m1 = static_cast<float>((mn[0] >> 8) & 0xffu);
+        const float m2 = static_cast<float>((mn[0] >> 16) & 0xffu), m3 = static_cast<float>(mn[0] >> 24);
+        const float m4 = static_cast<float>(mn[1] & 0xffu), m5 = static_cast<float>((mn[1] >> 8) & 0xffu);
+        const float m6 = static_cast<float>((mn[1] >> 16) & 0xffu), m7 = static_cast<float>(mn[1] >> 24);
 #pragma unroll
         for (int g = 0; g < VG; g++) {
             const float4 s0 = *reinterpret_cast<const float4*>(sums + 64 * g);

@@ -44,6 +44,15 @@ hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint6
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
                      hipStream_t stream);
 
+// ---- gemv_mma.hip: dequant-GEMV for 2..8 vectors on v_mfma_i32_16x16x32_i8 (Q4_K, Q4_0) -------
+// W is streamed once through LDS whatever the number of vectors; f32-accurate like gemv_limb.
+// x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
+constexpr uint32_t kGemvMmaMaxVectors = 8;
+bool gemv_mma_supported(int32_t codec, uint64_t rows, uint64_t columns, uint32_t vectors);
+hipError_t gemv_mma(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
+                    const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
+                    hipStream_t stream);
+
 // ---- gemv_generic.hip: every codec, any whole number of blocks, vectors <= 4 ----
 constexpr uint32_t kGemvGenericMaxVectors = 4;
 hipError_t gemv_generic(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,

@@ -150,7 +150,13 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
     } else if (plan->activation_mode == ET_ACT_F32) {
         const uint32_t limb_most = gemv_limb_max_vectors(plan->codec);
         const uint32_t limb_launch = static_cast<uint32_t>(plan->vectors < limb_most ? plan->vectors : limb_most);
-        if (plan->vectors >= kGemmMinVectors && gemm_h16_supported(plan->codec, plan->columns)) {
+        if (plan->vectors >= 2 && plan->vectors <= kGemvMmaMaxVectors &&
+            gemv_mma_supported(plan->codec, plan->rows, plan->columns, static_cast<uint32_t>(plan->vectors))) {
+            // the small-batch regime of the reference's GPU backend (runtime-metal/src/quantized.rs:1204-1220):
+            // one pass over W for all the vectors
+            plan->kernel = LinearKernel::kGemvMma;
+            plan->vectors_per_launch = kGemvMmaMaxVectors;
+        } else if (plan->vectors >= kGemmMinVectors && gemm_h16_supported(plan->codec, plan->columns)) {
             plan_matrix_core(LinearKernel::kGemmHalf, 2);
         } else if (plan->vectors >= kGemmMinVectors && gemm_i8_supported(plan->codec, plan->columns)) {
             plan_matrix_core(LinearKernel::kGemmLimb, 3);
@@ -265,6 +271,7 @@ const char* kernel_name(const et_linear_plan& plan) {
                        ? "gemv_limb_dma"
                        : "gemv_limb";
         case LinearKernel::kGemvGeneric: return "gemv_generic";
+        case LinearKernel::kGemvMma: return "gemv_mma";
         case LinearKernel::kGemmI8:
             return plan.k_splits > 1 ? "quantize_act+gemm_i8+reduce" : "quantize_act+gemm_i8";
         case LinearKernel::kGemmLimb:
@@ -730,7 +737,9 @@ int linear_enqueue(const et_linear_plan& plan, const float* x, uint64_t x_row_st
         const float* xv = x + v0 * x_row_stride;
         float* yv = y + v0 * plan.rows;
         hipError_t status;
-        if (plan.kernel == LinearKernel::kGemvLimb && gemv_limb_supported(plan.codec, plan.columns, count))
+        if (plan.kernel == LinearKernel::kGemvMma)
+            status = gemv_mma(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns, count, s);
+        else if (plan.kernel == LinearKernel::kGemvLimb && gemv_limb_supported(plan.codec, plan.columns, count))
             status = gemv_limb(plan.codec, weight, xv, x_row_stride, bias, yv, plan.rows, plan.columns,
                                count, s);
         else

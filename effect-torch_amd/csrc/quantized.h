@@ -31,6 +31,7 @@ enum class LinearKernel {
     kNone,         // empty output: nothing is enqueued
     kGemvLimb,     // dequant-GEMV on integer dot products (gemv_limb.hip)
     kGemvGeneric,  // portable dequant-GEMV (gemv_generic.hip)
+    kGemvMma,      // 2..8 vectors in one pass over W on the int8 matrix cores (gemv_mma.hip)
     kGemmI8,       // int8 activations: quantize_act.hip + gemm_i8.hip
     kGemmLimb,     // f32-accurate 3-limb activations on the same matrix-core kernel
     kGemmHalf,     // f32-accurate two-half activations on the half-float matrix cores (gemm_h16)

@@ -559,6 +559,23 @@ def _group_then_rotary(group: "LinearGroup", prepared, weights, ys, workspace, r
         ctypes.byref(after), _stream_handle(stream), cancelled.ptr if cancelled is not None else None))
 
 
+HANDOVER_DEFAULT_SPIN_LIMIT = 0xFFFFFFFF
+
+
+def handover_timeouts() -> int:
+    """Waves of this process that have abandoned a bounded wait on another wave in a GEMV kernel on the
+    current device (0 on a healthy run). Synchronises with the device."""
+    count = ctypes.c_uint64(0)
+    _check(N.lib().et_hip_handover_timeouts(ctypes.byref(count)))
+    return int(count.value)
+
+
+def set_handover_spin_limit(limit: int = HANDOVER_DEFAULT_SPIN_LIMIT) -> None:
+    """Test hook: polls after which a wave gives up such a wait (0: at once; the default restores the
+    library's own limit)."""
+    N.lib().et_hip_test_set_handover_spin_limit(ctypes.c_uint32(limit))
+
+
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""
     assert sink.numel() >= 4 * workgroups and sink.element_size() == 4

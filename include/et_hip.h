@@ -29,8 +29,11 @@
  *     from et_hip_last_error() on the calling thread.
  *   - `cancel` is an optional host flag (the reference's CancellationFlag,
  *     crates/runtime/src/cancellation.rs:18-35). It is polled before anything
- *     is enqueued; a set flag yields ET_ERR_CANCELLED / "operation aborted".
- *     Kernels already enqueued are not pre-empted.
+ *     is enqueued and again between the launches of one call (quantiser,
+ *     contraction, reduction; one GEMV launch after the other), where the
+ *     reference polls between rows and blocks (quantized.rs:451,459); a set
+ *     flag yields ET_ERR_CANCELLED / "operation aborted". Kernels already
+ *     enqueued are not pre-empted.
  *   - No C++ exception crosses this boundary.
  */
 #ifndef ET_HIP_H
@@ -585,6 +588,14 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
 
 /* Message of the last failed call on this thread ("" if none). */
 const char* et_hip_last_error(void);
+
+/* The GEMV kernels whose loader waves hand rows over to consumer waves through LDS bound every
+ * such wait: a wave that has polled a fixed number of times (about a second) gives up, and every
+ * wave of the launch still reaches its end. `*count` receives how many waves of this process have
+ * done so on the current device (0 on a healthy run; results of a launch that counted are
+ * meaningless). Synchronises with the device. No counterpart in the reference: its kernels have
+ * no cross-thread waits. */
+int et_hip_handover_timeouts(uint64_t* count);
 
 #ifdef __cplusplus
 }

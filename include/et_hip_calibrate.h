@@ -69,6 +69,13 @@ enum { ET_CONTRACTION_WHOLE = 0, ET_CONTRACTION_NO_ARITHMETIC = 1, ET_CONTRACTIO
 int et_hip_calibration_contraction(int32_t probe, const void* weight, const void* prepared, float* y,
                                    uint64_t rows, uint64_t columns, uint64_t vectors, void* stream);
 
+/* Test hook: the number of polls after which a wave of the GEMV kernels gives up a wait on another
+ * wave (see et_hip_handover_timeouts), for the launches that follow. 0 makes every wait that is not
+ * already satisfied give up at once, so that a test can see every wave leave the kernel;
+ * ET_HANDOVER_DEFAULT_SPIN_LIMIT restores the library's own value. */
+#define ET_HANDOVER_DEFAULT_SPIN_LIMIT 0xffffffffu
+void et_hip_test_set_handover_spin_limit(uint32_t limit);
+
 #ifdef __cplusplus
 }
 #endif
