@@ -1,8 +1,8 @@
-// Dequant-GEMV for a few activation vectors (2..8) on the int8 matrix cores of gfx950 (Q4_K, Q4_0):
+// Dequant-GEMV for a few activation vectors (2..8) on the int8 matrix cores of gfx950 (Q4_K, Q5_K, Q4_0, Q8_0):
 //     y[v, r] = sum_k x[v, k] * decode(W[r])[k] (+ bias[r])
 //
 // Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499) with decode_q4_k
-// (:180-199) in factored form; Q4_0 follows the public ggml block layout. The reference's own GPU
+// (:180-199) and decode_q5_k (:203-234) in factored form; Q4_0 and Q8_0 follow the public ggml block layouts. The reference's own GPU
 // backend keeps 2..8 vectors in its GEMV family (crates/runtime-metal/src/quantized.rs:1204-1220).
 // f32-accurate (24-bit fixed-point activations, exact integer dots).
 //
@@ -28,6 +28,7 @@
 // whose 16 bytes are padding are switched off.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdint>
 #include <cstdlib>
@@ -42,20 +43,21 @@ namespace {
 
 constexpr int kConsumers = 8;
 constexpr uint32_t kLdsBytes = 160u * 1024u;
-constexpr uint32_t kUnitBytes = 144u;   // 256 columns of either codec
 constexpr uint32_t kGroupRows = 16u;    // rows of W per matrix instruction
 constexpr float kLimbRange = 8323072.0f;  // 127 * 2^16: |X| <= this
 
+constexpr uint32_t kMostGroups = 4u;    // groups of a range: its rows' partial sums wait in LDS for the end
+
 // Per consumer wave: [limb planes of one vector, 544 bytes apart][sums per vector and 32 columns]
 // [units per vector and 256 columns]. Once the A operands are in registers the first part holds the
-// wave's partial sums: [group parity][vector group][lane].
+// wave's partial sums: [group][vector group][lane].
 constexpr uint32_t kLimbPitch = 544u;  // 512 bytes of a limb plane + 32: the three planes start in different banks
-constexpr uint32_t kSumsAt = 1664u, kUnitsAt = 2176u, kWaveScratch = 2304u;
+constexpr uint32_t kSumsAt = 2048u, kUnitsAt = 2560u, kWaveScratch = 2624u;
+static_assert(3u * kLimbPitch <= kSumsAt && kMostGroups * 2u * 256u <= kSumsAt, "planes and partial sums share the first part");
 struct Control {
-    uint32_t landed[8];   // copies of loader w that have landed
-    uint32_t arrived[2];  // consumers that have left their partial sums of a group (by group parity)
-    uint32_t reduced;     // groups whose partial sums have been added
-    uint32_t pad[5];
+    uint32_t landed[8];  // copies of loader w that have landed
+    uint32_t summed;     // consumers that have left the partial sums of all their groups
+    uint32_t pad[7];
 };
 static_assert(sizeof(Control) == 64, "sixteen words, zeroed by sixteen lanes");
 constexpr uint32_t kControlAt = kLdsBytes - 64u;
@@ -71,6 +73,18 @@ __device__ __forceinline__ float dpp(float v) {
 }
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+
+#ifdef ET_MMA_PROBES
+// timing experiments only: [workgroup][wave][slot] wall-clock stamps (100 MHz)
+__device__ uint64_t mma_stamps[1024 * 16 * 16];
+#define ET_STAMP(slot)                                                                                          \
+    do {                                                                                                        \
+        if (PROBE == 4 && lane_id == 0 && blockIdx.x < 1024)                                                    \
+            mma_stamps[(blockIdx.x * 16 + wave) * 16 + (slot)] = wall_clock64();                                \
+    } while (0)
+#else
+#define ET_STAMP(slot) do {} while (0)
+#endif
 
 __device__ __forceinline__ long pack(uint32_t low, uint32_t high) {
     return static_cast<long>((static_cast<uint64_t>(high) << 32) | low);
@@ -89,7 +103,7 @@ __device__ __forceinline__ void split_quad(int x0, int x1, int x2, int x3, uint3
 }
 
 // ---------------------------------------------------------------------------
-// Codec traits: one 256-column unit (144 bytes) of sixteen rows against the A operands.
+// Codec traits: one 256-column unit (kUnitBytes) of sixteen rows against the A operands.
 //   rp     the unit in the lane's row of the LDS image
 //   q      the lane's K index: which 8 of a block's 32 columns its operand registers hold
 //   a      A operands of the wave's sixteen 32-column blocks, per group of four vectors
@@ -97,6 +111,7 @@ __device__ __forceinline__ void split_quad(int x0, int x1, int x2, int x3, uint3
 //   units  value of one unit of limb 0 of the lane's vector in this unit (next vector group: + 8 floats)
 // ---------------------------------------------------------------------------
 struct Q4KMma {
+    static constexpr uint32_t kUnitBytes = 144u;  // one super-block
     static __device__ __forceinline__ uint32_t chunk(uint32_t q) { return q; }
     template <int VG, int UNIT>
     static __device__ __forceinline__ void contract(const uint8_t* rp, uint32_t q, const long (&a)[VG][16],
@@ -105,7 +120,9 @@ struct Q4KMma {
         const float d = half_bits_to_float(h.x & 0xffffu), dmin = half_bits_to_float(h.x >> 16);
         // (scale, min) of the eight sub-blocks, a byte each: crates/runtime-cpu/src/quantized.rs:77-86
         const uint32_t sc[2] = {h.y & 0x3f3f3f3fu, (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u)};
-        const uint32_t mn[2] = {h.z & 0x3f3f3f3fu, ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u)};
+        uint32_t mn[2] = {h.z & 0x3f3f3f3fu, ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u)};
+        // keeps the minima packed, a byte-to-float conversion each, instead of a mask per byte
+        asm volatile("" : "+v"(mn[0]), "+v"(mn[1]));
         int acc[VG][3];
 #pragma unroll
         for (int g = 0; g < VG; g++) acc[g][0] = acc[g][1] = acc[g][2] = 0;
@@ -158,6 +175,7 @@ struct Q4KMma {
 // 16 * (q & 1) + 8 * (q >> 1) .. + 7. value = d * (nibble - 8): the - 8 meets the f32 sums of the
 // activations once per block.
 struct Q40Mma {
+    static constexpr uint32_t kUnitBytes = 144u;  // eight blocks of 18 bytes
     static __device__ __forceinline__ uint32_t chunk(uint32_t q) { return ((q & 1u) << 1) | (q >> 1); }
     template <int VG, int UNIT>
     static __device__ __forceinline__ void contract(const uint8_t* rp, uint32_t q, const long (&a)[VG][16],
@@ -202,6 +220,105 @@ struct Q40Mma {
     }
 };
 
+// Q5_K (decode_q5_k, crates/runtime-cpu/src/quantized.rs:203-234): Q4_K's layout with a fifth bit per
+// value in qh[32] between the scales and the nibbles - bit g of qh[i] belongs to column i of sub-block g.
+struct Q5KMma {
+    static constexpr uint32_t kUnitBytes = 176u;
+    static __device__ __forceinline__ uint32_t chunk(uint32_t q) { return q; }
+    template <int VG, int UNIT>
+    static __device__ __forceinline__ void contract(const uint8_t* rp, uint32_t q, const long (&a)[VG][16],
+                                                    const float* sums, const float* units, float (&total)[VG]) {
+        const uint4 h = *reinterpret_cast<const uint4*>(rp);
+        const float d = half_bits_to_float(h.x & 0xffffu), dmin = half_bits_to_float(h.x >> 16);
+        const uint32_t sc[2] = {h.y & 0x3f3f3f3fu, (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u)};
+        uint32_t mn[2] = {h.z & 0x3f3f3f3fu, ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u)};
+        asm volatile("" : "+v"(mn[0]), "+v"(mn[1]));
+        const uint2 fifth = *reinterpret_cast<const uint2*>(rp + 16 + 8 * q);  // columns 8q..8q+7, all sub-blocks
+        int acc[VG][3];
+#pragma unroll
+        for (int g = 0; g < VG; g++) acc[g][0] = acc[g][1] = acc[g][2] = 0;
+        const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint2 w = *reinterpret_cast<const uint2*>(rp + 48 + 32 * p + 8 * q);
+            const uint32_t fx = fifth.x >> (2 * p), fy = fifth.y >> (2 * p);
+            const long lo = pack((w.x & 0x0f0f0f0fu) | ((fx & 0x01010101u) << 4), (w.y & 0x0f0f0f0fu) | ((fy & 0x01010101u) << 4));
+            const long hi = pack(((w.x >> 4) & 0x0f0f0f0fu) | ((fx & 0x02020202u) << 3),
+                                 ((w.y >> 4) & 0x0f0f0f0fu) | ((fy & 0x02020202u) << 3));
+            const int s_lo = static_cast<int>((sc[p >> 1] >> (16 * (p & 1))) & 0xffu);
+            const int s_hi = static_cast<int>((sc[p >> 1] >> (16 * (p & 1) + 8)) & 0xffu);
+#pragma unroll
+            for (int g = 0; g < VG; g++) {
+                const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[g][UNIT * 8 + 2 * p], lo, zero, 0, 0, 0);
+                const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[g][UNIT * 8 + 2 * p + 1], hi, zero, 0, 0, 0);
+                // block dots are below 2^18, scales below 2^6
+#pragma unroll
+                for (int k = 0; k < 3; k++) acc[g][k] += __mul24(c0[k], s_lo) + __mul24(c1[k], s_hi);
+            }
+        }
+        const float m0 = static_cast<float>(mn[0] & 0xffu), m1 = static_cast<float>((mn[0] >> 8) & 0xffu);
+        const float m2 = static_cast<float>((mn[0] >> 16) & 0xffu), m3 = static_cast<float>(mn[0] >> 24);
+        const float m4 = static_cast<float>(mn[1] & 0xffu), m5 = static_cast<float>((mn[1] >> 8) & 0xffu);
+        const float m6 = static_cast<float>((mn[1] >> 16) & 0xffu), m7 = static_cast<float>(mn[1] >> 24);
+#pragma unroll
+        for (int g = 0; g < VG; g++) {
+            const float4 s0 = *reinterpret_cast<const float4*>(sums + 64 * g);
+            const float4 s1 = *reinterpret_cast<const float4*>(sums + 64 * g + 4);
+            float neg = m0 * s0.x;
+            neg = fmaf(m1, s0.y, neg);
+            neg = fmaf(m2, s0.z, neg);
+            neg = fmaf(m3, s0.w, neg);
+            neg = fmaf(m4, s1.x, neg);
+            neg = fmaf(m5, s1.y, neg);
+            neg = fmaf(m6, s1.z, neg);
+            neg = fmaf(m7, s1.w, neg);
+            float f = static_cast<float>(acc[g][0]);
+            f = fmaf(256.0f, static_cast<float>(acc[g][1]), f);
+            f = fmaf(65536.0f, static_cast<float>(acc[g][2]), f);
+            total[g] += d * (units[8 * g] * f) - dmin * neg;
+        }
+    }
+};
+
+// Q8_0: a unit is four pairs of 34-byte blocks, 68 bytes = 17 dwords each. Block: half-float d, then
+// 32 signed bytes. The lanes with K index q take columns 8q..8q+7.
+struct Q80Mma {
+    static constexpr uint32_t kUnitBytes = 272u;
+    static __device__ __forceinline__ uint32_t chunk(uint32_t q) { return q; }
+    template <int VG, int UNIT>
+    static __device__ __forceinline__ void contract(const uint8_t* rp, uint32_t q, const long (&a)[VG][16],
+                                                    const float*, const float* units, float (&total)[VG]) {
+        float pos[VG];
+#pragma unroll
+        for (int g = 0; g < VG; g++) pos[g] = 0.f;
+        const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t* pair = reinterpret_cast<const uint32_t*>(rp + 68 * c);
+            const uint32_t* mine = pair + 2 * q;
+            // even block: quants at bytes 2..33 of the pair (2 bytes off dword alignment); odd: 36..67
+            const uint32_t e0 = mine[0], e1 = mine[1], e2 = mine[2], o0 = mine[9], o1 = mine[10];
+            const long even = pack(__builtin_amdgcn_alignbit(e1, e0, 16), __builtin_amdgcn_alignbit(e2, e1, 16));
+            const long odd = pack(o0, o1);
+            const float da = half_bits_to_float(pair[0] & 0xffffu), db = half_bits_to_float(pair[8] >> 16);
+#pragma unroll
+            for (int g = 0; g < VG; g++) {
+                const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[g][UNIT * 8 + 2 * c], even, zero, 0, 0, 0);
+                const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[g][UNIT * 8 + 2 * c + 1], odd, zero, 0, 0, 0);
+                float f0 = static_cast<float>(c0[0]);
+                f0 = fmaf(256.0f, static_cast<float>(c0[1]), f0);
+                f0 = fmaf(65536.0f, static_cast<float>(c0[2]), f0);
+                float f1 = static_cast<float>(c1[0]);
+                f1 = fmaf(256.0f, static_cast<float>(c1[1]), f1);
+                f1 = fmaf(65536.0f, static_cast<float>(c1[2]), f1);
+                pos[g] = fmaf(db, f1, fmaf(da, f0, pos[g]));
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < VG; g++) total[g] += units[8 * g] * pos[g];
+    }
+};
+
 // Waits until the loaders have brought the first `need` copies of the image (taken in turn: copy i
 // is loader i % LOADERS's). One poll reads all the loaders' words, a lane each.
 template <int LOADERS>
@@ -219,7 +336,7 @@ __device__ __forceinline__ bool await_copies(const Control* control, uint32_t la
     return false;
 }
 
-template <class T, int VG, int LOADERS, int DEPTH>
+template <class T, int VG, int LOADERS, int DEPTH, int PROBE = 0>
 __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
     const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns, uint32_t rows_per_wg,
@@ -233,9 +350,10 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t wg_row0 = blockIdx.x * rows_per_wg;
     if (wg_row0 >= rows) return;
+    ET_STAMP(0);
     const uint32_t wg_rows = min(rows_per_wg, rows - wg_row0);
     const uint32_t row_units = columns >> 8;
-    const uint32_t row_bytes = row_units * kUnitBytes;
+    const uint32_t row_bytes = row_units * T::kUnitBytes;
     const uint32_t pitch = image_pitch(row_bytes);
     const uint32_t image_bytes = (wg_rows - 1u) * pitch + row_bytes;  // ends with the last row's last byte
 
@@ -254,7 +372,7 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
         uint32_t next = loader;  // number of the wave's next copy
         const auto copy = [&]() {
             // never a copy without a lane: the image ends with bytes of W and padding is shorter than a copy
-            if (row < wg_rows && column < row_bytes)
+            if (PROBE != 2 && PROBE != 3 && row < wg_rows && column < row_bytes)
                 // streamed once: non-temporal (aux bit 1), the caches keep nothing of it
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + row * row_bytes + column),
                                                  reinterpret_cast<uint4*>(lds + next * 1024u), 16, 0, 2);
@@ -268,20 +386,26 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
         };
         // The first copies wait for the barrier, i.e. until the consumers have issued their activation
         // loads: issued ahead of it they delay those loads, and with them everything else.
+        // (measured: issued ahead of the barrier, 0.9 to 1.5 us per launch slower)
         __syncthreads();
+        ET_STAMP(1);
         const uint32_t head = min(mine, static_cast<uint32_t>(DEPTH));
         for (uint32_t i = 0; i < head; i++) copy();
+        ET_STAMP(2);
         uint32_t landed = 0;
         for (uint32_t i = head; i < mine; i++) {  // only with DEPTH copies in flight
             // the oldest copy in flight has landed: say so, then take its place in the queue
             __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));
             lds_store_unseen(landed_address, ++landed);
+            if (landed == 1u) ET_STAMP(3);
             copy();
         }
+        ET_STAMP(4);
         for (uint32_t left = head; left > 0u; left--) {
             wait_copies_in_flight(left - 1u);
             lds_store_unseen(landed_address, ++landed);
         }
+        ET_STAMP(5);
         return;
     }
 
@@ -310,6 +434,7 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     }
     if (threadIdx.x < 16) reinterpret_cast<uint32_t*>(control)[threadIdx.x] = 0u;
     __syncthreads();  // the only barrier: the counters are zero before anybody counts
+    ET_STAMP(1);
 
     // 24-bit fixed point per vector and 256-column unit, X = rint(x * 127 * 2^16 / max|x|), in three
     // balanced signed-byte limbs; the limbs go through the wave's scratch into the lanes that hold
@@ -359,76 +484,72 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
         }
     }
     asm volatile("" ::: "memory");
+    ET_STAMP(2);
 
     const uint32_t n = lane_id & 15u, q = lane_id >> 4;
     const uint32_t groups = (wg_rows + kGroupRows - 1u) / kGroupRows;
-    float* partial = reinterpret_cast<float*>(scratch);  // [group parity][vector group][lane]
-    const uint32_t reduced_address = lds_address(&control->reduced);
+    float* partial = reinterpret_cast<float*>(scratch);  // [group][vector group][lane]
     for (uint32_t group = 0; group < groups; group++) {
         const uint32_t last_row = min(group * kGroupRows + kGroupRows, wg_rows) - 1u;
         const bool landed = await_copies<LOADERS>(control, lane_id, (last_row * pitch + row_bytes + 1023u) >> 10, patience);
+        ET_STAMP(3 + 3 * group);
         float total[VG];
 #pragma unroll
         for (int g = 0; g < VG; g++) total[g] = 0.f;
-        if (landed && my_units != 0u) {
+        if (PROBE != 1 && PROBE != 3 && landed && my_units != 0u) {
             // rows past the end of the range read its last row again and are not stored
-            const uint8_t* rp = lds + min(group * kGroupRows + n, wg_rows - 1u) * pitch + first_unit * kUnitBytes;
-            T::template contract<VG, 0>(rp, q, a, sums + q * 16u, units + q * 2u, total);
-            if (my_units > 1u)
-                T::template contract<VG, 1>(rp + kUnitBytes, q, a, sums + q * 16u + 8u, units + q * 2u + 1u, total);
-        }
-        // the slot of this parity is free once the group two before has been added up
-        if (group >= 2u) lds_await(reduced_address, group - 1u, patience);
-        const uint32_t parity = group & 1u;
-#pragma unroll
-        for (int g = 0; g < VG; g++) partial[(parity * VG + g) * 64u + lane_id] = total[g];
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        uint32_t before = 0;
-        const uint32_t arrived_address = lds_address(&control->arrived[parity]);
-        if (lane_id == 0)
-            asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=v"(before) : "v"(arrived_address), "v"(1u) : "memory");
-        before = __builtin_amdgcn_readfirstlane(before);
-        if (before == static_cast<uint32_t>(kConsumers - 1)) {
-            // the last to arrive adds the eight partial sums in wave order and stores the group
-            const uint32_t row = group * kGroupRows + n;
-#pragma unroll
-            for (int g = 0; g < VG; g++) {
-                float value = 0.f;
-#pragma unroll
-                for (int w = 0; w < kConsumers; w++)
-                    value += reinterpret_cast<const float*>(lds + kScratchAt + w * kWaveScratch)[(parity * VG + g) * 64u + lane_id];
-                const uint32_t vector = 4u * g + q;
-                if (vector < vectors && row < wg_rows) {
-                    if (bias != nullptr) value += bias[wg_row0 + row];
-                    y[static_cast<uint64_t>(vector) * rows + wg_row0 + row] = value;
-                }
+            const uint8_t* rp = lds + min(group * kGroupRows + n, wg_rows - 1u) * pitch + first_unit * T::kUnitBytes;
+            if (my_units > 1u) {  // both in one block: the second unit's LDS reads overtake the first's arithmetic
+                T::template contract<VG, 0>(rp, q, a, sums + q * 16u, units + q * 2u, total);
+                T::template contract<VG, 1>(rp + T::kUnitBytes, q, a, sums + q * 16u + 8u, units + q * 2u + 1u, total);
+            } else {
+                T::template contract<VG, 0>(rp, q, a, sums + q * 16u, units + q * 2u, total);
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            lds_store_unseen(arrived_address, 0u);
-            lds_store_unseen(reduced_address, group + 1u);
+        }
+        ET_STAMP(4 + 3 * group);
+#pragma unroll
+        for (int g = 0; g < VG; g++) partial[(group * VG + g) * 64u + lane_id] = total[g];
+    }
+    // The eight partial sums of every (group, vector group) meet here: each consumer adds those of one
+    // pair in wave order (the same bits on every run) and stores sixteen rows of four vectors.
+    const uint32_t summed_address = lds_address(&control->summed);
+    lds_arrive(summed_address, lane_id == 0);
+    ET_STAMP(15);
+    if (!lds_await(summed_address, kConsumers, patience)) return;
+    for (uint32_t pair = wave; pair < groups * VG; pair += kConsumers) {
+        const uint32_t group = pair / VG, g = pair - group * VG;
+        float value = 0.f;
+#pragma unroll
+        for (int w = 0; w < kConsumers; w++)
+            value += reinterpret_cast<const float*>(lds + kScratchAt + w * kWaveScratch)[pair * 64u + lane_id];
+        const uint32_t vector = 4u * g + q, row = group * kGroupRows + n;
+        if (vector < vectors && row < wg_rows) {
+            if (bias != nullptr) value += bias[wg_row0 + row];
+            y[static_cast<uint64_t>(vector) * rows + wg_row0 + row] = value;
         }
     }
+    ET_STAMP(14);
 }
 
-// Rows of a workgroup's range: a two-hundred-fifty-sixth of the matrix when its image fits LDS,
-// else the most whole groups that fit.
-uint32_t range_rows(uint32_t rows, uint32_t columns) {
-    const uint32_t row_bytes = (columns >> 8) * kUnitBytes;
+// Rows of a workgroup's range: a two-hundred-fifty-sixth of the matrix when its image fits LDS (and
+// its groups the partial sums' slots); else the matrix is cut into the fewest rounds of 256 ranges that do.
+uint32_t range_rows(uint32_t rows, uint32_t row_bytes) {
     const uint32_t pitch = image_pitch(row_bytes);
-    const uint32_t most = (kScratchAt - row_bytes) / pitch + 1u;
+    const uint32_t most = std::min((kScratchAt - row_bytes) / pitch + 1u, kMostGroups * kGroupRows);
     const uint32_t share = (rows + 255u) / 256u;
     if (share <= most) return share;
-    return most >= kGroupRows ? most / kGroupRows * kGroupRows : most;
+    const uint32_t rounds = (share + most - 1u) / most;
+    return (rows + 256u * rounds - 1u) / (256u * rounds);
 }
 
-template <class T, int VG, int LOADERS, int DEPTH>
+template <class T, int VG, int LOADERS, int DEPTH, int PROBE = 0>
 hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias, float* y,
                   uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
     static std::atomic<bool> allowed[64];
     int device = 0;
     if (hipError_t status = hipGetDevice(&device)) return status;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    const auto kernel = gemv_mma_kernel<T, VG, LOADERS, DEPTH>;
+    const auto kernel = gemv_mma_kernel<T, VG, LOADERS, DEPTH, PROBE>;
     if (!allowed[device].load(std::memory_order_acquire)) {
         if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes))
@@ -437,7 +558,7 @@ hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, 
     }
     HandoverState handover;
     if (hipError_t status = handover_state(&handover)) return status;
-    const uint32_t rows_per_wg = range_rows(rows, columns);
+    const uint32_t rows_per_wg = range_rows(rows, (columns >> 8) * T::kUnitBytes);
     const uint32_t grid = (rows + rows_per_wg - 1u) / rows_per_wg;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * (kConsumers + LOADERS)), kLdsBytes, stream, weight, x, x_row_stride,
                        bias, y, rows, columns, rows_per_wg, vectors, handover.limit, handover.timeouts);
@@ -447,6 +568,21 @@ hipError_t launch(const uint8_t* weight, const float* x, uint64_t x_row_stride, 
 template <class T>
 hipError_t launch_vectors(const uint8_t* weight, const float* x, uint64_t x_row_stride, const float* bias, float* y,
                           uint32_t rows, uint32_t columns, uint32_t vectors, hipStream_t stream) {
+#ifdef ET_MMA_PROBES
+    // timing experiments only (never in the product build): ET_HIP_MMA_VARIANT picks a launch shape or a probe
+    static const int variant = [] { const char* v = std::getenv("ET_HIP_MMA_VARIANT"); return v ? std::atoi(v) : 0; }();
+#define ET_V(N, ...) case N: return launch<T, __VA_ARGS__>(weight, x, x_row_stride, bias, y, rows, columns, vectors, stream)
+    if (vectors <= 4) switch (variant) {
+        ET_V(1, 1, 8, 4, 1); ET_V(2, 1, 8, 4, 2); ET_V(3, 1, 8, 5); ET_V(4, 1, 8, 6); ET_V(5, 1, 4, 8); ET_V(6, 1, 8, 8);
+        ET_V(7, 1, 8, 3); ET_V(8, 1, 4, 6); ET_V(9, 1, 8, 4, 3); ET_V(10, 1, 8, 4, 4);
+        default: break;
+    } else switch (variant) {
+        ET_V(1, 2, 4, 8, 1); ET_V(2, 2, 4, 8, 2); ET_V(3, 2, 8, 4); ET_V(4, 2, 8, 5); ET_V(5, 2, 4, 6); ET_V(6, 2, 2, 8);
+        ET_V(9, 2, 4, 8, 3); ET_V(10, 2, 4, 8, 4);
+        default: break;
+    }
+#undef ET_V
+#endif
     if (vectors <= 4) return launch<T, 1, 8, 4>(weight, x, x_row_stride, bias, y, rows, columns, vectors, stream);
     // two vector groups keep 64 registers of A operands: twelve waves leave each 168
     return launch<T, 2, 4, 8>(weight, x, x_row_stride, bias, y, rows, columns, vectors, stream);
@@ -454,10 +590,16 @@ hipError_t launch_vectors(const uint8_t* weight, const float* x, uint64_t x_row_
 
 }  // namespace
 
+#ifdef ET_MMA_PROBES
+extern "C" int et_hip_mma_stamps(uint64_t* out, uint64_t count) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(mma_stamps), count * 8);
+}
+#endif
+
 bool gemv_mma_supported(int32_t codec, uint64_t rows, uint64_t columns, uint32_t vectors) {
-    if (codec != kQ4_K && codec != kQ4_0) return false;
+    if (codec != kQ4_K && codec != kQ4_0 && codec != kQ5_K && codec != kQ8_0) return false;
     if (vectors < 2 || vectors > kGemvMmaMaxVectors) return false;
-    // one image row is at most 16 units; the copies are 16 bytes wide (144 bytes per 256 columns)
+    // one image row is at most 16 units; the copies are 16 bytes wide (a unit is a multiple of 16 bytes)
     if (columns == 0 || columns % 256 != 0 || columns > 4096) return false;
     // with less than a group of rows to a compute unit most of every matrix instruction is padding
     return rows >= 256u * 8u && rows <= 0xffffffffull;
@@ -467,8 +609,13 @@ hipError_t gemv_mma(int32_t codec, const uint8_t* weight, const float* x, uint64
                     float* y, uint64_t rows, uint64_t columns, uint32_t vectors, hipStream_t stream) {
     const uint32_t n = static_cast<uint32_t>(rows), k = static_cast<uint32_t>(columns);
     if (!gemv_mma_supported(codec, rows, columns, vectors)) return hipErrorInvalidValue;
-    if (codec == kQ4_K) return launch_vectors<Q4KMma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
-    return launch_vectors<Q40Mma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+    switch (codec) {
+        case kQ4_K: return launch_vectors<Q4KMma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ5_K: return launch_vectors<Q5KMma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ4_0: return launch_vectors<Q40Mma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        case kQ8_0: return launch_vectors<Q80Mma>(weight, x, x_row_stride, bias, y, n, k, vectors, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace et

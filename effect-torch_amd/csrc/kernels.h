@@ -44,7 +44,7 @@ hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint6
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
                      hipStream_t stream);
 
-// ---- gemv_mma.hip: dequant-GEMV for 2..8 vectors on v_mfma_i32_16x16x32_i8 (Q4_K, Q4_0) -------
+// ---- gemv_mma.hip: dequant-GEMV for 2..8 vectors on v_mfma_i32_16x16x32_i8 (Q4_K, Q5_K, Q4_0, Q8_0) ----
 // W is streamed once through LDS whatever the number of vectors; f32-accurate like gemv_limb.
 // x rows must be 16-byte aligned (x pointer and x_row_stride * 4).
 constexpr uint32_t kGemvMmaMaxVectors = 8;

@@ -1,4 +1,4 @@
-"""GPU parity of the one-pass small-batch GEMV (2..8 activation vectors, Q4_K and Q4_0; the regime
+"""GPU parity of the one-pass small-batch GEMV (2..8 activation vectors; Q4_K, Q5_K, Q4_0, Q8_0; the regime
 crates/runtime-metal/src/quantized.rs:1204-1220 keeps in its GEMV family): the HIP path through the C
 ABI against the CPU oracle (linear_into, crates/runtime-cpu/src/quantized.rs:419-499) on the same
 seeded inputs. Bar: |a-b| <= 1e-3 * max(|b|, 1), once against the oracle and once, with no allowance,
@@ -14,7 +14,7 @@ from test_gpu_parity import close, run_linear, to_dev
 
 pytestmark = pytest.mark.gpu
 
-CODECS = [oracle.Q4_K, oracle.Q4_0]
+CODECS = [oracle.Q4_K, oracle.Q4_0, oracle.Q5_K, oracle.Q8_0]
 
 
 def planned_kernel(et, codec, rows, columns, vectors, bias=False):
@@ -54,7 +54,7 @@ def test_every_vector_count(et, device, codec, vectors):
     (3, 5003, 256),      # one unit per row: seven of the eight consumer waves hold no columns
     (8, 3000, 2048),     # four consumer waves hold columns
     (5, 30000, 512),     # 118 rows per range, images of 36 KiB
-    (8, 40000, 4096),    # more rows than 256 images hold: ranges of 48 rows, a grid of 834
+    (8, 40000, 4096),    # more rows than 256 images hold: three rounds of 256 ranges of 53 rows
     (6, 9000, 1024),
     (4, 12000, 3072),    # the last consumer waves hold one unit / none
     (7, 2300, 3840),     # fifteen units: the last wave holds one
@@ -65,7 +65,7 @@ def test_shapes(et, device, codec, vectors, rows, columns):
     check(et, device, codec, rows, columns, vectors, rng, bias)
 
 
-@pytest.mark.parametrize("name", ["q4_0_gemv_11008x4096", "q4_k_gemv_14336x4096"])
+@pytest.mark.parametrize("name", ["q4_0_gemv_11008x4096", "q4_k_gemv_14336x4096", "q8_0_gemv_4096x4096"])
 @pytest.mark.parametrize("vectors", [2, 3, 4, 5, 6, 7, 8])
 def test_full_size(et, device, name, vectors):
     cfg = synth.CONFIGS[name]
@@ -75,7 +75,9 @@ def test_full_size(et, device, name, vectors):
 
 @pytest.mark.parametrize("codec", CODECS)
 def test_special_activations(et, device, codec):
-    # unit vectors select one decoded weight (exact: every other product is an exact zero); a vector of
+    # unit vectors select one decoded weight (every other product is an exact zero; what is left is the
+    # rounding of d * (scale * quant) against the decoder's (d * scale) * quant, and for Q4_0 of d * quant - 8 * d: a
+    # few 1e-8 of the largest weight); a vector of
     # zeros gives zeros; a vector whose 256-column units differ by 2^20 in size keeps every unit's precision
     rows, columns, vectors = 2304, 4096, 4
     rng = np.random.default_rng(31 + codec)
@@ -87,7 +89,7 @@ def test_special_activations(et, device, codec):
         x[v, k] = 1.0
     got = run_linear(et, device, codec, rows, columns, x, weight)
     for v, k in enumerate(picks):
-        assert np.array_equal(got[v], decoded[:, k])
+        np.testing.assert_allclose(got[v], decoded[:, k], rtol=5e-7, atol=1e-7 * np.abs(decoded[:, k]).max())
     assert not got[3].any()
     x = synth.random_activations(vectors, columns, rng)
     x[:, :256] *= 2.0 ** 20
