@@ -11,6 +11,7 @@ import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libet_hip.so")
+CALIBRATE_LIB_PATH = os.path.join(HERE, "lib", "libet_hip_calibrate.so")
 
 # et_status
 OK, ERR_UNSUPPORTED, ERR_EXECUTION, ERR_CANCELLED, ERR_UNAVAILABLE, ERR_INVALID = range(6)
@@ -223,15 +224,21 @@ SIGNATURES = {
     "et_hip_quantize_activations": (ctypes.c_int, [_vp, _u64, _u64, _u64, _vp, _vp, _vp, _vp]),
     "et_hip_handover_timeouts": (ctypes.c_int, [_vp]),
     "et_hip_test_set_handover_spin_limit": (None, [ctypes.c_uint32]),
+    "et_hip_last_error": (ctypes.c_char_p, []),
+}
+
+# libet_hip_calibrate.so: the measurement aids (include/et_hip_calibrate.h)
+CALIBRATE_SIGNATURES = {
     "et_hip_calibration_read": (ctypes.c_int, [_vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_read_variant": (ctypes.c_int, [_i32, _vp, _u64, _vp, ctypes.c_uint32, _vp]),
     "et_hip_calibration_copy": (ctypes.c_int, [_vp, _vp, _u64, _vp]),
     "et_hip_calibration_contraction": (ctypes.c_int, [_i32, _vp, _vp, _vp, _u64, _u64, _u64, _vp]),
     "et_hip_calibration_mfma": (ctypes.c_int, [_i32, ctypes.c_uint32, ctypes.c_uint32, _vp, _vp]),
-    "et_hip_last_error": (ctypes.c_char_p, []),
+    "et_hip_calibration_last_error": (ctypes.c_char_p, []),
 }
 
 _lib = None
+_calibrate_lib = None
 
 
 class NativeLibraryMissing(ImportError):
@@ -253,6 +260,22 @@ def lib() -> ctypes.CDLL:
             fn.argtypes = argtypes
         _lib = handle
     return _lib
+
+
+def calibrate_lib() -> ctypes.CDLL:
+    """Loads the measurement library (after the operators' library, which it links against)."""
+    global _calibrate_lib
+    if _calibrate_lib is None:
+        lib()
+        if not os.path.exists(CALIBRATE_LIB_PATH):
+            raise NativeLibraryMissing(f"{CALIBRATE_LIB_PATH} is missing: build it with `python effect-torch_amd/build.py`")
+        handle = ctypes.CDLL(CALIBRATE_LIB_PATH)
+        for name, (restype, argtypes) in CALIBRATE_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _calibrate_lib = handle
+    return _calibrate_lib
 
 
 def last_error() -> str:

@@ -10,7 +10,6 @@
 
 #include "et_codecs.h"
 #include "et_hip.h"
-#include "et_hip_calibrate.h"
 #include "kernels.h"
 #include "lds_handover.h"
 #include "decode_host.h"
@@ -807,99 +806,6 @@ int et_hip_quantize_activations(const float* x, uint64_t x_row_stride, uint64_t 
     });
 }
 
-int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
-                            void* stream) {
-    return guarded([&](std::string* error) -> int {
-        if (src == nullptr || sink == nullptr || workgroups == 0 || (bytes >> 36) != 0 ||
-            reinterpret_cast<uintptr_t>(src) % 16 != 0) {
-            *error = "calibration_read: source must be 16-byte aligned, sink non-NULL, workgroups > 0";
-            return ET_ERR_INVALID;
-        }
-        const hipError_t status =
-            et::calibration_read(src, bytes, sink, workgroups, static_cast<hipStream_t>(stream));
-        if (status != hipSuccess) {
-            *error = std::string("calibration_read: HIP error: ") + hipGetErrorString(status);
-            return ET_ERR_EXECUTION;
-        }
-        return ET_OK;
-    });
-}
-
-int et_hip_calibration_read_variant(int32_t variant, const void* src, uint64_t bytes, uint32_t* sink,
-                                    uint32_t workgroups, void* stream) {
-    return guarded([&](std::string* error) -> int {
-        if (src == nullptr || sink == nullptr || workgroups == 0 || workgroups > 65536 || (bytes >> 36) != 0 ||
-            reinterpret_cast<uintptr_t>(src) % 16 != 0 || variant < ET_READ_PLAIN || variant > ET_READ_LDS_8) {
-            *error = "calibration_read_variant: variant 0..4, source 16-byte aligned, sink non-NULL, "
-                     "1 <= workgroups <= 65536";
-            return ET_ERR_INVALID;
-        }
-        const hipError_t status =
-            et::calibration_read_variant(variant, src, bytes, sink, workgroups, static_cast<hipStream_t>(stream));
-        if (status != hipSuccess) {
-            *error = std::string("calibration_read_variant: HIP error: ") + hipGetErrorString(status);
-            return ET_ERR_EXECUTION;
-        }
-        return ET_OK;
-    });
-}
-
-int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* stream) {
-    return guarded([&](std::string* error) -> int {
-        if (src == nullptr || dst == nullptr || reinterpret_cast<uintptr_t>(src) % 16 != 0 ||
-            reinterpret_cast<uintptr_t>(dst) % 16 != 0) {
-            *error = "calibration_copy: buffers must be non-NULL and 16-byte aligned";
-            return ET_ERR_INVALID;
-        }
-        const hipError_t status =
-            et::calibration_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
-        if (status != hipSuccess) {
-            *error = std::string("calibration_copy: HIP error: ") + hipGetErrorString(status);
-            return ET_ERR_EXECUTION;
-        }
-        return ET_OK;
-    });
-}
-
-int et_hip_calibration_mfma(int32_t kind, uint32_t iterations, uint32_t workgroups, float* sink, void* stream) {
-    return guarded([&](std::string* error) -> int {
-        if (sink == nullptr || workgroups == 0 || workgroups > 65536 || iterations == 0 || iterations > (1u << 20) ||
-            kind < ET_MFMA_I8 || kind > ET_MFMA_I8_BIASED_VALU_ONLY) {
-            *error = "calibration_mfma: kind 0..7, 1 <= iterations <= 2^20, 1 <= workgroups <= 65536, sink non-NULL";
-            return ET_ERR_INVALID;
-        }
-        const hipError_t status = et::calibration_mfma(kind, iterations, workgroups, sink, static_cast<hipStream_t>(stream));
-        if (status != hipSuccess) {
-            *error = std::string("calibration_mfma: HIP error: ") + hipGetErrorString(status);
-            return ET_ERR_EXECUTION;
-        }
-        return ET_OK;
-    });
-}
-
-int et_hip_calibration_contraction(int32_t probe, const void* weight, const void* prepared, float* y, uint64_t rows,
-                                   uint64_t columns, uint64_t vectors, void* stream) {
-    return guarded([&](std::string* error) -> int {
-        if (weight == nullptr || prepared == nullptr || y == nullptr || probe < ET_CONTRACTION_WHOLE ||
-            probe > ET_CONTRACTION_ACTIVATION_COPIES_ONLY || reinterpret_cast<uintptr_t>(prepared) % 16 != 0) {
-            *error = "calibration_contraction: probe 0..6, operands non-NULL, prepared input 16-byte aligned";
-            return ET_ERR_INVALID;
-        }
-        const hipError_t status =
-            et::gemm_h16_probe(probe, static_cast<const uint8_t*>(weight), static_cast<const uint8_t*>(prepared), y, rows,
-                               columns, vectors, static_cast<hipStream_t>(stream));
-        if (status == hipErrorInvalidValue) {
-            *error = "calibration_contraction: a Q4_K shape of 64-row tiles without K shares and at most 32 vectors";
-            return ET_ERR_UNSUPPORTED;
-        }
-        if (status != hipSuccess) {
-            *error = std::string("calibration_contraction: HIP error: ") + hipGetErrorString(status);
-            return ET_ERR_EXECUTION;
-        }
-        return ET_OK;
-    });
-}
-
 const char* et_hip_last_error(void) { return g_last_error.c_str(); }
 
 int et_hip_handover_timeouts(uint64_t* count) {
@@ -919,7 +825,7 @@ int et_hip_handover_timeouts(uint64_t* count) {
 }
 
 void et_hip_test_set_handover_spin_limit(uint32_t limit) {
-    et::handover_set_spin_limit(limit == ET_HANDOVER_DEFAULT_SPIN_LIMIT ? et::kHandoverSpinLimit : limit);
+    et::handover_set_spin_limit(limit == ET_HIP_HANDOVER_DEFAULT_SPIN_LIMIT ? et::kHandoverSpinLimit : limit);
 }
 
 }  // extern "C"

@@ -816,6 +816,7 @@ hipError_t gemm_h16_group(int32_t codec, const GemmMember* members, uint32_t cou
     return launch_group<kQ4_K, 2, 2, 3>(members, count, tiles, partials, columns, vectors, g.k_splits, stream, leave_shares, rotary);
 }
 
+#ifdef ET_HIP_CALIBRATE  // the measurement library's build of this file: the kernel minus one part, per probe
 hipError_t gemm_h16_probe(int probe, const uint8_t* weight, const uint8_t* tiles, float* y, uint64_t rows,
                           uint64_t columns, uint64_t vectors, hipStream_t stream) {
     if (!gemm_h16_supported(kQ4_K, columns) || rows == 0 || rows > 0xffffffffull || vectors == 0 || vectors > 32)
@@ -845,6 +846,7 @@ hipError_t gemm_h16_probe(int probe, const uint8_t* weight, const uint8_t* tiles
     };
     return vectors <= 16 ? run(std::true_type{}) : run(std::false_type{});
 }
+#endif
 
 hipError_t gemm_h16(int32_t codec, const uint8_t* weight, const uint8_t* tiles, const GemmOutput& out,
                     uint64_t rows, uint64_t columns, uint64_t vectors, hipStream_t stream) {

@@ -1180,6 +1180,11 @@ bool dma_takes(uint32_t rows, uint32_t columns, uint32_t* rows_per_wg) {
     // first instructions, is the faster one (Q8_0 4096 x 4096, two rows to a range: 5.1 against 5.5 us).
     if (share < 4u * kDmaPairs) return false;
     const uint64_t row_bytes = (static_cast<uint64_t>(columns) / T::kBlockColumns) * T::kBlockBytes;
+    // A loader lane copies 16 bytes: rows that are not whole 16-byte pieces (Q2_K unless columns % 1024 == 0,
+    // Q4_0 / Q8_0 unless columns % 256 == 0) would let the last lane of a range read up to 12 bytes past it -
+    // for the last range of the matrix, past the weight buffer. Those widths stay on gemv_limb_kernel,
+    // which reads exact dwords.
+    if (row_bytes % 16u != 0u) return false;
     const uint64_t per_pair = (share + kDmaPairs - 1u) / kDmaPairs;
     const uint64_t range_bytes = ((per_pair * row_bytes + 1023u) / 1024u) * 1024u;  // as laid out in LDS
     const uint64_t stage_at = kDmaControlAt - M * sizeof(StageMemory);

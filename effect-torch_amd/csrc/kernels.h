@@ -186,7 +186,7 @@ GemmShares gemm_h16_shares_layout(int32_t codec, uint64_t rows, uint64_t columns
 // ---- kv_attention.hip: paged key/value-cache attention ---------------------------
 constexpr int kKvTableEntries = 1024;     // blocks one context split of the streaming kernel may touch
 constexpr int kKvAnyWidthPerLane = 8;     // the any-width kernel covers head widths up to 64 * 8
-// The device status block holds one word per slot: 0, or code << 32 | value.
+// The device status block holds one word per slot: 0, or code << 56 | value (56 bits of value).
 enum : uint32_t {
     kKvBadAdvance = 1,    // value = the advance
     kKvOverCapacity = 2,  // value = live context

@@ -285,6 +285,7 @@ const char* kernel_name(const et_linear_plan& plan) {
 int linear_requirements(const TensorView& input, const TensorView& weight, const TensorView* bias,
                         int32_t codec, uint64_t rows, uint64_t columns, int32_t activation_mode,
                         et_linear_plan* plan, std::string* error) {
+    warm_device_symbols();
     if (input.dtype != ET_DTYPE_F32 || input.shape.size() < 2)
         return fail(error, ET_ERR_UNSUPPORTED, "quantized_linear: input must be rank >= 2 f32");
     if (input.shape.back() != columns)
@@ -326,6 +327,7 @@ int linear_requirements(const TensorView& input, const TensorView& weight, const
 int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
                            bool has_bias, int32_t activation_mode, et_linear_plan* plan,
                            std::string* error) {
+    warm_device_symbols();
     TensorView input;
     input.dtype = ET_DTYPE_F32;
     input.shape = {vectors, columns};

@@ -78,6 +78,10 @@ namespace quantized {
 int linear_requirements(const TensorView& input, const TensorView& weight, const TensorView* bias,
                         int32_t codec, uint64_t rows, uint64_t columns, int32_t activation_mode,
                         et_linear_plan* plan, std::string* error);
+// Resolves the device addresses of the library's own device symbols on the current device (a no-op
+// without a device). Called when a plan is made, so that no launch has to do it - a launch may be
+// recorded into a stream capture, where such a lookup does not belong.
+void warm_device_symbols();
 int linear_plan_from_sizes(int32_t codec, uint64_t rows, uint64_t columns, uint64_t vectors,
                            bool has_bias, int32_t activation_mode, et_linear_plan* plan,
                            std::string* error);

@@ -16,6 +16,7 @@
 #include <string>
 
 #include "et_hip.h"
+#include "lds_handover.h"
 #include "quantized.h"
 
 static __device__ __align__(256) uint8_t scratch[ET_HIP_STATIC_WORKSPACE_BYTES];
@@ -60,6 +61,22 @@ int scratch_pointer(uint8_t** out, std::string* error) {
 }  // namespace
 
 namespace quantized {
+
+void warm_device_symbols() {
+    // Looks up, outside any stream capture, the device addresses that launches need later: the static
+    // workspace's and the hand-over status word's (hipGetSymbolAddress may load the code object).
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();  // no device: plans can still be made (and checked) on the host
+        return;
+    }
+    uint8_t* pointer = nullptr;
+    std::string ignored;
+    (void)scratch_pointer(&pointer, &ignored);
+    HandoverState handover;
+    (void)handover_state(&handover);
+    (void)hipGetLastError();
+}
 
 int linear_enqueue_static_workspace(const et_linear_plan& plan, const float* x, uint64_t x_row_stride,
                                     const uint8_t* weight, const float* bias, float* y, void* stream,

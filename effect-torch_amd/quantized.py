@@ -94,6 +94,12 @@ def _check(status: int) -> None:
     raise QuantizedError(status, message)
 
 
+def _check_calibration(status: int) -> None:
+    """:func:`_check` for the measurement library, which keeps its own error message."""
+    if status != N.OK:
+        raise QuantizedError(status, (N.calibrate_lib().et_hip_calibration_last_error() or b"").decode())
+
+
 class _Desc:
     """Keeps the ctypes arrays of an ``et_tensor`` alive."""
 
@@ -579,7 +585,7 @@ def set_handover_spin_limit(limit: int = HANDOVER_DEFAULT_SPIN_LIMIT) -> None:
 def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """Plain streaming read of ``src`` (measurement aid, ``et_hip_calibration_read``)."""
     assert sink.numel() >= 4 * workgroups and sink.element_size() == 4
-    _check(N.lib().et_hip_calibration_read(src.data_ptr(), src.numel() * src.element_size(),
+    _check_calibration(N.calibrate_lib().et_hip_calibration_read(src.data_ptr(), src.numel() * src.element_size(),
                                            sink.data_ptr(), workgroups, _stream_handle(stream)))
 
 
@@ -589,14 +595,14 @@ READ_VARIANTS = {"plain": 0, "deep": 1, "streaming": 2, "lds4": 3, "lds8": 4}
 def calibration_read_variant(variant: str, src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:
     """The streaming read by one of several kernels (measurement aid, ``et_hip_calibration_read_variant``)."""
     assert sink.numel() >= max(4 * workgroups, 1024) and sink.element_size() == 4
-    _check(N.lib().et_hip_calibration_read_variant(READ_VARIANTS[variant], src.data_ptr(),
+    _check_calibration(N.calibrate_lib().et_hip_calibration_read_variant(READ_VARIANTS[variant], src.data_ptr(),
                                                    src.numel() * src.element_size(), sink.data_ptr(), workgroups,
                                                    _stream_handle(stream)))
 
 
 def calibration_copy(src: torch.Tensor, dst: torch.Tensor, stream=None) -> None:
     """Plain copy ``dst <- src`` (measurement aid, ``et_hip_calibration_copy``)."""
-    _check(N.lib().et_hip_calibration_copy(src.data_ptr(), dst.data_ptr(),
+    _check_calibration(N.calibrate_lib().et_hip_calibration_copy(src.data_ptr(), dst.data_ptr(),
                                            src.numel() * src.element_size(), _stream_handle(stream)))
 
 
@@ -617,7 +623,7 @@ def calibration_contraction(probe: str, plan: "RawLinear", weight: torch.Tensor,
     plan._holds("prepared input", prepared, plan.prepared_input_bytes)
     plan._check_weight(weight)
     plan._check_output(y)
-    _check(N.lib().et_hip_calibration_contraction(CONTRACTION_PROBES[probe], weight.data_ptr(), prepared.data_ptr(),
+    _check_calibration(N.calibrate_lib().et_hip_calibration_contraction(CONTRACTION_PROBES[probe], weight.data_ptr(), prepared.data_ptr(),
                                                   y.data_ptr(), plan.rows, plan.columns, plan.vectors,
                                                   _stream_handle(stream)))
 
@@ -627,5 +633,5 @@ def calibration_mfma(kind: str, iterations: int, sink: torch.Tensor, stream=None
     aid, ``et_hip_calibration_mfma``); ``sink`` is f32 with 256 elements per workgroup."""
     if sink.dtype != torch.float32 or sink.numel() % 256 != 0 or sink.numel() == 0:
         raise ValueError("calibration_mfma: sink must be f32 with a multiple of 256 elements")
-    _check(N.lib().et_hip_calibration_mfma(MFMA_KINDS[kind], iterations, sink.numel() // 256, sink.data_ptr(),
+    _check_calibration(N.calibrate_lib().et_hip_calibration_mfma(MFMA_KINDS[kind], iterations, sink.numel() // 256, sink.data_ptr(),
                                            _stream_handle(stream)))

@@ -83,7 +83,10 @@ typedef enum {
     ET_ACT_F32 = 0, /* f32 activations, f32 accumulate; tolerance 1e-3 against the CPU path */
     ET_ACT_INT8 = 1 /* activations quantised on the fly to int8 per 32 columns with an f32
                        absmax scale, int8 MFMA, f32 block-scale epilogue; tolerance 2e-2.
-                       The reference has no such mode. */
+                       The reference has no such mode. Codecs: Q8_0, Q4_0 and Q4_K (whole
+                       256-column stages); a plan for Q2_K, Q3_K, Q5_K or Q6_K in this mode is
+                       refused with ET_ERR_UNSUPPORTED ("int8 activation mode is not available
+                       for ...") - their batches run in ET_ACT_F32. */
 } et_activation_mode;
 
 /* A strided view of caller-owned storage, in ELEMENTS - the reference's Tensor
@@ -174,7 +177,10 @@ int et_hip_linear_enqueue(const et_linear_plan* plan, const float* x, uint64_t x
  * exceeds the array is refused (ET_ERR_UNSUPPORTED, "... the static workspace holds ..."): such
  * callers bring their own workspace to et_hip_linear_enqueue. Every call on a GPU uses the same
  * array: calls that overlap in time on one GPU race on it - serialise them (one stream, or events).
- * Results are those of et_hip_linear_enqueue, bit for bit. */
+ * Results are those of et_hip_linear_enqueue, bit for bit. The array's device address is looked up
+ * when a plan is made on that GPU (et_hip_linear_plan_create / et_hip_linear_requirements), not by
+ * this call, so that the call may be recorded into a stream capture: make the plan, with the GPU
+ * current, before the capture begins. */
 #define ET_HIP_STATIC_WORKSPACE_BYTES (16u << 20)
 int et_hip_linear_enqueue_static_workspace(const et_linear_plan* plan, const float* x, uint64_t x_row_stride,
                                            const uint8_t* weight, const float* bias, float* y, void* stream,
@@ -412,7 +418,6 @@ int et_hip_kv_attention_projected_into(const et_kv_layer* layer, const et_kv_pro
  * (napi/mod.rs:3590-3594). */
 int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
                                      const void* status_host);
-/* Name of the kernel variant these sizes select, for profiles and diagnostics. */
 /* The commit of a step (crates/runtime-cpu/src/napi/mod.rs:4511-4517): cursor += advance for the
  * layer's active slots, on the device, after the step's last attention call - so that a decode loop
  * replays one captured graph per step without a host round trip. Writes layer->cursors (the caller's
@@ -420,6 +425,7 @@ int et_hip_kv_attention_status_check(const et_kv_layer* layer, uint64_t tokens,
  * one call. */
 int et_hip_kv_commit(const et_kv_layer* layer, void* stream);
 
+/* Name of the kernel variant these sizes select, for profiles and diagnostics. */
 const char* et_hip_kv_attention_kernel(const et_kv_layer* layer, uint64_t query_heads,
                                        uint64_t tokens);
 
@@ -596,6 +602,11 @@ const char* et_hip_last_error(void);
  * meaningless). Synchronises with the device. No counterpart in the reference: its kernels have
  * no cross-thread waits. */
 int et_hip_handover_timeouts(uint64_t* count);
+/* Test hook: the number of polls after which a wave gives up such a wait, for the launches that
+ * follow. 0 makes every wait that is not already satisfied give up at once, so that a test can see
+ * every wave leave the kernel; ET_HIP_HANDOVER_DEFAULT_SPIN_LIMIT restores the library's own value. */
+#define ET_HIP_HANDOVER_DEFAULT_SPIN_LIMIT 0xffffffffu
+void et_hip_test_set_handover_spin_limit(uint32_t limit);
 
 #ifdef __cplusplus
 }

@@ -1,9 +1,11 @@
-/* Measurement aids of libet_hip.so: plain reads, a plain copy and matrix-core loops.
+/* Measurement aids: plain reads, a plain copy, matrix-core loops and the batched contraction taken apart.
  *
- * These entry points are exported by the same library as the operator boundary (et_hip.h) but are
- * not part of it: they mirror nothing in the reference and nothing on the operator path calls
- * them. The benchmark uses them to put the rates this device sustains next to the published peaks
- * and to calibrate hardware counters against a known number of bytes.
+ * These entry points live in a library of their own, libet_hip_calibrate.so, apart from the
+ * operator boundary (et_hip.h, libet_hip.so): they mirror nothing in the reference and nothing on
+ * the operator path calls them. The benchmark's calibrate_* workloads and two tests load it to put
+ * the rates this device sustains next to the published peaks and to calibrate hardware counters
+ * against a known number of bytes. Failures return an et_status (et_hip.h); the message is
+ * et_hip_calibration_last_error() on the calling thread.
  */
 #ifndef ET_HIP_CALIBRATE_H
 #define ET_HIP_CALIBRATE_H
@@ -69,12 +71,7 @@ enum { ET_CONTRACTION_WHOLE = 0, ET_CONTRACTION_NO_ARITHMETIC = 1, ET_CONTRACTIO
 int et_hip_calibration_contraction(int32_t probe, const void* weight, const void* prepared, float* y,
                                    uint64_t rows, uint64_t columns, uint64_t vectors, void* stream);
 
-/* Test hook: the number of polls after which a wave of the GEMV kernels gives up a wait on another
- * wave (see et_hip_handover_timeouts), for the launches that follow. 0 makes every wait that is not
- * already satisfied give up at once, so that a test can see every wave leave the kernel;
- * ET_HANDOVER_DEFAULT_SPIN_LIMIT restores the library's own value. */
-#define ET_HANDOVER_DEFAULT_SPIN_LIMIT 0xffffffffu
-void et_hip_test_set_handover_spin_limit(uint32_t limit);
+const char* et_hip_calibration_last_error(void);
 
 #ifdef __cplusplus
 }

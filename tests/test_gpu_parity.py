@@ -255,7 +255,10 @@ def test_linear_few_tiles_share_k_over_workgroups(et, device, mode, codec, vecto
     # decode-batch shapes: far fewer 64-row tiles than compute units, so the stages of K are shared
     # out over several workgroups per tile and summed by a second kernel, in a fixed order
     if codec in (oracle.Q2_K, oracle.Q3_K, oracle.Q5_K, oracle.Q6_K) and mode == "INT8":
-        pytest.skip("the int8-activation mode has no kernel for this codec")
+        # the documented refusal (include/et_hip.h, et_activation_mode): these codecs' batches run in f32 mode
+        with pytest.raises(et.QuantizedError, match="int8 activation mode is not available for"):
+            et.RawLinear(et.GgmlQuant(codec), rows, columns, vectors, True, et.ActivationMode.INT8)
+        return
     rng = np.random.default_rng(rows + columns + vectors)
     weight = synth.random_weight(codec, rows, columns, rng)
     x = synth.random_activations(vectors, columns, rng)
@@ -413,14 +416,27 @@ def test_linear_full_size_q4k_batched_row_ranges(et, device, vectors):
 
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q5_K, oracle.Q8_0, oracle.Q4_0, oracle.Q2_K])
 @pytest.mark.parametrize("vectors,rows,columns", [(1, 2048, 4096), (2, 2100, 4096), (1, 4099, 1024), (2, 5003, 256),
-                                                  (3, 3000, 2048), (1, 30000, 512), (1, 1793, 4096)])
+                                                  (3, 3000, 2048), (1, 30000, 512), (1, 1793, 4096), (1, 8193, 4096),
+                                                  (1, 9000, 1024), (1, 12000, 2048), (1, 14336, 4096), (1, 20000, 768)])
 def test_gemv_with_weights_copied_through_lds(et, device, codec, vectors, rows, columns):
     if columns % 256 and codec not in (oracle.Q8_0, oracle.Q4_0):
         pytest.skip("the K-quants take whole 256-column blocks")
-    # one or two vectors, one slice of columns, eight or more rows per compute unit: the loader waves
-    # copy the workgroup's share of W into LDS and the consumer waves fold it as it lands. Ragged last
-    # shares, shares that end inside a 1 KiB copy, narrow rows, bias; three vectors stay on the
-    # register-streaming kernel and must agree just the same.
+    # One vector, one slice of columns, 32 or more rows per compute unit whose packed bytes fit LDS, rows of
+    # whole 16-byte pieces: the loader waves copy the workgroup's share of W into LDS and the consumer waves
+    # fold it as it lands (gemv_limb_dma). Ragged last shares (8193 rows: a last share of one row), shares
+    # that end inside a 1 KiB copy, narrow rows, bias. The other shapes - fewer rows, more vectors, rows that
+    # are not whole 16-byte pieces (a loader lane copies 16 bytes and must not read past the matrix) - run on
+    # another GEMV kernel and must agree just the same.
+    share = -(-rows // 256)
+    row_bytes = columns // synth.BLOCK_VALUES[codec] * synth.BLOCK_BYTES[codec]
+    # eight ranges of whole KiB below the activation stage (13056 bytes) and the control block (1 KiB)
+    fits = -(-(-(-share // 8) * row_bytes) // 1024) * 1024 * 8 <= 160 * 1024 - 1024 - 13056
+    copied = vectors == 1 and share >= 32 and row_bytes % 16 == 0 and fits
+    plan = et.RawLinear(et.GgmlQuant(codec), rows, columns, vectors, bool(rows % 2))
+    if copied:
+        assert plan.requirements.kernel == "gemv_limb_dma"
+    else:
+        assert plan.requirements.kernel != "gemv_limb_dma"
     rng = np.random.default_rng(codec * 17 + vectors + rows + columns)
     weight = synth.random_weight(codec, rows, columns, rng)
     x = synth.random_activations(vectors, columns, rng)
@@ -634,7 +650,8 @@ def test_k_quant_gemv_at_full_size(et, device, codec, vectors):
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   None, et.GgmlQuant(codec), (rows, columns))
     copied = vectors == 1 and codec == oracle.Q2_K  # shares of 56 rows that fit LDS
-    assert plan.kernel == ("gemv_limb_dma" if copied else "gemv_limb")
+    one_pass = vectors > 1 and codec == oracle.Q5_K  # 2..8 vectors of Q5_K: the small-batch kernel
+    assert plan.kernel == ("gemv_mma" if one_pass else "gemv_limb_dma" if copied else "gemv_limb")
     got = run_linear(et, device, codec, rows, columns, x, weight)
     for start in (0, rows - 128):
         want = oracle.linear_rows(codec, rows, columns, x, weight, None, start, start + 128)[:, start:start + 128]

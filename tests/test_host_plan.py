@@ -16,19 +16,21 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_library_exports_every_declared_symbol(et):
+    # the operator boundary <-> libet_hip.so, the measurement aids <-> libet_hip_calibrate.so: each library
+    # exports what its header declares, and the operators' library carries none of the aids
     from effect_torch_amd import _native
-    declared = set()
-    for name in ("et_hip.h", "et_hip_calibrate.h"):  # the operator boundary, and the measurement aids
-        header = open(os.path.join(ROOT, "include", name)).read()
-        found = set(re.findall(r"\b(et_hip_[a-z0-9_]+)\s*\(", header))
-        assert found, f"no declarations found in {name}"
-        declared |= found
     boundary = open(os.path.join(ROOT, "include", "et_hip.h")).read()
     assert "calibration" not in boundary, "measurement aids belong in et_hip_calibrate.h"
-    lib = _native.lib()
-    for name in sorted(declared):
-        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
-    assert declared == set(_native.SIGNATURES), declared ^ set(_native.SIGNATURES)
+    for name, lib, signatures in (("et_hip.h", _native.lib(), _native.SIGNATURES),
+                                  ("et_hip_calibrate.h", _native.calibrate_lib(), _native.CALIBRATE_SIGNATURES)):
+        header = open(os.path.join(ROOT, "include", name)).read()
+        declared = set(re.findall(r"\b(et_hip_[a-z0-9_]+)\s*\(", header))
+        assert declared, f"no declarations found in {name}"
+        for symbol in sorted(declared):
+            assert hasattr(lib, symbol), f"{symbol} is declared in include/{name} but not exported"
+        assert declared == set(signatures), declared ^ set(signatures)
+    for symbol in _native.CALIBRATE_SIGNATURES:
+        assert not hasattr(_native.lib(), symbol), f"{symbol} belongs in the measurement library"
 
 
 def test_codec_tables(et):

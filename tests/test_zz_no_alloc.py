@@ -54,6 +54,43 @@ def test_static_workspace_entry_point_matches_the_workspace_one(et, device):
     both_ways(et, device, oracle.Q4_K, 4096, 14336, 32, F32, rng, False)
 
 
+def test_static_workspace_entry_point_under_stream_capture(et, device):
+    # What the entry point is for: a caller that records the call into a graph. The plan is made before the
+    # capture (that is when the library looks up the array's device address); the recorded call then
+    # allocates nothing - device memory in use is the same after it - and every replay, with eager work
+    # and synchronisations in between, gives the eager result.
+    rng = np.random.default_rng(22)
+    codec, rows, columns, vectors = oracle.Q4_K, 4096, 4096, 32
+    weight = torch.from_numpy(synth.random_weight(codec, rows, columns, rng)).to(device)
+    x = torch.from_numpy(synth.random_activations(vectors, columns, rng)).to(device)
+    plan = et.RawLinear(et.GgmlQuant(codec), rows, columns, vectors)
+    assert 0 < plan.requirements.workspace_bytes <= et.STATIC_WORKSPACE_BYTES
+    eager = torch.empty((vectors, rows), device=device)
+    plan.enqueue_static_workspace(x, weight, None, eager)  # warm-up, and the result to compare with
+    torch.cuda.synchronize()
+    out = torch.full((vectors, rows), float("nan"), device=device)
+    free_before = torch.cuda.mem_get_info()[0]
+    plan.enqueue_static_workspace(x, weight, None, out)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before  # nothing was allocated
+    assert torch.equal(out, eager)
+    graph = torch.cuda.CUDAGraph()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            plan.enqueue_static_workspace(x, weight, None, out)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        other = torch.empty((9, 1000), device=device)  # eager work in between, on the same array
+        small = et.RawLinear(et.GgmlQuant(codec), 1000, columns, 9)
+        small.enqueue_static_workspace(x[:9], weight[:1000], None, other)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay} differs from the eager call"
+
+
 def test_static_workspace_entry_point_refuses_what_does_not_fit(et, device):
     # 2048 vectors of 14336 columns need 120 MiB of tiles: more than the array holds
     plan = et.RawLinear(et.GgmlQuant.Q4_K, 256, 14336, 2048)
