@@ -4,7 +4,7 @@
 // Same contraction as linear_into (crates/runtime-cpu/src/quantized.rs:419-499) with decode_q4_k
 // (:180-199) and decode_q5_k (:203-234) in factored form; Q4_0 and Q8_0 follow the public ggml block layouts. The reference's own GPU
 // backend keeps 2..8 vectors in its GEMV family (crates/runtime-metal/src/quantized.rs:1204-1220).
-// f32-accurate (24-bit fixed-point activations, exact integer dots).
+// f32-accurate (23-bit fixed-point activations per 256 columns, exact integer dots).
 //
 // The kernel is HBM-bound and streams W exactly once, whatever the number of vectors. What a few
 // vectors cost on v_dot4 (gemv_limb.hip: 48 dots per vector, row and lane) is here one matrix
@@ -44,7 +44,11 @@ namespace {
 constexpr int kConsumers = 8;
 constexpr uint32_t kLdsBytes = 160u * 1024u;
 constexpr uint32_t kGroupRows = 16u;    // rows of W per matrix instruction
-constexpr float kLimbRange = 8323072.0f;  // 127 * 2^16: |X| <= this
+// Activations as fixed point: X = rint(x * kLimbRange / max|x|), |X| < 2^22. Adding kLimbMagic to the
+// scaled value makes the float's mantissa the integer X + 0x408080 (the sum lies in [2^23, 2^24), where
+// floats are the integers): one fused multiply-add quantises, rounds to nearest even and offsets.
+constexpr float kLimbRange = 4161000.0f;                // X + 0x8080 stays below 2^22 with room for the reciprocal's ulp
+constexpr float kLimbMagic = 12582912.0f + 32896.0f;    // 1.5 * 2^23 + 0x8080
 
 constexpr uint32_t kMostGroups = 4u;    // groups of a range: its rows' partial sums wait in LDS for the end
 
@@ -90,8 +94,10 @@ __device__ __forceinline__ long pack(uint32_t low, uint32_t high) {
     return static_cast<long>((static_cast<uint64_t>(high) << 32) | low);
 }
 
-// 4x3 byte transpose: limb k of four 24-bit values (already + 0x8080) into one dword each. The two
-// low bytes are offset digits (flip the top bit to get the signed limb), the third is signed as it is.
+// 4x3 byte transpose: limb k of four 23-bit values X + 0x408080 (the low three bytes of the words) into
+// one dword each. With X = 65536 l2 + 256 l1 + l0 in balanced digits (l0, l1 in [-128, 127], l2 in
+// [-64, 63]) the bytes are l0 + 128, l1 + 128 and l2 + 64: flipping the top bit gives the signed limb,
+// for the third after another 64 (no byte carries: it is below 128).
 __device__ __forceinline__ void split_quad(int x0, int x1, int x2, int x3, uint32_t (&limb)[3]) {
     const uint32_t a = __builtin_amdgcn_perm(x1, x0, 0x05010400u);  // x0.b0 x1.b0 x0.b1 x1.b1
     const uint32_t b = __builtin_amdgcn_perm(x3, x2, 0x05010400u);
@@ -99,7 +105,7 @@ __device__ __forceinline__ void split_quad(int x0, int x1, int x2, int x3, uint3
     const uint32_t d = __builtin_amdgcn_perm(x3, x2, 0x0c0c0602u);
     limb[0] = __builtin_amdgcn_perm(b, a, 0x05040100u) ^ 0x80808080u;
     limb[1] = __builtin_amdgcn_perm(b, a, 0x07060302u) ^ 0x80808080u;
-    limb[2] = __builtin_amdgcn_perm(d, c, 0x05040100u);
+    limb[2] = (__builtin_amdgcn_perm(d, c, 0x05040100u) + 0x40404040u) ^ 0x80808080u;
 }
 
 // ---------------------------------------------------------------------------
@@ -362,26 +368,29 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
         const uint32_t loader = wave - kConsumers;
         const uint32_t copies = (image_bytes + 1023u) >> 10;
         const uint32_t mine = copies > loader ? (copies - loader + LOADERS - 1u) / LOADERS : 0u;
-        // where this lane's 16 bytes of the wave's next copy lie in the image
+        // where this lane's 16 bytes of the wave's next copy lie in the image, and in W (from the range's first byte)
         uint32_t at = loader * 1024u + lane_id * 16u;
         uint32_t row = at / pitch, column = at - row * pitch;
-        constexpr uint32_t kStep = LOADERS * 1024u;
+        uint32_t from = row * row_bytes + column;
+        constexpr uint32_t kStep = LOADERS * 1024u;  // between two copies of a wave
         const uint32_t step_rows = kStep / pitch, step_columns = kStep - step_rows * pitch;
+        const uint32_t step_from = step_rows * row_bytes + step_columns;
+        const uint32_t end = wg_rows * row_bytes;  // rows past the range start there
         const uint8_t* source = weight + static_cast<uint64_t>(wg_row0) * row_bytes;
         const uint32_t landed_address = lds_address(&control->landed[loader]);
         uint32_t next = loader;  // number of the wave's next copy
         const auto copy = [&]() {
             // never a copy without a lane: the image ends with bytes of W and padding is shorter than a copy
-            if (PROBE != 2 && PROBE != 3 && row < wg_rows && column < row_bytes)
+            if (PROBE != 2 && PROBE != 3 && column < row_bytes && from < end)
                 // streamed once: non-temporal (aux bit 1), the caches keep nothing of it
-                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + row * row_bytes + column),
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + from),
                                                  reinterpret_cast<uint4*>(lds + next * 1024u), 16, 0, 2);
             next += LOADERS;
-            row += step_rows;
             column += step_columns;
-            if (column >= pitch) {
+            from += step_from;
+            if (column >= pitch) {  // into the next row: its padding is not in W
                 column -= pitch;
-                row += 1u;
+                from += row_bytes - pitch;
             }
         };
         // The first copies wait for the barrier, i.e. until the consumers have issued their activation
@@ -436,7 +445,7 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     __syncthreads();  // the only barrier: the counters are zero before anybody counts
     ET_STAMP(1);
 
-    // 24-bit fixed point per vector and 256-column unit, X = rint(x * 127 * 2^16 / max|x|), in three
+    // 23-bit fixed point per vector and 256-column unit, X = rint(x * kLimbRange / max|x|), in three
     // balanced signed-byte limbs; the limbs go through the wave's scratch into the lanes that hold
     // them as A operands: lane l, as row l % 16 = 4 * vector + limb, K index l / 16.
     long a[VG][16];
@@ -448,8 +457,10 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     for (int v = 0; v < VEC; v++) {
         if (static_cast<uint32_t>(v) >= vectors) break;
         const float4 f0 = xv[v][0], f1 = xv[v][1];
-        float amax = fmaxf(fmaxf(fmaxf(fabsf(f0.x), fabsf(f0.y)), fmaxf(fabsf(f0.z), fabsf(f0.w))),
-                           fmaxf(fmaxf(fabsf(f1.x), fabsf(f1.y)), fmaxf(fabsf(f1.z), fabsf(f1.w))));
+        float amax = fmaxf(fmaxf(fabsf(f0.x), fabsf(f0.y)), fabsf(f0.z));  // three-input maxima
+        amax = fmaxf(fmaxf(amax, fabsf(f0.w)), fabsf(f1.x));
+        amax = fmaxf(fmaxf(amax, fabsf(f1.y)), fabsf(f1.z));
+        amax = fmaxf(amax, fabsf(f1.w));
         amax = fmaxf(amax, dpp<0xB1>(amax));   // quad_perm [1,0,3,2]
         amax = fmaxf(amax, dpp<0x4E>(amax));   // quad_perm [2,3,0,1]
         amax = fmaxf(amax, dpp<0x141>(amax));  // row_half_mirror
@@ -458,15 +469,15 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
         float total = ((f0.x + f0.y) + (f0.z + f0.w)) + ((f1.x + f1.y) + (f1.z + f1.w));
         total += dpp<0xB1>(total);
         total += dpp<0x4E>(total);  // the block's 32 columns
-        // 1 ulp of the reciprocal moves |X| by at most 1, far inside the headroom of the limbs.
+        // 1 ulp of the reciprocal moves |X| by at most 1, far inside the headroom of the range.
         const bool nonzero = amax >= 1e-30f;
         const float inv = nonzero ? kLimbRange * __builtin_amdgcn_rcpf(amax) : 0.f;
         const float unit = nonzero ? amax * (1.0f / kLimbRange) : 0.f;
         uint32_t low[3], high[3];
-        split_quad(static_cast<int>(rintf(f0.x * inv)) + 0x8080, static_cast<int>(rintf(f0.y * inv)) + 0x8080,
-                   static_cast<int>(rintf(f0.z * inv)) + 0x8080, static_cast<int>(rintf(f0.w * inv)) + 0x8080, low);
-        split_quad(static_cast<int>(rintf(f1.x * inv)) + 0x8080, static_cast<int>(rintf(f1.y * inv)) + 0x8080,
-                   static_cast<int>(rintf(f1.z * inv)) + 0x8080, static_cast<int>(rintf(f1.w * inv)) + 0x8080, high);
+        split_quad(__float_as_int(fmaf(f0.x, inv, kLimbMagic)), __float_as_int(fmaf(f0.y, inv, kLimbMagic)),
+                   __float_as_int(fmaf(f0.z, inv, kLimbMagic)), __float_as_int(fmaf(f0.w, inv, kLimbMagic)), low);
+        split_quad(__float_as_int(fmaf(f1.x, inv, kLimbMagic)), __float_as_int(fmaf(f1.y, inv, kLimbMagic)),
+                   __float_as_int(fmaf(f1.z, inv, kLimbMagic)), __float_as_int(fmaf(f1.w, inv, kLimbMagic)), high);
         asm volatile("" ::: "memory");  // the reads of the vector before are done with the planes
 #pragma unroll
         for (int k = 0; k < 3; k++)
