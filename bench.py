@@ -41,9 +41,17 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # When either differs from what runs now, `roofline.traffic` is null until the profile is re-taken.
 MEASURED_TRAFFIC = {
     ("q4_k_gemv_14336x4096", 1, "f32"): {
-        "bytes": 33316300, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
-        "sha256": "c97830386ce6b1bbaa1f8903e935411df72db510501e31dcf2e961dfcea3d1d8",
+        "bytes": 33315000, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
+        "sha256": "04f8f05ea8735a1c4f7d99d5a64519ec8b5e4cfaae344241ac54612d96a88da2",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
+    ("q4_k_gemv_14336x4096", 4, "f32"): {
+        "bytes": 33895000, "kernel": "gemv_mma", "source": "gemv_mma.hip",
+        "sha256": "7a5f713f6923c9fcdfce7e5f2ca29da604d0f069669b3f2b769e23a27a7233fa",
+        "profile": "profiles/gemv_mma_small_batch_2_to_8_vectors.md"},
+    ("q4_k_gemv_14336x4096", 8, "f32"): {
+        "bytes": 34757400, "kernel": "gemv_mma", "source": "gemv_mma.hip",
+        "sha256": "7a5f713f6923c9fcdfce7e5f2ca29da604d0f069669b3f2b769e23a27a7233fa",
+        "profile": "profiles/gemv_mma_small_batch_2_to_8_vectors.md"},
     ("kv_attention_decode", 2048): {
         "bytes": 270024900, "kernel": "kv_attend", "source": "kv_attention.hip",
         "sha256": "590105a686a613206e4bfe632266890d8f03aa1f6a00829b1aa81122a1f041fd",
