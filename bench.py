@@ -999,6 +999,61 @@ def decode_leg(args, et):
             "leg_wall_s": round(time.perf_counter() - t0, 1)}
 
 
+BASELINE_CONFIGS = [
+    # (BASELINE.json config, arguments after `python bench.py`)
+    ("0: Q8_0 4096x4096, M=1", ["--workload", "q8_0_gemv_4096x4096", "--vectors", "1"]),
+    ("1: Q4_0 11008x4096, M=1", ["--workload", "q4_0_gemv_11008x4096", "--vectors", "1"]),
+    ("1: Q4_0 11008x4096, M=4", ["--workload", "q4_0_gemv_11008x4096", "--vectors", "4"]),
+    ("1: Q4_0 11008x4096, M=8", ["--workload", "q4_0_gemv_11008x4096", "--vectors", "8"]),
+    ("2: Q4_K 14336x4096, M=1 (headline)", ["--workload", "q4_k_gemv_14336x4096", "--vectors", "1"]),
+    ("2: Q4_K 14336x4096, M=16", ["--workload", "q4_k_gemv_14336x4096", "--vectors", "16"]),
+    ("2: Q4_K 14336x4096, M=64", ["--workload", "q4_k_gemv_14336x4096", "--vectors", "64"]),
+    ("3: Q8_0 4096x14336, M=512, int8 activations", ["--workload", "q8_0_gemm_i8_512x14336x4096", "--vectors", "512"]),
+    ("4: Llama-3-8B-shaped batched decode, 32 x 2048, 128 steps", ["--workload", "llama3_8b_batched_decode"]),
+    ("f-1: paged KV attention, 32 slots, context 2048, f16", ["--workload", "kv_attention_decode"]),
+]
+
+
+def baseline_configs(args):
+    """Workload ``baseline_configs``: every BASELINE configuration (and the attention kernel) as the driver
+    would run it - one ``python bench.py ... --steps 20 --warmup 5 --no-cpu`` process each, one after the
+    other - gathered into one markdown table (stdout) with the JSON lines behind it; what
+    ``profiles/baseline_configs.md`` is made from."""
+    import hashlib
+    import subprocess
+
+    lines, table = [], []
+    for label, extra in BASELINE_CONFIGS:
+        decode = "llama3" in extra[1]
+        command = [sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--no-cpu", "--no-decode"] + extra
+        if not decode:
+            command += ["--steps", "20", "--warmup", "5"]
+        done = subprocess.run(command, capture_output=True, text=True, timeout=600)
+        text = [line for line in done.stdout.splitlines() if line.startswith("{")]
+        if done.returncode != 0 or not text:
+            table.append(f"| {label} | failed (exit {done.returncode}) | | | | |")
+            continue
+        result = json.loads(text[-1])
+        lines.append(text[-1])
+        roofline = result["roofline"]
+        unit = roofline.get("unit", "")
+        kernel = roofline.get("kernel", "")
+        table.append(f"| {label} | `{' '.join(extra)}` | {kernel} | {result['ms_per_step'] * 1e3:.2f} "
+                     f"({(result.get('ms_per_step_min') or 0) * 1e3:.2f} - {(result.get('ms_per_step_max') or 0) * 1e3:.2f}) | "
+                     f"{result['value']} {result['unit']} | {roofline['achieved']} {unit} = {roofline['frac']:.4f} of {roofline['peak']:g} |")
+    sources = sorted(name for name in os.listdir(os.path.join(ROOT, "effect-torch_amd", "csrc")) if name.endswith(".hip"))
+    digest = hashlib.sha256()
+    for name in sources:
+        with open(os.path.join(ROOT, "effect-torch_amd", "csrc", name), "rb") as source:
+            digest.update(source.read())
+    print("| BASELINE config | arguments (after `python bench.py --gpus 1 --no-cpu --no-decode`, plus `--steps 20 --warmup 5`) | kernel | us per step (min - max of the timed replays) | value | roofline |")
+    print("|---|---|---|---|---|---|")
+    print("\n".join(table))
+    print(f"\nSHA-256 over the kernel sources (effect-torch_amd/csrc/*.hip, in name order): {digest.hexdigest()}; {cpu_model()}\n")
+    for line in lines:
+        print(line)
+
+
 def gguf_upload(args, et):
     """Workload ``gguf_upload``: a synthetic GGUF v3 file with the tensor catalog of a Llama-3-8B Q4_K
     model (291 tensors; ``--layers`` of them carry payloads, the default 4 make a 0.5 GB file) is
@@ -1114,6 +1169,9 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
               file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "baseline_configs":
+        return baseline_configs(args)
 
     import numpy as np
     import torch

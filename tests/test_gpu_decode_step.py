@@ -41,7 +41,7 @@ def tiled_rows(base, rows):
 
 
 class Model:
-    def __init__(self, et, device, layers, slots, fused):
+    def __init__(self, et, device, layers, slots, fused, contexts=(40, 200)):
         rng = np.random.default_rng(0x11A3A + layers)
         self.shape = shape = et.LlamaShape(layers=layers)
         self.shapes = shapes = shape.linear_shapes()
@@ -63,7 +63,7 @@ class Model:
         self.embedding_base = rng.standard_normal((4096, shape.hidden)).astype(np.float16)  # row t = base[t % 4096]
         block = 16
         self.block = block
-        self.contexts = rng.integers(40, 200, slots).astype(np.uint32)
+        self.contexts = rng.integers(contexts[0], contexts[1], slots).astype(np.uint32)
         self.max_context = int(self.contexts.max()) + STEPS
         blocks_per_slot = -(-self.max_context // block)
         total_blocks = slots * blocks_per_slot + 5
@@ -107,12 +107,14 @@ class Model:
                                                                          self.linear("up", layer, h))))
 
 
-@pytest.mark.parametrize("fused,slots", [(True, 32), (False, 32), (True, 12)],
-                         ids=["fused", "one_operator_per_launch", "fused_12_slots"])
-def test_decode_steps_follow_the_oracle_chain(et, device, fused, slots):
-    # 12 slots: the contractions' narrow tile, attention workgroups of four waves with the context split
+@pytest.mark.parametrize("fused,slots,contexts", [(True, 32, (40, 200)), (False, 32, (40, 200)), (True, 12, (40, 200)),
+                                                  (True, 32, (2030, 2060))],
+                         ids=["fused", "one_operator_per_launch", "fused_12_slots", "fused_context_2048"])
+def test_decode_steps_follow_the_oracle_chain(et, device, fused, slots, contexts):
+    # 12 slots: the contractions' narrow tile, attention workgroups of four waves with the context split;
+    # contexts around 2048: the end-to-end configuration's cache length (130 blocks of 16 per slot)
     layers = 2
-    model = Model(et, device, layers, slots, fused)
+    model = Model(et, device, layers, slots, fused, contexts)
     dec, shape = model.decoder, model.shape
     if fused:
         assert dec.on_the_fly, "the Q4_K plans of these shapes take their inputs on the fly"

@@ -414,6 +414,20 @@ def test_linear_full_size_q4k_batched_row_ranges(et, device, vectors):
     close(y12, got.astype(np.float64) + y2, 2e-3)
 
 
+@pytest.mark.parametrize("vectors", [16, 64])
+def test_linear_full_size_q4k_batched_whole_matrix(et, device, vectors):
+    # config 2 at M = 16 and 64, every output: against the oracle (the reference's scalar loop: a few seconds of
+    # one host core) and, with no allowance, against the f64-exact value of the same contraction
+    cfg = synth.CONFIGS["q4_k_gemv_14336x4096"]
+    rng = np.random.default_rng(cfg["seed"] + 2000 + vectors)
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(vectors, cfg["columns"], rng)
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight)
+    close(got, oracle.linear_into(cfg["codec"], cfg["rows"], cfg["columns"], x, weight))
+    exact = x.astype(np.float64) @ oracle.decode_rows(cfg["codec"], weight, cfg["columns"]).astype(np.float64).T
+    close(got, exact, oracle_noise=0)
+
+
 @pytest.mark.parametrize("codec", [oracle.Q4_K, oracle.Q5_K, oracle.Q8_0, oracle.Q4_0, oracle.Q2_K])
 @pytest.mark.parametrize("vectors,rows,columns", [(1, 2048, 4096), (2, 2100, 4096), (1, 4099, 1024), (2, 5003, 256),
                                                   (3, 3000, 2048), (1, 30000, 512), (1, 1793, 4096), (1, 8193, 4096),
@@ -536,6 +550,18 @@ def test_int8_full_size_prefill_row_ranges(et, device):
         want = oracle.linear_q8_rows(cfg["codec"], cfg["rows"], cfg["columns"], q, scale, total, weight,
                                      None, begin, begin + 16)
         close(got[:, begin:begin + 16], want[:, begin:begin + 16])
+
+
+def test_int8_full_size_prefill_whole_matrix(et, device):
+    # config 3, every one of the 512 x 4096 outputs against the oracle's int8 path (15 s of one host core)
+    cfg = synth.CONFIGS["q8_0_gemm_i8_512x14336x4096"]
+    rng = np.random.default_rng(cfg["seed"] + 1)
+    weight = synth.random_weight(cfg["codec"], cfg["rows"], cfg["columns"], rng)
+    x = synth.random_activations(512, cfg["columns"], rng, cfg["x_scale"])
+    got = run_linear(et, device, cfg["codec"], cfg["rows"], cfg["columns"], x, weight, None, et.ActivationMode.INT8)
+    q, scale, total = oracle.quantize_q8(x)
+    want = oracle.linear_q8_rows(cfg["codec"], cfg["rows"], cfg["columns"], q, scale, total, weight, None, 0, cfg["rows"])
+    close(got, want)
 
 
 def test_int8_full_size_prefill_against_the_f32_reference(et, device, capsys):
