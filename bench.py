@@ -141,6 +141,8 @@ def parse_args():
     p.add_argument("--no-decode", action="store_true", help="headline workload: skip the batched-decode leg that fills "
                                                             "the line's `decode` object")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
+    p.add_argument("--sizes-mib", default=None, help="calibrate_read_sweep: comma-separated sizes in MiB instead of "
+                   "8 ... 1024 (the headline weight's size is always measured as well)")
     args = p.parse_args()
     decode = args.workload == "llama3_8b_batched_decode"
     if args.steps is None:
@@ -330,9 +332,13 @@ def calibrate_read_sweep(args, et):
     sink = torch.zeros(4 * 4096, dtype=torch.int32, device=device)
     headline = 14336 * 2304
     sizes = [8 << 20, 16 << 20, headline, 64 << 20, 128 << 20, 256 << 20, 512 << 20, 1024 << 20]
+    if args.sizes_mib:
+        sizes = sorted({int(float(m) * (1 << 20)) for m in args.sizes_mib.split(",")} | {headline})
+    at_headline = sizes.index(headline)
     # (variant, workgroups): the LDS kernels hold a whole compute unit's LDS, one workgroup each
     kernels = [("plain", 512), ("plain", 2048), ("deep", 512), ("deep", 1024), ("streaming", 1024), ("lds4", 256),
-               ("lds8", 256)]
+               ("lds8", 256), ("lds8_nt", 256), ("lds8_nt_shallow", 256), ("lds8_nt_ranges", 256),
+               ("lds8_nt_ranges_shallow", 256)]
     table, fits = [], []
     for variant, workgroups in kernels:
         times = []
@@ -352,7 +358,7 @@ def calibrate_read_sweep(args, et):
         fits.append({"kernel": f"{variant} x{workgroups}", "t0_us": round(t0 * 1e6, 3),
                      "BW_GBps": round(1.0 / slope / 1e9, 1),
                      "predicted_us_at_headline_bytes": round((t0 + headline * slope) * 1e6, 3),
-                     "measured_us_at_headline_bytes": round(times[2] * 1e6, 3)})
+                     "measured_us_at_headline_bytes": round(times[at_headline] * 1e6, 3)})
     best = min(fits, key=lambda f: f["measured_us_at_headline_bytes"])
     gbs = headline / (best["measured_us_at_headline_bytes"] * 1e-6) / 1e9
     print(json.dumps({

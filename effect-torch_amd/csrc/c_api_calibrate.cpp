@@ -63,8 +63,8 @@ int et_hip_calibration_read_variant(int32_t variant, const void* src, uint64_t b
                                     uint32_t workgroups, void* stream) {
     return guarded([&](std::string* error) -> int {
         if (src == nullptr || sink == nullptr || workgroups == 0 || workgroups > 65536 || (bytes >> 36) != 0 ||
-            reinterpret_cast<uintptr_t>(src) % 16 != 0 || variant < ET_READ_PLAIN || variant > ET_READ_LDS_8) {
-            *error = "calibration_read_variant: variant 0..4, source 16-byte aligned, sink non-NULL, "
+            reinterpret_cast<uintptr_t>(src) % 16 != 0 || variant < ET_READ_PLAIN || variant > ET_READ_LDS_8_NT_RANGES_SHALLOW) {
+            *error = "calibration_read_variant: variant 0..8, source 16-byte aligned, sink non-NULL, "
                      "1 <= workgroups <= 65536";
             return ET_ERR_INVALID;
         }

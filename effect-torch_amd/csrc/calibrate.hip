@@ -85,8 +85,10 @@ constexpr int vmcnt_only(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 
 // A read that uses no registers and no arithmetic: every wave only issues 1 KiB global-to-LDS
 // copies into its own ring of DEPTH slots and, once the ring is full, waits for the oldest copy
 // before it issues the next one - DEPTH KiB in flight per wave for the whole launch. One workgroup
-// per compute unit (WAVES * DEPTH = 128 KiB of LDS); workgroup w takes the w-th contiguous range.
-template <int WAVES, int DEPTH>
+// per compute unit (WAVES * DEPTH <= 128 KiB of LDS); workgroup w takes the w-th contiguous range.
+// NT: non-temporal copies (the caches keep nothing of the bytes). RANGES: wave v of a workgroup copies
+// the v-th contiguous part of the workgroup's range instead of every WAVES-th KiB of it.
+template <int WAVES, int DEPTH, bool NT = false, bool RANGES = false>
 __global__ __launch_bounds__(64 * WAVES) void read_lds_kernel(const uint8_t* __restrict__ src, uint32_t kib,
                                                               uint32_t* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) uint8_t ring[];
@@ -96,12 +98,14 @@ __global__ __launch_bounds__(64 * WAVES) void read_lds_kernel(const uint8_t* __r
     const uint32_t begin = blockIdx.x * per_wg;
     const uint32_t end = min(begin + per_wg, kib);
     uint8_t* mine = ring + wave * DEPTH * 1024u;
-    // jobs of this wave: begin + wave, begin + wave + WAVES, ...
-    uint32_t job = begin + wave, slot = 0;
-    for (; job < end; job += WAVES) {
+    const uint32_t per_wave = (per_wg + WAVES - 1) / WAVES;
+    // jobs of this wave: begin + wave, begin + wave + WAVES, ... or a contiguous part of the range
+    uint32_t job = RANGES ? begin + wave * per_wave : begin + wave, slot = 0;
+    const uint32_t last = RANGES ? min(job + per_wave, end) : end;
+    for (; job < last; job += RANGES ? 1u : static_cast<uint32_t>(WAVES)) {
         if (slot >= static_cast<uint32_t>(DEPTH)) __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));  // the slot's last copy has landed
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(src + static_cast<uint64_t>(job) * 1024u + lane * 16u),
-                                         reinterpret_cast<uint4*>(mine + (slot % DEPTH) * 1024u), 16, 0, 0);
+                                         reinterpret_cast<uint4*>(mine + (slot % DEPTH) * 1024u), 16, 0, NT ? 2 : 0);
         slot += 1;
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
@@ -342,6 +346,14 @@ hipError_t calibration_read_variant(int variant, const void* src, uint64_t bytes
     const uint4* quads = static_cast<const uint4*>(src);
     const uint32_t count = static_cast<uint32_t>(bytes / 16);
     constexpr uint32_t kRingBytes = 128u * 1024u;
+    const auto launch_lds = [&](auto kernel, uint32_t waves) -> hipError_t {
+        if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, kRingBytes))
+            return status;
+        hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(64 * waves), kRingBytes, stream,
+                           static_cast<const uint8_t*>(src), static_cast<uint32_t>(bytes / 1024), sink);
+        return hipGetLastError();
+    };
     switch (variant) {
         case kReadPlain: return calibration_read(src, bytes, sink, workgroups, stream);
         case kReadDeep:
@@ -350,24 +362,12 @@ hipError_t calibration_read_variant(int variant, const void* src, uint64_t bytes
         case kReadStreaming:
             hipLaunchKernelGGL((read_deep_kernel<16, true>), dim3(workgroups), dim3(256), 0, stream, quads, count, sink);
             break;
-        case kReadLds4: {
-            const auto kernel = read_lds_kernel<4, 32>;
-            if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRingBytes))
-                return status;
-            hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(256), kRingBytes, stream,
-                               static_cast<const uint8_t*>(src), static_cast<uint32_t>(bytes / 1024), sink);
-            break;
-        }
-        case kReadLds8: {
-            const auto kernel = read_lds_kernel<8, 16>;
-            if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kRingBytes))
-                return status;
-            hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(512), kRingBytes, stream,
-                               static_cast<const uint8_t*>(src), static_cast<uint32_t>(bytes / 1024), sink);
-            break;
-        }
+        case kReadLds4: return launch_lds(read_lds_kernel<4, 32>, 4);
+        case kReadLds8: return launch_lds(read_lds_kernel<8, 16>, 8);
+        case kReadLds8Nt: return launch_lds(read_lds_kernel<8, 16, true>, 8);
+        case kReadLds8NtShallow: return launch_lds(read_lds_kernel<8, 4, true>, 8);
+        case kReadLds8NtRanges: return launch_lds(read_lds_kernel<8, 16, true, true>, 8);
+        case kReadLds8NtRangesShallow: return launch_lds(read_lds_kernel<8, 4, true, true>, 8);
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -146,8 +146,8 @@ __device__ __forceinline__ float limb_value(const XLimbs& x, int d0, int d1, int
 
 struct Q4KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 144u;
-    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
-    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
+    static constexpr bool kLdsCopies = true;     // its weights can come through LDS copies
+    static constexpr bool kCopiesInTurn = true;  // ... on gemv_limb_turns_kernel
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -230,8 +230,8 @@ struct Q4KLimb {
 // sub-block g. 176 bytes per block, every field 16-byte aligned.
 struct Q5KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 176u;
-    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
-    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
+    static constexpr bool kLdsCopies = true;     // its weights can come through LDS copies
+    static constexpr bool kCopiesInTurn = true;  // ... on gemv_limb_turns_kernel
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -326,8 +326,8 @@ struct __attribute__((packed, aligned(4))) Dwords17 {
 // Q4_0: two 18-byte blocks = 36 bytes = 9 dwords (dword aligned when columns % 64 == 0).
 struct Q40Limb {
     static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 18u;
-    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
-    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
+    static constexpr bool kLdsCopies = true;     // its weights can come through LDS copies
+    static constexpr bool kCopiesInTurn = true;  // ... on gemv_limb_turns_kernel
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -387,8 +387,8 @@ struct Q40Limb {
 // Q8_0: two 34-byte blocks = 68 bytes = 17 dwords (dword aligned when columns % 64 == 0).
 struct Q80Limb {
     static constexpr uint32_t kBlockColumns = 32u, kBlockBytes = 34u;
-    static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec
-    static constexpr bool kLoaderFolds = true;   // its loader waves fold the last row of their range (load_limbs_unseen)
+    static constexpr bool kLdsCopies = true;     // its weights can come through LDS copies
+    static constexpr bool kCopiesInTurn = true;  // ... on gemv_limb_turns_kernel
     static __device__ __forceinline__ void load_activations(const StageMemory& stage, uint32_t lane, bool active,
                                                             XLimbs& out) {
         load_limbs(stage, lane, active, out);
@@ -489,7 +489,6 @@ __device__ __forceinline__ void load_run_activations(const StageMemory& stage, u
 struct Q6KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 210u;
     static constexpr bool kLdsCopies = false;    // gemv_limb_kernel only: a share of 14336 rows (56 x 3360 bytes) does not fit LDS
-    static constexpr bool kLoaderFolds = false;
     struct Lane {
         uint32_t offset;  // byte offset of the lane's block within a row
         uint32_t half, j;
@@ -601,7 +600,7 @@ typedef struct __attribute__((packed, aligned(2))) { uint32_t v[3]; } Dwords3_a2
 struct Q2KLimb {
     static constexpr uint32_t kBlockColumns = 256u, kBlockBytes = 84u;
     static constexpr bool kLdsCopies = true;     // gemv_limb_dma_kernel takes this codec; LDS serves the lanes' loads at any alignment
-    static constexpr bool kLoaderFolds = false;  // the loaders only copy: the run-wise activation gather is the consumers'
+    static constexpr bool kCopiesInTurn = false; // ... on gemv_limb_dma_kernel, whose loaders fold the end of their ranges
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -679,7 +678,6 @@ struct Q3KLimb {
     // gemv_limb_kernel only. LDS serves the lanes' 2-byte-aligned 16-byte reads, but slowly: through
     // gemv_limb_dma_kernel 14336 x 4096 measured 10.5 us against 9.6.
     static constexpr bool kLdsCopies = false;
-    static constexpr bool kLoaderFolds = false;
     struct Lane {
         uint32_t offset, half, j;
     };
@@ -943,7 +941,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_limb_kernel(
 // loader keeps DEPTH copies in flight; before it issues the next one it waits for the oldest
 // (loads return in order per wave: one counted s_waitcnt) and publishes in LDS how many of its
 // copies have landed; its consumer polls that one word until it covers the next row.
-// The last row of a range is folded by its loader, which knows first when its last copy has landed.
+// This kernel serves the 2-bit codec, whose folds are long against its bytes: a loader has issued its
+// few copies early and would idle, so once they have all landed it folds the last quarter of its range.
+// The other codecs run on gemv_limb_turns_kernel below.
 // The consumers meet each other through one LDS counter (`staged`).
 // LDS: [the ranges, whole KiB each][...][StageMemory x M][control]; shapes whose ranges would reach
 // into the stages stay on gemv_limb_kernel.
@@ -960,8 +960,6 @@ bool gemv_limb_dma_enabled() {
 constexpr int kDmaPairs = 8;  // ranges of a share: one loader and one consumer wave each (a workgroup has at most
                               // sixteen waves)
 constexpr int kDmaConsumers = kDmaPairs;
-constexpr int kDmaLoaderRows = 1;  // rows at the end of a range that its loader folds (two and three measured slower:
-                                   // a loader that folds is late with the word its consumer waits for)
 constexpr int kDmaDepth = 4;  // copies a loader keeps in flight: more only lengthen the queue, and a loader says that a
                               // copy has landed only when it may issue the copy DEPTH places later
 constexpr int kDmaHead = kDmaDepth;  // copies a loader issues before it does anything else, at most eight
@@ -969,6 +967,9 @@ constexpr int kDmaHead = kDmaDepth;  // copies a loader issues before it does an
                                      // 7.9 and 8.2 against 7.7 us): a longer queue only delays everybody's first rows.
 constexpr uint32_t kDmaLateEighths = 2;  // share of a range that a loader which only copies folds at the end
 constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaPairs);
+constexpr int kTurnConsumers = 11, kTurnLoaders = 5, kTurnDepth = 6;  // gemv_limb_turns_kernel: waves that fold, waves that
+                                                                      // copy, copies in flight per loader
+static_assert(64 * (kTurnConsumers + kTurnLoaders) == kDmaThreads, "sixteen waves either way");
 constexpr uint32_t kDmaLdsBytes = 160u * 1024u;
 struct DmaControl {
     uint32_t landed[kDmaPairs];  // copies of loader w that have landed
@@ -977,36 +978,6 @@ struct DmaControl {
 };
 constexpr uint32_t kDmaControlAt = kDmaLdsBytes - 1024u;
 static_assert(sizeof(DmaControl) == 64, "sixteen words, zeroed by sixteen lanes");
-
-// load_limbs for a wave with copies in flight: the same reads, unseen by the compiler.
-__device__ __forceinline__ void load_limbs_unseen(const StageMemory& stage, uint32_t lane, bool active, XLimbs& out) {
-    typedef uint32_t v4u __attribute__((ext_vector_type(4)));
-#pragma unroll
-    for (int k = 0; k < 3; k++) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            v4u v;
-            asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(lds_address(&stage.limbs[k][limb_slot(4u * lane + j) * 4u])) : "memory");
-            out.limb[k][4 * j + 0] = static_cast<int>(v.x);
-            out.limb[k][4 * j + 1] = static_cast<int>(v.y);
-            out.limb[k][4 * j + 2] = static_cast<int>(v.z);
-            out.limb[k][4 * j + 3] = static_cast<int>(v.w);
-        }
-    }
-    uint32_t unit, sum0, sum1;
-    asm volatile("ds_read_b32 %0, %1" : "=v"(unit) : "v"(lds_address(&stage.unit[lane])) : "memory");
-    asm volatile("ds_read_b32 %0, %1" : "=v"(sum0) : "v"(lds_address(&stage.sum[0][lane])) : "memory");
-    asm volatile("ds_read_b32 %0, %1" : "=v"(sum1) : "v"(lds_address(&stage.sum[1][lane])) : "memory");
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // the values are used only from here on: every register above is written by now
-#pragma unroll
-    for (int k = 0; k < 3; k++)
-#pragma unroll
-        for (int j = 0; j < 16; j++) out.limb[k][j] = active ? out.limb[k][j] : 0;
-    out.s = active ? __uint_as_float(unit) : 0.f;
-    out.sum[0] = active ? __uint_as_float(sum0) : 0.f;
-    out.sum[1] = active ? __uint_as_float(sum1) : 0.f;
-}
 
 template <class T, int M, int DEPTH>
 __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
@@ -1018,10 +989,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     constexpr uint32_t kStageAt = kDmaControlAt - M * static_cast<uint32_t>(sizeof(StageMemory));
     constexpr int NI = kSliceQuads / (64 * kDmaConsumers);  // float4s per consumer thread and vector
     static_assert(DEPTH <= kDmaHead && kDmaHead <= 8, "the steady loop starts with DEPTH copies in flight; wait_copies_in_flight counts to seven");
-    constexpr int kLoaderRows = T::kLoaderFolds ? kDmaLoaderRows : 0;  // rows at the end of a range that its loader folds
-    // Codecs whose fold is long against their bytes (the 2- and 3-bit ones): a loader has issued its few copies
-    // early and would idle; once they have all landed it folds the last kDmaLateEighths / 8 of the range.
-    constexpr bool kLate = !T::kLoaderFolds;
+    static_assert(!T::kCopiesInTurn, "the other codecs run on gemv_limb_turns_kernel");
     DmaControl* control = reinterpret_cast<DmaControl*>(lds + kDmaControlAt);
     StageMemory* stage = reinterpret_cast<StageMemory*>(lds + kStageAt);
 
@@ -1039,7 +1007,7 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     const uint32_t count = min(per_pair, wg_rows - first);
     const uint32_t range_kib = (per_pair * row_bytes + 1023u) >> 10;
     uint8_t* range = lds + pair * (range_kib << 10);
-    const uint32_t late = kLate ? count * kDmaLateEighths / 8u : 0u;  // rows the loader folds after its last copy
+    const uint32_t late = count * kDmaLateEighths / 8u;  // rows the loader folds after its last copy
 
     const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
     const bool active = chunk < columns / kChunk;
@@ -1090,15 +1058,6 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
         __syncthreads();
         const uint32_t head = min(copies, static_cast<uint32_t>(kDmaHead));
         for (uint32_t i = 0; i < head; i++) copy(i);
-        // The loader folds the last row of its range itself (below), next to the consumer folding the
-        // row before: one fold after the last byte instead of two. Its
-        // limbs come out of the stages as soon as the consumers have written them, while its first
-        // copies are on their way (measured: later in the stream this costs a quarter microsecond).
-        if constexpr (kLoaderRows > 0) {
-            lds_await(lds_address(&control->staged), kDmaConsumers, patience);
-#pragma unroll
-            for (int m = 0; m < M; m++) load_limbs_unseen(stage[m], lane_id, active, xr[m]);
-        }
         uint32_t landed = 0, in_flight = head;
         if (in_flight > static_cast<uint32_t>(DEPTH)) {  // down to the steady depth
             __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH));
@@ -1112,36 +1071,19 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
             lds_store_unseen(landed_address, ++landed);
             copy(i);
         }
-        // With every copy issued the loader is free: it folds the last kLoaderRows rows of the range
-        // itself, each the moment its last copy has landed.
-        const uint32_t own = min(count, static_cast<uint32_t>(kLoaderRows));
-        uint32_t next_own = count - own;
-        const auto fold_landed = [&](uint32_t have) {
-            if constexpr (kLoaderRows > 0) {
-                while (next_own < count && have >= (((next_own + 1u) * row_bytes + 1023u) >> 10)) {
-                    typename T::Data data;
-                    T::load(range + next_own * row_bytes, lane, data);
-                    fold_row(next_own, data);
-                    next_own += 1u;
-                }
-            }
-        };
         for (uint32_t left = in_flight; left > 0u; left--) {
             wait_copies_in_flight(left - 1u);
             lds_store_unseen(landed_address, ++landed);
-            fold_landed(landed);
         }
-        if constexpr (kLate) {
-            // nothing of this wave is in flight any more: ordinary LDS reads from here on
-            if (late != 0u) {
-                lds_await(lds_address(&control->staged), kDmaConsumers, patience);
+        // nothing of this wave is in flight any more: ordinary LDS reads from here on
+        if (late != 0u) {
+            lds_await(lds_address(&control->staged), kDmaConsumers, patience);
 #pragma unroll
-                for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
-                for (uint32_t r = count - late; r < count; r++) {
-                    typename T::Data data;
-                    T::load(range + r * row_bytes, lane, data);
-                    fold_row(r, data);
-                }
+            for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
+            for (uint32_t r = count - late; r < count; r++) {
+                typename T::Data data;
+                T::load(range + r * row_bytes, lane, data);
+                fold_row(r, data);
             }
         }
         return;
@@ -1161,12 +1103,133 @@ __global__ __launch_bounds__(kDmaThreads) void gemv_limb_dma_kernel(
     // Row r needs the copies that hold bytes [0, (r + 1) * row_bytes) of the range. (Reading row r + 1
     // out of LDS ahead of the fold of row r, when it has landed by then, measured slower: the consumers
     // are bound by their arithmetic, two of them and two loaders to a SIMD, not by LDS latency.)
-    const uint32_t mine = count - (kLate ? late : min(count, static_cast<uint32_t>(kLoaderRows)));  // the last rows are the loader's
+    const uint32_t mine = count - late;  // the last rows are the loader's
     for (uint32_t r = 0; r < mine; r++) {
         lds_await(landed_address, ((r + 1u) * row_bytes + 1023u) >> 10, patience);
         typename T::Data data;
         T::load(range + r * row_bytes, lane, data);
         fold_row(r, data);
+    }
+}
+
+// The same split of the work with the copies taken in turn (the 4-, 5- and 8-bit codecs): the
+// workgroup's share of W is ONE image in LDS, exactly as it lies in memory, whose 1 KiB copies the
+// loaders take in turn (copy i is loader i % LOADERS's), so the image lands front to back at the rate of
+// all loaders together. Rows are not tied to waves: a consumer that is free takes the next row from a
+// counter in LDS, waits until the row's last byte has landed (one poll reads all the loaders' words) and
+// folds it. The loaders do nothing but copy: a launch whose loaders read the staged activations while
+// their first copies are on the way, to fold a row each at the end, measured half a microsecond slower
+// than one whose loaders only copy - and such a launch, with its consumers switched off, runs as fast
+// as the same copies alone (Q4_K 14336 x 4096: 6.2 - 6.6 us). What the launch waits for is its folds:
+// they start when the activations are in registers (1.3 us after the barrier) and then keep the vector
+// ALU busy for about 70 % of the time, so eleven of the sixteen waves fold and five copy, six copies in
+// flight each (8 + 8 x 4: 8.2 - 8.4 us, 11 + 5 x 6: 7.9 - 8.1 on the same box; Q4_0 11008 x 4096: 7.1 -> 6.5).
+template <class T, int M, int CONSUMERS, int LOADERS, int DEPTH>
+__global__ __launch_bounds__(64 * (CONSUMERS + LOADERS)) void gemv_limb_turns_kernel(
+    const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
+    const float* __restrict__ bias, float* __restrict__ y, uint32_t rows, uint32_t columns,
+    uint32_t rows_per_wg, uint32_t spin_limit, uint32_t* timeouts) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr uint32_t kStageAt = kDmaControlAt - M * static_cast<uint32_t>(sizeof(StageMemory));
+    constexpr int kStagers = 8;                            // consumer waves that prepare the activations
+    constexpr int NI = kSliceQuads / (64 * kStagers);      // float4s per such thread and vector
+    static_assert(DEPTH >= 1 && DEPTH <= 8, "wait_copies_in_flight counts to seven");
+    static_assert(CONSUMERS >= kStagers && LOADERS <= kDmaPairs, "eight waves stage; DmaControl has eight loader words");
+    DmaControl* control = reinterpret_cast<DmaControl*>(lds + kDmaControlAt);
+    StageMemory* stage = reinterpret_cast<StageMemory*>(lds + kStageAt);
+    Patience patience{spin_limit, timeouts};  // every wait on another wave is bounded (lds_handover.h)
+
+    const uint32_t lane_id = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wg_row0 = blockIdx.x * rows_per_wg;
+    if (wg_row0 >= rows) return;
+    const uint32_t wg_rows = min(rows_per_wg, rows - wg_row0);
+    const uint32_t row_bytes = static_cast<uint32_t>(T::row_bytes(columns));
+    const uint32_t bytes = wg_rows * row_bytes;
+    const uint32_t chunk = lane_id;  // one slice: the lane's 64-column stretch of the row
+    const bool active = chunk < columns / kChunk;
+    const uint32_t staged_address = lds_address(&control->staged);
+    const uint32_t next_row_address = lds_address(&control->pad[0]);
+
+    if (wave >= static_cast<uint32_t>(CONSUMERS)) {
+        // ---- loaders ------------------------------------------------------------------------
+        const uint32_t loader = wave - CONSUMERS;
+        const uint32_t copies = (bytes + 1023u) >> 10;
+        const uint32_t mine = copies > loader ? (copies - loader + LOADERS - 1u) / LOADERS : 0u;
+        const uint8_t* source = weight + static_cast<uint64_t>(wg_row0) * row_bytes + lane_id * 16u;
+        const uint32_t landed_address = lds_address(&control->landed[loader]);
+        uint32_t at = loader * 1024u;  // of this loader's next copy in the image
+        const auto copy = [&]() {
+            if (at + lane_id * 16u < bytes)  // the last copy of the image stops where the share ends
+                // streamed once: non-temporal (aux bit 1), the caches keep nothing of it
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(source + at),
+                                                 reinterpret_cast<uint4*>(lds + at), 16, 0, 2);
+            at += LOADERS * 1024u;
+        };
+        // The first copies wait for the barrier, i.e. until the consumers have issued their activation
+        // loads: issued ahead of it they delay those loads, and with them every fold.
+        __syncthreads();
+        const uint32_t head = min(mine, static_cast<uint32_t>(DEPTH));
+        for (uint32_t i = 0; i < head; i++) copy();
+        uint32_t landed = 0;
+        for (uint32_t i = head; i < mine; i++) {  // only with DEPTH copies in flight
+            // the oldest copy in flight has landed: say so, then take its place in the queue
+            __builtin_amdgcn_s_waitcnt(vmcnt_only(DEPTH - 1));
+            lds_store_unseen(landed_address, ++landed);
+            copy();
+        }
+        for (uint32_t left = head; left > 0u; left--) {
+            wait_copies_in_flight(left - 1u);
+            lds_store_unseen(landed_address, ++landed);
+        }
+        return;
+    }
+
+    // ---- consumers ------------------------------------------------------------------------------
+    {
+        // Activation loads go first: nothing of the consumers' may queue behind a copy.
+        float4 xv[M][NI];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                const uint32_t quad = threadIdx.x + i * 64u * kStagers;
+                xv[m][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (wave < kStagers && quad < (columns >> 2))
+                    xv[m][i] = reinterpret_cast<const float4*>(x + m * x_row_stride)[quad];
+            }
+        if (threadIdx.x < 16) reinterpret_cast<uint32_t*>(control)[threadIdx.x] = 0u;
+        __syncthreads();  // the only barrier: the counters are zero before anybody counts
+        if (wave < kStagers) {
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int i = 0; i < NI; i++) stage_quad(stage[m], xv[m][i], threadIdx.x + i * 64u * kStagers);
+            lds_arrive(staged_address, lane_id == 0);
+        }
+        if (!lds_await(staged_address, kStagers, patience)) return;
+    }
+
+    // ---- take a row, wait for it, fold it -------------------------------------------------------
+    const typename T::Lane lane = T::lane_setup(active ? chunk : 0u);
+    XLimbs xr[M];
+#pragma unroll
+    for (int m = 0; m < M; m++) T::load_activations(stage[m], lane_id, active, xr[m]);
+    for (;;) {
+        const uint32_t r = lds_take(next_row_address, lane_id == 0);
+        if (r >= wg_rows) break;
+        if (!await_copies_in_turn<LOADERS>(control->landed, lane_id, ((r + 1u) * row_bytes + 1023u) >> 10, patience)) break;
+        typename T::Data data;
+        T::load(lds + r * row_bytes, lane, data);
+        float value[M];
+        T::template fold<M>(data, lane, xr, value);
+        const uint32_t row = wg_row0 + r;
+        const float b = bias != nullptr ? bias[row] : 0.f;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float total = wave_sum(active ? value[m] : 0.f);
+            if (lane_id == 0) y[static_cast<uint64_t>(m) * rows + row] = bias != nullptr ? total + b : total;
+        }
     }
 }
 
@@ -1200,19 +1263,24 @@ hipError_t launch_dma(const uint8_t* weight, const float* x, uint64_t x_row_stri
     int device = 0;
     if (hipError_t status = hipGetDevice(&device)) return status;
     if (device < 0 || device >= 64) return hipErrorInvalidDevice;
-    const auto kernel = gemv_limb_dma_kernel<T, M, kDmaDepth>;
-    if (!allowed[device].load(std::memory_order_acquire)) {
-        if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLdsBytes))
-            return status;
-        allowed[device].store(true, std::memory_order_release);
-    }
     HandoverState handover;
     if (hipError_t status = handover_state(&handover)) return status;
     const uint32_t grid = (rows + rows_per_wg - 1) / rows_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kDmaThreads), kDmaLdsBytes, stream, weight, x, x_row_stride, bias, y,
-                       rows, columns, rows_per_wg, handover.limit, handover.timeouts);
-    return hipGetLastError();
+    const auto go = [&](auto kernel, uint32_t threads) -> hipError_t {
+        if (!allowed[device].load(std::memory_order_acquire)) {
+            if (hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDmaLdsBytes))
+                return status;
+            allowed[device].store(true, std::memory_order_release);
+        }
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), kDmaLdsBytes, stream, weight, x, x_row_stride, bias, y,
+                           rows, columns, rows_per_wg, handover.limit, handover.timeouts);
+        return hipGetLastError();
+    };
+    if constexpr (T::kCopiesInTurn)
+        return go(gemv_limb_turns_kernel<T, M, kTurnConsumers, kTurnLoaders, kTurnDepth>, kDmaThreads);
+    else
+        return go(gemv_limb_dma_kernel<T, M, kDmaDepth>, kDmaThreads);
 }
 
 template <class T, int M, int R, int WAVES, int NK, bool LOOP>

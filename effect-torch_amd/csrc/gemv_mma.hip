@@ -325,23 +325,6 @@ struct Q80Mma {
     }
 };
 
-// Waits until the loaders have brought the first `need` copies of the image (taken in turn: copy i
-// is loader i % LOADERS's). One poll reads all the loaders' words, a lane each.
-template <int LOADERS>
-__device__ __forceinline__ bool await_copies(const Control* control, uint32_t lane_id, uint32_t need, Patience& patience) {
-    const uint32_t loader = lane_id < LOADERS ? lane_id : LOADERS - 1;
-    const uint32_t wanted = need > loader ? (need - loader + LOADERS - 1) / LOADERS : 0u;
-    const uint32_t address = lds_address(&control->landed[loader]);
-    for (uint32_t polls = 0;; polls++) {
-        const uint32_t have = lds_read_unseen(address);
-        if (__builtin_amdgcn_ballot_w64(have < wanted) == 0ull) return true;
-        if (polls >= patience.limit) break;
-        __builtin_amdgcn_s_sleep(1);
-    }
-    patience.give_up();
-    return false;
-}
-
 template <class T, int VG, int LOADERS, int DEPTH, int PROBE = 0>
 __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     const uint8_t* __restrict__ weight, const float* __restrict__ x, uint64_t x_row_stride,
@@ -502,7 +485,7 @@ __global__ __launch_bounds__(64 * (kConsumers + LOADERS)) void gemv_mma_kernel(
     float* partial = reinterpret_cast<float*>(scratch);  // [group][vector group][lane]
     for (uint32_t group = 0; group < groups; group++) {
         const uint32_t last_row = min(group * kGroupRows + kGroupRows, wg_rows) - 1u;
-        const bool landed = await_copies<LOADERS>(control, lane_id, (last_row * pitch + row_bytes + 1023u) >> 10, patience);
+        const bool landed = await_copies_in_turn<LOADERS>(control->landed, lane_id, (last_row * pitch + row_bytes + 1023u) >> 10, patience);
         ET_STAMP(3 + 3 * group);
         float total[VG];
 #pragma unroll

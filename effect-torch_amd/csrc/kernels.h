@@ -282,7 +282,10 @@ hipError_t gather_rows(const void* table, uint64_t table_rows, uint64_t row_byte
 // sink must hold 4 * `workgroups` words; bytes < 2^36.
 hipError_t calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups,
                             hipStream_t stream);
-enum : int { kReadPlain = 0, kReadDeep = 1, kReadStreaming = 2, kReadLds4 = 3, kReadLds8 = 4 };
+enum : int {
+    kReadPlain = 0, kReadDeep = 1, kReadStreaming = 2, kReadLds4 = 3, kReadLds8 = 4, kReadLds8Nt = 5,
+    kReadLds8NtShallow = 6, kReadLds8NtRanges = 7, kReadLds8NtRangesShallow = 8
+};
 hipError_t calibration_read_variant(int variant, const void* src, uint64_t bytes, uint32_t* sink,
                                     uint32_t workgroups, hipStream_t stream);
 hipError_t calibration_copy(const void* src, void* dst, uint64_t bytes, hipStream_t stream);

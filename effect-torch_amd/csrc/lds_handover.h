@@ -59,6 +59,13 @@ __device__ __forceinline__ void lds_arrive(uint32_t address, bool one_lane) {
     if (one_lane) asm volatile("ds_add_u32 %0, %1" : : "v"(address), "v"(1u) : "memory");
 }
 
+// Takes the next number from a counter in LDS (what the word held; the word grows by one). Wave-uniform.
+__device__ __forceinline__ uint32_t lds_take(uint32_t address, bool one_lane) {
+    uint32_t old = 0u;
+    if (one_lane) asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=v"(old) : "v"(address), "v"(1u) : "memory");
+    return __builtin_amdgcn_readfirstlane(old);
+}
+
 // What a wave remembers of its waits.
 struct Patience {
     uint32_t limit;      // polls per wait; 0 once a wait has been abandoned
@@ -74,6 +81,25 @@ struct Patience {
 __device__ __forceinline__ bool lds_await(uint32_t address, uint32_t count, Patience& patience) {
     for (uint32_t polls = 0;; polls++) {
         if (lds_count(address) >= count) return true;
+        if (polls >= patience.limit) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    patience.give_up();
+    return false;
+}
+
+// Waits until the first `need` copies of an image have landed whose copies LOADERS loader waves take in
+// turn (copy i is loader i % LOADERS's; landed[j] counts loader j's). One poll reads all the loaders'
+// words, a lane each. Returns false when the wave gave up.
+template <int LOADERS>
+__device__ __forceinline__ bool await_copies_in_turn(const uint32_t* landed, uint32_t lane_id, uint32_t need,
+                                                     Patience& patience) {
+    const uint32_t loader = lane_id < LOADERS ? lane_id : LOADERS - 1;
+    const uint32_t wanted = need > loader ? (need - loader + LOADERS - 1) / LOADERS : 0u;
+    const uint32_t address = lds_address(&landed[loader]);
+    for (uint32_t polls = 0;; polls++) {
+        const uint32_t have = lds_read_unseen(address);
+        if (__builtin_amdgcn_ballot_w64(have < wanted) == 0ull) return true;
         if (polls >= patience.limit) break;
         __builtin_amdgcn_s_sleep(1);
     }

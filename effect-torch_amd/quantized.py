@@ -589,7 +589,8 @@ def calibration_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, str
                                            sink.data_ptr(), workgroups, _stream_handle(stream)))
 
 
-READ_VARIANTS = {"plain": 0, "deep": 1, "streaming": 2, "lds4": 3, "lds8": 4}
+READ_VARIANTS = {"plain": 0, "deep": 1, "streaming": 2, "lds4": 3, "lds8": 4, "lds8_nt": 5, "lds8_nt_shallow": 6,
+                 "lds8_nt_ranges": 7, "lds8_nt_ranges_shallow": 8}
 
 
 def calibration_read_variant(variant: str, src: torch.Tensor, sink: torch.Tensor, workgroups: int, stream=None) -> None:

@@ -33,8 +33,15 @@ int et_hip_calibration_read(const void* src, uint64_t bytes, uint32_t* sink, uin
  *   ET_READ_STREAMING ET_READ_DEEP with non-temporal loads
  *   ET_READ_LDS_4 / ET_READ_LDS_8   one workgroup of 4 / 8 waves per `workgroups` entry that only issue
  *                     1 KiB global-to-LDS copies (no registers, no arithmetic), each wave keeping
- *                     32 / 16 KiB of copies in flight in a ring of LDS slots. */
-enum { ET_READ_PLAIN = 0, ET_READ_DEEP = 1, ET_READ_STREAMING = 2, ET_READ_LDS_4 = 3, ET_READ_LDS_8 = 4 };
+ *                     32 / 16 KiB of copies in flight in a ring of LDS slots.
+ * ET_READ_LDS_8_NT: ET_READ_LDS_8 with non-temporal copies; _NT_SHALLOW: the same with 4 KiB in
+ *                     flight per wave; _NT_RANGES: every wave copies its own contiguous eighth of the
+ *                     workgroup's range instead of every eighth KiB of it; _NT_RANGES_SHALLOW: both. */
+enum {
+    ET_READ_PLAIN = 0, ET_READ_DEEP = 1, ET_READ_STREAMING = 2, ET_READ_LDS_4 = 3, ET_READ_LDS_8 = 4,
+    ET_READ_LDS_8_NT = 5, ET_READ_LDS_8_NT_SHALLOW = 6, ET_READ_LDS_8_NT_RANGES = 7,
+    ET_READ_LDS_8_NT_RANGES_SHALLOW = 8
+};
 int et_hip_calibration_read_variant(int32_t variant, const void* src, uint64_t bytes, uint32_t* sink,
                                     uint32_t workgroups, void* stream);
 int et_hip_calibration_copy(const void* src, void* dst, uint64_t bytes, void* stream);
