@@ -41,8 +41,12 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # When either differs from what runs now, `roofline.traffic` is null until the profile is re-taken.
 MEASURED_TRAFFIC = {
     ("q4_k_gemv_14336x4096", 1, "f32"): {
-        "bytes": 33315000, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
-        "sha256": "04f8f05ea8735a1c4f7d99d5a64519ec8b5e4cfaae344241ac54612d96a88da2",
+        "bytes": 33284100, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
+        "sha256": "6f805d2b51dcf23f7d33b56f542d357e03b569b6bc7902eec1784db847f25b36",
+        "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
+    ("q4_0_gemv_11008x4096", 1, "f32"): {
+        "bytes": 25614000, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
+        "sha256": "6f805d2b51dcf23f7d33b56f542d357e03b569b6bc7902eec1784db847f25b36",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("q4_k_gemv_14336x4096", 4, "f32"): {
         "bytes": 33895000, "kernel": "gemv_mma", "source": "gemv_mma.hip",
@@ -317,7 +321,7 @@ def calibrate(args, et):
 
 
 def calibrate_read_sweep(args, et):
-    """Workload ``calibrate_read_sweep``: plain reads of 8 MiB ... 1 GiB by five different read kernels
+    """Workload ``calibrate_read_sweep``: plain reads of 8 MiB ... 1 GiB by different read kernels
     (``et_hip_calibration_read_variant``), cold (the buffers of a size rotate through a 2.25 GiB pool),
     each as a HIP-graph replay timed like every other workload; per kernel the launch times are fitted
     to t = t0 + bytes / BW. What this answers: how long a read of the headline weight's 33 MB takes on
@@ -366,7 +370,7 @@ def calibrate_read_sweep(args, et):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(best["measured_us_at_headline_bytes"] * 1e-3, 6), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "calibrate_read_sweep: plain reads of 8 MiB ... 1 GiB by five read kernels, cold, "
+        "config": {"workload": "calibrate_read_sweep: plain reads of 8 MiB ... 1 GiB by read kernels of eleven launch shapes, cold, "
                                "graph replay; fit t = t0 + bytes / BW per kernel",
                    "best_kernel_at_headline_bytes": best["kernel"], "fits": fits, "table": table},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
