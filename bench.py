@@ -145,6 +145,8 @@ def parse_args():
     p.add_argument("--no-decode", action="store_true", help="headline workload: skip the batched-decode leg that fills "
                                                             "the line's `decode` object")
     p.add_argument("--cpu-seconds", type=float, default=10.0)
+    p.add_argument("--waves-per-simd", type=int, default=2, help="calibrate_mfma_*: resident waves per SIMD (one workgroup of "
+                   "four waves per compute unit each)")
     p.add_argument("--sizes-mib", default=None, help="calibrate_read_sweep: comma-separated sizes in MiB instead of "
                    "8 ... 1024 (the headline weight's size is always measured as well)")
     args = p.parse_args()
@@ -438,7 +440,8 @@ def calibrate_mfma(args, et):
     if kind not in et.MFMA_OPERATIONS:
         sys.exit(f"unknown workload {args.workload}; kinds: {sorted(et.MFMA_OPERATIONS)}")
     device = torch.device("cuda:0")
-    workgroups, iterations = 512, 2000  # two workgroups of four waves per compute unit: two waves per SIMD
+    # one workgroup of four waves per compute unit and resident wave per SIMD (two by default)
+    workgroups, iterations = 256 * max(1, args.waves_per_simd), 2000
     sink = torch.zeros(256 * workgroups, dtype=torch.float32, device=device)
     step = lambda i: et.calibration_mfma(kind, iterations, sink)  # noqa: E731
     ms, graphed, wall = time_steps(step, args.steps, args.warmup, not args.no_graph)
@@ -459,7 +462,7 @@ def calibrate_mfma(args, et):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8" if kind.startswith("i8") else "f16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {workgroups} workgroups of four waves, {iterations} rounds of four "
+        "config": {"workload": f"{args.workload}: {workgroups} workgroups of four waves ({workgroups // 256} per SIMD), {iterations} rounds of four "
                                "independent instructions per wave, no memory traffic",
                    "launch": "hipgraph replay of the K steps" if graphed else "K plain enqueues"},
         "roofline": {"bound": "mfma", "achieved": round(tops, 1), "peak": peak, "unit": "TFLOP/s",
