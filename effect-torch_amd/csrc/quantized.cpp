@@ -163,6 +163,18 @@ int select_kernel(et_linear_plan* plan, std::string* error) {
         } else if (gemv_limb_supported(plan->codec, plan->columns, limb_launch)) {
             plan->kernel = LinearKernel::kGemvLimb;
             plan->vectors_per_launch = limb_launch;
+            // One call is vectors / limb_launch launches of limb_launch vectors and one of the rest; a
+            // launch of one vector may take its weights through LDS copies. The name says all of it.
+            const auto launch_name = [&](uint64_t vectors) {
+                return std::string(gemv_limb_copies_through_lds(plan->codec, plan->rows, plan->columns,
+                                                                static_cast<uint32_t>(vectors))
+                                       ? "gemv_limb_dma"
+                                       : "gemv_limb");
+            };
+            const uint64_t whole = plan->vectors / limb_launch, rest = plan->vectors % limb_launch;
+            plan->kernel_label = launch_name(limb_launch);
+            if (whole > 1) plan->kernel_label += " x" + std::to_string(whole);
+            if (rest != 0) plan->kernel_label += "+" + launch_name(rest);
         } else {
             plan->kernel = LinearKernel::kGemvGeneric;
             plan->vectors_per_launch = kGemvGenericMaxVectors;
@@ -265,11 +277,7 @@ bool TensorView::is_contiguous() const {
 const char* kernel_name(const et_linear_plan& plan) {
     switch (plan.kernel) {
         case LinearKernel::kNone: return "none";
-        case LinearKernel::kGemvLimb:
-            return gemv_limb_copies_through_lds(plan.codec, plan.rows, plan.columns,
-                                                static_cast<uint32_t>(plan.vectors_per_launch))
-                       ? "gemv_limb_dma"
-                       : "gemv_limb";
+        case LinearKernel::kGemvLimb: return plan.kernel_label.c_str();
         case LinearKernel::kGemvGeneric: return "gemv_generic";
         case LinearKernel::kGemvMma: return "gemv_mma";
         case LinearKernel::kGemmI8:

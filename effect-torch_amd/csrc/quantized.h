@@ -52,6 +52,7 @@ struct et_linear_plan {
     uint64_t output_bytes;
     et::quantized::LinearKernel kernel;
     uint32_t vectors_per_launch;
+    std::string kernel_label;              // kGemvLimb plans: what the launches of one call are (kernel_name)
     // workspace sections (byte offsets), all 256-byte aligned
     uint64_t gather_offset, gather_bytes;  // densified f32 input
     uint64_t bias_offset;                  // densified f32 bias

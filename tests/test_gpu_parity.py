@@ -675,9 +675,12 @@ def test_k_quant_gemv_at_full_size(et, device, codec, vectors):
     x = synth.random_activations(vectors, columns, rng)
     plan = et.linear_requirements(torch.zeros(vectors, columns), torch.zeros((rows, weight.shape[1]), dtype=torch.uint8),
                                   None, et.GgmlQuant(codec), (rows, columns))
-    copied = vectors == 1 and codec == oracle.Q2_K  # shares of 56 rows that fit LDS
-    one_pass = vectors > 1 and codec == oracle.Q5_K  # 2..8 vectors of Q5_K: the small-batch kernel
-    assert plan.kernel == ("gemv_mma" if one_pass else "gemv_limb_dma" if copied else "gemv_limb")
+    single = "gemv_limb_dma" if codec == oracle.Q2_K else "gemv_limb"  # one vector of Q2_K: shares of 56 rows that fit LDS
+    if vectors > 1 and codec == oracle.Q5_K:
+        expected = "gemv_mma"  # 2..8 vectors of Q5_K: the small-batch kernel
+    else:  # at most two vectors per launch (Q5_K: one vector here), the name lists the launches of a call
+        expected = {1: single, 2: "gemv_limb", 5: "gemv_limb x2+" + single}[vectors]
+    assert plan.kernel == expected
     got = run_linear(et, device, codec, rows, columns, x, weight)
     for start in (0, rows - 128):
         want = oracle.linear_rows(codec, rows, columns, x, weight, None, start, start + 128)[:, start:start + 128]

@@ -66,9 +66,17 @@ def test_linear_plan_shapes(et):
         assert batch.kernel in ("quantize_halves+gemm_h16", "quantize_halves+gemm_h16+reduce")
     plan8 = et.linear_requirements(torch.zeros(10, 512), _w(7, 544), None, et.GgmlQuant.Q8_0, (7, 512))
     assert plan8.kernel in ("quantize_limbs+gemm_i8", "quantize_limbs+gemm_i8+reduce")
-    for few in (3, 6):
+    # the name says what the launches of one call are: three vectors per launch, the rest in one more
+    for few, name in ((3, "gemv_limb"), (6, "gemv_limb x2"), (4, "gemv_limb+gemv_limb"), (5, "gemv_limb+gemv_limb")):
         plan3 = et.linear_requirements(torch.zeros(few, 512), _w(7, 288), None, et.GgmlQuant.Q4_K, (7, 512))
-        assert plan3.kernel == "gemv_limb"
+        assert plan3.kernel == name
+    # a trailing launch of one vector takes its weights through LDS copies where a single vector would
+    tall = et.linear_requirements(torch.zeros(4, 8192), _w(14336, 4608), None, et.GgmlQuant.Q4_K, (14336, 8192))
+    assert tall.kernel == "gemv_limb+gemv_limb", tall.kernel
+    three = et.linear_requirements(torch.zeros(3, 4096), _w(14336, 1344), None, et.GgmlQuant.Q2_K, (14336, 4096))
+    assert three.kernel == "gemv_limb+gemv_limb_dma", three.kernel
+    four = et.linear_requirements(torch.zeros(4, 4096), _w(1024 * 9, 2304), None, et.GgmlQuant.Q4_K, (1024 * 9, 4096))
+    assert four.kernel == "gemv_mma"
     assert plan.algorithmic_bytes == 7 * 288 + 4 * 10 * 512 + 4 * 10 * 7 + 4 * 7
     plan = et.linear_requirements(torch.zeros(1, 256), _w(2, 210), None, et.GgmlQuant.Q6_K, (2, 256))
     assert plan.kernel == "gemv_limb"
