@@ -49,12 +49,12 @@ MEASURED_TRAFFIC = {
         "sha256": "6f805d2b51dcf23f7d33b56f542d357e03b569b6bc7902eec1784db847f25b36",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("q4_k_gemv_14336x4096", 4, "f32"): {
-        "bytes": 33895000, "kernel": "gemv_mma", "source": "gemv_mma.hip",
-        "sha256": "7a5f713f6923c9fcdfce7e5f2ca29da604d0f069669b3f2b769e23a27a7233fa",
+        "bytes": 33895200, "kernel": "gemv_mma", "source": "gemv_mma.hip",
+        "sha256": "f3bf93df89988bc17bec99050bd1b47eecb979a5c848917aad42700dfb58aba2",
         "profile": "profiles/gemv_mma_small_batch_2_to_8_vectors.md"},
     ("q4_k_gemv_14336x4096", 8, "f32"): {
-        "bytes": 34757400, "kernel": "gemv_mma", "source": "gemv_mma.hip",
-        "sha256": "7a5f713f6923c9fcdfce7e5f2ca29da604d0f069669b3f2b769e23a27a7233fa",
+        "bytes": 34754600, "kernel": "gemv_mma", "source": "gemv_mma.hip",
+        "sha256": "f3bf93df89988bc17bec99050bd1b47eecb979a5c848917aad42700dfb58aba2",
         "profile": "profiles/gemv_mma_small_batch_2_to_8_vectors.md"},
     ("kv_attention_decode", 2048): {
         "bytes": 270024900, "kernel": "kv_attend", "source": "kv_attention.hip",
