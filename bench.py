@@ -41,12 +41,12 @@ ROTATE_BYTES = 640 << 20       # > 2x the 256 MB Infinity Cache
 # When either differs from what runs now, `roofline.traffic` is null until the profile is re-taken.
 MEASURED_TRAFFIC = {
     ("q4_k_gemv_14336x4096", 1, "f32"): {
-        "bytes": 33284100, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
-        "sha256": "6f805d2b51dcf23f7d33b56f542d357e03b569b6bc7902eec1784db847f25b36",
+        "bytes": 33283900, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
+        "sha256": "4fa7d816114655dcc55c2445c3543c2c2a4ee75ef28d65d3e37a1ac4883848cb",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("q4_0_gemv_11008x4096", 1, "f32"): {
         "bytes": 25614000, "kernel": "gemv_limb_dma", "source": "gemv_limb.hip",
-        "sha256": "6f805d2b51dcf23f7d33b56f542d357e03b569b6bc7902eec1784db847f25b36",
+        "sha256": "4fa7d816114655dcc55c2445c3543c2c2a4ee75ef28d65d3e37a1ac4883848cb",
         "profile": "profiles/gemv_limb_q4k_14336x4096_m1_hbm_traffic.md"},
     ("q4_k_gemv_14336x4096", 4, "f32"): {
         "bytes": 33895200, "kernel": "gemv_mma", "source": "gemv_mma.hip",

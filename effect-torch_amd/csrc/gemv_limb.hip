@@ -963,8 +963,8 @@ constexpr int kDmaConsumers = kDmaPairs;
 constexpr int kDmaDepth = 4;  // copies a loader keeps in flight: more only lengthen the queue, and a loader says that a
                               // copy has landed only when it may issue the copy DEPTH places later
 constexpr int kDmaHead = kDmaDepth;  // copies a loader issues before it does anything else, at most eight
-                                     // (wait_copies_in_flight). Six and eight measured slower (Q4_K 14336 x 4096:
-                                     // 7.9 and 8.2 against 7.7 us): a longer queue only delays everybody's first rows.
+                                     // (wait_copies_in_flight). Six and eight measured slower when the 4-bit codec ran
+                                     // on this kernel (14336 x 4096: 7.9 and 8.2 against 7.7 us).
 constexpr uint32_t kDmaLateEighths = 2;  // share of a range that a loader which only copies folds at the end
 constexpr int kDmaThreads = 64 * (kDmaConsumers + kDmaPairs);
 constexpr int kTurnConsumers = 11, kTurnLoaders = 5, kTurnDepth = 6;  // gemv_limb_turns_kernel: waves that fold, waves that

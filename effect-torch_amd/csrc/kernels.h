@@ -38,7 +38,8 @@ hipError_t gather_f32(const float* src, const IndexLayout& layout, uint64_t coun
 constexpr uint32_t kGemvLimbMaxVectors = 3;
 uint32_t gemv_limb_max_vectors(int32_t codec);  // per launch: 3, or 2 for Q6_K
 bool gemv_limb_supported(int32_t codec, uint64_t columns, uint32_t vectors);
-// whether that launch runs as gemv_limb_dma_kernel (weights copied through LDS by loader waves)
+// whether that launch takes its weights through LDS copies issued by loader waves
+// (gemv_limb_turns_kernel, or gemv_limb_dma_kernel for the 2-bit codec)
 bool gemv_limb_copies_through_lds(int32_t codec, uint64_t rows, uint64_t columns, uint32_t vectors);
 hipError_t gemv_limb(int32_t codec, const uint8_t* weight, const float* x, uint64_t x_row_stride,
                      const float* bias, float* y, uint64_t rows, uint64_t columns, uint32_t vectors,
